@@ -1,0 +1,148 @@
+/*
+ * tlq.h -- C ABI of libtlq.so: MI355X (gfx950) quantized-matmul kernels.
+ *
+ * Drop-in boundary for the quantized-matmul hot path of tile-ai/tilelang-ascend.  The
+ * reference compiles one shared object per kernel exposing
+ *     extern "C" void call(uint8_t* p0, ..., uint8_t* pn, [int64_t dyn...], aclrtStream stream)
+ * (emitter: src/target/codegen_ascend.cc:1061-1112; ctypes caller:
+ * tilelang/jit/adapter/cython/cython_wrapper.pyx:189-197).  The entry points below keep
+ * that ordering rule -- raw device pointers first, then sizes, then option codes, the
+ * stream last -- with one named symbol per operator instead of one anonymous `call` per
+ * specialisation.
+ *
+ * Conventions
+ *   * all pointers are DEVICE pointers owned by the caller; the library borrows them for
+ *     the duration of the (asynchronous) launch and never allocates or frees memory;
+ *   * `stream` is a hipStream_t passed as void* (NULL = the legacy default stream);
+ *   * return value 0 = launched; non-zero = rejected before launch, with the reason
+ *     available from tlq_last_error() (thread local).  This is the
+ *     `int init()/const char* get_last_error()` protocol the reference declares in
+ *     tilelang/jit/adapter/wrapper.py:30-50 but leaves unwired for its NPU backend
+ *     (tilelang/jit/adapter/cython/adapter.py:269-275);
+ *   * packed int4 weights are uint8 [N, K/2]: element k of row n is nibble (k % 2) of byte
+ *     k / 2, low nibble first (examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:27-29,
+ *     tilelang/quantize/utils.py:64-67);
+ *   * per-group scales / zeros are [N, K/group] in the activation dtype.
+ */
+#ifndef TLQ_H_
+#define TLQ_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TLQ_ABI_VERSION 1
+
+/* element type codes */
+enum {
+  TLQ_F16 = 0,
+  TLQ_BF16 = 1,
+  TLQ_F32 = 2,
+  TLQ_I8 = 3,
+  TLQ_I32 = 4
+};
+
+/* int4 sign conventions (how a nibble u in 0..15 becomes an integer) */
+enum {
+  TLQ_U4 = 0,        /* u            tilelang/quantize/quantization.py:198-206; fine_grained.py:10-57 */
+  TLQ_S4_TWOS = 1,   /* u>=8 ? u-16 : u   quantization.py:221-231; example_dequant_gemm_w4a8.py:124-145 */
+  TLQ_S4_OFFSET8 = 2,/* u - 8        quantization.py:186-195; lop3.py:14 (isSigned) */
+  TLQ_S4_OFFSET7 = 3 /* u - 7        quantization.py:56-65 */
+};
+
+/* layout of the second GEMM operand */
+enum {
+  TLQ_B_KN = 0, /* B[K, N] row-major (example_quant_batch_matmul.py:39, fine_grained.py:85) */
+  TLQ_B_NK = 1  /* B[N, K] row-major, i.e. transpose_B (examples/deepseek_v4/int8_gemm.py:58,77) */
+};
+
+/* kernel selection for tlq_gemm_w4a16 */
+enum {
+  TLQ_ALGO_AUTO = 0,
+  TLQ_ALGO_GEMV = 1, /* split-K wavefront GEMV (M <= 16) */
+  TLQ_ALGO_MFMA = 2  /* LDS-staged MFMA dequant-GEMM */
+};
+
+int tlq_abi_version(void);
+const char* tlq_last_error(void);
+
+/* Number of compute units of the current device (0 on failure). */
+int tlq_device_cu_count(void);
+
+/* Nibble unpack, replaces torch_unpack_uint4_to_fp16 / torch_unpack_uint4_to_int8
+ * (example_dequant_gemm_fine_grained.py:10-57), torch_convert (example_dequant_gemm_w4a8.py:124-145)
+ * and the vector-core unpack of w4a8_gemm_cv (:69-106).
+ * out[n, k] = convert(sign_mode, nibble) as out_dtype (TLQ_F16 / TLQ_BF16 / TLQ_I8).  K even. */
+int tlq_unpack_int4(const void* w_packed, void* out, int64_t N, int64_t K, int out_dtype, int sign_mode, void* stream);
+
+/* Per-group dequantisation W[n,k] = rn_T( rn_T(T(u) - T(z)) * s ), T = dtype (TLQ_F16 / TLQ_BF16):
+ * the "original" zeros mode of tilelang/quantize/lop3.py:135-175 and gen_quant4's
+ * ref = (q - 8).half() * s (tilelang/quantize/utils.py:33).
+ * scales: [N, K/group] or NULL (=1).  zeros: [N, K/group] or NULL (then zero_scalar is used).
+ * group must divide K and be even. */
+int tlq_dequant_w4(const void* w_packed, const void* scales, const void* zeros, void* out, int64_t N, int64_t K,
+                   int64_t group, float zero_scalar, int dtype, void* stream);
+
+/* Fused weight-only GEMM / GEMV, replaces dequant_gemm_fp16_wrapper + fp16_gemm
+ * (example_dequant_gemm_fine_grained.py:60-115,176-223) extended with per-group scale / zero:
+ *   C[M,N] = rn_out( sum_k f32(A[m,k]) * f32(W[n,k]) ),  W as in tlq_dequant_w4, fp32 accumulate.
+ * A: [M,K] in_dtype (TLQ_F16 / TLQ_BF16); C: [M,N] out_dtype (TLQ_F16 / TLQ_BF16 / TLQ_F32).
+ * Requires K % 64 == 0 and group % 32 == 0 (group divides K). */
+int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
+                   int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
+                   void* stream);
+
+/* `batch` independent decode GEMVs in one launch (one grid row per problem): A [batch,M,K],
+ * w_packed [batch,N,K/2], scales / zeros [batch,N,K/group], C [batch,M,N], all contiguous.
+ * Same arithmetic as tlq_gemm_w4a16 with TLQ_ALGO_GEMV; M <= 16.  This is the shape of a decode
+ * step that applies many weight-only-quantized projections (layers, experts) of one size; the
+ * reference has no batched form of its GEMV (examples/gemv/example_gemv_c.py:27-46 is one
+ * vector x one matrix), its batched operators are examples/batch_gemm/batch_gemm.py:28-60 and
+ * quant_batch_matmul. */
+int tlq_gemv_w4a16_batched(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C,
+                           int64_t batch, int64_t M, int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype,
+                           int out_dtype, void* stream);
+
+/* Plain fp16 / bf16 GEMM with fp32 accumulate, replaces fp16_gemm
+ * (example_dequant_gemm_fine_grained.py:60-115): C[M,N] = A[M,K] . B, B laid out per b_layout. */
+int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
+                 int b_layout, void* stream);
+
+/* int8 x int8 -> int32 GEMM (bit exact), replaces int8_gemm
+ * (example_dequant_gemm_fine_grained.py:118-173); batched when batch > 1 (A [B,M,K], B [B,K,N] or
+ * [B,N,K], C [B,M,N]). */
+int tlq_gemm_i8(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,
+                void* stream);
+
+/* int8 activations x packed int4 weights -> int32, replaces w4a8_gemm_cv
+ * (example_dequant_gemm_w4a8.py:25-121) and dequant_gemm_int8_wrapper
+ * (example_dequant_gemm_fine_grained.py:226-266): C[M,N] = A[M,K] . convert(sign_mode, Wp)[N,K]^T.
+ * The reference's caller-supplied int8 [N,K] workspace is not needed (unpack is fused). */
+int tlq_gemm_w4a8(const void* A, const void* w_packed, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
+                  void* stream);
+
+/* W8A8 matmul with fused rescale epilogue, replaces simple_quant_batch_matmul
+ * (examples/quant_batch_matmul/example_quant_batch_matmul.py:8-91), simple_quant_matmul
+ * (example_quant_matmul.py:8-90) and int8_gemm_kernel_corrected
+ * (examples/deepseek_v4/int8_gemm.py:25-104):
+ *   acc = A[b] . B[b]            (int32, exact)
+ *   C   = rn_out( rn_f32( rn_f32(f32(acc) * scale_a[b,m]) * scale_b[n] ) )
+ * scale_a: fp32 [batch*M] or NULL (skipped).  scale_b: fp32 [n_scale_b], n_scale_b = 1 (per
+ * tensor) or N (per channel), or NULL.  The reference's int32 [B,M,N] workspace round trip
+ * (:42,66-68) is fused away. */
+int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
+                  int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, void* stream);
+
+/* Tuning hooks for benchmark sweeps (process-global, not thread safe; 0 = automatic choice).
+ * They play the role of the reference's block_M / block_N / block_K factory arguments
+ * (example_dequant_gemm_fine_grained.py:437,462), which here select among pre-built tilings. */
+void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4, waves 1..4 */
+void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256|512 (512 = 256x256, 8 waves) */
+void tlq_tune_i8_tile(int block_m);                         /* 32|128|256 */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TLQ_H_ */

@@ -1,0 +1,381 @@
+"""TEST INFRASTRUCTURE ONLY -- numpy / torch-CPU restatement of the reference arithmetic.
+
+Every function cites the reference lines it follows (paths relative to the reference
+checkout).  The restatement is written from the reference's source text; the
+reference itself cannot be imported (it needs TVM and torch_npu).
+
+What pins each function (so that a dropped term, wrong nibble order or transposed
+operand fails a test):
+
+* unpack_uint4 / torch_unpack_uint4_to_{fp16,int8}: the reference's own known-answer
+  vector [[0x12, 0x34]] -> [2, 1, 4, 3]; the literal per-element loop on small shapes;
+  an exhaustive 256-byte x 2-position table; the independent C restatement (oracle.c).
+* torch_convert (two's-complement int4): exhaustive table; round trip with
+  generate_quantized_weight; C restatement.
+* general_compress: inverse of the unpackers; brute force on tiny shapes.
+* interleave_weight (nbits=4): explicit permutation tables e0,e2,e4,e6,e1,e3,e5,e7
+  (fp16) and e0,e4,e1,e5,e2,e6,e3,e7 (int8).  The 1-bit / 2-bit special branches call
+  ``torch.int32(...)`` in the reference, which raises; they are restated by intent and
+  are PARITY UNPINNED.
+* gen_quant4: invariants only (ref == (q-8).half()*s, shapes, ranges, seed
+  reproducibility) -- the random stream itself is torch's.
+* dequant_w4 (per-group scale / zero): float64 evaluation followed by one correctly
+  rounded conversion per operation (C restatement uses a different rounding routine).
+* int8 matmuls: exact int64 brute force on small shapes, float64 matmul (exact below
+  2**53) on large ones, the closed form for constant inputs.
+* rescale epilogues: pure functions of (acc, scale) -- compared with a float64
+  evaluation rounded once.
+* lop3 decoders: closed forms (u-8 for signed, (u-z)*s, fma(u,s,-z), (u-qz)*s).
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+TORCH_DTYPE = {
+    "float16": torch.float16,
+    "bfloat16": torch.bfloat16,
+    "float32": torch.float32,
+    "int8": torch.int8,
+    "int32": torch.int32,
+}
+
+
+def _np_u8(t) -> np.ndarray:
+    if isinstance(t, torch.Tensor):
+        t = t.cpu()
+        if t.dtype == torch.int8:
+            t = t.view(torch.uint8)
+        return t.numpy()
+    a = np.asarray(t)
+    return a.view(np.uint8) if a.dtype == np.int8 else a
+
+
+# --------------------------------------------------------------------------------------
+# U1 / U2: unsigned nibble unpack
+# --------------------------------------------------------------------------------------
+def unpack_uint4_loop(packed, out_dtype=torch.float16) -> torch.Tensor:
+    """Literal per-element loop of examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:10-32
+    (fp16) and :35-57 (int8).  N*K Python iterations: small inputs only."""
+    assert packed.dtype == torch.uint8
+    N, K_packed = packed.shape
+    K = K_packed * 2
+    result = torch.empty(N, K, dtype=out_dtype)
+    for i in range(N):
+        for j in range(K):
+            val = packed[i, j // 2].item()
+            pos = j % 2
+            u4 = (val >> (pos * 4)) & 0xF
+            result[i, j] = float(u4) if out_dtype.is_floating_point else u4
+    return result
+
+
+def unpack_uint4(packed) -> np.ndarray:
+    """Vectorised form of the same loop: element k of row n is nibble (k % 2) of byte k // 2,
+    low nibble first.  Returns uint8 values 0..15, shape [..., 2*K_packed]."""
+    p = _np_u8(packed)
+    out = np.empty(p.shape[:-1] + (p.shape[-1] * 2,), dtype=np.uint8)
+    out[..., 0::2] = p & 0xF
+    out[..., 1::2] = p >> 4
+    return out
+
+
+def torch_unpack_uint4_to_fp16(tensor: torch.Tensor) -> torch.Tensor:
+    """example_dequant_gemm_fine_grained.py:10-32, vectorised."""
+    assert tensor.dtype == torch.uint8
+    return torch.from_numpy(unpack_uint4(tensor).astype(np.float16))
+
+
+def torch_unpack_uint4_to_int8(tensor: torch.Tensor) -> torch.Tensor:
+    """example_dequant_gemm_fine_grained.py:35-57, vectorised."""
+    assert tensor.dtype == torch.uint8
+    return torch.from_numpy(unpack_uint4(tensor).astype(np.int8))
+
+
+# --------------------------------------------------------------------------------------
+# U3 / P4: two's-complement signed int4
+# --------------------------------------------------------------------------------------
+def torch_convert_loop(tensor: torch.Tensor) -> torch.Tensor:
+    """Literal loop of examples/dequantize_gemm/example_dequant_gemm_w4a8.py:124-145."""
+
+    def _convert(val, pos):
+        assert val.dtype == torch.uint8
+        val = val.view(torch.int8)
+        mask = (1 << 4) - 1
+        i4_shifted = (val >> (pos * 4)) & mask
+        i4 = (i4_shifted << 4) >> 4
+        return i4.view(torch.int8)
+
+    N, K = tensor.shape
+    new_tensor = torch.empty(N, K * 2, dtype=torch.int8)
+    for i in range(N):
+        for j in range(K * 2):
+            new_tensor[i][j] = _convert(tensor[i][j // 2], j % 2)
+    return new_tensor
+
+
+def torch_convert(tensor) -> torch.Tensor:
+    """Vectorised example_dequant_gemm_w4a8.py:124-145: nibble -> sign-extended int8 (-8..7)."""
+    u = unpack_uint4(tensor).astype(np.int16)
+    return torch.from_numpy(np.where(u >= 8, u - 16, u).astype(np.int8))
+
+
+def generate_quantized_weight(N: int, K: int, generator: torch.Generator | None = None):
+    """example_dequant_gemm_w4a8.py:156-165 with the loop vectorised:
+    qB[n, j] = (B[n, 2j+1] & 15) << 4 | (B[n, 2j] & 15)."""
+    B_int8 = torch.randint(-8, 8, (N, K), dtype=torch.int8, generator=generator)
+    b = B_int8.numpy().view(np.uint8)
+    qB = ((b[:, 1::2] & 0xF) << 4) | (b[:, 0::2] & 0xF)
+    return torch.from_numpy(qB.astype(np.uint8)), B_int8
+
+
+# --------------------------------------------------------------------------------------
+# Q1..Q5: tilelang.quantize element converters, restated on integer arrays
+# --------------------------------------------------------------------------------------
+def _field(val, pos, nbit):
+    v = np.asarray(val).astype(np.int64) & 0xFFFFFFFF
+    return (v >> (np.asarray(pos).astype(np.int64) * nbit)) & ((1 << nbit) - 1)
+
+
+def packed_to_unsigned(val, pos, nbit=4):
+    """tilelang/quantize/quantization.py:198-206: (val >> pos*nbit) & mask."""
+    return _field(val, pos, nbit)
+
+
+def packed_to_unsigned_with_zeros(val, pos, zero, nbit=4):
+    """quantization.py:209-218: ((val >> pos*nbit) & mask) - zero, exact integer subtraction."""
+    return _field(val, pos, nbit) - np.asarray(zero).astype(np.int64)
+
+
+def packed_to_signed_offset(val, pos, nbit=4):
+    """quantization.py:186-195: offset-binary, u - 2**(nbit-1)."""
+    return _field(val, pos, nbit) - (1 << (nbit - 1))
+
+
+def packed_int_to_int(val, pos, nbit=4):
+    """quantization.py:221-231 (and :68-78): two's-complement sign extension of the field."""
+    u = _field(val, pos, nbit)
+    return np.where(u >= (1 << (nbit - 1)), u - (1 << nbit), u)
+
+
+def packed_uint_to_uint_to_float(val, pos, nbit=4):
+    """quantization.py:56-65: u - (2**(nbit-1) - 1)."""
+    return _field(val, pos, nbit) - ((1 << (nbit - 1)) - 1)
+
+
+# --------------------------------------------------------------------------------------
+# P1..P3: tilelang/quantize/utils.py
+# --------------------------------------------------------------------------------------
+def general_compress(lowprecision_weight: torch.Tensor, source_bits=4, storage_dtype=None) -> torch.Tensor:
+    """tilelang/quantize/utils.py:53-69.  out[..., j] |= (w[..., j*epb+k] << bits*k) truncated to
+    8 bits, accumulated in int8, then cast to storage_dtype."""
+    if storage_dtype is None:
+        storage_dtype = torch.int8
+    epb = 8 // source_bits
+    w = lowprecision_weight
+    if w.dtype == torch.float16:
+        w = w.to(torch.int8)
+    a = w.cpu().numpy().astype(np.int64)
+    out = np.zeros(a.shape[:-1] + (a.shape[-1] // epb,), dtype=np.int64)
+    for k in range(epb):
+        out |= (a[..., k::epb][..., : out.shape[-1]] << (source_bits * k)) & 0xFF
+    return torch.from_numpy(out.astype(np.uint8).view(np.int8).copy()).to(storage_dtype)
+
+
+def interleave_weight(qweight: torch.Tensor, nbits=4, target_dtype="float16") -> torch.Tensor:
+    """tilelang/quantize/utils.py:73-126.  Per 32-bit word, field i moves to bit
+    (i % G) * stride + (i // G) * nbits with stride 16 (fp16) / 8 (int8), G = 32 // stride."""
+    assert target_dtype in ["float16", "int8"]
+    q = qweight.cpu().contiguous().view(torch.int32).numpy().view(np.uint32)
+    new = np.zeros_like(q)
+    stride = 8 if target_dtype == "int8" else 16
+    mask = np.uint32((1 << nbits) - 1)
+    G = 32 // stride
+    per = stride // nbits
+    for i in range(G):
+        for j in range(per):
+            off = i * per + j
+            shift = (off % G) * stride + (off // G) * nbits
+            new |= ((q >> np.uint32(nbits * off)) & mask) << np.uint32(shift)
+
+    def mv(x, m, down, up):
+        return ((x & np.uint32(m)) >> np.uint32(down)) << np.uint32(up)
+
+    # The three special branches below are restated by intent (utils.py:103-124); the
+    # reference text calls torch.int32(...) there, which is not callable.  PARITY UNPINNED.
+    if nbits == 1 and target_dtype == "int8":
+        r = new & np.uint32(0xF0F00F0F)
+        r |= mv(new, 0x000000F0, 4, 16) | mv(new, 0x0000F000, 12, 24)
+        r |= mv(new, 0x000F0000, 16, 4) | mv(new, 0x0F000000, 24, 12)
+        new = r
+    elif nbits == 2 and target_dtype == "float16":
+        r = new & np.uint32(0xFF0000FF)
+        r |= mv(new, 0x0000FF00, 8, 16) | mv(new, 0x00FF0000, 16, 8)
+        new = r
+    elif nbits == 1 and target_dtype == "float16":
+        r = new & np.uint32(0xF000000F)
+        r |= mv(new, 0x000000F0, 4, 8) | mv(new, 0x00000F00, 8, 16) | mv(new, 0x0000F000, 12, 24)
+        r |= mv(new, 0x000F0000, 16, 4) | mv(new, 0x00F00000, 20, 12) | mv(new, 0x0F000000, 24, 20)
+        new = r
+    return torch.from_numpy(new.view(np.int32).copy()).view(torch.int8)
+
+
+def gen_quant4(k, n, groupsize=-1):
+    """tilelang/quantize/utils.py:5-50, same torch calls in the same order (so the same seed
+    gives the same stream).  Note maxq = 16 and the clamp to [0, 16] (sic)."""
+    import torch.nn as nn
+
+    maxq = 2**4
+    w = torch.randn((k, n), dtype=torch.half, device="cpu")
+    original_w = w.clone()
+    if groupsize == -1:
+        groupsize = k
+    w = w.reshape((-1, groupsize, n)).permute(1, 0, 2).reshape((groupsize, -1))
+    s = torch.max(torch.abs(w), 0, keepdim=True)[0]
+    s *= 2 / maxq
+    w = torch.round(w / s).int()
+    w += maxq // 2
+    w = torch.clamp(w, 0, maxq)
+    ref = (w - maxq // 2).half() * s
+
+    def reshape(x):
+        return x.reshape((groupsize, -1, n)).permute(1, 0, 2).reshape((k, n)).contiguous()
+
+    ref = reshape(ref)
+    w = reshape(w)
+    s = s.reshape((-1, n)).contiguous()
+    linear = nn.Linear(k, n, bias=False)
+    linear.weight.data = ref.t()
+    return original_w, linear, s, (w - maxq // 2)
+
+
+# --------------------------------------------------------------------------------------
+# Per-group dequantisation: W[n,k] = rn_T( rn_T(T(u) - T(z[n,k//g])) * s[n,k//g] )
+# ("original" zeros mode of tilelang/quantize/lop3.py:135-175: sub.f16x2 then fma.rn.f16x2
+#  with a zero addend; gen_quant4's ref = (q-8).half()*s, utils.py:33)
+# --------------------------------------------------------------------------------------
+def dequant_w4(B_packed, scales=None, zeros=None, group_size=128, dtype=torch.float16) -> torch.Tensor:
+    """scales: [N, K/g] tensor of dtype T or None (=1).  zeros: None (=0), a python number, or a
+    [N, K/g] tensor of dtype T.  Each arithmetic step rounds to T (torch CPU half/bfloat16
+    arithmetic computes in fp32 and rounds once per operation, which equals native rounding)."""
+    u = torch.from_numpy(unpack_uint4(B_packed).astype(np.float32)).to(dtype)
+    N, K = u.shape
+    if zeros is not None:
+        if isinstance(zeros, torch.Tensor):
+            z = zeros.cpu().to(dtype).repeat_interleave(group_size, dim=1)
+            assert z.shape == (N, K)
+        else:
+            z = torch.tensor(float(zeros), dtype=dtype)
+        u = u - z
+    if scales is not None:
+        s = scales.cpu().to(dtype).repeat_interleave(group_size, dim=1)
+        assert s.shape == (N, K)
+        u = u * s
+    return u
+
+
+def ref_program_w4a16(A, B_packed, scales=None, zeros=None, group_size=128, output_dtype="float16"):
+    """ref_program_fp16 (example_dequant_gemm_fine_grained.py:269-289) extended with the group
+    dequant above: (A.f32 @ W.f32.T).to(out).  A is NOT down-cast (line :283)."""
+    W = dequant_w4(B_packed, scales, zeros, group_size, A.dtype)
+    C = torch.matmul(A.cpu().to(torch.float32), W.to(torch.float32).T)
+    return C.to(TORCH_DTYPE[output_dtype])
+
+
+def ref_program_fp16(A, B_packed, output_dtype):
+    """example_dequant_gemm_fine_grained.py:269-289 (vectorised unpack)."""
+    B_fp16 = torch_unpack_uint4_to_fp16(B_packed)
+    C = torch.matmul(A.to(torch.float32), B_fp16.to(torch.float32).T)
+    return C.to(TORCH_DTYPE[output_dtype])
+
+
+def ref_program_fp16_loop(A, B_packed, output_dtype):
+    """Same, with the literal per-element unpack loop (small shapes only)."""
+    B_fp16 = unpack_uint4_loop(B_packed, torch.float16)
+    C = torch.matmul(A.to(torch.float32), B_fp16.to(torch.float32).T)
+    return C.to(TORCH_DTYPE[output_dtype])
+
+
+# --------------------------------------------------------------------------------------
+# Integer matmuls
+# --------------------------------------------------------------------------------------
+def int_matmul_exact(A, B) -> torch.Tensor:
+    """Exact integer A @ B through float64 (every partial sum is an integer < 2**53).
+    Batched when the inputs are 3-D.  Returns int64."""
+    return torch.matmul(A.cpu().to(torch.float64), B.cpu().to(torch.float64)).to(torch.int64)
+
+
+def ref_program_int8(A, B_packed, output_dtype):
+    """example_dequant_gemm_fine_grained.py:292-312: (A.i32 @ U2(Wp).i32.T).to(out)."""
+    B_int8 = torch_unpack_uint4_to_int8(B_packed)
+    C = int_matmul_exact(A, B_int8.T).to(torch.int32)
+    return C.to(TORCH_DTYPE[output_dtype])
+
+
+def ref_program_w4a8(A, qB):
+    """example_dequant_gemm_w4a8.py:148-153: returns the TRANSPOSE [N, M] (int32)."""
+    B = torch_convert(qB)
+    C = torch.matmul(A.cpu().to(torch.float), B.T.to(torch.float)).to(torch.int32)
+    return C.transpose(0, 1)
+
+
+def ref_program_quant(A, B, scale, out_dtype, accum_dtype=torch.int32, literal=False):
+    """examples/quant_batch_matmul/example_quant_batch_matmul.py:93-95 and
+    example_quant_matmul.py:92-94: ((A.acc @ B.acc).to(scale.dtype) * scale).to(out).
+    literal=True runs torch's own integer matmul (slow); otherwise the exact float64 route."""
+    if literal:
+        C = A.cpu().to(accum_dtype) @ B.cpu().to(accum_dtype)
+    else:
+        C = int_matmul_exact(A, B).to(accum_dtype)
+    return (C.to(scale.dtype) * scale.cpu()).to(out_dtype)
+
+
+def ref_int8_gemm_sequential(A, B_nk, scale_a, scale_b, out_dtype):
+    """Kernel order of examples/deepseek_v4/int8_gemm.py:95-102: cast acc to fp32 (RINT),
+    multiply by scale_a[m], then by scale_b[n] (two fp32 roundings), cast to out (RINT)."""
+    acc = int_matmul_exact(A, B_nk.transpose(-1, -2)).to(torch.int32)
+    c = acc.to(torch.float32)
+    c = c * scale_a.cpu().reshape(*scale_a.shape[: A.dim() - 1], 1).to(torch.float32)
+    c = c * scale_b.cpu().reshape(-1).to(torch.float32)
+    return c.to(out_dtype)
+
+
+def int8_gemm_torch_optimized(a_int8, a_scales, b_int8, b_scales, out_dtype=torch.float32):
+    """Golden of examples/deepseek_v4/int8_gemm.py:108-139: fp32 matmul times outer(a_s, b_s).
+    The fp32 matmul is inexact for full-range int8 at large K -- a tolerance oracle only."""
+    shape = a_int8.shape
+    a2 = a_int8.reshape(-1, shape[-1]).to(torch.float32)
+    out = torch.matmul(a2, b_int8.to(torch.float32).T)
+    out = out * torch.outer(a_scales.reshape(-1), b_scales.reshape(-1))
+    if out_dtype == torch.bfloat16:
+        out = out.bfloat16()
+    return out.view(*shape[:-1], b_int8.shape[0])
+
+
+# --------------------------------------------------------------------------------------
+# Q6: closed forms of the lop3 decoders (tilelang/quantize/lop3.py:5-421), 4-bit -> fp16
+# --------------------------------------------------------------------------------------
+LOP3_F16_ORDER = (0, 4, 1, 5, 2, 6, 3, 7)  # output slot j holds field LOP3_F16_ORDER[j] of the u32
+
+
+def lop3_decode_i4_to_f16(words_u32, signed=False, scale=None, zeros=None, zeros_mode=None):
+    """One u32 -> 8 fp16.  h[i] (a half2) = fields (i, i+4) of the word (lop3.py:17-24), so the
+    flat output order is field 0,4,1,5,2,6,3,7: the weights must have been passed through
+    interleave_weight for the flat order to be the logical one.  signed subtracts 8 (:14).
+    zeros_mode: None | 'original' (u - z) * s (:165-166) | 'rescale' fma(u, s, -z) (:247,260) |
+    'quantized' (u - qz) * s with integer qz (:340,351-353)."""
+    w = np.asarray(words_u32, dtype=np.uint32).reshape(-1)
+    f = np.stack([(w >> np.uint32(4 * i)) & np.uint32(0xF) for i in LOP3_F16_ORDER], axis=1)
+    h = f.astype(np.float16)
+    if signed:
+        h = h - np.float16(8)
+    if zeros_mode in ("original", "quantized"):
+        h = (h - np.float16(zeros)).astype(np.float16)
+    if scale is not None:
+        if zeros_mode == "rescale":
+            h = (h.astype(np.float64) * np.float64(np.float16(scale)) - np.float64(np.float16(zeros))).astype(
+                np.float16
+            )
+        else:
+            h = (h * np.float16(scale)).astype(np.float16)
+    return h

@@ -1,0 +1,93 @@
+"""ctypes binding of libtlq.so (the C ABI declared in include/tlq.h).
+
+Plays the part of the reference's ``lib.call(*void_ptrs, [dyn ints], stream)`` step
+(tilelang/jit/adapter/cython/cython_wrapper.pyx:189-197): raw device pointers first, sizes
+after, the stream last.  There is no CPU fallback: if the library cannot be loaded the
+operators raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+from . import build as _build
+
+# type codes of include/tlq.h
+F16, BF16, F32, I8, I32 = 0, 1, 2, 3, 4
+U4, S4_TWOS, S4_OFFSET8, S4_OFFSET7 = 0, 1, 2, 3
+B_KN, B_NK = 0, 1
+ALGO_AUTO, ALGO_GEMV, ALGO_MFMA = 0, 1, 2
+ABI_VERSION = 1
+
+_vp, _i64, _int, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+
+# name -> (restype, argtypes); kept in step with include/tlq.h (a test compares the two)
+SIGNATURES = {
+    "tlq_abi_version": (_int, []),
+    "tlq_last_error": (ctypes.c_char_p, []),
+    "tlq_device_cu_count": (_int, []),
+    "tlq_unpack_int4": (_int, [_vp, _vp, _i64, _i64, _int, _int, _vp]),
+    "tlq_dequant_w4": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _int, _vp]),
+    "tlq_gemm_w4a16": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp]),
+    "tlq_gemv_w4a16_batched": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _int, _int, _vp]),
+    "tlq_gemm_f16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int, _vp]),
+    "tlq_gemm_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "tlq_gemm_w4a8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "tlq_tune_gemv": (None, [_int, _int]),
+    "tlq_tune_w4a16_tile": (None, [_int]),
+    "tlq_tune_i8_tile": (None, [_int]),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+def library_path() -> str:
+    return os.environ.get("TLQ_LIBRARY", _build.LIB_PATH)
+
+
+def load():
+    """Load libtlq.so once per process (mutex; the reference guards its library cache the same
+    way, tilelang/jit/adapter/cython/adapter.py:79-98).  Builds it when it is absent and hipcc
+    is available; otherwise raises -- there is no other implementation to fall back to."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = library_path()
+        if not os.path.exists(path):
+            try:
+                path = _build.build_library(force=True)
+            except Exception as e:  # noqa: BLE001
+                raise RuntimeError(
+                    f"libtlq.so not found at {path} and could not be built ({e}); "
+                    "run `python -m tilelang_ascend_amd.build`"
+                ) from e
+        lib = ctypes.CDLL(path)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        if lib.tlq_abi_version() != ABI_VERSION:
+            raise RuntimeError(f"libtlq.so ABI version {lib.tlq_abi_version()} != expected {ABI_VERSION}")
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    msg = load().tlq_last_error()
+    return msg.decode() if msg else ""
+
+
+def check(rc: int) -> None:
+    """Non-zero return -> RuntimeError carrying the library's message."""
+    if rc != 0:
+        raise RuntimeError(last_error() or f"libtlq call failed with code {rc}")
+
+
+def ptr(t) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())

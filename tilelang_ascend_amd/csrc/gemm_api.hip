@@ -1,0 +1,136 @@
+// extern "C" entry points of the GEMM family: argument validation, then dispatch.
+// Every shape assumption a kernel makes is checked here, before anything is launched.
+#include "tlq_common.h"
+
+namespace tlq {
+int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch, int64_t M,
+               int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
+int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                    int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
+int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
+                   int b_layout, hipStream_t st);
+int gemm_i8_i32(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,
+                hipStream_t st);
+int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
+                      int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, hipStream_t st);
+int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
+                  hipStream_t st);
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+static const int64_t kMaxDim = (int64_t)1 << 30;
+}  // namespace tlq
+
+using namespace tlq;
+
+#define TLQ_CHECK_DIMS(name)                                                                                      \
+  TLQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim, name ": bad shape M=%lld N=%lld K=%lld", \
+              (long long)M, (long long)N, (long long)K)
+
+extern "C" {
+
+int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
+                   int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
+                   void* stream) {
+  TLQ_CHECK_DIMS("tlq_gemm_w4a16");
+  TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_w4a16: in_dtype must be float16 or bfloat16 (got %d)",
+              in_dtype);
+  TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32,
+              "tlq_gemm_w4a16: out_dtype must be float16, bfloat16 or float32 (got %d)", out_dtype);
+  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_MFMA, "tlq_gemm_w4a16: bad algo %d", algo);
+  if (M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(K > 0 && K % 64 == 0, "tlq_gemm_w4a16: K=%lld must be a positive multiple of 64", (long long)K);
+  TLQ_REQUIRE(group > 0 && K % group == 0 && group % 32 == 0,
+              "tlq_gemm_w4a16: group=%lld must divide K=%lld and be a multiple of 32", (long long)group, (long long)K);
+  TLQ_REQUIRE(A && w_packed && C, "tlq_gemm_w4a16: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(w_packed) && aligned16(C), "tlq_gemm_w4a16: A, w_packed and C must be 16-byte aligned");
+  TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16: scales / zeros misaligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (algo == TLQ_ALGO_AUTO) algo = (M <= 4) ? TLQ_ALGO_GEMV : TLQ_ALGO_MFMA;
+  if (algo == TLQ_ALGO_GEMV) {
+    TLQ_REQUIRE(M <= 16, "tlq_gemm_w4a16: the GEMV kernel handles M <= 16 (got %lld)", (long long)M);
+    return gemv_w4a16(A, w_packed, scales, zeros, C, 1, M, N, K, group, zero_scalar, in_dtype, out_dtype, st);
+  }
+  TLQ_REQUIRE(N % 4 == 0, "tlq_gemm_w4a16: the MFMA kernel needs N %% 4 == 0 (got %lld)", (long long)N);
+  return gemm_w4a16_mfma(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, st);
+}
+
+int tlq_gemv_w4a16_batched(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C,
+                           int64_t batch, int64_t M, int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype,
+                           int out_dtype, void* stream) {
+  TLQ_CHECK_DIMS("tlq_gemv_w4a16_batched");
+  TLQ_REQUIRE(batch >= 0 && batch <= 65535, "tlq_gemv_w4a16_batched: batch=%lld must be in 0..65535", (long long)batch);
+  TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemv_w4a16_batched: bad in_dtype %d", in_dtype);
+  TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemv_w4a16_batched: bad out_dtype %d",
+              out_dtype);
+  if (batch == 0 || M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(M <= 16, "tlq_gemv_w4a16_batched: M=%lld must be <= 16", (long long)M);
+  TLQ_REQUIRE(K > 0 && K % 64 == 0, "tlq_gemv_w4a16_batched: K=%lld must be a positive multiple of 64", (long long)K);
+  TLQ_REQUIRE(group > 0 && K % group == 0 && group % 32 == 0,
+              "tlq_gemv_w4a16_batched: group=%lld must divide K=%lld and be a multiple of 32", (long long)group, (long long)K);
+  TLQ_REQUIRE(A && w_packed && C, "tlq_gemv_w4a16_batched: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(w_packed), "tlq_gemv_w4a16_batched: A and w_packed must be 16-byte aligned");
+  return gemv_w4a16(A, w_packed, scales, zeros, C, batch, M, N, K, group, zero_scalar, in_dtype, out_dtype,
+                    (hipStream_t)stream);
+}
+
+int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
+                 int b_layout, void* stream) {
+  TLQ_CHECK_DIMS("tlq_gemm_f16");
+  TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_f16: in_dtype must be float16 or bfloat16 (got %d)",
+              in_dtype);
+  TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_f16: bad out_dtype %d",
+              out_dtype);
+  TLQ_REQUIRE(b_layout == TLQ_B_KN || b_layout == TLQ_B_NK, "tlq_gemm_f16: bad b_layout %d", b_layout);
+  if (M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(K > 0 && K % 8 == 0, "tlq_gemm_f16: K=%lld must be a positive multiple of 8", (long long)K);
+  TLQ_REQUIRE(N % 8 == 0, "tlq_gemm_f16: N=%lld must be a multiple of 8", (long long)N);
+  TLQ_REQUIRE(A && B && C, "tlq_gemm_f16: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_f16: pointers must be 16-byte aligned");
+  return gemm_f16_plain(A, B, C, M, N, K, in_dtype, out_dtype, b_layout, (hipStream_t)stream);
+}
+
+int tlq_gemm_i8(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,
+                void* stream) {
+  TLQ_CHECK_DIMS("tlq_gemm_i8");
+  TLQ_REQUIRE(batch >= 0 && batch < kMaxDim, "tlq_gemm_i8: bad batch %lld", (long long)batch);
+  TLQ_REQUIRE(b_layout == TLQ_B_KN || b_layout == TLQ_B_NK, "tlq_gemm_i8: bad b_layout %d", b_layout);
+  if (batch == 0 || M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(K > 0 && K % 16 == 0, "tlq_gemm_i8: K=%lld must be a positive multiple of 16", (long long)K);
+  TLQ_REQUIRE(N % 16 == 0, "tlq_gemm_i8: N=%lld must be a multiple of 16", (long long)N);
+  TLQ_REQUIRE(A && B && C, "tlq_gemm_i8: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_i8: pointers must be 16-byte aligned");
+  return gemm_i8_i32(A, B, C, batch, M, N, K, b_layout, (hipStream_t)stream);
+}
+
+int tlq_gemm_w4a8(const void* A, const void* w_packed, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
+                  void* stream) {
+  TLQ_CHECK_DIMS("tlq_gemm_w4a8");
+  TLQ_REQUIRE(sign_mode >= TLQ_U4 && sign_mode <= TLQ_S4_OFFSET7, "tlq_gemm_w4a8: bad sign_mode %d", sign_mode);
+  if (M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(K > 0 && K % 32 == 0, "tlq_gemm_w4a8: K=%lld must be a positive multiple of 32", (long long)K);
+  TLQ_REQUIRE(N % 4 == 0, "tlq_gemm_w4a8: N=%lld must be a multiple of 4", (long long)N);
+  TLQ_REQUIRE(A && w_packed && C, "tlq_gemm_w4a8: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(w_packed) && aligned16(C), "tlq_gemm_w4a8: pointers must be 16-byte aligned");
+  return gemm_w4a8_i32(A, w_packed, C, M, N, K, sign_mode, (hipStream_t)stream);
+}
+
+int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
+                  int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, void* stream) {
+  TLQ_CHECK_DIMS("tlq_gemm_w8a8");
+  TLQ_REQUIRE(batch >= 0 && batch < kMaxDim, "tlq_gemm_w8a8: bad batch %lld", (long long)batch);
+  TLQ_REQUIRE(b_layout == TLQ_B_KN || b_layout == TLQ_B_NK, "tlq_gemm_w8a8: bad b_layout %d", b_layout);
+  TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_w8a8: bad out_dtype %d",
+              out_dtype);
+  if (batch == 0 || M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(K > 0 && K % 16 == 0, "tlq_gemm_w8a8: K=%lld must be a positive multiple of 16", (long long)K);
+  TLQ_REQUIRE(N % 16 == 0, "tlq_gemm_w8a8: N=%lld must be a multiple of 16", (long long)N);
+  TLQ_REQUIRE(scale_b == nullptr || n_scale_b == 1 || n_scale_b == N,
+              "tlq_gemm_w8a8: n_scale_b=%lld must be 1 or N=%lld", (long long)n_scale_b, (long long)N);
+  TLQ_REQUIRE(A && B && C, "tlq_gemm_w8a8: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_w8a8: pointers must be 16-byte aligned");
+  TLQ_REQUIRE(((uintptr_t)scale_a & 3) == 0 && ((uintptr_t)scale_b & 3) == 0, "tlq_gemm_w8a8: scales misaligned");
+  return gemm_w8a8_rescale(A, B, scale_a, scale_b, C, batch, M, N, K, n_scale_b, b_layout, out_dtype,
+                           (hipStream_t)stream);
+}
+
+}  // extern "C"

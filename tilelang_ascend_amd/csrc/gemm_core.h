@@ -1,0 +1,387 @@
+// LDS-staged MFMA GEMM main loop for gfx950, shared by the W4A16, fp16/bf16 and int8 paths.
+//
+//   D[n, m] += sum_k Wt[n, k] * At[m, k]
+//
+// Everything is expressed in BYTES of K: one stage is 128 bytes of K per row (64 fp16/bf16
+// or 128 int8 values).  Both operand tiles live in LDS as [rows][128 B] with the 16-byte
+// chunk index XOR-swizzled by the row, and one 16x16 MFMA k-step consumes one 16-byte chunk
+// per lane from each operand (v_mfma_f32_16x16x32_{f16,bf16}: 8 values, v_mfma_i32_16x16x64_i8:
+// 16 values), so the loop body is identical for all element types.
+//
+// MFMA operand roles: the WEIGHT tile is the first (row) operand and the ACTIVATION tile
+// the second (column) operand.  Lane l then holds D[n = 4*(l/16) + i][m = l%16], i = 0..3,
+// i.e. four consecutive output columns of one row of the row-major C[M, N]: the epilogue
+// writes 8/16-byte vectors.
+//
+// Pipeline: global -> registers -> (convert / dequantise / transpose) -> LDS, double
+// buffered.  The global loads of stage t+1 are issued before the MFMAs of stage t; their
+// conversion and LDS store follow the MFMAs; one barrier per stage.
+#pragma once
+
+#include "tlq_common.h"
+
+namespace tlq {
+
+constexpr int kStageBytes = 128;
+
+// 16-byte chunk swizzle.  Makes the MFMA operand reads (16 consecutive rows, same logical
+// chunk), the row-copy stores (8 lanes per row) and the transposing stores (rows 16 apart)
+// spread over the LDS banks.
+__device__ __forceinline__ int lds_swz(int row) { return (row & 7) ^ ((row >> 3) & 1) ^ ((row >> 4) & 7); }
+__device__ __forceinline__ int lds_off(int row, int chunk) { return row * kStageBytes + ((chunk ^ lds_swz(row)) << 4); }
+
+// ---- MFMA wrappers ----------------------------------------------------------------------
+struct MmaF16 {
+  typedef float4_t acc_t;
+  static constexpr int elem_bytes = 2;
+  static __device__ __forceinline__ acc_t mma(const uint4_t& a, const uint4_t& b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<half8_t>(a), bitcast<half8_t>(b), c, 0, 0, 0);
+  }
+};
+struct MmaBF16 {
+  typedef float4_t acc_t;
+  static constexpr int elem_bytes = 2;
+  static __device__ __forceinline__ acc_t mma(const uint4_t& a, const uint4_t& b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<bf16x8_t>(a), bitcast<bf16x8_t>(b), c, 0, 0, 0);
+  }
+};
+struct MmaI8 {
+  typedef int4_t acc_t;
+  static constexpr int elem_bytes = 1;
+  static __device__ __forceinline__ acc_t mma(const uint4_t& a, const uint4_t& b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(bitcast<int4_t>(a), bitcast<int4_t>(b), c, 0, 0, 0);
+  }
+};
+
+// ---- tile loaders -----------------------------------------------------------------------
+// A loader owns a Regs type (what one thread keeps in flight for one stage) and two phases:
+//   gload (regs, kt, tid): issue the global loads of stage kt
+//   lstore(regs, lds, tid): convert and write the stage into an LDS tile of ROWS x 128 B
+
+// Plain row-major [rows, k_bytes] source (activations of every kind, weights stored [N, K]).
+template <int ROWS, int NT>
+struct RowLoader {
+  static constexpr int SLOTS = ROWS * 8;  // 16-byte chunks per stage
+  static constexpr int PASSES = (SLOTS + NT - 1) / NT;
+  static constexpr bool PARTIAL = SLOTS % NT != 0;
+  struct Params {
+    const uint8_t* base;   // element [0, 0] of batch 0
+    int64_t ld;            // row pitch in bytes
+    int64_t batch_stride;  // bytes between batches
+    int64_t k_bytes;       // bytes of K per row (multiple of 16)
+  };
+  struct Regs {
+    uint4_t v[PASSES];
+  };
+  const uint8_t* base;
+  int64_t ld;
+  int rows_valid;
+  int k_bytes;
+
+  __device__ __forceinline__ RowLoader(const Params& p, int batch, int row0, int rows_total)
+      : base(p.base + batch * p.batch_stride + (int64_t)row0 * p.ld), ld(p.ld), rows_valid(rows_total - row0),
+        k_bytes((int)p.k_bytes) {}
+
+  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
+    const int chunk = tid & 7;
+    const int kb = kt * kStageBytes + chunk * 16;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int slot = p * NT + tid;
+      int row = slot >> 3;
+      row = row < rows_valid ? row : rows_valid - 1;
+      uint4_t v = {0u, 0u, 0u, 0u};
+      if (kb < k_bytes && (!PARTIAL || slot < SLOTS)) v = *(const uint4_t*)(base + (int64_t)row * ld + kb);
+      r.v[p] = v;
+    }
+  }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
+    const int chunk = tid & 7;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int slot = p * NT + tid;
+      if (PARTIAL && slot >= SLOTS) continue;
+      *(uint4_t*)(lds + lds_off(slot >> 3, chunk)) = r.v[p];
+    }
+  }
+};
+
+// int8 source stored [K, N] (N contiguous): 4(k) x 16(n) register blocks are byte-transposed
+// with v_perm_b32 so that the LDS tile is [n][k] like every other operand.
+template <int ROWS, int NT>
+struct I8KNLoader {
+  static constexpr int NBLK = ROWS / 16;                // 16-column blocks per tile
+  static constexpr int PASSES = (32 * NBLK) / NT;       // 128 k = 32 blocks of 4 rows
+  static_assert(PASSES >= 1 && (32 * NBLK) % NT == 0 && NT % NBLK == 0, "bad transposing loader shape");
+  struct Params {
+    const uint8_t* base;   // B[0, 0] of batch 0
+    int64_t ld;            // bytes per k row (= N)
+    int64_t batch_stride;
+    int64_t k_total;       // K
+  };
+  struct Regs {
+    uint4_t v[PASSES][4];
+  };
+  const uint8_t* base;
+  int64_t ld;
+  int k_total;
+
+  // cols_total must be a multiple of 16 (checked on the host)
+  __device__ __forceinline__ I8KNLoader(const Params& p, int batch, int col0, int cols_total)
+      : base(p.base + batch * p.batch_stride + col0), ld(p.ld), k_total((int)p.k_total), cols_valid(cols_total - col0) {}
+  int cols_valid;
+
+  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
+    const int nblk = tid % NBLK;
+    int col = nblk * 16;
+    col = col < cols_valid ? col : cols_valid - 16;  // clamp whole 16-column blocks
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int kblk = p * (NT / NBLK) + tid / NBLK;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = kt * kStageBytes + kblk * 4 + i;
+        uint4_t v = {0u, 0u, 0u, 0u};
+        if (k < k_total) v = *(const uint4_t*)(base + (int64_t)k * ld + col);
+        r.v[p][i] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
+    const int nblk = tid % NBLK;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int kblk = p * (NT / NBLK) + tid / NBLK;
+      const int chunk = kblk >> 2;
+      const int within = (kblk & 3) * 4;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint32_t a = r.v[p][0][c], b = r.v[p][1][c], cc = r.v[p][2][c], d = r.v[p][3][c];
+        // 4x4 byte transpose: t[j] = (a.byte j, b.byte j, c.byte j, d.byte j)
+        const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400u);
+        const uint32_t ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602u);
+        const uint32_t cd_lo = __builtin_amdgcn_perm(d, cc, 0x05010400u);
+        const uint32_t cd_hi = __builtin_amdgcn_perm(d, cc, 0x07030602u);
+        const uint32_t t[4] = {__builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u),
+                               __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u),
+                               __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u),
+                               __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u)};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int row = nblk * 16 + c * 4 + j;
+          *(uint32_t*)(lds + lds_off(row, chunk) + within) = t[j];
+        }
+      }
+    }
+  }
+};
+
+// ---- epilogues ----------------------------------------------------------------------------
+// store(m, n, acc): acc holds C[m, n .. n+3]
+struct EpiFloat {  // fp32 accumulators -> f16 / bf16 / f32
+  struct Params {
+    void* C;
+    int64_t ldc;
+    int64_t batch_stride;  // elements
+    int out_dtype;
+  };
+  Params p;
+  int64_t boff;
+  __device__ __forceinline__ EpiFloat(const Params& pp, int batch) : p(pp), boff(batch * pp.batch_stride) {}
+  __device__ __forceinline__ void store(int m, int n, const float4_t& acc, int M, int N) const {
+    if (m >= M || n >= N) return;
+    const int64_t idx = boff + (int64_t)m * p.ldc + n;
+    if (n + 3 < N) {
+      if (p.out_dtype == TLQ_F32) {
+        *(float4_t*)((float*)p.C + idx) = acc;
+      } else if (p.out_dtype == TLQ_F16) {
+        half_t h[4] = {(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
+        *(uint2_t*)((half_t*)p.C + idx) = bitcast<uint2_t>(h);
+      } else {
+        uint2_t o;
+        o.x = float_to_bf16_bits(acc[0]) | (float_to_bf16_bits(acc[1]) << 16);
+        o.y = float_to_bf16_bits(acc[2]) | (float_to_bf16_bits(acc[3]) << 16);
+        *(uint2_t*)((uint16_t*)p.C + idx) = o;
+      }
+    } else {
+      for (int i = 0; i < 4 && n + i < N; ++i) store_out(p.C, idx + i, acc[i], p.out_dtype);
+    }
+  }
+};
+
+struct EpiInt32 {  // raw int32 accumulators
+  struct Params {
+    int32_t* C;
+    int64_t ldc;
+    int64_t batch_stride;
+  };
+  Params p;
+  int64_t boff;
+  __device__ __forceinline__ EpiInt32(const Params& pp, int batch) : p(pp), boff(batch * pp.batch_stride) {}
+  __device__ __forceinline__ void store(int m, int n, const int4_t& acc, int M, int N) const {
+    if (m >= M || n >= N) return;
+    const int64_t idx = boff + (int64_t)m * p.ldc + n;
+    if (n + 3 < N) {
+      *(int4_t*)(p.C + idx) = acc;
+    } else {
+      for (int i = 0; i < 4 && n + i < N; ++i) p.C[idx + i] = acc[i];
+    }
+  }
+};
+
+// int32 accumulators -> fp32 (RNE) -> * scale_a[m] -> * scale_b[n] -> out dtype (RNE); each
+// multiply rounds to fp32 on its own (the file is compiled with -ffp-contract=off).
+struct EpiRescale {
+  struct Params {
+    void* C;
+    int64_t ldc;
+    int64_t batch_stride;  // elements of C per batch
+    const float* scale_a;  // [batch * M] or null
+    const float* scale_b;  // [n_scale_b] or null
+    int64_t n_scale_b;     // 1 or N
+    int64_t scale_a_batch_stride;
+    int out_dtype;
+  };
+  Params p;
+  int64_t boff;
+  const float* sa;
+  __device__ __forceinline__ EpiRescale(const Params& pp, int batch)
+      : p(pp), boff(batch * pp.batch_stride), sa(pp.scale_a ? pp.scale_a + batch * pp.scale_a_batch_stride : nullptr) {}
+  __device__ __forceinline__ void store(int m, int n, const int4_t& acc, int M, int N) const {
+    if (m >= M || n >= N) return;
+    float4_t f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = (float)acc[i];
+    if (sa) {
+      const float a = sa[m];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[i] = f[i] * a;
+    }
+    if (p.scale_b) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int nn = (n + i < N) ? n + i : N - 1;
+        f[i] = f[i] * (p.n_scale_b == 1 ? p.scale_b[0] : p.scale_b[nn]);
+      }
+    }
+    EpiFloat::Params fp{p.C, p.ldc, 0, p.out_dtype};
+    EpiFloat ef(fp, 0);
+    ef.boff = boff;
+    ef.store(m, n, f, M, N);
+  }
+};
+
+// ---- the kernel -----------------------------------------------------------------------------
+template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64, 1) void gemm_mfma_kernel(typename AL::Params pa, typename WL::Params pw,
+                                                                    typename Epi::Params pe, int M, int N, int KT,
+                                                                    int tiles_m, int tiles_n) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int TM = BM / WM / 16;  // 16-row activation tiles per wave
+  constexpr int TN = BN / WN / 16;  // 16-row weight tiles per wave
+  extern __shared__ __align__(16) uint8_t smem[];
+  uint8_t* const ldsA0 = smem;
+  uint8_t* const ldsW0 = smem + 2 * BM * kStageBytes;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int r16 = lane & 15;
+  const int q = lane >> 4;
+  const int wave_m0 = (wave % WM) * (BM / WM);
+  const int wave_n0 = (wave / WM) * (BN / WN);
+
+  // Work-group -> tile.  Consecutive hardware ids are dealt round-robin to the 8 XCDs; give
+  // every XCD a contiguous range of logical tiles so that tiles sharing an activation panel
+  // also share an L2.
+  const int total = gridDim.x;
+  int lid = blockIdx.x;
+  if ((total & 7) == 0) lid = (lid & 7) * (total >> 3) + (lid >> 3);
+  const int per_batch = tiles_m * tiles_n;
+  const int batch = lid / per_batch;
+  const int rem = lid - batch * per_batch;
+  const int m0 = (rem / tiles_n) * BM;
+  const int n0 = (rem % tiles_n) * BN;
+
+  AL al(pa, batch, m0, M);
+  WL wl(pw, batch, n0, N);
+  typename AL::Regs ra;
+  typename WL::Regs rw;
+
+  typename Mma::acc_t acc[TN][TM];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = typename Mma::acc_t{0, 0, 0, 0};
+
+  al.gload(ra, 0, tid);
+  wl.gload(rw, 0, tid);
+  al.lstore(ra, ldsA0, tid);
+  wl.lstore(rw, ldsW0, tid);
+  __syncthreads();
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int cur = kt & 1;
+    const uint8_t* la = ldsA0 + cur * BM * kStageBytes;
+    const uint8_t* lw = ldsW0 + cur * BN * kStageBytes;
+    const bool more = kt + 1 < KT;
+    if (more) {
+      al.gload(ra, kt + 1, tid);
+      wl.gload(rw, kt + 1, tid);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int chunk = ks * 4 + q;
+      uint4_t wf[TN], af[TM];
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) wf[tn] = *(const uint4_t*)(lw + lds_off(wave_n0 + tn * 16 + r16, chunk));
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) af[tm] = *(const uint4_t*)(la + lds_off(wave_m0 + tm * 16 + r16, chunk));
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = Mma::mma(wf[tn], af[tm], acc[tn][tm]);
+    }
+    if (more) {
+      al.lstore(ra, ldsA0 + (cur ^ 1) * BM * kStageBytes, tid);
+      wl.lstore(rw, ldsW0 + (cur ^ 1) * BN * kStageBytes, tid);
+    }
+    __syncthreads();
+  }
+
+  Epi epi(pe, batch);
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+      epi.store(m0 + wave_m0 + tm * 16 + r16, n0 + wave_n0 + tn * 16 + q * 4, acc[tn][tm], M, N);
+}
+
+// Host-side launcher: sets the dynamic LDS size and launches one work-group per tile.
+template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
+int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,
+                int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what) {
+  auto kern = gemm_mfma_kernel<Mma, AL, WL, Epi, BM, BN, WM, WN>;
+  constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes;
+  static bool attr_set = false;  // per instantiation; idempotent, so a race only repeats the call
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) {
+      set_error("%s: cannot reserve %d bytes of LDS: %s", what, lds_bytes, hipGetErrorString(e));
+      return 1;
+    }
+    attr_set = true;
+  }
+  const int64_t tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
+  const int64_t blocks = batch * tiles_m * tiles_n;
+  if (blocks <= 0) return 0;
+  if (blocks > 0x7fffffff) {
+    set_error("%s: too many tiles", what);
+    return 1;
+  }
+  const int KT = (int)ceil_div(k_bytes, kStageBytes);
+  kern<<<(unsigned)blocks, WM * WN * 64, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, KT, (int)tiles_m, (int)tiles_n);
+  return check_launch(what) ? 0 : 1;
+}
+
+}  // namespace tlq

@@ -1,0 +1,101 @@
+// Plain fp16 / bf16 GEMM with fp32 accumulation: C[M, N] = A[M, K] . B, B stored [K, N]
+// (transposed on the fly) or [N, K].
+#include "gemm_core.h"
+
+namespace tlq {
+
+// 16-bit source stored [K, N] (N contiguous): 4(k) x 8(n) register blocks are transposed with
+// v_perm_b32 and written as 8-byte pieces (4 consecutive k of one n) into the [n][k] LDS tile.
+template <int ROWS, int NT>
+struct H16KNLoader {
+  static constexpr int NBLK = ROWS / 8;            // 8-column blocks per tile
+  static constexpr int PASSES = (16 * NBLK) / NT;  // 64 k = 16 blocks of 4 rows
+  static_assert(PASSES >= 1 && (16 * NBLK) % NT == 0 && NT % NBLK == 0, "bad transposing loader shape");
+  struct Params {
+    const uint8_t* base;  // B[0, 0]
+    int64_t ld;           // bytes per k row (= 2 N)
+    int64_t batch_stride;
+    int64_t k_total;
+  };
+  struct Regs {
+    uint4_t v[PASSES][4];
+  };
+  const uint8_t* base;
+  int64_t ld;
+  int k_total;
+  int cols_valid;
+
+  // cols_total must be a multiple of 8 (checked on the host)
+  __device__ __forceinline__ H16KNLoader(const Params& p, int batch, int col0, int cols_total)
+      : base(p.base + batch * p.batch_stride + (int64_t)col0 * 2), ld(p.ld), k_total((int)p.k_total),
+        cols_valid(cols_total - col0) {}
+
+  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
+    int col = (tid % NBLK) * 8;
+    col = col < cols_valid ? col : cols_valid - 8;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int kblk = p * (NT / NBLK) + tid / NBLK;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = kt * 64 + kblk * 4 + i;
+        uint4_t v = {0u, 0u, 0u, 0u};
+        if (k < k_total) v = *(const uint4_t*)(base + (int64_t)k * ld + col * 2);
+        r.v[p][i] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
+    const int nblk = tid % NBLK;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int kblk = p * (NT / NBLK) + tid / NBLK;
+      const int chunk = kblk >> 1;
+      const int within = (kblk & 1) * 8;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {  // word w of each row holds columns 2w, 2w+1
+        const uint32_t a = r.v[p][0][w], b = r.v[p][1][w], c = r.v[p][2][w], d = r.v[p][3][w];
+        uint2_t even, odd;
+        even.x = __builtin_amdgcn_perm(b, a, 0x05040100u);  // (a.lo, b.lo)
+        even.y = __builtin_amdgcn_perm(d, c, 0x05040100u);  // (c.lo, d.lo)
+        odd.x = __builtin_amdgcn_perm(b, a, 0x07060302u);   // (a.hi, b.hi)
+        odd.y = __builtin_amdgcn_perm(d, c, 0x07060302u);
+        *(uint2_t*)(lds + lds_off(nblk * 8 + 2 * w, chunk) + within) = even;
+        *(uint2_t*)(lds + lds_off(nblk * 8 + 2 * w + 1, chunk) + within) = odd;
+      }
+    }
+  }
+};
+
+template <class Mma, int BM, int BN, int WM, int WN>
+static int run_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int out_dtype, int b_layout,
+                   hipStream_t st) {
+  constexpr int NT = WM * WN * 64;
+  typedef RowLoader<BM, NT> AL;
+  typename AL::Params pa{(const uint8_t*)A, K * 2, 0, K * 2};
+  EpiFloat::Params pe{C, N, 0, out_dtype};
+  if (b_layout == TLQ_B_NK) {
+    typedef RowLoader<BN, NT> WL;
+    typename WL::Params pw{(const uint8_t*)B, K * 2, 0, K * 2};
+    return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16");
+  }
+  typedef H16KNLoader<BN, NT> WL;
+  typename WL::Params pw{(const uint8_t*)B, N * 2, 0, K};
+  return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16");
+}
+
+template <class Mma>
+static int dispatch_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int out_dtype,
+                        int b_layout, hipStream_t st) {
+  if (M <= 128 || ceil_div(M, 256) * ceil_div(N, 256) < 128)
+    return run_f16<Mma, 128, 128, 2, 2>(A, B, C, M, N, K, out_dtype, b_layout, st);
+  return run_f16<Mma, 256, 256, 2, 2>(A, B, C, M, N, K, out_dtype, b_layout, st);
+}
+
+int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
+                   int b_layout, hipStream_t st) {
+  if (in_dtype == TLQ_F16) return dispatch_f16<MmaF16>(A, B, C, M, N, K, out_dtype, b_layout, st);
+  return dispatch_f16<MmaBF16>(A, B, C, M, N, K, out_dtype, b_layout, st);
+}
+
+}  // namespace tlq

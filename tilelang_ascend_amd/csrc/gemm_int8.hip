@@ -1,0 +1,175 @@
+// int8 MFMA GEMMs (v_mfma_i32_16x16x64_i8, int32 accumulate, bit exact):
+//   * W8A8 with the fused rescale epilogue  C = rn_out(f32(acc) * scale_a[m] * scale_b[n])
+//   * raw int32 output
+//   * W4A8: packed int4 weights expanded to int8 on the way into LDS
+// The second operand may be stored [K, N] (transposed on the fly) or [N, K].
+#include "gemm_core.h"
+
+namespace tlq {
+
+// Packed int4 [N, K/2] -> int8 LDS tile.  One stage is 128 values of K = 64 packed bytes per
+// row; a thread expands 16 packed bytes into two 16-byte chunks.
+template <int ROWS, int NT>
+struct W4I8Loader {
+  static constexpr int SLOTS = ROWS * 4;
+  static constexpr int PASSES = (SLOTS + NT - 1) / NT;
+  static constexpr bool PARTIAL = SLOTS % NT != 0;
+  struct Params {
+    const uint8_t* wp;
+    int64_t row_bytes;  // K / 2
+    int sign_mode;
+  };
+  struct Regs {
+    uint4_t v[PASSES];
+  };
+  const uint8_t* base;
+  int64_t row_bytes;
+  int rows_valid;
+  int sign_mode;
+
+  __device__ __forceinline__ W4I8Loader(const Params& p, int /*batch*/, int row0, int rows_total)
+      : base(p.wp + (int64_t)row0 * p.row_bytes), row_bytes(p.row_bytes), rows_valid(rows_total - row0),
+        sign_mode(p.sign_mode) {}
+
+  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+      const int slot = ps * NT + tid;
+      int row = slot >> 2;
+      row = row < rows_valid ? row : rows_valid - 1;
+      const int kb = kt * 64 + (slot & 3) * 16;
+      uint4_t v = {0u, 0u, 0u, 0u};
+      if (kb < row_bytes && (!PARTIAL || slot < SLOTS)) v = *(const uint4_t*)(base + (int64_t)row * row_bytes + kb);
+      r.v[ps] = v;
+    }
+  }
+  // four nibbles held one per byte (0..15) -> four int8 under the sign convention
+  __device__ __forceinline__ uint32_t sign4(uint32_t x) const {
+    if (sign_mode == TLQ_U4) return x;
+    if (sign_mode == TLQ_S4_TWOS) x ^= 0x08080808u;  // two's complement == offset-8 of (u ^ 8)
+    const uint32_t c = (sign_mode == TLQ_S4_OFFSET7) ? 0x07070707u : 0x08080808u;
+    // per-byte u - c without borrows between bytes: bias by 128, subtract, remove the bias
+    return ((x | 0x80808080u) - c) ^ 0x80808080u;
+  }
+  __device__ __forceinline__ void expand(uint32_t v, uint32_t& d0, uint32_t& d1) const {
+    const uint32_t lo = sign4(v & 0x0f0f0f0fu);         // k0 k2 k4 k6
+    const uint32_t hi = sign4((v >> 4) & 0x0f0f0f0fu);  // k1 k3 k5 k7
+    d0 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);    // k0 k1 k2 k3
+    d1 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);    // k4 k5 k6 k7
+  }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+      const int slot = ps * NT + tid;
+      if (PARTIAL && slot >= SLOTS) continue;
+      const int row = slot >> 2;
+      const int quarter = slot & 3;
+      uint32_t d[8];
+      expand(r.v[ps].x, d[0], d[1]);
+      expand(r.v[ps].y, d[2], d[3]);
+      expand(r.v[ps].z, d[4], d[5]);
+      expand(r.v[ps].w, d[6], d[7]);
+      *(uint4_t*)(lds + lds_off(row, quarter * 2 + 0)) = uint4_t{d[0], d[1], d[2], d[3]};
+      *(uint4_t*)(lds + lds_off(row, quarter * 2 + 1)) = uint4_t{d[4], d[5], d[6], d[7]};
+    }
+  }
+};
+
+// ---- launch helpers -----------------------------------------------------------------------
+template <class WL, class Epi, int BM, int BN, int WM, int WN>
+static int run_i8(const void* A, const typename WL::Params& pw, const typename Epi::Params& pe, int64_t batch,
+                  int64_t M, int64_t N, int64_t K, hipStream_t st, const char* what) {
+  constexpr int NT = WM * WN * 64;
+  typedef RowLoader<BM, NT> AL;
+  typename AL::Params pa{(const uint8_t*)A, K, M * K, K};
+  return launch_gemm<MmaI8, AL, WL, Epi, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K, st, what);
+}
+
+static int g_i8_tile = 0;
+
+static int pick_tile(int64_t batch, int64_t M, int64_t N) {
+  if (g_i8_tile) return g_i8_tile;
+  if (M <= 32) return 32;
+  if (M <= 128 || batch * ceil_div(M, 256) * ceil_div(N, 256) < 128) return 128;
+  return 256;
+}
+
+template <class Epi>
+static int dispatch_i8(const void* A, const void* B, const typename Epi::Params& pe, int64_t batch, int64_t M,
+                       int64_t N, int64_t K, int b_layout, hipStream_t st, const char* what) {
+  const int tile = pick_tile(batch, M, N);
+  if (b_layout == TLQ_B_KN) {
+#define TLQ_RUN(BM, BN, WM, WN)                                               \
+  {                                                                           \
+    typedef I8KNLoader<BN, WM * WN * 64> WL;                                  \
+    typename WL::Params pw{(const uint8_t*)B, N, K * N, K};                   \
+    return run_i8<WL, Epi, BM, BN, WM, WN>(A, pw, pe, batch, M, N, K, st, what); \
+  }
+    switch (tile) {
+      case 32:
+        TLQ_RUN(32, 128, 1, 4)
+      case 128:
+        TLQ_RUN(128, 128, 2, 2)
+      default:
+        TLQ_RUN(256, 256, 2, 2)
+    }
+#undef TLQ_RUN
+  } else {
+#define TLQ_RUN(BM, BN, WM, WN)                                               \
+  {                                                                           \
+    typedef RowLoader<BN, WM * WN * 64> WL;                                   \
+    typename WL::Params pw{(const uint8_t*)B, K, N * K, K};                   \
+    return run_i8<WL, Epi, BM, BN, WM, WN>(A, pw, pe, batch, M, N, K, st, what); \
+  }
+    switch (tile) {
+      case 32:
+        TLQ_RUN(32, 128, 1, 4)
+      case 128:
+        TLQ_RUN(128, 128, 2, 2)
+      default:
+        TLQ_RUN(256, 256, 2, 2)
+    }
+#undef TLQ_RUN
+  }
+}
+
+int gemm_i8_i32(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,
+                hipStream_t st) {
+  EpiInt32::Params pe{(int32_t*)C, N, M * N};
+  return dispatch_i8<EpiInt32>(A, B, pe, batch, M, N, K, b_layout, st, "tlq_gemm_i8");
+}
+
+int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
+                      int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, hipStream_t st) {
+  EpiRescale::Params pe{C, N, M * N, (const float*)scale_a, (const float*)scale_b, n_scale_b, M, out_dtype};
+  return dispatch_i8<EpiRescale>(A, B, pe, batch, M, N, K, b_layout, st, "tlq_gemm_w8a8");
+}
+
+int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
+                  hipStream_t st) {
+  EpiInt32::Params pe{(int32_t*)C, N, M * N};
+  const int tile = pick_tile(1, M, N);
+#define TLQ_RUN(BM, BN, WM, WN)                                                                  \
+  {                                                                                              \
+    typedef W4I8Loader<BN, WM * WN * 64> WL;                                                     \
+    typename WL::Params pw{(const uint8_t*)Wp, K / 2, sign_mode};                                \
+    return run_i8<WL, EpiInt32, BM, BN, WM, WN>(A, pw, pe, 1, M, N, K, st, "tlq_gemm_w4a8");     \
+  }
+  switch (tile) {
+    case 32:
+      TLQ_RUN(32, 128, 1, 4)
+    case 128:
+      TLQ_RUN(128, 128, 2, 2)
+    default:
+      TLQ_RUN(256, 256, 2, 2)
+  }
+#undef TLQ_RUN
+}
+
+}  // namespace tlq
+
+extern "C" {
+// Tuning hook used by the benchmark sweeps: forces the activation-tile height (32, 128, 256)
+// of the int8 kernels; 0 restores the automatic choice.
+void tlq_tune_i8_tile(int block_m) { tlq::g_i8_tile = block_m; }
+}
