@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|prefill|w8a8] [--units U]
+
+Headline workload (default): the W4A16 decode GEMV -- M=1, N=11008, K=4096, fp16 activations,
+uint4 weights packed low-nibble-first, group 128, fp16 scales U[0.005,0.02] and fp16 zeros U{6..9},
+fp16 output, fp32 accumulation.  One "step" is one launch of the GEMV kernel over `units`
+independent weight sets (default 1).  The weight sets rotate through a pool larger than the
+256 MB last-level cache, so every step streams its weights from HBM.  Inputs are resident in
+HBM before the timed region starts.
+
+Prints ONE JSON line.  `value` is algorithmic bytes / wall time (GB/s); `roofline` describes the
+dominant kernel from HIP events recorded on the launch stream around the timed region;
+`cpu_baseline` is the CPU oracle (the reference's torch ref_program arithmetic) timed on the
+host cores on a bounded sample; `other_workloads` carries the prefill GEMM and W8A8 figures.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+MFMA_I8_PEAK_TOPS = 5000.0
+POOL_BYTES = 576 * 1024 * 1024  # weight pool > 2x the 256 MB last-level cache
+
+
+def w4a16_bytes(M, N, K, group, zeros_tensor=True, elem=2):
+    """Algorithmic bytes of one W4A16 problem: packed weights + scales (+ zeros) + A + C."""
+    return N * K // 2 + (2 if zeros_tensor else 1) * elem * N * K // group + elem * M * K + elem * M * N
+
+
+def w8a8_bytes(B, M, N, K):
+    return B * M * K + B * K * N + 2 * B * M * N + 4 * B * M + 4 * N
+
+
+def timed(fn, steps, warmup):
+    """Returns (wall seconds per step, event-measured seconds per step)."""
+    import torch
+
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def bench_gemv(args):
+    import torch
+
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dev = torch.device("cuda:0")
+    M, N, K, g = 1, 11008, 4096, 128
+    units = args.units
+    unit_bytes = w4a16_bytes(M, N, K, g)
+    sets = max(2 * units, -(-POOL_BYTES // unit_bytes))
+    sets = -(-sets // units) * units
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    Wp = torch.randint(0, 256, (sets, N, K // 2), dtype=torch.uint8, generator=gen).to(dev)
+    S = (torch.rand(sets, N, K // g, generator=gen) * 0.015 + 0.005).to(torch.float16).to(dev)
+    Z = torch.randint(6, 10, (sets, N, K // g), generator=gen).to(torch.float16).to(dev)
+    A = torch.randn(sets, M, K, generator=gen).to(torch.float16).to(dev)
+    C = torch.empty(sets, M, N, dtype=torch.float16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    groups = sets // units
+
+    if units == 1:
+        def step(i):
+            j = i % sets
+            rc = lib.tlq_gemm_w4a16(P(A[j]), P(Wp[j]), P(S[j]), P(Z[j]), P(C[j]), M, N, K, g, 0.0, _abi.F16, _abi.F16,
+                                    _abi.ALGO_GEMV, stream)
+            if rc:
+                raise RuntimeError(_abi.last_error())
+    else:
+        def step(i):
+            j = (i % groups) * units
+            rc = lib.tlq_gemv_w4a16_batched(P(A[j]), P(Wp[j]), P(S[j]), P(Z[j]), P(C[j]), units, M, N, K, g, 0.0,
+                                            _abi.F16, _abi.F16, stream)
+            if rc:
+                raise RuntimeError(_abi.last_error())
+
+    wall, ev = timed(step, args.steps, args.warmup)
+    step_bytes = unit_bytes * units
+    # spot check of the last result against the oracle (outside the timed region)
+    from oracle import ref
+
+    j = ((args.steps - 1) % groups) * units if units > 1 else (args.steps - 1) % sets
+    want = ref.ref_program_w4a16(A[j].cpu(), Wp[j].cpu(), S[j].cpu(), Z[j].cpu(), g, "float32")
+    rel = ((C[j].float().cpu() - want).norm() / want.norm()).item()
+    if rel > 1e-3:
+        raise RuntimeError(f"GEMV result differs from the oracle: relative L2 {rel}")
+
+    cpu = cpu_baseline_gemv(A[0].cpu(), Wp[0].cpu(), S[0].cpu(), Z[0].cpu(), g, unit_bytes)
+    return {
+        "metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
+        "value": round(step_bytes / wall / 1e9, 1),
+        "unit": "GB/s",
+        "ms_per_step": wall * 1e3,
+        "dtype": "f16",
+        "config": {"workload": f"W4A16 decode GEMV M=1 N=11008 K=4096 group=128 fp16 scales+zeros, {units} weight set(s) per launch, "
+                               f"{sets} sets rotating ({sets * unit_bytes >> 20} MiB)",
+                   "M": M, "N": N, "K": K, "group": g, "units_per_launch": units},
+        "roofline": {"kernel": "gemv_w4a16_kernel", "bound": "hbm", "achieved": round(step_bytes / ev / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(step_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "bytes_per_launch": step_bytes, "avg_launch_us": round(ev * 1e6, 3)},
+        "cpu_baseline": cpu,
+        "parity_rel_l2": rel,
+    }
+
+
+def cpu_baseline_gemv(A, Wp, S, Z, g, unit_bytes, budget_s=10.0):
+    """The reference's CPU path for this workload: vectorised nibble unpack, (u - z) * s in fp16,
+    fp32 matmul, cast (oracle.ref.ref_program_w4a16), timed on the host cores."""
+    import torch
+
+    from oracle import ref
+
+    ref.ref_program_w4a16(A, Wp, S, Z, g, "float16")  # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        ref.ref_program_w4a16(A, Wp, S, Z, g, "float16")
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s and reps >= 3 or reps >= 200:
+            break
+    per = dt / reps
+    return {"value": round(unit_bytes / per / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{reps} evaluations of the same M=1 N=11008 K=4096 GEMV (unpack + dequant + fp32 matmul) in {dt:.1f} s",
+            "ms_per_eval": round(per * 1e3, 2), "host_cpus": os.cpu_count()}
+
+
+def bench_prefill(args, steps=None):
+    import torch
+
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dev = torch.device("cuda:0")
+    M = N = K = 4096
+    g = 128
+    gen = torch.Generator(device="cpu").manual_seed(1)
+    Wp = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=gen).to(dev)
+    S = (torch.rand(N, K // g, generator=gen) * 0.015 + 0.005).to(torch.bfloat16).to(dev)
+    A = torch.randn(M, K, generator=gen).to(torch.bfloat16).to(dev)
+    C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step(i):
+        rc = lib.tlq_gemm_w4a16(P(A), P(Wp), P(S), None, P(C), M, N, K, g, 8.0, _abi.BF16, _abi.BF16, _abi.ALGO_MFMA, stream)
+        if rc:
+            raise RuntimeError(_abi.last_error())
+
+    wall, ev = timed(step, steps or args.steps, args.warmup)
+    flops = 2.0 * M * N * K
+    return {"workload": "W4A16 prefill GEMM M=N=K=4096 bf16 group=128 zero=8", "dtype": "bf16",
+            "value": round(flops / wall / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": wall * 1e3,
+            "roofline": {"kernel": "gemm_mfma_kernel<MmaBF16,W4Loader>", "bound": "mfma", "achieved": round(flops / ev / 1e12, 1),
+                         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                         "traffic": None, "flops_per_launch": flops, "avg_launch_us": round(ev * 1e6, 2)}}
+
+
+def bench_w8a8(args, steps=None):
+    import torch
+
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dev = torch.device("cuda:0")
+    B, M, N, K = 8, 2048, 4096, 4096
+    gen = torch.Generator(device="cpu").manual_seed(2)
+    A = torch.randint(-127, 128, (B, M, K), dtype=torch.int8, generator=gen).to(dev)
+    W = torch.randint(-127, 128, (B, K, N), dtype=torch.int8, generator=gen).to(dev)
+    sa = (torch.rand(B, M, generator=gen) * 0.04 + 0.01).to(dev)
+    sb = (torch.rand(N, generator=gen) * 0.009 + 0.001).to(dev)
+    C = torch.empty(B, M, N, dtype=torch.float16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step(i):
+        rc = lib.tlq_gemm_w8a8(P(A), P(W), P(sa), P(sb), P(C), B, M, N, K, N, _abi.B_KN, _abi.F16, stream)
+        if rc:
+            raise RuntimeError(_abi.last_error())
+
+    wall, ev = timed(step, steps or args.steps, args.warmup)
+    ops = 2.0 * B * M * N * K
+    return {"workload": "W8A8 quant batch matmul B=8 M=2048 N=K=4096, per-token x per-channel rescale, fp16 out",
+            "dtype": "i8", "value": round(ops / wall / 1e12, 1), "unit": "TOP/s", "ms_per_step": wall * 1e3,
+            "roofline": {"kernel": "gemm_mfma_kernel<MmaI8,I8KNLoader,EpiRescale>", "bound": "mfma",
+                         "achieved": round(ops / ev / 1e12, 1), "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
+                         "frac": round(ops / ev / 1e12 / MFMA_I8_PEAK_TOPS, 4), "traffic": None, "ops_per_launch": ops,
+                         "avg_launch_us": round(ev * 1e6, 2)}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=480)
+    ap.add_argument("--warmup", type=int, default=48)
+    ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8"])
+    ap.add_argument("--units", type=int, default=1, help="independent weight sets per GEMV launch")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU's share of the path; --gpus {args.gpus} is not supported in this build "
+              "(the path shards over N with no exchange, see DESIGN.md).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+
+    if args.workload == "gemv":
+        line = bench_gemv(args)
+        if not args.no_extra:
+            line["other_workloads"] = [bench_prefill(args, steps=20), bench_w8a8(args, steps=10)]
+    else:
+        res = bench_prefill(args) if args.workload == "prefill" else bench_w8a8(args)
+        line = {"metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
+                "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
+                "config": {"workload": res["workload"]}, "roofline": res["roofline"], "cpu_baseline": None}
+    line.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+                 "vs_baseline": None, "data": "synthetic"})
+    order = ["metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+             "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"]
+    out = {k: line[k] for k in order if k in line}
+    out.update({k: v for k, v in line.items() if k not in out})
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

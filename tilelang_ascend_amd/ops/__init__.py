@@ -11,6 +11,6 @@ from .dequant_gemm import (  # noqa: F401
     unpack_int4,
     w4a16_gemm,
 )
-from .int8_gemm import int8_gemm_kernel_corrected, quant_batch_matmul_per_token  # noqa: F401
+from .int8_per_token import int8_gemm_kernel_corrected, quant_batch_matmul_per_token  # noqa: F401
 from .quant_matmul import simple_quant_batch_matmul, simple_quant_matmul  # noqa: F401
 from .w4a8 import torch_convert, w4a8_gemm_cv  # noqa: F401
