@@ -12,7 +12,7 @@
 // expands them to four 16-byte LDS chunks.
 //
 // fp16 expansion, per 32-bit word (8 nibbles k0..k7):
-//   (x    & 0x000f000f) | 0x64006400 -> half2 (1024+k0, 1024+k4)     one v_and_or_b32 each
+//   (x    & 0x000f000f) | 0x64006400 -> half2 (1024+k0, 1024+k4)     one v_bfi_b32 each
 //   (x    & 0x00f000f0) | 0x54005400 -> half2 (  64+k1,   64+k5)
 //   (x>>8 & ...) likewise             -> (k2, k6), (k3, k7)
 //   packed subtract of the bias (and of an integer zero point folded into it, exact), packed
@@ -29,8 +29,9 @@ struct Expand8;
 template <>
 struct Expand8<half_t> {
   half2_t s2, z2, b_lo, b_hi;
+  NibbleMagic mg;
   bool fold;
-  __device__ __forceinline__ Expand8(half_t s, half_t z, bool fold_) : fold(fold_) {
+  __device__ __forceinline__ Expand8(half_t s, half_t z, bool fold_, const NibbleMagic& mg_) : mg(mg_), fold(fold_) {
     s2 = half2_t{s, s};
     z2 = half2_t{z, z};
     // with an integer zero point 1024+z and 64+z are exact binary16 values
@@ -41,10 +42,10 @@ struct Expand8<half_t> {
   }
   __device__ __forceinline__ uint4_t operator()(uint32_t v) const {
     const uint32_t v8 = v >> 8;
-    half2_t p0 = bitcast<half2_t>(and_or(v, 0x000f000fu, 0x64006400u)) - b_lo;   // (k0, k4)
-    half2_t p1 = bitcast<half2_t>(and_or(v, 0x00f000f0u, 0x54005400u)) - b_hi;   // (k1, k5)
-    half2_t p2 = bitcast<half2_t>(and_or(v8, 0x000f000fu, 0x64006400u)) - b_lo;  // (k2, k6)
-    half2_t p3 = bitcast<half2_t>(and_or(v8, 0x00f000f0u, 0x54005400u)) - b_hi;  // (k3, k7)
+    half2_t p0 = bitcast<half2_t>(bfi(mg.m_lo, v, mg.b_lo)) - b_lo;   // (k0, k4)
+    half2_t p1 = bitcast<half2_t>(bfi(mg.m_hi, v, mg.b_hi)) - b_hi;   // (k1, k5)
+    half2_t p2 = bitcast<half2_t>(bfi(mg.m_lo, v8, mg.b_lo)) - b_lo;  // (k2, k6)
+    half2_t p3 = bitcast<half2_t>(bfi(mg.m_hi, v8, mg.b_hi)) - b_hi;  // (k3, k7)
     if (!fold) {
       p0 = p0 - z2;
       p1 = p1 - z2;
@@ -70,7 +71,7 @@ template <>
 struct Expand8<bf16_t> {
   float sf, zf, c;
   bool fold;
-  __device__ __forceinline__ Expand8(bf16_t s, bf16_t z, bool fold_) : fold(fold_) {
+  __device__ __forceinline__ Expand8(bf16_t s, bf16_t z, bool fold_, const NibbleMagic&) : fold(fold_) {
     sf = to_float(s);
     zf = to_float(z);
     c = -(zf * sf);  // exact in fp32 for a small integer zero point (8 x 8 significant bits)
@@ -114,9 +115,11 @@ struct W4Loader {
   Params p;
   const uint8_t* base;
   int row0, rows_valid;
+  NibbleMagic mg;
 
   __device__ __forceinline__ W4Loader(const Params& pp, int /*batch*/, int row0_, int rows_total)
-      : p(pp), base(pp.wp + (int64_t)row0_ * pp.row_bytes), row0(row0_), rows_valid(rows_total - row0_) {}
+      : p(pp), base(pp.wp + (int64_t)row0_ * pp.row_bytes), row0(row0_), rows_valid(rows_total - row0_),
+        mg(make_nibble_magic()) {}
 
   __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
     const T one = from_float<T>(1.0f);
@@ -148,7 +151,7 @@ struct W4Loader {
       if (PARTIAL && slot >= SLOTS) continue;
       const int row = slot >> 1;
       const int half = slot & 1;
-      const Expand8<T> ex(r.s[ps], r.z[ps], p.fold != 0);
+      const Expand8<T> ex(r.s[ps], r.z[ps], p.fold != 0, mg);
       *(uint4_t*)(lds + lds_off(row, half * 4 + 0)) = ex(r.v[ps].x);
       *(uint4_t*)(lds + lds_off(row, half * 4 + 1)) = ex(r.v[ps].y);
       *(uint4_t*)(lds + lds_off(row, half * 4 + 2)) = ex(r.v[ps].z);

@@ -8,7 +8,7 @@
 // in registers, multiplied with the matching activation slice and the 64 partial sums are
 // combined with a cross-lane butterfly at the end (split-K inside the wavefront).
 //
-// fp16 path: two nibbles at a time are turned into a half2 with one v_and_or_b32
+// fp16 path: two nibbles at a time are turned into a half2 with one v_bfi_b32
 // ((x & 0x000f000f) | 0x64006400 = 1024+u, (x & 0x00f000f0) | 0x54005400 = 64+u), the bias
 // is removed exactly with one packed subtract and v_dot2_f32_f16 accumulates in fp32.  Scale
 // and zero point are applied once per chunk in fp32:  s * (sum A*u - z * sum A), which is
@@ -25,16 +25,33 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Sum over the 64 lanes with DPP moves (no LDS traffic); the total lands in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, bitcast<int>(v), CTRL, ROW_MASK, 0xf, false);
+  return v + bitcast<float>(moved);
+}
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v = dpp_add<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141, 0xf>(v);  // row_half_mirror
+  v = dpp_add<0x140, 0xf>(v);  // row_mirror: every lane of a row holds the row total
+  v = dpp_add<0x142, 0xa>(v);  // row_bcast15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v);  // row_bcast31 into rows 2 and 3
+  return v;
+}
+
 // ---- fp16: activations kept as half2 pairs in the order the nibble unpack produces ----------
 // pair p = 4*j + i of a 32-element chunk holds elements (8*j + i, 8*j + i + 4).
 struct ActF16 {
   half2_t a[16];
-  float sum;
+  float sum;   // sum of the 32 activations
+  float bsum;  // 1024 * (sum over even k) + 64 * (sum over odd k): what the unpack bias adds to the dot
 };
 
 __device__ __forceinline__ void load_act(ActF16& r, const half_t* __restrict__ A, int64_t off) {
   const uint4_t* p = (const uint4_t*)(A + off);
-  float s = 0.f;
+  float s = 0.f, se = 0.f;
   const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -47,12 +64,34 @@ __device__ __forceinline__ void load_act(ActF16& r, const half_t* __restrict__ A
     r.a[4 * j + 3] = half2_t{q1.y, q3.y};
 #pragma unroll
     for (int i = 0; i < 4; ++i) s = __builtin_amdgcn_fdot2(r.a[4 * j + i], ones, s, false);
+    se = __builtin_amdgcn_fdot2(r.a[4 * j + 0], ones, se, false);  // pairs 0 and 2 hold the even k
+    se = __builtin_amdgcn_fdot2(r.a[4 * j + 2], ones, se, false);
   }
   r.sum = s;
+  r.bsum = 1024.0f * se + 64.0f * (s - se);
+}
+
+// Sum over the chunk of A[k] * (bias_k + u[k]) with the unpack bias left in (1024 for even k,
+// 64 for odd k); the caller subtracts act.bsum.  fp32 accumulation keeps the cancellation error
+// near 1e-5 relative, far below the fp16 output rounding.
+__device__ __forceinline__ float dot_chunk_biased(const uint4_t& w, const ActF16& act, const NibbleMagic& mg) {
+  float acc = 0.f;
+  const uint32_t x[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t v = x[j];
+    const uint32_t v8 = v >> 8;
+    acc = __builtin_amdgcn_fdot2(bitcast<half2_t>(bfi(mg.m_lo, v, mg.b_lo)), act.a[4 * j + 0], acc, false);
+    acc = __builtin_amdgcn_fdot2(bitcast<half2_t>(bfi(mg.m_hi, v, mg.b_hi)), act.a[4 * j + 1], acc, false);
+    acc = __builtin_amdgcn_fdot2(bitcast<half2_t>(bfi(mg.m_lo, v8, mg.b_lo)), act.a[4 * j + 2], acc, false);
+    acc = __builtin_amdgcn_fdot2(bitcast<half2_t>(bfi(mg.m_hi, v8, mg.b_hi)), act.a[4 * j + 3], acc, false);
+  }
+  return acc;
 }
 
 // sum over the chunk of A[k] * u[k] (u = raw nibble value), fp32
 __device__ __forceinline__ float dot_chunk(const uint4_t& w, const ActF16& act) {
+  const NibbleMagic mg = make_nibble_magic();
   const half2_t b1024 = {(half_t)1024.0f, (half_t)1024.0f};
   const half2_t b64 = {(half_t)64.0f, (half_t)64.0f};
   float acc = 0.f;
@@ -61,10 +100,10 @@ __device__ __forceinline__ float dot_chunk(const uint4_t& w, const ActF16& act) 
   for (int j = 0; j < 4; ++j) {
     uint32_t v = x[j];
     uint32_t v8 = v >> 8;
-    half2_t p0 = bitcast<half2_t>(and_or(v, 0x000f000fu, 0x64006400u)) - b1024;   // (k0, k4)
-    half2_t p1 = bitcast<half2_t>(and_or(v, 0x00f000f0u, 0x54005400u)) - b64;     // (k1, k5)
-    half2_t p2 = bitcast<half2_t>(and_or(v8, 0x000f000fu, 0x64006400u)) - b1024;  // (k2, k6)
-    half2_t p3 = bitcast<half2_t>(and_or(v8, 0x00f000f0u, 0x54005400u)) - b64;    // (k3, k7)
+    half2_t p0 = bitcast<half2_t>(bfi(mg.m_lo, v, mg.b_lo)) - b1024;   // (k0, k4)
+    half2_t p1 = bitcast<half2_t>(bfi(mg.m_hi, v, mg.b_hi)) - b64;     // (k1, k5)
+    half2_t p2 = bitcast<half2_t>(bfi(mg.m_lo, v8, mg.b_lo)) - b1024;  // (k2, k6)
+    half2_t p3 = bitcast<half2_t>(bfi(mg.m_hi, v8, mg.b_hi)) - b64;    // (k3, k7)
     acc = __builtin_amdgcn_fdot2(p0, act.a[4 * j + 0], acc, false);
     acc = __builtin_amdgcn_fdot2(p1, act.a[4 * j + 1], acc, false);
     acc = __builtin_amdgcn_fdot2(p2, act.a[4 * j + 2], acc, false);
@@ -76,6 +115,12 @@ __device__ __forceinline__ float dot_chunk(const uint4_t& w, const ActF16& act) 
 __device__ __forceinline__ float chunk_term(const uint4_t& w, const ActF16& act, half_t s, half_t z) {
   float d = dot_chunk(w, act);
   return (float)s * (d - (float)z * act.sum);
+}
+// same value through the biased dot: s * (sum A*(bias+u) - sum A*bias - z * sum A)
+__device__ __forceinline__ float chunk_term_biased(const uint4_t& w, const ActF16& act, half_t s, half_t z,
+                                                   const NibbleMagic& mg) {
+  const float d = dot_chunk_biased(w, act, mg);
+  return (float)s * (d - __builtin_fmaf((float)z, act.sum, act.bsum));
 }
 
 // ---- bf16: activations as floats, element-wise exact dequantisation ----------------------------
@@ -112,6 +157,159 @@ __device__ __forceinline__ float chunk_term(const uint4_t& w, const ActBF16& act
     }
   }
   return acc;
+}
+
+// ---- fp16 kernel: persistent wavefronts, activations pre-processed once per block into LDS -----
+// LDS layout for MT activation rows and `chunks` = K/32 chunks:
+//   pairs[m][j][c]  uint4  (j = 0..3: pairs 4j..4j+3 of chunk c, in unpack order)   -> lane c reads 16 B
+//   sums [m][c]     float2 (sum of the 32 activations of chunk c, bias correction of chunk c)
+// so that consecutive lanes read consecutive 16-byte words (no bank conflicts).
+//
+// A wavefront walks over "steps": step (rg, it) covers R rows (row group rg) x one 16-byte chunk
+// per lane (chunk it*64 + lane).  Row groups are dealt round-robin to all wavefronts of the grid;
+// the loads of the next step are always issued before the current step is computed, so a
+// wavefront keeps 2*R*1 KB in flight from its first instruction to its last.
+template <int R, int MT>
+__global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __restrict__ A,
+                                                                const uint8_t* __restrict__ Wp,
+                                                                const half_t* __restrict__ scales,
+                                                                const half_t* __restrict__ zeros,
+                                                                void* __restrict__ C, int m_count, int N, int K,
+                                                                int group_shift, float zero_scalar, int out_dtype) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int chunks = K >> 5;
+  uint4_t* const lds_pairs = (uint4_t*)smem;                            // [MT][4][chunks]
+  float2* const lds_sums = (float2*)(smem + (size_t)MT * chunks * 64);  // [MT][chunks]
+  const int groups = K >> group_shift;
+  {
+    const int64_t b = blockIdx.y;
+    const int64_t gsz = (int64_t)N * groups;
+    A += b * m_count * K;
+    Wp += b * N * (int64_t)(K >> 1);
+    if (scales) scales += b * gsz;
+    if (zeros) zeros += b * gsz;
+    const int64_t coff = b * m_count * N;
+    C = out_dtype == TLQ_F32 ? (void*)((float*)C + coff) : (void*)((uint16_t*)C + coff);
+  }
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: row pointers stay scalar
+  const int waves_per_block = blockDim.x >> 6;
+  const int wave_id = blockIdx.x * waves_per_block + wave;
+  const int wave_count = gridDim.x * waves_per_block;
+  const int row_groups = (N + R - 1) / R;
+  const int row_bytes = K >> 1;
+  const int iters = (chunks + 63) >> 6;  // chunk iterations per row
+  const half_t one = (half_t)1.0f;
+  const half_t zs = (half_t)zero_scalar;
+
+  // Absent scale / zero tensors: read a valid dummy location (the activations) and discard the
+  // value, so that the load sequence is branch free.
+  const bool has_s = scales != nullptr, has_z = zeros != nullptr;
+  const half_t* const sp = has_s ? scales : A;
+  const half_t* const zp = has_z ? zeros : A;
+
+  struct Stage {
+    uint4_t w[R];
+    half_t s[R], z[R];
+  };
+  auto issue = [&](Stage& st, int rg, int it) {
+    const int c = (it << 6) + lane;
+    const bool ok = c < chunks;
+    const int cc = ok ? c : chunks - 1;
+    const int gi = (cc << 5) >> group_shift;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int row = rg * R + r;
+      row = row < N ? row : N - 1;  // clamp: loads stay in bounds
+      st.w[r] = *(const uint4_t*)(Wp + (uint32_t)(row * row_bytes + (cc << 4)));
+      const uint32_t go = (uint32_t)(row * groups + gi);
+      const half_t sv = sp[has_s ? go : 0u];
+      const half_t zv = zp[has_z ? go : 0u];
+      st.s[r] = ok ? (has_s ? sv : one) : (half_t)0.0f;  // a chunk past the end contributes 0
+      st.z[r] = has_z ? zv : zs;
+    }
+  };
+
+  const NibbleMagic mg = make_nibble_magic();
+  Stage cur, nxt;
+  int rg = wave_id, it = 0;
+  const bool any = rg < row_groups;
+  if (any) issue(cur, rg, it);  // first weight loads go out before the activation staging
+
+  for (int m0 = 0; m0 < m_count; m0 += MT) {
+    if (m0 > 0) __syncthreads();  // previous pass has finished reading LDS
+    for (int i = threadIdx.x; i < chunks * MT; i += blockDim.x) {
+      const int m = (MT == 1) ? 0 : i / chunks;
+      const int c = i - m * chunks;
+      const int mm = (m0 + m < m_count) ? m0 + m : m_count - 1;
+      ActF16 act;
+      load_act(act, A, (int64_t)mm * K + (c << 5));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint4_t v = {bitcast<uint32_t>(act.a[4 * j + 0]), bitcast<uint32_t>(act.a[4 * j + 1]),
+                     bitcast<uint32_t>(act.a[4 * j + 2]), bitcast<uint32_t>(act.a[4 * j + 3])};
+        lds_pairs[(m * 4 + j) * chunks + c] = v;
+      }
+      lds_sums[m * chunks + c] = make_float2(act.sum, act.bsum);
+    }
+    __syncthreads();
+
+    if (m0 > 0) {
+      rg = wave_id;
+      it = 0;
+      if (any) issue(cur, rg, it);
+    }
+    float acc[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MT; ++m) acc[r][m] = 0.f;
+
+    while (rg < row_groups) {
+      // next step of this wavefront
+      int rg2 = rg, it2 = it + 1;
+      if (it2 == iters) {
+        it2 = 0;
+        rg2 = rg + wave_count;
+      }
+      if (rg2 < row_groups) issue(nxt, rg2, it2);
+
+      int c = (it << 6) + lane;
+      c = c < chunks ? c : chunks - 1;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        ActF16 act;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint4_t v = lds_pairs[(m * 4 + j) * chunks + c];
+          act.a[4 * j + 0] = bitcast<half2_t>(v.x);
+          act.a[4 * j + 1] = bitcast<half2_t>(v.y);
+          act.a[4 * j + 2] = bitcast<half2_t>(v.z);
+          act.a[4 * j + 3] = bitcast<half2_t>(v.w);
+        }
+        const float2 sb = lds_sums[m * chunks + c];
+        act.sum = sb.x;
+        act.bsum = sb.y;
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r][m] += chunk_term_biased(cur.w[r], act, cur.s[r], cur.z[r], mg);
+      }
+
+      if (it == iters - 1) {  // row group finished: reduce over the lanes and store
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            const float v = wave_sum_to_lane63(acc[r][m]);
+            const int row = rg * R + r;
+            if (lane == 63 && row < N && m0 + m < m_count) store_out(C, (int64_t)(m0 + m) * N + row, v, out_dtype);
+            acc[r][m] = 0.f;
+          }
+      }
+      cur = nxt;
+      rg = rg2;
+      it = it2;
+    }
+  }
 }
 
 template <typename T>
@@ -206,37 +404,80 @@ static void launch_gemv(const void* A, const void* Wp, const void* scales, const
                                                                      out_dtype);
 }
 
-// rows-per-wave / waves-per-block overrides for tuning runs (0 = automatic)
-static int g_gemv_rows = 0, g_gemv_waves = 0;
+// rows-per-wave / waves-per-block / blocks-per-CU overrides for tuning runs (0 = automatic)
+static int g_gemv_rows = 0, g_gemv_waves = 0, g_gemv_unroll = 0;
+
+static int cu_count() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+  }
+  return n;
+}
+
+template <int R, int MT>
+static int launch_gemv_f16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int batch,
+                           int M, int N, int K, int group_shift, float zero_scalar, int out_dtype, int waves_per_block,
+                           int blocks_per_cu, hipStream_t st) {
+  const size_t lds = (size_t)MT * (K / 32) * 72;
+  if (lds > 64 * 1024) {
+    set_error("tlq_gemm_w4a16(gemv): K=%d needs %zu bytes of LDS for the activations (limit 65536)", K, lds);
+    return 1;
+  }
+  const int row_groups = (int)ceil_div(N, R);
+  int blocks = (int)ceil_div(row_groups, waves_per_block);
+  const int cap = (int)ceil_div((int64_t)cu_count() * blocks_per_cu, batch);
+  if (blocks > cap) blocks = cap < 1 ? 1 : cap;
+  gemv_w4a16_f16_kernel<R, MT><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
+      (const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C, M, N, K, group_shift,
+      zero_scalar, out_dtype);
+  return 0;
+}
 
 int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch, int64_t M,
                int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st) {
-  int R = g_gemv_rows ? g_gemv_rows : 2;
-  int wpb = g_gemv_waves ? g_gemv_waves : 4;
-  const bool f16 = in_dtype == TLQ_F16;
-#define TLQ_GEMV_CASE(RR, MTT)                                                                                       \
-  if (f16)                                                                                                           \
-    launch_gemv<half_t, RR, MTT>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, (int)group, zero_scalar, out_dtype, \
-                                 wpb, st);                                                                           \
-  else                                                                                                               \
-    launch_gemv<bf16_t, RR, MTT>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, (int)group, zero_scalar, out_dtype, \
-                                 wpb, st)
-  if (M == 1) {
-    if (R == 1) {
-      TLQ_GEMV_CASE(1, 1);
+  const int wpb = g_gemv_waves ? g_gemv_waves : 4;
+  int rc = 0;
+  const bool pow2 = (group & (group - 1)) == 0;
+  if (in_dtype == TLQ_F16 && pow2) {
+    int shift = 0;
+    while (((int64_t)1 << shift) < group) ++shift;
+    // One problem of a few tens of MB is latency bound: one row per wavefront and a grid of 8
+    // blocks per CU (each wavefront then walks ~3 rows with the next row's loads in flight).
+    // Large / batched problems stream: two rows per wavefront, one block per 8 rows.
+    const bool streaming = batch * N * (K / 2) > ((int64_t)64 << 20);
+    const int R = g_gemv_rows ? g_gemv_rows : (streaming ? 2 : 1);
+    const int bpc = g_gemv_unroll ? g_gemv_unroll : (streaming ? 64 : 8);  // grid size cap, blocks per CU
+    const bool two_rows = M > 1 && (size_t)2 * (K / 32) * 72 <= 64 * 1024;
+#define TLQ_F16_CASE(RR, MTT)                                                                                       \
+  rc = launch_gemv_f16<RR, MTT>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, shift, zero_scalar,   \
+                                out_dtype, wpb, bpc, st)
+    if (two_rows) {
+      TLQ_F16_CASE(2, 2);
+    } else if (R == 1) {
+      TLQ_F16_CASE(1, 1);
     } else if (R == 4) {
-      TLQ_GEMV_CASE(4, 1);
+      TLQ_F16_CASE(4, 1);
     } else {
-      TLQ_GEMV_CASE(2, 1);
+      TLQ_F16_CASE(2, 1);
     }
+#undef TLQ_F16_CASE
+    if (rc) return rc;
+  } else if (in_dtype == TLQ_F16) {
+    // group size that is not a power of two: generic kernel
+    launch_gemv<half_t, 2, 1>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, (int)group, zero_scalar,
+                              out_dtype, wpb, st);
   } else {
-    if (R >= 2) {
-      TLQ_GEMV_CASE(2, 2);
-    } else {
-      TLQ_GEMV_CASE(1, 2);
-    }
+    // bfloat16: element-wise exact dequantisation (generic kernel)
+    if (M == 1)
+      launch_gemv<bf16_t, 2, 1>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, (int)group, zero_scalar,
+                                out_dtype, wpb, st);
+    else
+      launch_gemv<bf16_t, 1, 2>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, (int)group, zero_scalar,
+                                out_dtype, wpb, st);
   }
-#undef TLQ_GEMV_CASE
   return check_launch("tlq_gemm_w4a16(gemv)") ? 0 : 1;
 }
 
@@ -249,4 +490,5 @@ void tlq_tune_gemv(int rows_per_wave, int waves_per_block) {
   tlq::g_gemv_rows = rows_per_wave;
   tlq::g_gemv_waves = (waves_per_block < 0 || waves_per_block > 4) ? 0 : waves_per_block;
 }
+void tlq_tune_gemv_unroll(int blocks_per_cu) { tlq::g_gemv_unroll = blocks_per_cu; }
 }

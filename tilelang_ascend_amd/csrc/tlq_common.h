@@ -38,13 +38,26 @@ __device__ __forceinline__ To bitcast(const From& v) {
   return __builtin_bit_cast(To, v);
 }
 
-// (x & mask) | orv in one VALU instruction.  gfx9 VOP3 encodings cannot carry literals, so
-// the two constants live in VGPRs (the compiler hoists them out of loops).
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t orv) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(mask), "v"(orv));
-  return r;
+// Nibble-pair extraction constants, made opaque to the optimiser so that
+// (x & mask) | (magic & ~mask) is selected as one v_bfi_b32 with register operands (gfx9 VOP3
+// encodings cannot carry literals; with visible constants the compiler emits v_and + v_or).
+//   lo: bits 0..3 and 16..19  ->  fp16 1024 + u     hi: bits 4..7 and 20..23  ->  fp16 64 + u
+struct NibbleMagic {
+  uint32_t m_lo, b_lo, m_hi, b_hi;
+};
+__device__ __forceinline__ uint32_t opaque_u32(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
 }
+__device__ __forceinline__ NibbleMagic make_nibble_magic() {
+  NibbleMagic m;
+  m.m_lo = opaque_u32(0x000f000fu);
+  m.b_lo = opaque_u32(0x64006400u);
+  m.m_hi = opaque_u32(0x00f000f0u);
+  m.b_hi = opaque_u32(0x54005400u);
+  return m;
+}
+__device__ __forceinline__ uint32_t bfi(uint32_t mask, uint32_t x, uint32_t y) { return (x & mask) | (y & ~mask); }
 
 // ---- 16-bit float helpers ----------------------------------------------------------------
 // bfloat16 <-> float.  The narrowing is round-to-nearest-even (what torch's .to(bfloat16)
