@@ -17,6 +17,8 @@ int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, 
                   hipStream_t st);
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+// the tile loaders address one matrix with 32-bit byte offsets
+static bool fits32(int64_t rows, int64_t row_bytes) { return rows * row_bytes < ((int64_t)1 << 32); }
 static const int64_t kMaxDim = (int64_t)1 << 30;
 }  // namespace tlq
 
@@ -51,6 +53,7 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
     return gemv_w4a16(A, w_packed, scales, zeros, C, 1, M, N, K, group, zero_scalar, in_dtype, out_dtype, st);
   }
   TLQ_REQUIRE(N % 4 == 0, "tlq_gemm_w4a16: the MFMA kernel needs N %% 4 == 0 (got %lld)", (long long)N);
+  TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K / 2), "tlq_gemm_w4a16: a matrix spans 4 GiB or more");
   return gemm_w4a16_mfma(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, st);
 }
 
@@ -86,6 +89,7 @@ int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, in
   TLQ_REQUIRE(N % 8 == 0, "tlq_gemm_f16: N=%lld must be a multiple of 8", (long long)N);
   TLQ_REQUIRE(A && B && C, "tlq_gemm_f16: null pointer");
   TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_f16: pointers must be 16-byte aligned");
+  TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K * 2), "tlq_gemm_f16: a matrix spans 4 GiB or more");
   return gemm_f16_plain(A, B, C, M, N, K, in_dtype, out_dtype, b_layout, (hipStream_t)stream);
 }
 
@@ -99,6 +103,7 @@ int tlq_gemm_i8(const void* A, const void* B, void* C, int64_t batch, int64_t M,
   TLQ_REQUIRE(N % 16 == 0, "tlq_gemm_i8: N=%lld must be a multiple of 16", (long long)N);
   TLQ_REQUIRE(A && B && C, "tlq_gemm_i8: null pointer");
   TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_i8: pointers must be 16-byte aligned");
+  TLQ_REQUIRE(fits32(M, K) && fits32(N, K), "tlq_gemm_i8: a matrix spans 4 GiB or more");
   return gemm_i8_i32(A, B, C, batch, M, N, K, b_layout, (hipStream_t)stream);
 }
 
@@ -111,6 +116,7 @@ int tlq_gemm_w4a8(const void* A, const void* w_packed, void* C, int64_t M, int64
   TLQ_REQUIRE(N % 4 == 0, "tlq_gemm_w4a8: N=%lld must be a multiple of 4", (long long)N);
   TLQ_REQUIRE(A && w_packed && C, "tlq_gemm_w4a8: null pointer");
   TLQ_REQUIRE(aligned16(A) && aligned16(w_packed) && aligned16(C), "tlq_gemm_w4a8: pointers must be 16-byte aligned");
+  TLQ_REQUIRE(fits32(M, K) && fits32(N, K / 2), "tlq_gemm_w4a8: a matrix spans 4 GiB or more");
   return gemm_w4a8_i32(A, w_packed, C, M, N, K, sign_mode, (hipStream_t)stream);
 }
 
@@ -129,6 +135,7 @@ int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void*
   TLQ_REQUIRE(A && B && C, "tlq_gemm_w8a8: null pointer");
   TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_w8a8: pointers must be 16-byte aligned");
   TLQ_REQUIRE(((uintptr_t)scale_a & 3) == 0 && ((uintptr_t)scale_b & 3) == 0, "tlq_gemm_w8a8: scales misaligned");
+  TLQ_REQUIRE(fits32(M, K) && fits32(N, K), "tlq_gemm_w8a8: a matrix spans 4 GiB or more");
   return gemm_w8a8_rescale(A, B, scale_a, scale_b, C, batch, M, N, K, n_scale_b, b_layout, out_dtype,
                            (hipStream_t)stream);
 }

@@ -4,7 +4,7 @@
 //
 // Everything is expressed in BYTES of K: one stage is 128 bytes of K per row (64 fp16/bf16
 // or 128 int8 values).  Both operand tiles live in LDS as [rows][128 B] with the 16-byte
-// chunk index XOR-swizzled by the row, and one 16x16 MFMA k-step consumes one 16-byte chunk
+// chunk index XOR-swizzled by (row & 7), and one 16x16 MFMA k-step consumes one 16-byte chunk
 // per lane from each operand (v_mfma_f32_16x16x32_{f16,bf16}: 8 values, v_mfma_i32_16x16x64_i8:
 // 16 values), so the loop body is identical for all element types.
 //
@@ -14,9 +14,15 @@
 // writes 8/16-byte vectors.
 //
 // Pipeline: global -> registers -> (convert / dequantise / transpose) -> LDS, double
-// buffered.  The global loads of stage t+1 are issued before the MFMAs of stage t; their
-// conversion and LDS store follow the MFMAs; one barrier per stage.
+// buffered.  The global loads of stage t+1 are issued at the top of stage t; their conversion
+// and LDS stores are cut into pieces that follow every group of MFMAs of stage t; one barrier
+// per stage.  Addressing is arranged so that the loop needs almost no address arithmetic:
+// global loads use a scalar base that advances per stage plus a loop-invariant 32-bit lane
+// offset, LDS accesses use a loop-invariant lane offset plus an immediate (the swizzle depends
+// only on row bits 0..2, so rows 8 apart differ by a constant).
 #pragma once
+
+#include <type_traits>
 
 #include "tlq_common.h"
 
@@ -24,39 +30,41 @@ namespace tlq {
 
 constexpr int kStageBytes = 128;
 
-// 16-byte chunk swizzle.  Makes the MFMA operand reads (16 consecutive rows, same logical
-// chunk), the row-copy stores (8 lanes per row) and the transposing stores (rows 16 apart)
-// spread over the LDS banks.
-__device__ __forceinline__ int lds_swz(int row) { return (row & 7) ^ ((row >> 3) & 1) ^ ((row >> 4) & 7); }
+// 16-byte chunk swizzle.  Measured on gfx950 with the LDS bank-conflict counter: conflict free
+// for the MFMA operand reads (16 consecutive rows, one logical chunk per 16 lanes), the row-copy
+// stores (8 lanes per row) and the dequantising stores (2 lanes per row, 4 chunks each).
+__device__ __forceinline__ int lds_swz(int row) { return row & 7; }
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * kStageBytes + ((chunk ^ lds_swz(row)) << 4); }
 
 // ---- MFMA wrappers ----------------------------------------------------------------------
 struct MmaF16 {
   typedef float4_t acc_t;
-  static constexpr int elem_bytes = 2;
   static __device__ __forceinline__ acc_t mma(const uint4_t& a, const uint4_t& b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<half8_t>(a), bitcast<half8_t>(b), c, 0, 0, 0);
   }
 };
 struct MmaBF16 {
   typedef float4_t acc_t;
-  static constexpr int elem_bytes = 2;
   static __device__ __forceinline__ acc_t mma(const uint4_t& a, const uint4_t& b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<bf16x8_t>(a), bitcast<bf16x8_t>(b), c, 0, 0, 0);
   }
 };
 struct MmaI8 {
   typedef int4_t acc_t;
-  static constexpr int elem_bytes = 1;
   static __device__ __forceinline__ acc_t mma(const uint4_t& a, const uint4_t& b, acc_t c) {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(bitcast<int4_t>(a), bitcast<int4_t>(b), c, 0, 0, 0);
   }
 };
 
 // ---- tile loaders -----------------------------------------------------------------------
-// A loader owns a Regs type (what one thread keeps in flight for one stage) and two phases:
-//   gload (regs, kt, tid): issue the global loads of stage kt
-//   lstore(regs, lds, tid): convert and write the stage into an LDS tile of ROWS x 128 B
+// A loader owns a Regs type (what one thread keeps in flight for one stage) and
+//   Loader(params, batch, row0, rows_total, tid)   per-thread offsets, computed once
+//   gload<TAIL>(regs, kt)                          issue the global loads of stage kt; TAIL = the
+//                                                  stage may extend past the end of K (zero fill)
+//   lstore_piece(regs, lds_tile, pc, np)           convert + store piece pc of np of the stage
+//   lstore(regs, lds_tile)                         the whole stage
+// Store work is counted in UNITS; piece pc handles the units u with u * np / UNITS == pc.
+// Loaders assume a matrix (one batch) spans less than 4 GiB (checked on the host).
 
 // Plain row-major [rows, k_bytes] source (activations of every kind, weights stored [N, K]).
 template <int ROWS, int NT>
@@ -64,6 +72,8 @@ struct RowLoader {
   static constexpr int SLOTS = ROWS * 8;  // 16-byte chunks per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
+  static constexpr int UNITS = PASSES;
+  static_assert(PASSES == 1 || (NT / 8) % 8 == 0, "pass stride must keep the swizzle phase");
   struct Params {
     const uint8_t* base;   // element [0, 0] of batch 0
     int64_t ld;            // row pitch in bytes
@@ -73,90 +83,119 @@ struct RowLoader {
   struct Regs {
     uint4_t v[PASSES];
   };
-  const uint8_t* base;
-  int64_t ld;
-  int rows_valid;
+  const uint8_t* base;    // uniform
+  uint32_t voff[PASSES];  // per lane: row * ld + chunk * 16
+  uint32_t loff;          // per lane: LDS offset of pass 0
+  int kb_lane;            // chunk * 16
   int k_bytes;
+  bool active;  // this thread has a slot in the (partial) last pass
 
-  __device__ __forceinline__ RowLoader(const Params& p, int batch, int row0, int rows_total)
-      : base(p.base + batch * p.batch_stride + (int64_t)row0 * p.ld), ld(p.ld), rows_valid(rows_total - row0),
-        k_bytes((int)p.k_bytes) {}
-
-  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
+  __device__ __forceinline__ RowLoader(const Params& p, int batch, int row0, int rows_total, int tid)
+      : base(p.base + batch * p.batch_stride + (int64_t)row0 * p.ld), k_bytes((int)p.k_bytes) {
+    const int rows_valid = rows_total - row0;
     const int chunk = tid & 7;
-    const int kb = kt * kStageBytes + chunk * 16;
+    kb_lane = chunk * 16;
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int slot = p * NT + tid;
-      int row = slot >> 3;
-      row = row < rows_valid ? row : rows_valid - 1;
-      uint4_t v = {0u, 0u, 0u, 0u};
-      if (kb < k_bytes && (!PARTIAL || slot < SLOTS)) v = *(const uint4_t*)(base + (int64_t)row * ld + kb);
-      r.v[p] = v;
+    for (int ps = 0; ps < PASSES; ++ps) {
+      int row = (ps * NT + tid) >> 3;
+      row = row < rows_valid ? row : rows_valid - 1;  // clamp: loads stay in bounds, results are masked later
+      voff[ps] = (uint32_t)row * (uint32_t)p.ld + (uint32_t)kb_lane;
+    }
+    loff = (uint32_t)lds_off(tid >> 3, chunk);
+    active = !PARTIAL || ((PASSES - 1) * NT + tid) < SLOTS;
+  }
+
+  template <bool TAIL>
+  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+    const uint8_t* sb = base + (int64_t)kt * kStageBytes;
+    if (!TAIL) {
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) r.v[ps] = *(const uint4_t*)(sb + voff[ps]);
+    } else {
+      const bool ok = kt * kStageBytes + kb_lane < k_bytes;
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) {
+        uint4_t v = *(const uint4_t*)(ok ? sb + voff[ps] : base + (voff[ps] - kb_lane));
+        if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
+        r.v[ps] = v;
+      }
     }
   }
-  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
-    const int chunk = tid & 7;
+  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int slot = p * NT + tid;
-      if (PARTIAL && slot >= SLOTS) continue;
-      *(uint4_t*)(lds + lds_off(slot >> 3, chunk)) = r.v[p];
+    for (int ps = 0; ps < PASSES; ++ps) {
+      if (ps * np / UNITS != pc) continue;
+      if (PARTIAL && ps == PASSES - 1 && !active) continue;
+      *(uint4_t*)(lds + loff + ps * (NT / 8) * kStageBytes) = r.v[ps];
     }
   }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
 };
 
 // int8 source stored [K, N] (N contiguous): 4(k) x 16(n) register blocks are byte-transposed
 // with v_perm_b32 so that the LDS tile is [n][k] like every other operand.
 template <int ROWS, int NT>
 struct I8KNLoader {
-  static constexpr int NBLK = ROWS / 16;                // 16-column blocks per tile
-  static constexpr int PASSES = (32 * NBLK) / NT;       // 128 k = 32 blocks of 4 rows
+  static constexpr int NBLK = ROWS / 16;           // 16-column blocks per tile
+  static constexpr int PASSES = (32 * NBLK) / NT;  // 128 k = 32 blocks of 4 rows
+  static constexpr int UNITS = PASSES * 4;
   static_assert(PASSES >= 1 && (32 * NBLK) % NT == 0 && NT % NBLK == 0, "bad transposing loader shape");
   struct Params {
-    const uint8_t* base;   // B[0, 0] of batch 0
-    int64_t ld;            // bytes per k row (= N)
+    const uint8_t* base;  // B[0, 0] of batch 0
+    int64_t ld;           // bytes per k row (= N)
     int64_t batch_stride;
-    int64_t k_total;       // K
+    int64_t k_total;  // K
   };
   struct Regs {
     uint4_t v[PASSES][4];
   };
-  const uint8_t* base;
-  int64_t ld;
+  const uint8_t* base;  // uniform
+  uint32_t ld;
+  uint32_t voff;  // per lane: kblk0 * 4 * ld + col
+  int kblk0, nblk;
   int k_total;
 
   // cols_total must be a multiple of 16 (checked on the host)
-  __device__ __forceinline__ I8KNLoader(const Params& p, int batch, int col0, int cols_total)
-      : base(p.base + batch * p.batch_stride + col0), ld(p.ld), k_total((int)p.k_total), cols_valid(cols_total - col0) {}
-  int cols_valid;
-
-  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
-    const int nblk = tid % NBLK;
+  __device__ __forceinline__ I8KNLoader(const Params& p, int batch, int col0, int cols_total, int tid)
+      : base(p.base + batch * p.batch_stride + col0), ld((uint32_t)p.ld), k_total((int)p.k_total) {
+    const int cols_valid = cols_total - col0;
+    nblk = tid % NBLK;
+    kblk0 = tid / NBLK;
     int col = nblk * 16;
     col = col < cols_valid ? col : cols_valid - 16;  // clamp whole 16-column blocks
+    voff = (uint32_t)(kblk0 * 4) * ld + (uint32_t)col;
+  }
+
+  template <bool TAIL>
+  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+    const uint8_t* sb = base + (int64_t)kt * kStageBytes * ld;
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int kblk = p * (NT / NBLK) + tid / NBLK;
+    for (int ps = 0; ps < PASSES; ++ps) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int k = kt * kStageBytes + kblk * 4 + i;
-        uint4_t v = {0u, 0u, 0u, 0u};
-        if (k < k_total) v = *(const uint4_t*)(base + (int64_t)k * ld + col);
-        r.v[p][i] = v;
+        const uint32_t o = voff + (uint32_t)(ps * (NT / NBLK) * 4 + i) * ld;
+        if (!TAIL) {
+          r.v[ps][i] = *(const uint4_t*)(sb + o);
+        } else {
+          const int k = kt * kStageBytes + (ps * (NT / NBLK) + kblk0) * 4 + i;
+          const bool ok = k < k_total;
+          uint4_t v = *(const uint4_t*)(ok ? sb + o : base + (voff - (uint32_t)(kblk0 * 4) * ld));
+          if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
+          r.v[ps][i] = v;
+        }
       }
     }
   }
-  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
-    const int nblk = tid % NBLK;
+  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int kblk = p * (NT / NBLK) + tid / NBLK;
+    for (int ps = 0; ps < PASSES; ++ps) {
+      const int kblk = ps * (NT / NBLK) + kblk0;
       const int chunk = kblk >> 2;
       const int within = (kblk & 3) * 4;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const uint32_t a = r.v[p][0][c], b = r.v[p][1][c], cc = r.v[p][2][c], d = r.v[p][3][c];
+        if ((ps * 4 + c) * np / UNITS != pc) continue;
+        const uint32_t a = r.v[ps][0][c], b = r.v[ps][1][c], cc = r.v[ps][2][c], d = r.v[ps][3][c];
         // 4x4 byte transpose: t[j] = (a.byte j, b.byte j, c.byte j, d.byte j)
         const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400u);
         const uint32_t ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602u);
@@ -174,6 +213,7 @@ struct I8KNLoader {
       }
     }
   }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
 };
 
 // ---- epilogues ----------------------------------------------------------------------------
@@ -199,8 +239,8 @@ struct EpiFloat {  // fp32 accumulators -> f16 / bf16 / f32
         *(uint2_t*)((half_t*)p.C + idx) = bitcast<uint2_t>(h);
       } else {
         uint2_t o;
-        o.x = float_to_bf16_bits(acc[0]) | (float_to_bf16_bits(acc[1]) << 16);
-        o.y = float_to_bf16_bits(acc[2]) | (float_to_bf16_bits(acc[3]) << 16);
+        o.x = pack_bf16x2(acc[0], acc[1]);
+        o.y = pack_bf16x2(acc[2], acc[3]);
         *(uint2_t*)((uint16_t*)p.C + idx) = o;
       }
     } else {
@@ -271,40 +311,50 @@ struct EpiRescale {
   }
 };
 
-// ---- the kernel -----------------------------------------------------------------------------
-template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(WM* WN * 64, 1) void gemm_mfma_kernel(typename AL::Params pa, typename WL::Params pw,
-                                                                    typename Epi::Params pe, int M, int N, int KT,
-                                                                    int tiles_m, int tiles_n) {
-  constexpr int NT = WM * WN * 64;
-  constexpr int TM = BM / WM / 16;  // 16-row activation tiles per wave
-  constexpr int TN = BN / WN / 16;  // 16-row weight tiles per wave
-  extern __shared__ __align__(16) uint8_t smem[];
-  uint8_t* const ldsA0 = smem;
-  uint8_t* const ldsW0 = smem + 2 * BM * kStageBytes;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int r16 = lane & 15;
-  const int q = lane >> 4;
-  const int wave_m0 = (wave % WM) * (BM / WM);
-  const int wave_n0 = (wave / WM) * (BN / WN);
-
-  // Work-group -> tile.  Consecutive hardware ids are dealt round-robin to the 8 XCDs; give
-  // every XCD a contiguous range of logical tiles so that tiles sharing an activation panel
-  // also share an L2.
+// Work-group -> tile.  Consecutive hardware ids are dealt round-robin to the 8 XCDs; give
+// every XCD a contiguous range of logical tiles so that tiles sharing an activation panel
+// also share an L2.
+struct TileCoord {
+  int batch, m0, n0;
+};
+template <int BM, int BN>
+__device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n) {
   const int total = gridDim.x;
   int lid = blockIdx.x;
   if ((total & 7) == 0) lid = (lid & 7) * (total >> 3) + (lid >> 3);
   const int per_batch = tiles_m * tiles_n;
-  const int batch = lid / per_batch;
-  const int rem = lid - batch * per_batch;
-  const int m0 = (rem / tiles_n) * BM;
-  const int n0 = (rem % tiles_n) * BN;
+  TileCoord t;
+  t.batch = lid / per_batch;
+  const int rem = lid - t.batch * per_batch;
+  t.m0 = (rem / tiles_n) * BM;
+  t.n0 = (rem % tiles_n) * BN;
+  return t;
+}
 
-  AL al(pa, batch, m0, M);
-  WL wl(pw, batch, n0, N);
+// ---- the kernel -----------------------------------------------------------------------------
+template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma_kernel(
+    typename AL::Params pa, typename WL::Params pw, typename Epi::Params pe, int M, int N, int KT, int k_tail,
+    int tiles_m, int tiles_n) {
+  constexpr int TM = BM / WM / 16;  // 16-row activation tiles per wave
+  constexpr int TN = BN / WN / 16;  // 16-row weight tiles per wave
+  constexpr int A_TILE = BM * kStageBytes, W_TILE = BN * kStageBytes;
+  extern __shared__ __align__(16) uint8_t smem[];
+  uint8_t* const ldsA0 = smem;
+  uint8_t* const ldsW0 = smem + 2 * A_TILE;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15;
+  const int q = lane >> 4;
+  const int wave_m0 = (wave % WM) * (BM / WM);
+  const int wave_n0 = (wave / WM) * (BN / WN);
+  const TileCoord tc = tile_of_block<BM, BN>(tiles_m, tiles_n);
+  const int m0 = tc.m0, n0 = tc.n0, batch = tc.batch;
+
+  AL al(pa, batch, m0, M, tid);
+  WL wl(pw, batch, n0, N, tid);
   typename AL::Regs ra;
   typename WL::Regs rw;
 
@@ -314,40 +364,76 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_mfma_kernel(typename AL::
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = typename Mma::acc_t{0, 0, 0, 0};
 
-  al.gload(ra, 0, tid);
-  wl.gload(rw, 0, tid);
-  al.lstore(ra, ldsA0, tid);
-  wl.lstore(rw, ldsW0, tid);
-  __syncthreads();
+  // Per-lane LDS offset of an operand fragment for k-step 0 (row r16 of a 16-row tile, logical
+  // chunk q).  K-step 1 uses chunk q + 4, i.e. this offset ^ 64; tiles 16 rows apart add 2048.
+  const uint32_t fo = (uint32_t)lds_off(r16, q);
+  const uint8_t* const fragA = ldsA0 + wave_m0 * kStageBytes;
+  const uint8_t* const fragW = ldsW0 + wave_n0 * kStageBytes;
 
-  for (int kt = 0; kt < KT; ++kt) {
-    const int cur = kt & 1;
-    const uint8_t* la = ldsA0 + cur * BM * kStageBytes;
-    const uint8_t* lw = ldsW0 + cur * BN * kStageBytes;
-    const bool more = kt + 1 < KT;
-    if (more) {
-      al.gload(ra, kt + 1, tid);
-      wl.gload(rw, kt + 1, tid);
-    }
+  // One stage: 2 k-steps x TN weight tiles x TM activation tiles of MFMAs on buffer CUR.  When
+  // FILL, the conversion + LDS stores of the next stage (already in registers) are cut into
+  // 2*TN pieces and one piece follows every TM MFMAs, so that the VALU / LDS-store work runs in
+  // the shadow of the MFMAs (this wavefront's and the other wavefront's on the same SIMD).
+  constexpr int NP = 2 * TN;   // pieces per stage
+  constexpr int NPA = NP / 2;  // first half: activation stores, second half: weight conversion
+  auto stage = [&](int cur, auto fill_tag) {
+    constexpr bool FILL = decltype(fill_tag)::value;
+    const uint8_t* la = fragA + cur * A_TILE;
+    const uint8_t* lw = fragW + cur * W_TILE;
+    uint8_t* na = ldsA0 + (cur ^ 1) * A_TILE;
+    uint8_t* nw = ldsW0 + (cur ^ 1) * W_TILE;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const int chunk = ks * 4 + q;
+      const uint32_t o = fo ^ (uint32_t)(ks << 6);
       uint4_t wf[TN], af[TM];
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) wf[tn] = *(const uint4_t*)(lw + lds_off(wave_n0 + tn * 16 + r16, chunk));
+      for (int tn = 0; tn < TN; ++tn) wf[tn] = *(const uint4_t*)(lw + o + tn * 16 * kStageBytes);
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) af[tm] = *(const uint4_t*)(la + lds_off(wave_m0 + tm * 16 + r16, chunk));
+      for (int tm = 0; tm < TM; ++tm) af[tm] = *(const uint4_t*)(la + o + tm * 16 * kStageBytes);
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn)
+      for (int tn = 0; tn < TN; ++tn) {
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = Mma::mma(wf[tn], af[tm], acc[tn][tm]);
+        if (FILL) {
+          const int pc = ks * TN + tn;
+          if (pc < NPA)
+            al.lstore_piece(ra, na, pc, NPA);
+          else
+            wl.lstore_piece(rw, nw, pc - NPA, NP - NPA);
+        }
+      }
     }
-    if (more) {
-      al.lstore(ra, ldsA0 + (cur ^ 1) * BM * kStageBytes, tid);
-      wl.lstore(rw, ldsW0 + (cur ^ 1) * BN * kStageBytes, tid);
-    }
+  };
+
+  // prologue: stage 0 into buffer 0
+  if (KT == 1 && k_tail) {
+    al.template gload<true>(ra, 0);
+    wl.template gload<true>(rw, 0);
+  } else {
+    al.template gload<false>(ra, 0);
+    wl.template gload<false>(rw, 0);
+  }
+  al.lstore(ra, ldsA0);
+  wl.lstore(rw, ldsW0);
+  __syncthreads();
+
+  // Stages 0 .. KT-2 compute and fill.  Only the load of stage KT-1 can be a partial stage.
+  const int last_full = k_tail ? KT - 2 : KT - 1;  // highest stage loadable without the tail path
+  int kt = 0;
+  for (; kt + 1 <= last_full; ++kt) {
+    al.template gload<false>(ra, kt + 1);
+    wl.template gload<false>(rw, kt + 1);
+    stage(kt & 1, std::true_type{});
     __syncthreads();
   }
+  if (kt + 1 < KT) {  // the partial last stage
+    al.template gload<true>(ra, kt + 1);
+    wl.template gload<true>(rw, kt + 1);
+    stage(kt & 1, std::true_type{});
+    __syncthreads();
+    ++kt;
+  }
+  if (KT > 0) stage((KT - 1) & 1, std::false_type{});
 
   Epi epi(pe, batch);
 #pragma unroll
@@ -380,7 +466,9 @@ int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, co
     return 1;
   }
   const int KT = (int)ceil_div(k_bytes, kStageBytes);
-  kern<<<(unsigned)blocks, WM * WN * 64, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, KT, (int)tiles_m, (int)tiles_n);
+  const int k_tail = (k_bytes % kStageBytes) != 0;
+  kern<<<(unsigned)blocks, WM * WN * 64, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, KT, k_tail, (int)tiles_m,
+                                                          (int)tiles_n);
   return check_launch(what) ? 0 : 1;
 }
 

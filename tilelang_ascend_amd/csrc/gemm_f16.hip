@@ -10,6 +10,7 @@ template <int ROWS, int NT>
 struct H16KNLoader {
   static constexpr int NBLK = ROWS / 8;            // 8-column blocks per tile
   static constexpr int PASSES = (16 * NBLK) / NT;  // 64 k = 16 blocks of 4 rows
+  static constexpr int UNITS = PASSES * 4;
   static_assert(PASSES >= 1 && (16 * NBLK) % NT == 0 && NT % NBLK == 0, "bad transposing loader shape");
   struct Params {
     const uint8_t* base;  // B[0, 0]
@@ -20,41 +21,54 @@ struct H16KNLoader {
   struct Regs {
     uint4_t v[PASSES][4];
   };
-  const uint8_t* base;
-  int64_t ld;
+  const uint8_t* base;  // uniform
+  uint32_t ld;
+  uint32_t voff;  // per lane: kblk0 * 4 * ld + col * 2
+  int kblk0, nblk;
   int k_total;
-  int cols_valid;
 
   // cols_total must be a multiple of 8 (checked on the host)
-  __device__ __forceinline__ H16KNLoader(const Params& p, int batch, int col0, int cols_total)
-      : base(p.base + batch * p.batch_stride + (int64_t)col0 * 2), ld(p.ld), k_total((int)p.k_total),
-        cols_valid(cols_total - col0) {}
-
-  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
-    int col = (tid % NBLK) * 8;
+  __device__ __forceinline__ H16KNLoader(const Params& p, int batch, int col0, int cols_total, int tid)
+      : base(p.base + batch * p.batch_stride + (int64_t)col0 * 2), ld((uint32_t)p.ld), k_total((int)p.k_total) {
+    const int cols_valid = cols_total - col0;
+    nblk = tid % NBLK;
+    kblk0 = tid / NBLK;
+    int col = nblk * 8;
     col = col < cols_valid ? col : cols_valid - 8;
+    voff = (uint32_t)(kblk0 * 4) * ld + (uint32_t)(col * 2);
+  }
+
+  template <bool TAIL>
+  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+    const uint8_t* sb = base + (int64_t)kt * 64 * ld;
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int kblk = p * (NT / NBLK) + tid / NBLK;
+    for (int ps = 0; ps < PASSES; ++ps) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int k = kt * 64 + kblk * 4 + i;
-        uint4_t v = {0u, 0u, 0u, 0u};
-        if (k < k_total) v = *(const uint4_t*)(base + (int64_t)k * ld + col * 2);
-        r.v[p][i] = v;
+        const uint32_t o = voff + (uint32_t)(ps * (NT / NBLK) * 4 + i) * ld;
+        if (!TAIL) {
+          r.v[ps][i] = *(const uint4_t*)(sb + o);
+        } else {
+          const int k = kt * 64 + (ps * (NT / NBLK) + kblk0) * 4 + i;
+          const bool ok = k < k_total;
+          uint4_t v = *(const uint4_t*)(ok ? sb + o : base + (voff - (uint32_t)(kblk0 * 4) * ld));
+          if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
+          r.v[ps][i] = v;
+        }
       }
     }
   }
-  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
-    const int nblk = tid % NBLK;
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
+  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int kblk = p * (NT / NBLK) + tid / NBLK;
+    for (int ps = 0; ps < PASSES; ++ps) {
+      const int kblk = ps * (NT / NBLK) + kblk0;
       const int chunk = kblk >> 1;
       const int within = (kblk & 1) * 8;
 #pragma unroll
       for (int w = 0; w < 4; ++w) {  // word w of each row holds columns 2w, 2w+1
-        const uint32_t a = r.v[p][0][w], b = r.v[p][1][w], c = r.v[p][2][w], d = r.v[p][3][w];
+        if ((ps * 4 + w) * np / UNITS != pc) continue;
+        const uint32_t a = r.v[ps][0][w], b = r.v[ps][1][w], c = r.v[ps][2][w], d = r.v[ps][3][w];
         uint2_t even, odd;
         even.x = __builtin_amdgcn_perm(b, a, 0x05040100u);  // (a.lo, b.lo)
         even.y = __builtin_amdgcn_perm(d, c, 0x05040100u);  // (c.lo, d.lo)
@@ -89,7 +103,7 @@ static int dispatch_f16(const void* A, const void* B, void* C, int64_t M, int64_
                         int b_layout, hipStream_t st) {
   if (M <= 128 || ceil_div(M, 256) * ceil_div(N, 256) < 128)
     return run_f16<Mma, 128, 128, 2, 2>(A, B, C, M, N, K, out_dtype, b_layout, st);
-  return run_f16<Mma, 256, 256, 2, 2>(A, B, C, M, N, K, out_dtype, b_layout, st);
+  return run_f16<Mma, 256, 256, 2, 4>(A, B, C, M, N, K, out_dtype, b_layout, st);
 }
 
 int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,

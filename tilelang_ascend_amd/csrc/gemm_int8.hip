@@ -14,6 +14,8 @@ struct W4I8Loader {
   static constexpr int SLOTS = ROWS * 4;
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
+  static constexpr int UNITS = PASSES;
+  static_assert(PASSES == 1 || (NT / 4) % 8 == 0, "pass stride must keep the swizzle phase");
   struct Params {
     const uint8_t* wp;
     int64_t row_bytes;  // K / 2
@@ -22,25 +24,42 @@ struct W4I8Loader {
   struct Regs {
     uint4_t v[PASSES];
   };
-  const uint8_t* base;
-  int64_t row_bytes;
-  int rows_valid;
-  int sign_mode;
+  const uint8_t* base;    // uniform
+  uint32_t voff[PASSES];  // per lane: row * row_bytes + quarter * 16
+  uint32_t loff[2];       // per lane: LDS offsets of the two chunks this lane writes (pass 0)
+  int kb_lane, row_bytes, sign_mode;
+  bool active;
 
-  __device__ __forceinline__ W4I8Loader(const Params& p, int /*batch*/, int row0, int rows_total)
-      : base(p.wp + (int64_t)row0 * p.row_bytes), row_bytes(p.row_bytes), rows_valid(rows_total - row0),
-        sign_mode(p.sign_mode) {}
-
-  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
+  __device__ __forceinline__ W4I8Loader(const Params& p, int /*batch*/, int row0, int rows_total, int tid)
+      : base(p.wp + (int64_t)row0 * p.row_bytes), row_bytes((int)p.row_bytes), sign_mode(p.sign_mode) {
+    const int rows_valid = rows_total - row0;
+    const int quarter = tid & 3;
+    kb_lane = quarter * 16;
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-      const int slot = ps * NT + tid;
-      int row = slot >> 2;
+      int row = (ps * NT + tid) >> 2;
       row = row < rows_valid ? row : rows_valid - 1;
-      const int kb = kt * 64 + (slot & 3) * 16;
-      uint4_t v = {0u, 0u, 0u, 0u};
-      if (kb < row_bytes && (!PARTIAL || slot < SLOTS)) v = *(const uint4_t*)(base + (int64_t)row * row_bytes + kb);
-      r.v[ps] = v;
+      voff[ps] = (uint32_t)row * (uint32_t)p.row_bytes + (uint32_t)kb_lane;
+    }
+    loff[0] = (uint32_t)lds_off(tid >> 2, quarter * 2 + 0);
+    loff[1] = (uint32_t)lds_off(tid >> 2, quarter * 2 + 1);
+    active = !PARTIAL || ((PASSES - 1) * NT + tid) < SLOTS;
+  }
+
+  template <bool TAIL>
+  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+    const uint8_t* sb = base + (int64_t)kt * 64;
+    if (!TAIL) {
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) r.v[ps] = *(const uint4_t*)(sb + voff[ps]);
+    } else {
+      const bool ok = kt * 64 + kb_lane < row_bytes;
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) {
+        uint4_t v = *(const uint4_t*)(ok ? sb + voff[ps] : base + (voff[ps] - kb_lane));
+        if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
+        r.v[ps] = v;
+      }
     }
   }
   // four nibbles held one per byte (0..15) -> four int8 under the sign convention
@@ -57,22 +76,22 @@ struct W4I8Loader {
     d0 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);    // k0 k1 k2 k3
     d1 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);    // k4 k5 k6 k7
   }
-  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
+  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-      const int slot = ps * NT + tid;
-      if (PARTIAL && slot >= SLOTS) continue;
-      const int row = slot >> 2;
-      const int quarter = slot & 3;
+      if (ps * np / UNITS != pc) continue;
+      if (PARTIAL && ps == PASSES - 1 && !active) continue;
       uint32_t d[8];
       expand(r.v[ps].x, d[0], d[1]);
       expand(r.v[ps].y, d[2], d[3]);
       expand(r.v[ps].z, d[4], d[5]);
       expand(r.v[ps].w, d[6], d[7]);
-      *(uint4_t*)(lds + lds_off(row, quarter * 2 + 0)) = uint4_t{d[0], d[1], d[2], d[3]};
-      *(uint4_t*)(lds + lds_off(row, quarter * 2 + 1)) = uint4_t{d[4], d[5], d[6], d[7]};
+      uint8_t* dst = lds + ps * (NT / 4) * kStageBytes;
+      *(uint4_t*)(dst + loff[0]) = uint4_t{d[0], d[1], d[2], d[3]};
+      *(uint4_t*)(dst + loff[1]) = uint4_t{d[4], d[5], d[6], d[7]};
     }
   }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
 };
 
 // ---- launch helpers -----------------------------------------------------------------------
@@ -111,7 +130,7 @@ static int dispatch_i8(const void* A, const void* B, const typename Epi::Params&
       case 128:
         TLQ_RUN(128, 128, 2, 2)
       default:
-        TLQ_RUN(256, 256, 2, 2)
+        TLQ_RUN(256, 256, 2, 4)
     }
 #undef TLQ_RUN
   } else {
@@ -127,7 +146,7 @@ static int dispatch_i8(const void* A, const void* B, const typename Epi::Params&
       case 128:
         TLQ_RUN(128, 128, 2, 2)
       default:
-        TLQ_RUN(256, 256, 2, 2)
+        TLQ_RUN(256, 256, 2, 4)
     }
 #undef TLQ_RUN
   }
@@ -161,7 +180,7 @@ int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, 
     case 128:
       TLQ_RUN(128, 128, 2, 2)
     default:
-      TLQ_RUN(256, 256, 2, 2)
+      TLQ_RUN(256, 256, 2, 4)
   }
 #undef TLQ_RUN
 }

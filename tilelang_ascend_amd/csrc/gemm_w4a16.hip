@@ -23,20 +23,20 @@
 
 namespace tlq {
 
-template <typename T>
+// FOLD is a compile-time flag: the decision is taken once per stage, not per element.
+template <typename T, bool FOLD>
 struct Expand8;
 
-template <>
-struct Expand8<half_t> {
+template <bool FOLD>
+struct Expand8<half_t, FOLD> {
   half2_t s2, z2, b_lo, b_hi;
   NibbleMagic mg;
-  bool fold;
-  __device__ __forceinline__ Expand8(half_t s, half_t z, bool fold_, const NibbleMagic& mg_) : mg(mg_), fold(fold_) {
+  __device__ __forceinline__ Expand8(half_t s, half_t z, const NibbleMagic& mg_) : mg(mg_) {
     s2 = half2_t{s, s};
     z2 = half2_t{z, z};
     // with an integer zero point 1024+z and 64+z are exact binary16 values
-    const half_t zl = fold_ ? (half_t)(1024.0f + (float)z) : (half_t)1024.0f;
-    const half_t zh = fold_ ? (half_t)(64.0f + (float)z) : (half_t)64.0f;
+    const half_t zl = FOLD ? (half_t)(1024.0f + (float)z) : (half_t)1024.0f;
+    const half_t zh = FOLD ? (half_t)(64.0f + (float)z) : (half_t)64.0f;
     b_lo = half2_t{zl, zl};
     b_hi = half2_t{zh, zh};
   }
@@ -46,7 +46,7 @@ struct Expand8<half_t> {
     half2_t p1 = bitcast<half2_t>(bfi(mg.m_hi, v, mg.b_hi)) - b_hi;   // (k1, k5)
     half2_t p2 = bitcast<half2_t>(bfi(mg.m_lo, v8, mg.b_lo)) - b_lo;  // (k2, k6)
     half2_t p3 = bitcast<half2_t>(bfi(mg.m_hi, v8, mg.b_hi)) - b_hi;  // (k3, k7)
-    if (!fold) {
+    if (!FOLD) {
       p0 = p0 - z2;
       p1 = p1 - z2;
       p2 = p2 - z2;
@@ -67,18 +67,17 @@ struct Expand8<half_t> {
   }
 };
 
-template <>
-struct Expand8<bf16_t> {
+template <bool FOLD>
+struct Expand8<bf16_t, FOLD> {
   float sf, zf, c;
-  bool fold;
-  __device__ __forceinline__ Expand8(bf16_t s, bf16_t z, bool fold_, const NibbleMagic&) : fold(fold_) {
+  __device__ __forceinline__ Expand8(bf16_t s, bf16_t z, const NibbleMagic&) {
     sf = to_float(s);
     zf = to_float(z);
     c = -(zf * sf);  // exact in fp32 for a small integer zero point (8 x 8 significant bits)
   }
   __device__ __forceinline__ float one(float u) const {
     // fold: (u - z) is an exact small integer, (u - z) * s = fma(u, s, -z*s) exactly
-    if (fold) return __builtin_fmaf(u, sf, c);
+    if (FOLD) return __builtin_fmaf(u, sf, c);
     return round_to_bf16(u - zf) * sf;
   }
   __device__ __forceinline__ uint4_t operator()(uint32_t v) const {
@@ -93,71 +92,88 @@ struct Expand8<bf16_t> {
   }
 };
 
-template <typename T, int ROWS, int NT>
+template <typename T, bool FOLD, int ROWS, int NT>
 struct W4Loader {
   static constexpr int SLOTS = ROWS * 2;  // 16-byte packed loads per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
+  static constexpr int UNITS = PASSES * 4;  // one unit = one 32-bit word -> one 16-byte LDS chunk
+  static_assert(PASSES == 1 || (NT / 2) % 8 == 0, "pass stride must keep the swizzle phase");
   struct Params {
     const uint8_t* wp;
-    const T* scales;
+    const T* scales;  // never null: the host passes a dummy readable pointer when there are no scales
     const T* zeros;
     int64_t row_bytes;  // K / 2
     int groups;         // K / group
-    int group;
+    int group_shift;    // log2(group); group is a power of two here
     float zero_scalar;
-    int fold;  // 1: zero point is one integer for the whole matrix and is folded into the bias
+    int has_scales, has_zeros;
   };
   struct Regs {
     uint4_t v[PASSES];
     T s[PASSES], z[PASSES];
   };
-  Params p;
-  const uint8_t* base;
-  int row0, rows_valid;
+  const uint8_t* base;  // uniform: first packed row of the tile
+  const T* sbase;       // uniform: scales / zeros row of the tile's first row
+  const T* zbase;
+  uint32_t voff[PASSES];  // per lane: row * row_bytes + half * 16
+  uint32_t goff[PASSES];  // per lane: row * groups + (lane-fixed part of the group index)
+  uint32_t loff[4];       // per lane: LDS offsets of the four chunks this lane writes (pass 0)
+  int group_shift;
+  bool has_s, has_z, active;
+  T one, zs;
   NibbleMagic mg;
 
-  __device__ __forceinline__ W4Loader(const Params& pp, int /*batch*/, int row0_, int rows_total)
-      : p(pp), base(pp.wp + (int64_t)row0_ * pp.row_bytes), row0(row0_), rows_valid(rows_total - row0_),
-        mg(make_nibble_magic()) {}
+  __device__ __forceinline__ W4Loader(const Params& p, int /*batch*/, int row0, int rows_total, int tid)
+      : base(p.wp + (int64_t)row0 * p.row_bytes), group_shift(p.group_shift), has_s(p.has_scales != 0),
+        has_z(p.has_zeros != 0), one(from_float<T>(1.0f)), zs(from_float<T>(p.zero_scalar)), mg(make_nibble_magic()) {
+    const int rows_valid = rows_total - row0;
+    sbase = p.scales + (has_s ? (int64_t)row0 * p.groups : 0);
+    zbase = p.zeros + (has_z ? (int64_t)row0 * p.groups : 0);
+    const int half = tid & 1;
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+      int row = (ps * NT + tid) >> 1;
+      row = row < rows_valid ? row : rows_valid - 1;  // clamp: loads stay in bounds, results are masked later
+      voff[ps] = (uint32_t)row * (uint32_t)p.row_bytes + (uint32_t)(half * 16);
+      goff[ps] = (uint32_t)row * (uint32_t)p.groups + (uint32_t)((half * 32) >> group_shift);
+    }
+    const int r0 = tid >> 1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) loff[j] = (uint32_t)lds_off(r0, half * 4 + j);
+    active = !PARTIAL || ((PASSES - 1) * NT + tid) < SLOTS;
+  }
 
-  __device__ __forceinline__ void gload(Regs& r, int kt, int tid) const {
-    const T one = from_float<T>(1.0f);
-    const T zs = from_float<T>(p.zero_scalar);
+  // K is a multiple of 64 on this path, so every stage is complete (TAIL is never needed).
+  // Group index of element (kt*64 + half*32) = ((kt*64) >> shift) + ((half*32) >> shift) for every
+  // power-of-two group >= 32.
+  template <bool TAIL>
+  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+    const uint8_t* sb = base + (int64_t)kt * 32;
+    const uint32_t gk = (uint32_t)((kt * 64) >> group_shift);
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-      const int slot = ps * NT + tid;
-      int row = slot >> 1;
-      const int half = slot & 1;
-      row = row < rows_valid ? row : rows_valid - 1;
-      const int kb = kt * 32 + half * 16;
-      uint4_t v = {0u, 0u, 0u, 0u};
-      T s = one, z = zs;
-      if (kb < p.row_bytes && (!PARTIAL || slot < SLOTS)) {
-        v = *(const uint4_t*)(base + (int64_t)row * p.row_bytes + kb);
-        const int64_t gi = (int64_t)(row0 + row) * p.groups + (kb * 2) / p.group;
-        if (p.scales) s = p.scales[gi];
-        if (p.zeros) z = p.zeros[gi];
+      r.v[ps] = *(const uint4_t*)(sb + voff[ps]);
+      const T sv = sbase[has_s ? goff[ps] + gk : 0u];
+      const T zv = zbase[has_z ? goff[ps] + gk : 0u];
+      r.s[ps] = has_s ? sv : one;
+      r.z[ps] = has_z ? zv : zs;
+    }
+  }
+  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+      if (PARTIAL && ps == PASSES - 1 && !active) continue;
+      const Expand8<T, FOLD> ex(r.s[ps], r.z[ps], mg);
+      const uint32_t w[4] = {r.v[ps].x, r.v[ps].y, r.v[ps].z, r.v[ps].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if ((ps * 4 + j) * np / UNITS != pc) continue;
+        *(uint4_t*)(lds + loff[j] + ps * (NT / 2) * kStageBytes) = ex(w[j]);
       }
-      r.v[ps] = v;
-      r.s[ps] = s;
-      r.z[ps] = z;
     }
   }
-  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds, int tid) const {
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-      const int slot = ps * NT + tid;
-      if (PARTIAL && slot >= SLOTS) continue;
-      const int row = slot >> 1;
-      const int half = slot & 1;
-      const Expand8<T> ex(r.s[ps], r.z[ps], p.fold != 0, mg);
-      *(uint4_t*)(lds + lds_off(row, half * 4 + 0)) = ex(r.v[ps].x);
-      *(uint4_t*)(lds + lds_off(row, half * 4 + 1)) = ex(r.v[ps].y);
-      *(uint4_t*)(lds + lds_off(row, half * 4 + 2)) = ex(r.v[ps].z);
-      *(uint4_t*)(lds + lds_off(row, half * 4 + 3)) = ex(r.v[ps].w);
-    }
-  }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
 };
 
 template <typename T>
@@ -171,28 +187,59 @@ struct MmaOf<bf16_t> {
   typedef MmaBF16 type;
 };
 
-template <typename T, int BM, int BN, int WM, int WN>
-static int run_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
-                     int64_t K, int64_t group, float zero_scalar, int fold, int out_dtype, hipStream_t st) {
+template <int ROWS, int NT>
+using W4LoaderF16Fold = W4Loader<half_t, true, ROWS, NT>;
+template <int ROWS, int NT>
+using W4LoaderF16Gen = W4Loader<half_t, false, ROWS, NT>;
+template <int ROWS, int NT>
+using W4LoaderBF16Fold = W4Loader<bf16_t, true, ROWS, NT>;
+template <int ROWS, int NT>
+using W4LoaderBF16Gen = W4Loader<bf16_t, false, ROWS, NT>;
+
+struct W4Args {
+  const void *A, *Wp, *scales, *zeros;
+  void* C;
+  int64_t M, N, K, group;
+  float zero_scalar;
+  int out_dtype;
+  hipStream_t st;
+};
+
+template <typename T, bool FOLD, int ROWS, int NT>
+static typename W4Loader<T, FOLD, ROWS, NT>::Params w4_params(const W4Args& a) {
+  int shift = 0;
+  while (((int64_t)1 << shift) < a.group) ++shift;
+  const T* dummy = (const T*)a.A;  // readable placeholder for absent scale / zero tensors
+  return {(const uint8_t*)a.Wp,
+          a.scales ? (const T*)a.scales : dummy,
+          a.zeros ? (const T*)a.zeros : dummy,
+          a.K / 2,
+          (int)(a.K / a.group),
+          shift,
+          a.zero_scalar,
+          a.scales ? 1 : 0,
+          a.zeros ? 1 : 0};
+}
+
+template <typename T, bool FOLD, int BM, int BN, int WM, int WN>
+static int run_w4a16(const W4Args& a) {
   constexpr int NT = WM * WN * 64;
   typedef RowLoader<BM, NT> AL;
-  typedef W4Loader<T, BN, NT> WL;
-  typename AL::Params pa{(const uint8_t*)A, K * 2, 0, K * 2};
-  typename WL::Params pw{(const uint8_t*)Wp, (const T*)scales, (const T*)zeros, K / 2, (int)(K / group), (int)group,
-                         zero_scalar,        fold};
-  EpiFloat::Params pe{C, N, 0, out_dtype};
-  return launch_gemm<typename MmaOf<T>::type, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, M, N, K * 2, st,
+  typedef W4Loader<T, FOLD, BN, NT> WL;
+  typename AL::Params pa{(const uint8_t*)a.A, a.K * 2, 0, a.K * 2};
+  auto pw = w4_params<T, FOLD, BN, NT>(a);
+  EpiFloat::Params pe{a.C, a.N, 0, a.out_dtype};
+  return launch_gemm<typename MmaOf<T>::type, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, a.M, a.N, a.K * 2, a.st,
                                                                                "tlq_gemm_w4a16(mfma)");
 }
 
 // tile override for tuning runs (0 = automatic)
 static int g_w4a16_tile = 0;
 
-template <typename T>
-static int dispatch_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M,
-                          int64_t N, int64_t K, int64_t group, float zero_scalar, int fold, int out_dtype,
-                          hipStream_t st) {
+template <typename T, bool FOLD>
+static int dispatch_w4a16(const W4Args& a) {
   int tile = g_w4a16_tile;
+  const int64_t M = a.M, N = a.N;
   if (tile == 0) {
     if (M <= 16)
       tile = 16;
@@ -205,35 +252,32 @@ static int dispatch_w4a16(const void* A, const void* Wp, const void* scales, con
     else
       tile = 256;
   }
-#define TLQ_RUN(BM, BN, WM, WN) \
-  return run_w4a16<T, BM, BN, WM, WN>(A, Wp, scales, zeros, C, M, N, K, group, zero_scalar, fold, out_dtype, st)
   switch (tile) {
     case 16:
-      TLQ_RUN(16, 64, 1, 4);
+      return run_w4a16<T, FOLD, 16, 64, 1, 4>(a);
     case 32:
-      TLQ_RUN(32, 128, 1, 4);
+      return run_w4a16<T, FOLD, 32, 128, 1, 4>(a);
     case 64:
-      TLQ_RUN(64, 256, 1, 4);
+      return run_w4a16<T, FOLD, 64, 256, 1, 4>(a);
     case 128:
-      TLQ_RUN(128, 128, 2, 2);
-    case 512:
-      TLQ_RUN(256, 256, 2, 4);
+      return run_w4a16<T, FOLD, 128, 128, 2, 2>(a);
     default:
-      TLQ_RUN(256, 256, 2, 2);
+      return run_w4a16<T, FOLD, 256, 256, 2, 4>(a);
   }
-#undef TLQ_RUN
 }
 
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st) {
+  if ((group & (group - 1)) != 0) {
+    set_error("tlq_gemm_w4a16(mfma): group=%lld must be a power of two", (long long)group);
+    return 1;
+  }
   // An integer zero point shared by the whole matrix folds exactly into the unpack bias.
-  const int fold = (zeros == nullptr && zero_scalar == (float)(int)zero_scalar && zero_scalar >= -256.0f &&
-                    zero_scalar <= 256.0f)
-                       ? 1
-                       : 0;
-  if (in_dtype == TLQ_F16)
-    return dispatch_w4a16<half_t>(A, Wp, scales, zeros, C, M, N, K, group, zero_scalar, fold, out_dtype, st);
-  return dispatch_w4a16<bf16_t>(A, Wp, scales, zeros, C, M, N, K, group, zero_scalar, fold, out_dtype, st);
+  const bool fold = zeros == nullptr && zero_scalar == (float)(int)zero_scalar && zero_scalar >= -256.0f &&
+                    zero_scalar <= 256.0f;
+  const W4Args a{A, Wp, scales, zeros, C, M, N, K, group, zero_scalar, out_dtype, st};
+  if (in_dtype == TLQ_F16) return fold ? dispatch_w4a16<half_t, true>(a) : dispatch_w4a16<half_t, false>(a);
+  return fold ? dispatch_w4a16<bf16_t, true>(a) : dispatch_w4a16<bf16_t, false>(a);
 }
 
 }  // namespace tlq
