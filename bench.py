@@ -60,7 +60,7 @@ def timed(fn, steps, warmup):
     return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
 
 
-def bench_gemv(args):
+def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
     import torch
 
     from tilelang_ascend_amd import _abi
@@ -68,7 +68,9 @@ def bench_gemv(args):
     lib, P = _abi.load(), _abi.ptr
     dev = torch.device("cuda:0")
     M, N, K, g = 1, 11008, 4096, 128
-    units = args.units
+    units = units or args.units
+    steps = steps or args.steps
+    warmup = args.warmup if warmup is None else warmup
     unit_bytes = w4a16_bytes(M, N, K, g)
     sets = max(2 * units, -(-POOL_BYTES // unit_bytes))
     sets = -(-sets // units) * units
@@ -81,33 +83,33 @@ def bench_gemv(args):
     stream = torch.cuda.current_stream().cuda_stream
     groups = sets // units
 
+    # argument tuples are prepared up front: per-step tensor indexing would cost more host time
+    # than the kernel runs for
     if units == 1:
-        def step(i):
-            j = i % sets
-            rc = lib.tlq_gemm_w4a16(P(A[j]), P(Wp[j]), P(S[j]), P(Z[j]), P(C[j]), M, N, K, g, 0.0, _abi.F16, _abi.F16,
-                                    _abi.ALGO_GEMV, stream)
-            if rc:
-                raise RuntimeError(_abi.last_error())
+        pre = [(P(A[j]), P(Wp[j]), P(S[j]), P(Z[j]), P(C[j]), M, N, K, g, 0.0, _abi.F16, _abi.F16, _abi.ALGO_GEMV, stream)
+               for j in range(sets)]
+        entry = lib.tlq_gemm_w4a16
     else:
-        def step(i):
-            j = (i % groups) * units
-            rc = lib.tlq_gemv_w4a16_batched(P(A[j]), P(Wp[j]), P(S[j]), P(Z[j]), P(C[j]), units, M, N, K, g, 0.0,
-                                            _abi.F16, _abi.F16, stream)
-            if rc:
-                raise RuntimeError(_abi.last_error())
+        pre = [(P(A[j]), P(Wp[j]), P(S[j]), P(Z[j]), P(C[j]), units, M, N, K, g, 0.0, _abi.F16, _abi.F16, stream)
+               for j in range(0, sets, units)]
+        entry = lib.tlq_gemv_w4a16_batched
 
-    wall, ev = timed(step, args.steps, args.warmup)
+    def step(i):
+        if entry(*pre[i % groups]):
+            raise RuntimeError(_abi.last_error())
+
+    wall, ev = timed(step, steps, warmup)
     step_bytes = unit_bytes * units
     # spot check of the last result against the oracle (outside the timed region)
     from oracle import ref
 
-    j = ((args.steps - 1) % groups) * units if units > 1 else (args.steps - 1) % sets
+    j = ((steps - 1) % groups) * units
     want = ref.ref_program_w4a16(A[j].cpu(), Wp[j].cpu(), S[j].cpu(), Z[j].cpu(), g, "float32")
     rel = ((C[j].float().cpu() - want).norm() / want.norm()).item()
     if rel > 1e-3:
         raise RuntimeError(f"GEMV result differs from the oracle: relative L2 {rel}")
 
-    cpu = cpu_baseline_gemv(A[0].cpu(), Wp[0].cpu(), S[0].cpu(), Z[0].cpu(), g, unit_bytes)
+    cpu = cpu_baseline_gemv(A[0].cpu(), Wp[0].cpu(), S[0].cpu(), Z[0].cpu(), g, unit_bytes) if cpu else None
     return {
         "metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
         "value": round(step_bytes / wall / 1e9, 1),
@@ -215,6 +217,10 @@ def main():
     ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8"])
     ap.add_argument("--units", type=int, default=1, help="independent weight sets per GEMV launch")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain elementwise copy of 256 MiB (int32 x+0 -> y) after the timed region, "
+                         "the known-size kernel that hardware traffic counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU's share of the path; --gpus {args.gpus} is not supported in this build "
@@ -229,14 +235,24 @@ def main():
     torch.cuda.set_device(0)
 
     if args.workload == "gemv":
-        line = bench_gemv(args)
+        line = bench_gemv(args, cpu=not args.no_cpu_baseline)
         if not args.no_extra:
-            line["other_workloads"] = [bench_prefill(args, steps=20), bench_w8a8(args, steps=10)]
+            many = bench_gemv(args, units=24, steps=20, warmup=4, cpu=False)
+            line["other_workloads"] = [
+                {"workload": many["config"]["workload"], "dtype": "f16", "value": many["value"], "unit": "GB/s",
+                 "ms_per_step": many["ms_per_step"], "roofline": many["roofline"]},
+                bench_prefill(args, steps=20), bench_w8a8(args, steps=10)]
     else:
         res = bench_prefill(args) if args.workload == "prefill" else bench_w8a8(args)
         line = {"metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
                 "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
                 "config": {"workload": res["workload"]}, "roofline": res["roofline"], "cpu_baseline": None}
+    if args.calibrate_copy:
+        src = torch.zeros(64 * 1024 * 1024, dtype=torch.int32, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        torch.add(src, 0, out=dst)
+        torch.cuda.synchronize()
     line.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
                  "vs_baseline": None, "data": "synthetic"})
     order = ["metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",

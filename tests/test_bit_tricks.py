@@ -152,7 +152,7 @@ def test_w4i8_expand_order():
 
 
 def lds_swz(row):
-    return (row & 7) ^ ((row >> 3) & 1) ^ ((row >> 4) & 7)
+    return row & 7
 
 
 def lds_off(row, chunk):
@@ -163,11 +163,11 @@ def test_lds_swizzle_is_a_bijection_and_spreads_banks():
     rows = 256
     offs = {lds_off(r, c) for r in range(rows) for c in range(8)}
     assert len(offs) == rows * 8 and max(offs) == rows * 128 - 16
-    # MFMA operand read: 16 consecutive rows, one logical chunk -> 16 distinct 16-byte slots of the
-    # 256-byte bank period (and 8 distinct slots of a 128-byte period for each aligned 8 rows)
-    for r0 in range(0, rows, 16):
+    # MFMA operand read: a 16-byte read is served 8 lanes at a time, i.e. 8 consecutive rows of one
+    # logical chunk; those must land in 8 distinct 16-byte slots of the 128-byte row pitch
+    for r0 in range(0, rows, 8):
         for c in range(8):
-            slots256 = {(lds_off(r0 + r, c) % 256) // 16 for r in range(16)}
-            assert len(slots256) == 16
-            for h in (0, 8):
-                assert len({(lds_off(r0 + h + r, c) % 128) // 16 for r in range(8)}) == 8
+            assert len({(lds_off(r0 + r, c) % 128) // 16 for r in range(8)}) == 8
+    # tile fill: 8 consecutive lanes write the 8 chunks of one row -> 8 distinct slots as well
+    for r in range(rows):
+        assert len({(lds_off(r, c) % 128) // 16 for c in range(8)}) == 8
