@@ -31,6 +31,12 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_I8_PEAK_TOPS = 5000.0
 POOL_BYTES = 576 * 1024 * 1024  # weight pool > 2x the 256 MB last-level cache
+# HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in separate
+# runs of this script with --calibrate-copy, each scaled by what the counter reads for the 256 MiB
+# copy kernel: x2.000 and x1.000); the summaries are the text files under profiles/.
+TRAFFIC_GEMV_1SET = 24_170_000
+TRAFFIC_PREFILL = 182_200_000
+TRAFFIC_W8A8 = 935_500_000
 
 
 def w4a16_bytes(M, N, K, group, zeros_tensor=True, elem=2):
@@ -121,7 +127,7 @@ def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
                    "M": M, "N": N, "K": K, "group": g, "units_per_launch": units},
         "roofline": {"kernel": "gemv_w4a16_kernel", "bound": "hbm", "achieved": round(step_bytes / ev / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(step_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": None, "bytes_per_launch": step_bytes, "avg_launch_us": round(ev * 1e6, 3)},
+                     "traffic": TRAFFIC_GEMV_1SET * units, "bytes_per_launch": step_bytes, "avg_launch_us": round(ev * 1e6, 3)},
         "cpu_baseline": cpu,
         "parity_rel_l2": rel,
     }
@@ -175,7 +181,7 @@ def bench_prefill(args, steps=None):
             "value": round(flops / wall / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": wall * 1e3,
             "roofline": {"kernel": "gemm_mfma_kernel<MmaBF16,W4Loader>", "bound": "mfma", "achieved": round(flops / ev / 1e12, 1),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                         "traffic": None, "flops_per_launch": flops, "avg_launch_us": round(ev * 1e6, 2)}}
+                         "traffic": TRAFFIC_PREFILL, "flops_per_launch": flops, "avg_launch_us": round(ev * 1e6, 2)}}
 
 
 def bench_w8a8(args, steps=None):
@@ -205,7 +211,7 @@ def bench_w8a8(args, steps=None):
             "dtype": "i8", "value": round(ops / wall / 1e12, 1), "unit": "TOP/s", "ms_per_step": wall * 1e3,
             "roofline": {"kernel": "gemm_mfma_kernel<MmaI8,I8KNLoader,EpiRescale>", "bound": "mfma",
                          "achieved": round(ops / ev / 1e12, 1), "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
-                         "frac": round(ops / ev / 1e12 / MFMA_I8_PEAK_TOPS, 4), "traffic": None, "ops_per_launch": ops,
+                         "frac": round(ops / ev / 1e12 / MFMA_I8_PEAK_TOPS, 4), "traffic": TRAFFIC_W8A8, "ops_per_launch": ops,
                          "avg_launch_us": round(ev * 1e6, 2)}}
 
 

@@ -85,11 +85,23 @@ int tlq_unpack_int4(const void* w_packed, void* out, int64_t N, int64_t K, int o
 int tlq_dequant_w4(const void* w_packed, const void* scales, const void* zeros, void* out, int64_t N, int64_t K,
                    int64_t group, float zero_scalar, int dtype, void* stream);
 
+/* Fast decode of INTERLEAVED 4-bit weights, the gfx950 counterpart of the CUDA decoders that
+ * get_lop3_intrin_group returns (tilelang/quantize/lop3.py:5-421, 998-1046, 1090-1202).  `words` are
+ * 32-bit words whose nibbles were permuted by interleave_weight (tilelang/quantize/utils.py:73-126)
+ * for the fp16 target (out_dtype TLQ_F16: 8 fp16 per word) or the int8 target (TLQ_I8: 16 int8 per
+ * word pair).  is_signed subtracts 8 (fp16) / 7 (int8), as the reference's decoders do.
+ * scales (fp16, one per `words_per_group` words) or NULL; zeros_mode 0 none | 1 original (u - z) * s |
+ * 2 rescale fma(u, s, -z) | 3 quantized (u - qz) * s with zeros an int16 array; zeros fp16 otherwise.
+ * The device functions themselves are in tilelang_ascend_amd/csrc/decode_i4.h. */
+int tlq_decode_i4_interleaved(const void* words, const void* scales, const void* zeros, void* out, int64_t n_words,
+                              int64_t words_per_group, int out_dtype, int is_signed, int zeros_mode, void* stream);
+
 /* Fused weight-only GEMM / GEMV, replaces dequant_gemm_fp16_wrapper + fp16_gemm
  * (example_dequant_gemm_fine_grained.py:60-115,176-223) extended with per-group scale / zero:
  *   C[M,N] = rn_out( sum_k f32(A[m,k]) * f32(W[n,k]) ),  W as in tlq_dequant_w4, fp32 accumulate.
  * A: [M,K] in_dtype (TLQ_F16 / TLQ_BF16); C: [M,N] out_dtype (TLQ_F16 / TLQ_BF16 / TLQ_F32).
- * Requires K % 64 == 0 and group % 32 == 0 (group divides K). */
+ * Requires K % 64 == 0 and group % 32 == 0 (group divides K).  The MFMA kernel additionally needs
+ * N % 4 == 0 and a power-of-two group (32, 64, 128, ...); the GEMV kernel takes any such group. */
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                    void* stream);

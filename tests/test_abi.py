@@ -1,0 +1,151 @@
+"""The C-ABI shared library: it loads without a GPU, exports every symbol include/tlq.h declares
+with the declared argument lists, and rejects bad arguments before touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from tilelang_ascend_amd import _abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tlq.h")
+
+CTYPE = {"const void*": ctypes.c_void_p, "void*": ctypes.c_void_p, "int64_t": ctypes.c_int64, "int": ctypes.c_int,
+         "float": ctypes.c_float}
+RESTYPE = {"int": ctypes.c_int, "void": None, "const char*": ctypes.c_char_p}
+
+
+def declared():
+    """name -> (return type, [argument types]) parsed from the header text."""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    out = {}
+    for m in re.finditer(r"(const char\*|int|void)\s+(tlq_\w+)\s*\(([^)]*)\)\s*;", text):
+        ret, name, args = m.group(1), m.group(2), " ".join(m.group(3).split())
+        types = []
+        if args != "void":
+            for a in args.split(","):
+                a = a.strip()
+                t = re.match(r"(const void\*|void\*|int64_t|int|float)\s*\w+$", a)
+                assert t, f"{name}: argument '{a}' is not a plain pointer / size / code"
+                types.append(t.group(1))
+        out[name] = (ret, types)
+    return out
+
+
+def test_header_declares_only_plain_c_types():
+    d = declared()
+    assert len(d) >= 15
+    assert "torch" not in open(HEADER).read().lower().replace("torch_unpack", "").replace("torch_convert", "")
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _abi.load()
+    for name in declared():
+        assert hasattr(lib, name), f"libtlq.so does not export {name}"
+    assert lib.tlq_abi_version() == _abi.ABI_VERSION
+    m = re.search(r"#define TLQ_ABI_VERSION (\d+)", open(HEADER).read())
+    assert int(m.group(1)) == _abi.ABI_VERSION
+
+
+def test_ctypes_signatures_match_the_header():
+    d = declared()
+    assert set(d) == set(_abi.SIGNATURES)
+    for name, (ret, types) in d.items():
+        res, args = _abi.SIGNATURES[name]
+        assert res is RESTYPE[ret], name
+        assert args == [CTYPE[t] for t in types], name
+
+
+def test_enum_codes_match_the_header():
+    text = open(HEADER).read()
+    for name, val in (("TLQ_F16", _abi.F16), ("TLQ_BF16", _abi.BF16), ("TLQ_F32", _abi.F32), ("TLQ_I8", _abi.I8),
+                      ("TLQ_I32", _abi.I32), ("TLQ_U4", _abi.U4), ("TLQ_S4_TWOS", _abi.S4_TWOS),
+                      ("TLQ_S4_OFFSET8", _abi.S4_OFFSET8), ("TLQ_S4_OFFSET7", _abi.S4_OFFSET7), ("TLQ_B_KN", _abi.B_KN),
+                      ("TLQ_B_NK", _abi.B_NK), ("TLQ_ALGO_AUTO", _abi.ALGO_AUTO), ("TLQ_ALGO_GEMV", _abi.ALGO_GEMV),
+                      ("TLQ_ALGO_MFMA", _abi.ALGO_MFMA)):
+        m = re.search(rf"\b{name}\s*=\s*(\d+)", text)
+        assert m and int(m.group(1)) == val, name
+
+
+# Argument validation runs on the host before any launch, so it can be exercised without a GPU.
+# The pointer values below are never dereferenced: every call is rejected.
+FAKE = ctypes.c_void_p(0x1000)
+ODD = ctypes.c_void_p(0x1004)
+ODD2 = ctypes.c_void_p(0x1002)
+NULL = ctypes.c_void_p(0)
+
+
+def _rejected(rc, *needles):
+    assert rc != 0
+    msg = _abi.last_error()
+    for n in needles:
+        assert n in msg, msg
+    with pytest.raises(RuntimeError):
+        _abi.check(rc)
+
+
+def test_rejects_bad_w4a16_arguments():
+    lib = _abi.load()
+    f = lib.tlq_gemm_w4a16
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 4, 64, 100, 32, 0.0, _abi.F16, _abi.F16, 0, NULL), "K=100", "multiple of 64")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 4, 64, 128, 48, 0.0, _abi.F16, _abi.F16, 0, NULL), "group=48")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 4, 64, 128, 32, 0.0, _abi.I8, _abi.F16, 0, NULL), "in_dtype")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 4, 64, 128, 32, 0.0, _abi.F16, _abi.I32, 0, NULL), "out_dtype")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 4, 64, 128, 32, 0.0, _abi.F16, _abi.F16, 7, NULL), "algo")
+    _rejected(f(NULL, FAKE, NULL, NULL, FAKE, 4, 64, 128, 32, 0.0, _abi.F16, _abi.F16, 0, NULL), "null pointer")
+    _rejected(f(ODD, FAKE, NULL, NULL, FAKE, 4, 64, 128, 32, 0.0, _abi.F16, _abi.F16, 0, NULL), "16-byte aligned")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, -1, 64, 128, 32, 0.0, _abi.F16, _abi.F16, 0, NULL), "bad shape")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 32, 64, 128, 32, 0.0, _abi.F16, _abi.F16, _abi.ALGO_GEMV, NULL), "M <= 16")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 32, 66, 128, 32, 0.0, _abi.F16, _abi.F16, _abi.ALGO_MFMA, NULL), "N % 4")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 32, 64, 192, 96, 0.0, _abi.F16, _abi.F16, _abi.ALGO_MFMA, NULL), "power of two")
+    _rejected(f(FAKE, FAKE, NULL, NULL, FAKE, 1 << 20, 64, 4096, 128, 0.0, _abi.F16, _abi.F16, _abi.ALGO_MFMA, NULL),
+              "4 GiB")
+    # empty problems are accepted and launch nothing
+    assert f(NULL, NULL, NULL, NULL, NULL, 0, 64, 128, 32, 0.0, _abi.F16, _abi.F16, 0, NULL) == 0
+    assert f(NULL, NULL, NULL, NULL, NULL, 4, 0, 128, 32, 0.0, _abi.F16, _abi.F16, 0, NULL) == 0
+
+
+def test_rejects_bad_integer_gemm_arguments():
+    lib = _abi.load()
+    _rejected(lib.tlq_gemm_i8(FAKE, FAKE, FAKE, 1, 8, 16, 24, _abi.B_KN, NULL), "K=24")
+    _rejected(lib.tlq_gemm_i8(FAKE, FAKE, FAKE, 1, 8, 20, 32, _abi.B_KN, NULL), "N=20")
+    _rejected(lib.tlq_gemm_i8(FAKE, FAKE, FAKE, 1, 8, 16, 32, 5, NULL), "b_layout")
+    _rejected(lib.tlq_gemm_i8(FAKE, FAKE, FAKE, -2, 8, 16, 32, _abi.B_KN, NULL), "batch")
+    _rejected(lib.tlq_gemm_w4a8(FAKE, FAKE, FAKE, 8, 16, 48, _abi.S4_TWOS, NULL), "K=48")
+    _rejected(lib.tlq_gemm_w4a8(FAKE, FAKE, FAKE, 8, 16, 64, 9, NULL), "sign_mode")
+    _rejected(lib.tlq_gemm_w8a8(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 8, 16, 32, 3, _abi.B_KN, _abi.F16, NULL), "n_scale_b=3")
+    _rejected(lib.tlq_gemm_w8a8(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 8, 16, 32, 16, _abi.B_KN, _abi.I32, NULL), "out_dtype")
+    _rejected(lib.tlq_gemm_w8a8(FAKE, FAKE, ODD2, FAKE, FAKE, 1, 8, 16, 32, 16, _abi.B_KN, _abi.F16, NULL), "misaligned")
+    _rejected(lib.tlq_gemm_f16(FAKE, FAKE, FAKE, 8, 16, 12, _abi.F16, _abi.F16, _abi.B_KN, NULL), "K=12")
+    _rejected(lib.tlq_gemv_w4a16_batched(FAKE, FAKE, NULL, NULL, FAKE, 70000, 1, 64, 128, 32, 0.0, 0, 0, NULL), "batch=70000")
+    assert lib.tlq_gemm_i8(NULL, NULL, NULL, 0, 8, 16, 32, _abi.B_KN, NULL) == 0
+
+
+def test_rejects_bad_unpack_arguments():
+    lib = _abi.load()
+    _rejected(lib.tlq_unpack_int4(FAKE, FAKE, 4, 7, _abi.I8, _abi.U4, NULL), "K")
+    _rejected(lib.tlq_unpack_int4(FAKE, FAKE, 4, 8, _abi.I32, _abi.U4, NULL), "out_dtype")
+    _rejected(lib.tlq_unpack_int4(NULL, FAKE, 4, 8, _abi.I8, _abi.U4, NULL), "null")
+    _rejected(lib.tlq_dequant_w4(FAKE, NULL, NULL, FAKE, 4, 64, 24, 0.0, _abi.F16, NULL), "group")
+    _rejected(lib.tlq_dequant_w4(FAKE, NULL, NULL, FAKE, 4, 64, 32, 0.0, _abi.I8, NULL), "dtype")
+
+
+def test_error_string_is_thread_local():
+    import threading
+
+    lib = _abi.load()
+    lib.tlq_gemm_i8(FAKE, FAKE, FAKE, 1, 8, 16, 24, _abi.B_KN, NULL)
+    seen = {}
+
+    def other():
+        seen["before"] = _abi.last_error()
+        lib.tlq_gemm_w4a8(FAKE, FAKE, FAKE, 8, 16, 48, _abi.S4_TWOS, NULL)
+        seen["after"] = _abi.last_error()
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen["before"] == "" and "tlq_gemm_w4a8" in seen["after"]
+    assert "tlq_gemm_i8" in _abi.last_error()

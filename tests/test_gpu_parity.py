@@ -320,3 +320,65 @@ def test_fp16_gemm_plain(ops):
     B = torch.randn(K, N, generator=gen(29)).to(torch.float16)
     got = ops.fp16_gemm(M, N, K, 128, 256, 64)(A.cuda(), B.cuda()).cpu()
     check_float_output(got, A.float() @ B.float(), "fp16_gemm")
+
+
+# ------------------------------------------------------------------------------------------
+# committed fixtures (tests/golden/*.npz): frozen inputs and outputs of the two oracles
+# ------------------------------------------------------------------------------------------
+GOLDEN = __import__("os").path.join(__import__("os").path.dirname(__import__("os").path.abspath(__file__)), "golden")
+
+
+def _from_bits(a, kind):
+    t = torch.from_numpy(a.view(np.int16).copy())
+    return t.view(torch.float16 if kind == 0 else torch.bfloat16)
+
+
+@pytest.mark.parametrize("name", ["f16_g128_tensorz", "f16_g32_scalar8", "bf16_g64_tensorz", "bf16_g128_scalar8", "f16_plain"])
+@pytest.mark.parametrize("algo", ["gemv", "mfma"])
+def test_golden_w4a16(ops, name, algo):
+    with np.load(f"{GOLDEN}/w4a16_small.npz") as f:
+        d = {k[len(name) + 1:]: f[k] for k in f.files if k.startswith(name + ".")}
+    M, N, K, g, kind, zs = (int(v) if i < 5 else float(v) for i, v in enumerate(d["meta"]))
+    if algo == "gemv" and M > 16:
+        pytest.skip("the GEMV kernel handles M <= 16")
+    dt = torch.float16 if kind == 0 else torch.bfloat16
+    A, Wp = _from_bits(d["A"], kind), torch.from_numpy(d["Wp"])
+    S = _from_bits(d["S"], kind) if "S" in d else None
+    Z = _from_bits(d["Z"], kind) if "Z" in d else (zs if zs else None)
+    W = ops.dequantize_w4(Wp.cuda(), None if S is None else S.cuda(), Z.cuda() if isinstance(Z, torch.Tensor) else Z, g, dt)
+    assert_bit_equal(W.cpu(), _from_bits(d["W"], kind), f"golden dequant {name}")
+    got = _run_w4a16(ops, A, Wp, S, Z, g, "float32", algo, "float16" if kind == 0 else "bfloat16")
+    check_float_output(got, torch.from_numpy(d["C"]), f"golden w4a16 {name} {algo}")
+
+
+def test_golden_int8(ops):
+    from tilelang_ascend_amd import _abi
+
+    with np.load(f"{GOLDEN}/int8_small.npz") as f:
+        d = {k: f[k] for k in f.files}
+    A, W = torch.from_numpy(d["i8.A"]), torch.from_numpy(d["i8.W_kn"])
+    B_, M, K = A.shape
+    N = W.shape[2]
+    lib, P = _abi.load(), _abi.ptr
+    st = torch.cuda.current_stream().cuda_stream
+    Ad, Wd = A.cuda(), W.cuda()
+    Wnk = W.transpose(1, 2).contiguous().cuda()
+    for layout, Bm in ((_abi.B_KN, Wd), (_abi.B_NK, Wnk)):
+        C = torch.empty(B_, M, N, dtype=torch.int32, device="cuda")
+        _abi.check(lib.tlq_gemm_i8(P(Ad), P(Bm), P(C), B_, M, N, K, layout, st))
+        assert_bit_equal(C.cpu(), torch.from_numpy(d["i8.acc"]), f"golden i8 layout {layout}")
+    sa, sb = torch.from_numpy(d["i8.scale_a"]).cuda(), torch.from_numpy(d["i8.scale_b"]).cuda()
+    got = ops.simple_quant_batch_matmul(B_, M, N, K, "N", 128, 256, 64)(Ad, Wd, sb).cpu()
+    assert_bit_equal(got, _from_bits(d["i8.C_scale_b_f16"], 0), "golden per-channel f16")
+    got = ops.simple_quant_batch_matmul(B_, M, N, K, "1", 128, 256, 64, out_dtype="bfloat16")(Ad, Wd, sb[:1].contiguous()).cpu()
+    assert_bit_equal(got, _from_bits(d["i8.C_scale_1_bf16"], 1), "golden per-tensor bf16")
+    got = ops.quant_batch_matmul_per_token(B_, M, N, K, out_dtype="float16")(Ad, Wd, sa, sb).cpu()
+    assert_bit_equal(got, _from_bits(d["i8.C_token_channel_f16"], 0), "golden per-token x per-channel")
+    Wp = torch.from_numpy(d["w4.Wp"])
+    assert_bit_equal(ops.torch_unpack_uint4_to_int8(Wp), torch.from_numpy(d["w4.unsigned"]), "golden unpack")
+    assert_bit_equal(ops.torch_convert(Wp), torch.from_numpy(d["w4.signed"]), "golden signed unpack")
+    got = ops.dequant_gemm_int8_wrapper(M, N, K, 128, 128, 64, "int32")(A[0], Wp)
+    assert_bit_equal(got, torch.from_numpy(d["w4.C_unsigned"]), "golden u4 x i8")
+    workspace = torch.empty(N, K, dtype=torch.int8, device="cuda")  # a caller-supplied input in the reference
+    got = ops.w4a8_gemm_cv(M, N, K)(Ad[0].contiguous(), Wp.cuda(), workspace).cpu()
+    assert_bit_equal(got.T.contiguous(), torch.from_numpy(d["w4.C_signed_t"]), "golden s4 x i8")

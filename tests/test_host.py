@@ -1,0 +1,156 @@
+"""Host-side logic that needs no GPU: the jit front door, the kernel cache and the launch
+contract's validation (reference: tilelang/jit/__init__.py:197-247, tilelang/jit/adapter/base.py:22-46,
+tilelang/jit/adapter/cython/cython_wrapper.pyx:102-203, tilelang/cache/kernel_cache.py)."""
+import os
+import threading
+
+import pytest
+import torch
+
+import tilelang_ascend_amd as tl
+from tilelang_ascend_amd import cache, ops
+from tilelang_ascend_amd.jit import JITKernel, KernelSpec, Param, _legalize_idx
+
+
+@pytest.fixture(autouse=True)
+def _cache_in_tmp(tmp_path, monkeypatch):
+    monkeypatch.setenv("TLQ_CACHE_DIR", str(tmp_path / "cache"))
+    tl.enable_cache()
+    cache.clear_cache()
+    yield
+    tl.enable_cache()
+
+
+def _spec(name="k", launch=None):
+    return KernelSpec(name, [Param("A", (4, 8), "int8"), Param("B", (8, 16), "int8"), Param("C", (4, 16), "int32"),
+                             Param("ws", (4, 16), "int32")], launch or (lambda t, s, st: None))
+
+
+def test_idx_legalisation():
+    assert _legalize_idx(None, 4, "result_idx") == []
+    assert _legalize_idx(2, 4, "result_idx") == [2]
+    assert _legalize_idx([-1, -2], 4, "result_idx") == [3, 2]
+    for bad in (4, -5, [0, 7]):
+        with pytest.raises(ValueError, match="should be an integer between -4 and 3"):
+            _legalize_idx(bad, 4, "result_idx")
+    with pytest.raises(ValueError, match="list of integers"):
+        _legalize_idx("1", 4, "result_idx")
+
+
+def test_factory_memoises_per_arguments():
+    k1 = ops.simple_quant_batch_matmul(2, 64, 64, 64, "N", 128, 256, 64)
+    k2 = ops.simple_quant_batch_matmul(2, 64, 64, 64, "N", 128, 256, 64)
+    k3 = ops.simple_quant_batch_matmul(2, 64, 64, 64, "1", 128, 256, 64)
+    k4 = ops.simple_quant_batch_matmul(2, 64, 64, 64, "N", 128, 256, 64, out_dtype="bfloat16")
+    assert k1 is k2 and k1 is not k3 and k1 is not k4
+    assert isinstance(k1, JITKernel)
+    assert k1.result_idx == [3] and k1.workspace_idx == [4] and k1.input_idx == [0, 1, 2]
+    assert [p.name for p in k1.params] == ["A", "B", "scale", "C", "workspace_1"]
+    assert k3.params[2].shape == (1,) and k1.params[2].shape == (64,)
+    assert k4.params[3].dtype == "bfloat16"
+    assert "simple_quant_batch_matmul" in k1.get_kernel_source()
+    with pytest.raises(ValueError, match='scale_size must be "1" or "N"'):
+        ops.simple_quant_batch_matmul(2, 64, 64, 64, "M", 128, 256, 64)
+
+
+def test_disable_cache_builds_fresh_kernels_and_clear_cache_is_harmless():
+    a = ops.w4a8_gemm_cv(64, 64, 128)
+    assert ops.w4a8_gemm_cv(64, 64, 128) is a
+    tl.disable_cache()
+    assert not tl.is_cache_enabled()
+    b = ops.w4a8_gemm_cv(64, 64, 128)
+    assert b is not a
+    tl.enable_cache()
+    from tilelang_ascend_amd import build
+
+    before = os.path.getmtime(build.LIB_PATH)
+    tl.cache.clear_cache()  # the reference's examples do this at import time
+    assert os.path.exists(build.LIB_PATH) and os.path.getmtime(build.LIB_PATH) == before
+    assert os.path.isdir(cache.cache_dir()) and os.listdir(cache.cache_dir()) == []
+
+
+def test_cache_key_covers_spec_indices_and_pass_configs():
+    s = _spec()
+    base = cache.make_key(s, [2], [3], "auto", "ctypes", None)
+    assert base == cache.make_key(_spec(), [2], [3], "auto", "ctypes", None)
+    assert base != cache.make_key(_spec("other"), [2], [3], "auto", "ctypes", None)
+    assert base != cache.make_key(s, [-2], [3], "auto", "ctypes", None)
+    assert base != cache.make_key(s, [2], None, "auto", "ctypes", None)
+    assert base != cache.make_key(s, [2], [3], "auto", "ctypes", {tl.PassConfigKey.TL_ASCEND_AUTO_SYNC: True})
+    assert base != cache.make_key(s, [2], [3], "auto", "ctypes", {"some.unknown.key": 1})  # unknown keys still count
+    k = tl.compile(s, out_idx=[2], workspace_idx=[3])
+    assert tl.compile(_spec(), out_idx=[2], workspace_idx=[3]) is k
+    assert len(os.listdir(cache.cache_dir())) == 1
+    with pytest.raises(TypeError):
+        tl.compile(lambda: None)
+
+
+def test_cache_is_thread_safe():
+    made = []
+
+    def builder():
+        made.append(1)
+        return JITKernel(_spec("threaded"), [2], [3])
+
+    got = []
+    ts = [threading.Thread(target=lambda: got.append(cache.cached("same-key", builder))) for _ in range(8)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert len({id(g) for g in got}) == 1  # every thread sees the one published kernel
+
+
+def test_forward_validation_errors():
+    seen = {}
+
+    def launch(tensors, symbols, stream):
+        seen["called"] = True
+
+    k = tl.compile(_spec("validate", launch), out_idx=[2], workspace_idx=[3])
+    A = torch.zeros(4, 8, dtype=torch.int8)
+    B = torch.zeros(8, 16, dtype=torch.int8)
+    with pytest.raises(ValueError, match="Expected 2 inputs, got 1 with 4 params"):
+        k(A)
+    with pytest.raises(ValueError, match="Unsupported tensor type"):
+        k(A, [1, 2])
+    with pytest.raises(ValueError, match="Input tensor at index 1 must be contiguous"):
+        k(A, torch.zeros(16, 8, dtype=torch.int8).t())
+    with pytest.raises(ValueError, match="Buffer dtype mismatch for parameter A"):
+        k(A.to(torch.int32), B)
+    with pytest.raises(ValueError, match="Static shape mismatch for parameter B"):
+        k(A, torch.zeros(8, 32, dtype=torch.int8))
+    with pytest.raises(ValueError, match="Static shape mismatch for parameter A"):
+        k(torch.zeros(4, 8, 1, dtype=torch.int8), B)
+    # every check passed, but the tensors are on the host: there is no CPU implementation
+    with pytest.raises(ValueError, match="Buffer device mismatch"):
+        k(A, B)
+    with pytest.raises(ValueError, match="Buffer device mismatch"):
+        k(A, B, torch.zeros(3))  # surplus positionals are ignored, as in the reference
+    assert "called" not in seen
+
+
+def test_symbolic_dimension_is_resolved_from_the_inputs():
+    k = ops.int8_gemm_kernel_corrected(64, 128)
+    assert k.params[0].shape[0] == "M" and k.result_idx == [4] and k.workspace_idx == [5]
+    sym = k._resolve([torch.zeros(24, 128, dtype=torch.int8), torch.zeros(64, 128, dtype=torch.int8)])
+    assert sym == {"M": 24}
+
+
+def test_cpu_wrappers_fail_loudly_without_a_gpu():
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    f = ops.dequant_gemm_fp16_wrapper(16, 64, 64, 128, 256, 64)
+    with pytest.raises((RuntimeError, ValueError, AssertionError)):
+        f(torch.zeros(16, 64, dtype=torch.float16), torch.zeros(64, 32, dtype=torch.uint8))
+    with pytest.raises((RuntimeError, ValueError, AssertionError)):
+        ops.torch_unpack_uint4_to_fp16(torch.zeros(4, 4, dtype=torch.uint8))
+
+
+def test_profiler_module_surface():
+    from tilelang_ascend_amd import profiler
+
+    k = tl.compile(_spec("prof"), out_idx=[2], workspace_idx=[3])
+    p = k.get_profiler()
+    assert isinstance(p, profiler.Profiler)
+    assert [q.name for q in p._get_params()] == ["A", "B"]
+    assert [q.name for q in p._get_params(with_output=True)] == ["A", "B", "C"]
+    assert profiler.TensorSupplyType.Auto.value == 7 and callable(profiler.do_bench)

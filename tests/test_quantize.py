@@ -1,0 +1,171 @@
+"""tilelang_ascend_amd.quantize (product code, torch) against the oracle and closed forms.
+The CPU cases run here; the GPU cases decode interleaved weights with the HIP fast decoders."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref
+from tilelang_ascend_amd import quantize as Q
+
+
+def _rng(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def test_import_surface():
+    for name in ("_tir_packed_int_to_int_convert", "_tir_packed_to_signed_convert", "_tir_packed_to_unsigned_convert",
+                 "_tir_packed_to_fp4_to_f16", "_tir_u8_to_f8_e4m3_to_f16", "_tir_packed_to_unsigned_convert_with_zeros",
+                 "gen_quant4", "general_compress", "interleave_weight", "get_lop3_intrin_group"):
+        assert hasattr(Q, name), name
+
+
+def test_element_converters_against_oracle_tables():
+    val = torch.randint(0, 256, (5, 7), dtype=torch.uint8, generator=_rng(1))
+    for pos in (0, 1):
+        u = Q._tir_packed_to_unsigned_convert("uint", 8)(4, val, pos, "float16")
+        assert u.dtype == torch.float16
+        assert np.array_equal(u.numpy().astype(np.int64), ref.packed_to_unsigned(val.numpy(), pos))
+        s = Q._tir_packed_to_signed_convert("uint", 8)(4, val, pos, "int8")
+        assert np.array_equal(s.numpy().astype(np.int64), ref.packed_to_signed_offset(val.numpy(), pos))
+        t = Q._tir_packed_int_to_int_convert("uint", 8)(4, val, pos, "int8")
+        assert np.array_equal(t.numpy().astype(np.int64), ref.packed_int_to_int(val.numpy(), pos))
+        f = Q._tir_packed_uint_to_uint_to_float(8)(4, val, pos, "float16")
+        assert np.array_equal(f.numpy().astype(np.int64), ref.packed_uint_to_uint_to_float(val.numpy(), pos))
+        z = Q._tir_packed_to_unsigned_convert_with_zeros("uint", 8)(4, val, pos, 9, "float16")
+        assert np.array_equal(z.numpy().astype(np.int64), ref.packed_to_unsigned_with_zeros(val.numpy(), pos, 9))
+        zf = Q._tir_packed_to_unsigned_convert_with_zeros("uint", 8)(4, val, pos, torch.tensor(7.5, dtype=torch.float16),
+                                                                    "float16")
+        assert torch.equal(zf, u - torch.tensor(7.5, dtype=torch.float16))
+    # int8 storage: the same bytes viewed as signed
+    sv = val.view(torch.int8)
+    assert torch.equal(Q._tir_packed_to_unsigned_convert("int", 8)(4, sv, 1, "int8"),
+                       Q._tir_packed_to_unsigned_convert("uint", 8)(4, val, 1, "int8"))
+    # per-element positions: unpack a whole row at once
+    packed = torch.tensor([[0x12, 0x34]], dtype=torch.uint8)
+    k = torch.arange(4)
+    got = Q._tir_packed_to_unsigned_convert("uint", 8)(4, packed[:, k // 2], k % 2, "int8")
+    assert got.tolist() == [[2, 1, 4, 3]]
+    with pytest.raises(AssertionError):
+        Q._tir_packed_to_unsigned_convert("uint", 8)(4, val.to(torch.int32), 0, "int8")
+
+
+def test_fp4_and_e4m3_closed_forms():
+    codes = torch.arange(16, dtype=torch.uint8)
+    got = Q._tir_packed_to_fp4_to_f16("uint", 8)(4, codes, 0, "float16")
+    want = [0.0 if (c & 7) == 0 else (-1.0 if c >> 3 else 1.0) * 2.0 ** ((c & 7) - 7) for c in range(16)]
+    assert got.tolist() == want
+    # e4m3: every normal finite code must equal torch's own float8_e4m3fn conversion
+    allc = torch.arange(256, dtype=torch.uint8)
+    mine = Q._tir_u8_to_f8_e4m3_to_f16(8, allc, "float16")
+    theirs = allc.view(torch.float8_e4m3fn).to(torch.float16)
+    normal = ((allc & 0x78) != 0) & ((allc & 0x7F) != 0x7F)
+    assert torch.equal(mine[normal], theirs[normal])
+
+
+def test_general_compress_and_interleave_match_oracle():
+    for bits in (4, 2, 1):
+        w = torch.randint(0, 1 << bits, (6, 64), dtype=torch.int8, generator=_rng(2))
+        assert torch.equal(Q.general_compress(w, bits, torch.int8), ref.general_compress(w, bits, torch.int8))
+    w = torch.randint(-8, 8, (3, 16), dtype=torch.int8, generator=_rng(3))  # unmasked negatives: same smear
+    assert torch.equal(Q.general_compress(w, 4, torch.int8), ref.general_compress(w, 4, torch.int8))
+    assert Q.general_compress(w.half(), 4, torch.int32).dtype == torch.int32
+    q = torch.randint(-128, 128, (5, 32), dtype=torch.int8, generator=_rng(4))
+    for nbits in (4, 2, 1):
+        for target in ("float16", "int8"):
+            assert torch.equal(Q.interleave_weight(q, nbits, target), ref.interleave_weight(q, nbits, target)), (nbits, target)
+    base = torch.tensor([[0x10, 0x32, 0x54, 0x76]], dtype=torch.uint8).view(torch.int8)
+    assert ref.unpack_uint4(Q.interleave_weight(base, 4, "float16")).tolist() == [[0, 2, 4, 6, 1, 3, 5, 7]]
+    assert ref.unpack_uint4(Q.interleave_weight(base, 4, "int8")).tolist() == [[0, 4, 1, 5, 2, 6, 3, 7]]
+
+
+def test_gen_quant4_same_stream_and_values_as_oracle():
+    for g in (64, -1):
+        torch.manual_seed(5)
+        a = Q.gen_quant4(256, 24, g)
+        torch.manual_seed(5)
+        b = ref.gen_quant4(256, 24, g)
+        assert torch.equal(a[0], b[0]) and torch.equal(a[2], b[2]) and torch.equal(a[3], b[3])
+        assert torch.equal(a[1].weight.data, b[1].weight.data)
+
+
+def test_lop3_group_naming_grammar():
+    g = Q.get_lop3_intrin_group("float16")
+    assert g["func_name"] == "decode_i4u_to_f16" and "decode_i4u_to_f16(" in g["c_source"]
+    assert Q.get_lop3_intrin_group("float16", source_format="int")["func_name"] == "decode_i4s_to_f16"
+    assert Q.get_lop3_intrin_group("float16", with_scaling=True)["func_name"] == "decode_i4u_to_f16_scale"
+    for mode in ("original", "rescale", "quantized"):
+        name = Q.get_lop3_intrin_group("float16", with_scaling=True, with_zeros=True, zeros_mode=mode)["func_name"]
+        assert name == f"decode_i4u_to_f16_scale_zeros_{mode}"
+    assert Q.get_lop3_intrin_group("int8", source_format="int")["func_name"] == "decode_i4s_to_i8s"
+    assert Q.get_lop3_intrin_group("int8")["func_name"] == "decode_i4u_to_i8s"
+    with pytest.raises(ValueError):
+        Q.get_lop3_intrin_group("float16", source_format="int", with_scaling=True, with_zeros=True)
+    with pytest.raises(ValueError):
+        Q.get_lop3_intrin_group("float16", source_format="float")
+    with pytest.raises(AssertionError):
+        Q.get_lop3_intrin_group("float32")
+    with pytest.raises(NotImplementedError):
+        Q.get_lop3_intrin_group("float16", source_bit=2)
+    with pytest.raises(NotImplementedError):
+        Q.get_lop3_intrin_group("float16", with_scaling=True, storage_scope="warp")
+
+
+# ------------------------------------------------------------------------------------------------
+# GPU: the HIP fast decoders on interleaved weights
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("signed", [False, True])
+def test_gpu_decode_plain_and_signed(signed):
+    from tilelang_ascend_amd.quantize import lop3
+
+    q = torch.randint(0, 256, (64, 96), dtype=torch.uint8, generator=_rng(10))
+    inter = Q.interleave_weight(q.view(torch.int8), 4, "float16").cuda()
+    got = lop3.decode(inter, "float16", "int" if signed else "uint").cpu()
+    want = ref.unpack_uint4(q).astype(np.float16) - (np.float16(8) if signed else np.float16(0))
+    assert got.dtype == torch.float16 and np.array_equal(got.numpy(), want)
+    inter8 = Q.interleave_weight(q.view(torch.int8), 4, "int8").cuda()
+    got8 = lop3.decode(inter8, "int8", "int" if signed else "uint").cpu()
+    want8 = ref.unpack_uint4(q).astype(np.int8) - (7 if signed else 0)
+    assert got8.dtype == torch.int8 and np.array_equal(got8.numpy(), want8)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", [None, "original", "rescale", "quantized"])
+def test_gpu_decode_scale_and_zeros(mode):
+    from tilelang_ascend_amd.quantize import lop3
+
+    N, K, g = 48, 256, 64
+    gen = _rng(11)
+    q = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=gen)
+    s = (torch.rand(N, K // g, generator=gen) * 0.015 + 0.005).half()
+    zf = (torch.rand(N, K // g, generator=gen) * 3 + 6).half()
+    zi = torch.randint(0, 16, (N, K // g), generator=gen)
+    inter = Q.interleave_weight(q.view(torch.int8), 4, "float16").cuda()
+    zeros = None if mode is None else (zi if mode == "quantized" else zf)
+    got = lop3.decode(inter, "float16", "uint", scale=s.cuda(), zeros=None if zeros is None else zeros.cuda(),
+                      zeros_mode=mode, group_size=g).cpu()
+    u = torch.from_numpy(ref.unpack_uint4(q).astype(np.float32)).half()
+    sx = s.repeat_interleave(g, dim=1)
+    if mode is None:
+        want = u * sx
+    elif mode == "original":
+        want = (u - zf.repeat_interleave(g, dim=1)) * sx
+    elif mode == "quantized":
+        want = (u - zi.half().repeat_interleave(g, dim=1)) * sx
+    else:  # one rounding
+        want = (u.double() * sx.double() - zf.repeat_interleave(g, dim=1).double()).half()
+    assert torch.equal(got, want)
+    # the word-level closed form of the oracle gives the same numbers for a single group
+    words = inter.cpu().contiguous().view(torch.int32).numpy().view(np.uint32).reshape(-1)[: g // 8]
+    if mode in ("original", "rescale"):
+        o = ref.lop3_decode_i4_to_f16(words, scale=float(s[0, 0]), zeros=float(zf[0, 0]), zeros_mode=mode)
+        assert np.array_equal(o.reshape(-1), got[0, :g].numpy())
+
+
+@pytest.mark.gpu
+def test_gpu_quantize_utils_run_on_device_tensors():
+    w = torch.randint(0, 16, (32, 128), dtype=torch.int8, generator=_rng(12))
+    packed = Q.general_compress(w.cuda(), 4, torch.int8)
+    assert packed.is_cuda and torch.equal(packed.cpu(), ref.general_compress(w, 4, torch.int8))
+    inter = Q.interleave_weight(packed, 4, "float16")
+    assert inter.is_cuda and torch.equal(inter.cpu(), ref.interleave_weight(packed.cpu(), 4, "float16"))

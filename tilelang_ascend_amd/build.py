@@ -28,6 +28,7 @@ ARCH = "gfx950"
 SOURCES = [
     "abi.hip",
     "unpack_dequant.hip",
+    "decode_i4.hip",
     "gemv_w4a16.hip",
     "gemm_w4a16.hip",
     "gemm_int8.hip",

@@ -1,0 +1,99 @@
+"""Fast-decode intrinsic groups for interleaved low-bit weights.
+
+Reference: ``get_lop3_intrin_group`` (tilelang/quantize/lop3.py:1090-1202) returns the name and the
+CUDA source of a device function that decodes one 32-bit word of interleaved nibbles with
+``lop3.b32`` + paired fp16 arithmetic.  The gfx950 counterparts (``v_and_or_b32`` +
+``v_pk_{add,mul,fma}_f16``) live in ``csrc/decode_i4.h``; this module hands out that header's text
+under the reference's naming grammar, and ``decode`` runs the same device functions on a tensor
+through the C ABI (``tlq_decode_i4_interleaved``).
+
+Only the 4-bit source width is built (the quantized-matmul path uses nothing else); asking for
+1- or 2-bit sources raises NotImplementedError rather than handing back untested code.
+"""
+from __future__ import annotations
+
+import os
+from typing import Dict, Literal, Optional
+
+_HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc", "decode_i4.h")
+ZEROS_MODES = {"original": 1, "rescale": 2, "quantized": 3}
+
+
+def get_lop3_intrin_group(
+    out_dtype: Literal["float16", "int8", "int4"],
+    source_format: Literal["int", "uint"] = "uint",
+    source_bit: int = 4,
+    storage_dtype: Literal["int32", "int8"] = "int8",
+    with_scaling: bool = False,
+    with_zeros: bool = False,
+    zeros_mode: Literal["original", "rescale", "quantized"] = "original",
+    storage_scope: str = "local",
+) -> Dict[str, str]:
+    """Same arguments, checks, ``func_name`` grammar and return shape as the reference
+    (lop3.py:1139-1202): {"func_name": "decode_i4u_to_f16_scale_zeros_original", "c_source": ...}.
+    ``c_source`` is HIP (namespace ``tlq_decode``)."""
+    assert out_dtype in ["float16", "int8", "int4"], (
+        f"Invalid out_dtype: {out_dtype}. Expected 'float16' or 'int8' or 'int4' .")
+    if source_format not in ["int", "uint"]:
+        raise ValueError(f"Invalid source_format. Expected 'int' or 'uint', but got {source_format}.")
+    if with_zeros and source_format == "int":
+        raise ValueError(f"Zeros are not supported for signed integers, but got {source_format}")
+    if with_zeros and zeros_mode not in ZEROS_MODES:
+        raise ValueError(f"Invalid zeros_mode: {zeros_mode}")
+    d4f = {"float16": "f16", "int8": "i8s", "int4": "i4s"}[out_dtype]
+    func_name = "decode_i{}{}_to_{}".format(source_bit, "u" if source_format == "uint" else "s", d4f)
+    if with_scaling:
+        func_name += "_scale"
+    if with_zeros:
+        func_name += f"_zeros_{zeros_mode}"
+    if storage_scope == "warp" and with_scaling:
+        func_name += "_offset"
+    if source_bit != 4 or out_dtype == "int4" or func_name.endswith("_offset"):
+        raise NotImplementedError(f"{func_name}: only 4-bit sources decoded to float16 / int8 in thread-local "
+                                  "storage are built for gfx950")
+    if out_dtype == "int8" and (with_scaling or with_zeros):
+        raise KeyError(f"i{source_bit}_to_i8" + ("_scale" if with_scaling else "") + " has no decoder")
+    if with_zeros and not with_scaling:
+        raise KeyError(f"i{source_bit}_to_f16_zeros_{zeros_mode} has no decoder (zeros need scaling)")
+    with open(_HEADER) as f:
+        source = f.read()
+    assert f" {func_name}(" in source, func_name
+    return {"func_name": func_name, "c_source": source}
+
+
+def decode(words, out_dtype: str = "float16", source_format: str = "uint", scale=None, zeros=None,
+           zeros_mode: Optional[str] = None, group_size: int = -1):
+    """Run the decoder named by the arguments on a device tensor of interleaved weights.
+
+    words: int8 / uint8 / int32 tensor, last dimension a whole number of 32-bit words.  Returns a
+    tensor with the last dimension expanded to one element per nibble (float16 or int8).
+    scale (fp16) / zeros (fp16, or an integer tensor for zeros_mode='quantized'): one value per
+    `group_size` consecutive weights (default: one value for everything)."""
+    import torch
+
+    from .. import _abi
+
+    lib = _abi.load()
+    assert out_dtype in ("float16", "int8")
+    w = words.contiguous()
+    n_bytes = w.numel() * w.element_size()
+    assert n_bytes % 4 == 0, "the weights must be whole 32-bit words"
+    n_words = n_bytes // 4
+    last = w.shape[-1] * w.element_size() * 2
+    out = torch.empty(*w.shape[:-1], last, dtype=torch.float16 if out_dtype == "float16" else torch.int8, device=w.device)
+    mode = 0 if zeros_mode is None else ZEROS_MODES[zeros_mode]
+    wpg = n_words if group_size in (-1, None) else group_size // 8
+    s = None if scale is None else scale.to(device=w.device, dtype=torch.float16).contiguous()
+    z = None
+    if zeros is not None:
+        z = zeros.to(device=w.device, dtype=torch.int16 if mode == 3 else torch.float16).contiguous()
+    if s is not None:
+        assert s.numel() * wpg >= n_words, "not enough scales for the weights"
+    if z is not None:
+        assert z.numel() * wpg >= n_words, "not enough zeros for the weights"
+    stream = torch.cuda.current_stream().cuda_stream
+    with torch.cuda.device(w.device):
+        _abi.check(lib.tlq_decode_i4_interleaved(_abi.ptr(w), _abi.ptr(s), _abi.ptr(z), _abi.ptr(out), n_words, max(wpg, 1),
+                                                 _abi.F16 if out_dtype == "float16" else _abi.I8,
+                                                 1 if source_format == "int" else 0, mode, stream))
+    return out
