@@ -36,6 +36,56 @@ constexpr int kStageBytes = 128;
 __device__ __forceinline__ int lds_swz(int row) { return row & 7; }
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * kStageBytes + ((chunk ^ lds_swz(row)) << 4); }
 
+// ---- MFMA operand fragments ---------------------------------------------------------------
+// A loader names the reader of its LDS tile layout as `Frag`:
+//   Frag(lane, wave_row0)     per-lane offsets, computed once
+//   read(tile, ks, t)         the 16 bytes lane (row = lane % 16, k-group = lane / 16) feeds to the
+//                             MFMA for 16-row tile t of this wavefront and k-step ks (0 | 1)
+// [rows][128 B] tiles with the (row & 7) chunk swizzle: one ds_read_b128.  K-step 1 uses logical
+// chunk q + 4, i.e. the k-step 0 offset ^ 64; tiles 16 rows apart add 2048.
+struct RowFrag {
+  uint32_t fo;
+  __device__ __forceinline__ RowFrag(int lane, int wave_row0)
+      : fo((uint32_t)lds_off(lane & 15, lane >> 4) + (uint32_t)(wave_row0 * kStageBytes)) {}
+  __device__ __forceinline__ uint4_t read(const uint8_t* tile, int ks, int t) const {
+    return *(const uint4_t*)(tile + (fo ^ (uint32_t)(ks << 6)) + t * 16 * kStageBytes);
+  }
+};
+
+// [128 k][BN bytes] tiles (a [K, N] int8 source copied as it is, n contiguous): the operand needs 16
+// consecutive k of one n per lane, which ds_read_b64_tr_b8 delivers straight from this layout.
+// Semantics of the instruction (established by probing): each group of 16 lanes supplies 16 row
+// addresses R[0..15] (8 bytes each); lane j of the group receives bytes b = 0..7 =
+// R[2b + j/8][j % 8].  With lane i supplying the row of k = i/2 at columns n_t + 8*(i%2), lane j
+// receives k = 0..7 of column n_t + j: two such reads (k 0..7, 8..15) make one operand.
+// 16-byte chunks of a k row are XOR-swizzled so that the 32 rows a wavefront touches per read, and
+// the row-wise fill stores, spread over all banks.
+template <int BN>
+__device__ __forceinline__ int kn_swz(int k) {
+  static_assert(BN == 128 || BN == 256, "tile width");
+  return BN == 256 ? ((k & 7) | (((k >> 4) & 1) << 3)) : (((k >> 1) & 3) | (((k >> 4) & 1) << 2));
+}
+template <int BN>
+struct KNFrag8 {
+  typedef int v2i_t __attribute__((ext_vector_type(2)));
+  uint32_t off[4];
+  __device__ __forceinline__ KNFrag8(int lane, int wave_row0) {
+    const int r16 = lane & 15, q = lane >> 4;
+    const int krow = q * 16 + (r16 >> 1);
+    const int sw = kn_swz<BN>(krow);  // unchanged by the +8 (second read) and +64 (k-step) row offsets
+    const uint32_t base = (uint32_t)(krow * BN + 8 * (r16 & 1));
+#pragma unroll
+    for (int t = 0; t < 4; ++t) off[t] = base + (uint32_t)((((wave_row0 >> 4) + t) ^ sw) << 4);
+  }
+  __device__ __forceinline__ uint4_t read(const uint8_t* tile, int ks, int t) const {
+    typedef __attribute__((address_space(3))) v2i_t* lds_ptr;
+    const uint8_t* p = tile + off[t] + ks * 64 * BN;
+    const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr)(p));
+    const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr)(p + 8 * BN));
+    return uint4_t{(uint32_t)lo.x, (uint32_t)lo.y, (uint32_t)hi.x, (uint32_t)hi.y};
+  }
+};
+
 // ---- MFMA wrappers ----------------------------------------------------------------------
 struct MmaF16 {
   typedef float4_t acc_t;
@@ -69,6 +119,7 @@ struct MmaI8 {
 // Plain row-major [rows, k_bytes] source (activations of every kind, weights stored [N, K]).
 template <int ROWS, int NT>
 struct RowLoader {
+  typedef RowFrag Frag;
   static constexpr int SLOTS = ROWS * 8;  // 16-byte chunks per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
@@ -132,14 +183,16 @@ struct RowLoader {
   __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
 };
 
-// int8 source stored [K, N] (N contiguous): 4(k) x 16(n) register blocks are byte-transposed
-// with v_perm_b32 so that the LDS tile is [n][k] like every other operand.
-template <int ROWS, int NT>
+// int8 source stored [K, N] (N contiguous): rows of k are copied unchanged into a [128 k][BN] LDS
+// tile; the transposition happens in the operand read (KNFrag8).
+template <int BN, int NT>
 struct I8KNLoader {
-  static constexpr int NBLK = ROWS / 16;           // 16-column blocks per tile
-  static constexpr int PASSES = (32 * NBLK) / NT;  // 128 k = 32 blocks of 4 rows
-  static constexpr int UNITS = PASSES * 4;
-  static_assert(PASSES >= 1 && (32 * NBLK) % NT == 0 && NT % NBLK == 0, "bad transposing loader shape");
+  typedef KNFrag8<BN> Frag;
+  static constexpr int CH = BN / 16;            // 16-byte chunks per k row
+  static constexpr int RPP = NT / CH;           // k rows per pass
+  static constexpr int PASSES = kStageBytes / RPP;
+  static constexpr int UNITS = PASSES;
+  static_assert(NT % CH == 0 && RPP % 32 == 0 && kStageBytes % RPP == 0, "pass stride must keep the swizzle phase");
   struct Params {
     const uint8_t* base;  // B[0, 0] of batch 0
     int64_t ld;           // bytes per k row (= N)
@@ -147,23 +200,25 @@ struct I8KNLoader {
     int64_t k_total;  // K
   };
   struct Regs {
-    uint4_t v[PASSES][4];
+    uint4_t v[PASSES];
   };
   const uint8_t* base;  // uniform
   uint32_t ld;
-  uint32_t voff;  // per lane: kblk0 * 4 * ld + col
-  int kblk0, nblk;
+  uint32_t voff;  // per lane: k0 * ld + col
+  uint32_t loff;  // per lane: LDS offset of pass 0
+  int k0;
   int k_total;
 
   // cols_total must be a multiple of 16 (checked on the host)
   __device__ __forceinline__ I8KNLoader(const Params& p, int batch, int col0, int cols_total, int tid)
       : base(p.base + batch * p.batch_stride + col0), ld((uint32_t)p.ld), k_total((int)p.k_total) {
     const int cols_valid = cols_total - col0;
-    nblk = tid % NBLK;
-    kblk0 = tid / NBLK;
-    int col = nblk * 16;
-    col = col < cols_valid ? col : cols_valid - 16;  // clamp whole 16-column blocks
-    voff = (uint32_t)(kblk0 * 4) * ld + (uint32_t)col;
+    const int c = tid % CH;
+    k0 = tid / CH;
+    int col = c * 16;
+    col = col < cols_valid ? col : cols_valid - 16;  // clamp whole chunks: loads stay in bounds, results are masked
+    voff = (uint32_t)k0 * ld + (uint32_t)col;
+    loff = (uint32_t)(k0 * BN + ((c ^ kn_swz<BN>(k0)) << 4));
   }
 
   template <bool TAIL>
@@ -171,46 +226,22 @@ struct I8KNLoader {
     const uint8_t* sb = base + (int64_t)kt * kStageBytes * ld;
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t o = voff + (uint32_t)(ps * (NT / NBLK) * 4 + i) * ld;
-        if (!TAIL) {
-          r.v[ps][i] = *(const uint4_t*)(sb + o);
-        } else {
-          const int k = kt * kStageBytes + (ps * (NT / NBLK) + kblk0) * 4 + i;
-          const bool ok = k < k_total;
-          uint4_t v = *(const uint4_t*)(ok ? sb + o : base + (voff - (uint32_t)(kblk0 * 4) * ld));
-          if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
-          r.v[ps][i] = v;
-        }
+      const uint32_t o = voff + (uint32_t)(ps * RPP) * ld;
+      if (!TAIL) {
+        r.v[ps] = *(const uint4_t*)(sb + o);
+      } else {
+        const bool ok = kt * kStageBytes + ps * RPP + k0 < k_total;
+        uint4_t v = *(const uint4_t*)(ok ? sb + o : base + (voff - (uint32_t)k0 * ld));
+        if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
+        r.v[ps] = v;
       }
     }
   }
   __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-      const int kblk = ps * (NT / NBLK) + kblk0;
-      const int chunk = kblk >> 2;
-      const int within = (kblk & 3) * 4;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        if ((ps * 4 + c) * np / UNITS != pc) continue;
-        const uint32_t a = r.v[ps][0][c], b = r.v[ps][1][c], cc = r.v[ps][2][c], d = r.v[ps][3][c];
-        // 4x4 byte transpose: t[j] = (a.byte j, b.byte j, c.byte j, d.byte j)
-        const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400u);
-        const uint32_t ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602u);
-        const uint32_t cd_lo = __builtin_amdgcn_perm(d, cc, 0x05010400u);
-        const uint32_t cd_hi = __builtin_amdgcn_perm(d, cc, 0x07030602u);
-        const uint32_t t[4] = {__builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u),
-                               __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u),
-                               __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u),
-                               __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u)};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int row = nblk * 16 + c * 4 + j;
-          *(uint32_t*)(lds + lds_off(row, chunk) + within) = t[j];
-        }
-      }
+      if (ps * np / UNITS != pc) continue;
+      *(uint4_t*)(lds + loff + ps * RPP * BN) = r.v[ps];
     }
   }
   __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
@@ -364,11 +395,8 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = typename Mma::acc_t{0, 0, 0, 0};
 
-  // Per-lane LDS offset of an operand fragment for k-step 0 (row r16 of a 16-row tile, logical
-  // chunk q).  K-step 1 uses chunk q + 4, i.e. this offset ^ 64; tiles 16 rows apart add 2048.
-  const uint32_t fo = (uint32_t)lds_off(r16, q);
-  const uint8_t* const fragA = ldsA0 + wave_m0 * kStageBytes;
-  const uint8_t* const fragW = ldsW0 + wave_n0 * kStageBytes;
+  const typename AL::Frag fragA(lane, wave_m0);
+  const typename WL::Frag fragW(lane, wave_n0);
 
   // One stage: 2 k-steps x TN weight tiles x TM activation tiles of MFMAs on buffer CUR.  When
   // FILL, the conversion + LDS stores of the next stage (already in registers) are cut into
@@ -378,18 +406,17 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   constexpr int NPA = NP / 2;  // first half: activation stores, second half: weight conversion
   auto stage = [&](int cur, auto fill_tag) {
     constexpr bool FILL = decltype(fill_tag)::value;
-    const uint8_t* la = fragA + cur * A_TILE;
-    const uint8_t* lw = fragW + cur * W_TILE;
+    const uint8_t* la = ldsA0 + cur * A_TILE;
+    const uint8_t* lw = ldsW0 + cur * W_TILE;
     uint8_t* na = ldsA0 + (cur ^ 1) * A_TILE;
     uint8_t* nw = ldsW0 + (cur ^ 1) * W_TILE;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const uint32_t o = fo ^ (uint32_t)(ks << 6);
       uint4_t wf[TN], af[TM];
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) wf[tn] = *(const uint4_t*)(lw + o + tn * 16 * kStageBytes);
+      for (int tn = 0; tn < TN; ++tn) wf[tn] = fragW.read(lw, ks, tn);
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) af[tm] = *(const uint4_t*)(la + o + tm * 16 * kStageBytes);
+      for (int tm = 0; tm < TM; ++tm) af[tm] = fragA.read(la, ks, tm);
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) {
 #pragma unroll

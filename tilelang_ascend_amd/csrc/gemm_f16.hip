@@ -8,6 +8,7 @@ namespace tlq {
 // v_perm_b32 and written as 8-byte pieces (4 consecutive k of one n) into the [n][k] LDS tile.
 template <int ROWS, int NT>
 struct H16KNLoader {
+  typedef RowFrag Frag;
   static constexpr int NBLK = ROWS / 8;            // 8-column blocks per tile
   static constexpr int PASSES = (16 * NBLK) / NT;  // 64 k = 16 blocks of 4 rows
   static constexpr int UNITS = PASSES * 4;

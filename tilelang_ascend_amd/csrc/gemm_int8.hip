@@ -11,6 +11,7 @@ namespace tlq {
 // row; a thread expands 16 packed bytes into two 16-byte chunks.
 template <int ROWS, int NT>
 struct W4I8Loader {
+  typedef RowFrag Frag;
   static constexpr int SLOTS = ROWS * 4;
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;

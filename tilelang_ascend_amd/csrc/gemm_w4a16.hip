@@ -94,6 +94,7 @@ struct Expand8<bf16_t, FOLD> {
 
 template <typename T, bool FOLD, int ROWS, int NT>
 struct W4Loader {
+  typedef RowFrag Frag;
   static constexpr int SLOTS = ROWS * 2;  // 16-byte packed loads per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
