@@ -120,6 +120,9 @@ struct MmaI8 {
 template <int ROWS, int NT>
 struct RowLoader {
   typedef RowFrag Frag;
+  static constexpr bool DIRECT = false;
+  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
+  static constexpr bool PREFETCH2 = false;
   static constexpr int SLOTS = ROWS * 8;  // 16-byte chunks per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
@@ -157,7 +160,7 @@ struct RowLoader {
   }
 
   template <bool TAIL>
-  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* /*lds_next*/ = nullptr) const {
     const uint8_t* sb = base + (int64_t)kt * kStageBytes;
     if (!TAIL) {
 #pragma unroll
@@ -183,11 +186,99 @@ struct RowLoader {
   __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
 };
 
+// Same source and LDS layout as RowLoader, but full stages travel global -> LDS without passing
+// through registers (global_load_lds_dwordx4): one wavefront instruction fills 8 rows x 128 B =
+// 1 KB of the tile, lane l landing at byte 16*l of that KB.  The chunk swizzle is therefore applied
+// on the global side: the lane that lands on (row, physical chunk pc) fetches logical chunk
+// pc ^ (row & 7) of that row (the 8 lanes of a row still cover one 128-byte line).  A partial
+// last stage needs zero fill, which the direct path cannot do; it goes through registers.
+template <int ROWS, int NT>
+struct RowLoaderDirect {
+  typedef RowFrag Frag;
+  static constexpr bool DIRECT = true;
+  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
+  static constexpr bool PREFETCH2 = false;
+  static constexpr int WAVES = NT / 64;
+  static constexpr int INSTR = ROWS / 8;          // wavefront-instructions per stage
+  static constexpr int PER_WAVE = INSTR / WAVES;  // ... per wavefront
+  static constexpr int UNITS = PER_WAVE;
+  static_assert(ROWS % 8 == 0 && INSTR % WAVES == 0 && PER_WAVE >= 1, "tile does not split into whole wavefront loads");
+  typedef typename RowLoader<ROWS, NT>::Params Params;
+  struct Regs {
+    uint4_t v[PER_WAVE];
+    bool pending;  // a register-path (tail) stage waits to be stored
+  };
+  const uint8_t* base;      // uniform
+  uint32_t voff[PER_WAVE];  // per lane: row * ld + logical chunk * 16
+  uint32_t wave_off;        // uniform: LDS offset of this wavefront's first KB
+  uint32_t lane_off;        // lane * 16
+  int kb_lane, k_bytes;
+
+  __device__ __forceinline__ RowLoaderDirect(const Params& p, int batch, int row0, int rows_total, int tid)
+      : base(p.base + batch * p.batch_stride + (int64_t)row0 * p.ld), k_bytes((int)p.k_bytes) {
+    const int rows_valid = rows_total - row0;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    wave_off = (uint32_t)wave * 1024u;
+    lane_off = (uint32_t)lane * 16u;
+    const int chunk = (lane & 7) ^ ((lane >> 3) & 7);  // rows of one instruction start at a multiple of 8
+    kb_lane = chunk * 16;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) {
+      int row = (j * WAVES + wave) * 8 + (lane >> 3);
+      row = row < rows_valid ? row : rows_valid - 1;
+      voff[j] = (uint32_t)row * (uint32_t)p.ld + (uint32_t)kb_lane;
+    }
+  }
+
+  // The direct loads are written as inline assembly on purpose: while a compiler-visible direct load is
+  // outstanding the compiler turns every LDS wait into a wait for everything (it must assume the load
+  // may also return through the LDS counter), which serialises the operand reads and LDS stores of the
+  // whole stage.  The kernel waits for them by hand (wait_direct) before the barrier that publishes
+  // the buffer.
+  template <bool TAIL>
+  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* lds_next) const {
+    typedef __attribute__((address_space(3))) uint8_t* lptr_t;
+    if (!TAIL) {
+      r.pending = false;
+      const uint8_t* sb = uniform_ptr(base + (int64_t)kt * kStageBytes);
+      const uint32_t l0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lptr_t)lds_next + wave_off);
+#pragma unroll
+      for (int j = 0; j < PER_WAVE; ++j)
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0 + (uint32_t)(j * WAVES * 1024)),
+                     "v"(voff[j]), "s"(sb)
+                     : "memory");
+    } else {
+      r.pending = true;
+      const uint8_t* sb = base + (int64_t)kt * kStageBytes;
+      const bool ok = kt * kStageBytes + kb_lane < k_bytes;
+#pragma unroll
+      for (int j = 0; j < PER_WAVE; ++j) {
+        uint4_t v = *(const uint4_t*)(ok ? sb + voff[j] : base + (voff[j] - kb_lane));
+        if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
+        r.v[j] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
+    if (!r.pending) return;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) {
+      if (j * np / UNITS != pc) continue;
+      *(uint4_t*)(lds + wave_off + j * WAVES * 1024 + lane_off) = r.v[j];
+    }
+  }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
+};
+
 // int8 source stored [K, N] (N contiguous): rows of k are copied unchanged into a [128 k][BN] LDS
 // tile; the transposition happens in the operand read (KNFrag8).
 template <int BN, int NT>
 struct I8KNLoader {
   typedef KNFrag8<BN> Frag;
+  static constexpr bool DIRECT = false;
+  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
+  static constexpr bool PREFETCH2 = false;
   static constexpr int CH = BN / 16;            // 16-byte chunks per k row
   static constexpr int RPP = NT / CH;           // k rows per pass
   static constexpr int PASSES = kStageBytes / RPP;
@@ -222,8 +313,8 @@ struct I8KNLoader {
   }
 
   template <bool TAIL>
-  __device__ __forceinline__ void gload(Regs& r, int kt) const {
-    const uint8_t* sb = base + (int64_t)kt * kStageBytes * ld;
+  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* /*lds_next*/ = nullptr) const {
+    const uint8_t* sb = uniform_ptr(base + (int64_t)kt * kStageBytes * ld);
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
       const uint32_t o = voff + (uint32_t)(ps * RPP) * ld;
@@ -402,8 +493,13 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   // FILL, the conversion + LDS stores of the next stage (already in registers) are cut into
   // 2*TN pieces and one piece follows every TM MFMAs, so that the VALU / LDS-store work runs in
   // the shadow of the MFMAs (this wavefront's and the other wavefront's on the same SIMD).
-  constexpr int NP = 2 * TN;   // pieces per stage
-  constexpr int NPA = NP / 2;  // first half: activation stores, second half: weight conversion
+  constexpr int NP = 2 * TN;  // pieces per stage
+  // first pieces: activation stores (none when they travel directly), the rest: weight conversion
+  constexpr int NPA = AL::DIRECT ? 0 : NP / 2;
+  // hand-issued direct loads are invisible to the compiler's wait insertion
+  auto wait_direct = [&]() {
+    if (AL::DIRECT || WL::DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
   auto stage = [&](int cur, auto fill_tag) {
     constexpr bool FILL = decltype(fill_tag)::value;
     const uint8_t* la = ldsA0 + cur * A_TILE;
@@ -427,6 +523,22 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
             al.lstore_piece(ra, na, pc, NPA);
           else
             wl.lstore_piece(rw, nw, pc - NPA, NP - NPA);
+          if (NPA == 0 && pc == 0) al.lstore(ra, na);  // direct loader: only a partial last stage stores anything
+        }
+      }
+    }
+    // Scheduling pipeline for the whole stage: left alone, the compiler gathers the conversion
+    // arithmetic of the fill into one long run after the last MFMA, where nothing hides it.
+    constexpr int VPM = WL::VALU_PER_MFMA;
+    if (FILL && VPM > 0) {
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        __builtin_amdgcn_sched_group_barrier(0x100, TN + TM, 0);  // operand fragment reads of this k-step
+#pragma unroll
+        for (int i = 0; i < TN * TM; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);  // VPM conversion instructions in its shadow
+          if (i % 16 == 15) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // an LDS store of converted weights
         }
       }
     }
@@ -434,31 +546,61 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
 
   // prologue: stage 0 into buffer 0
   if (KT == 1 && k_tail) {
-    al.template gload<true>(ra, 0);
-    wl.template gload<true>(rw, 0);
+    al.template gload<true>(ra, 0, ldsA0);
+    wl.template gload<true>(rw, 0, ldsW0);
   } else {
-    al.template gload<false>(ra, 0);
-    wl.template gload<false>(rw, 0);
+    al.template gload<false>(ra, 0, ldsA0);
+    wl.template gload<false>(rw, 0, ldsW0);
   }
   al.lstore(ra, ldsA0);
   wl.lstore(rw, ldsW0);
+  wait_direct();
   __syncthreads();
 
-  // Stages 0 .. KT-2 compute and fill.  Only the load of stage KT-1 can be a partial stage.
-  const int last_full = k_tail ? KT - 2 : KT - 1;  // highest stage loadable without the tail path
-  int kt = 0;
-  for (; kt + 1 <= last_full; ++kt) {
-    al.template gload<false>(ra, kt + 1);
-    wl.template gload<false>(rw, kt + 1);
-    stage(kt & 1, std::true_type{});
-    __syncthreads();
-  }
-  if (kt + 1 < KT) {  // the partial last stage
-    al.template gload<true>(ra, kt + 1);
-    wl.template gload<true>(rw, kt + 1);
-    stage(kt & 1, std::true_type{});
-    __syncthreads();
-    ++kt;
+  if constexpr (WL::PREFETCH2) {
+    // Converting loader: the weights of stage t+1 are converted during stage t from registers that were
+    // loaded during stage t-1, so the conversion never waits on a load issued in the same stage and the
+    // compiler is free to spread it between the MFMAs.  Costs one more register set (a few registers).
+    typename WL::Regs rw_next;
+    auto wload = [&](typename WL::Regs& r, int s) {
+      if (s < KT) {
+        if (k_tail && s == KT - 1)
+          wl.template gload<true>(r, s, ldsW0 + (s & 1) * W_TILE);
+        else
+          wl.template gload<false>(r, s, ldsW0 + (s & 1) * W_TILE);
+      }
+    };
+    wload(rw_next, 1);
+    for (int kt = 0; kt + 1 < KT; ++kt) {
+      rw = rw_next;
+      wload(rw_next, kt + 2);
+      if (k_tail && kt + 1 == KT - 1)
+        al.template gload<true>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
+      else
+        al.template gload<false>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
+      stage(kt & 1, std::true_type{});
+      wait_direct();
+      __syncthreads();
+    }
+  } else {
+    // Stages 0 .. KT-2 compute and fill.  Only the load of stage KT-1 can be a partial stage.
+    const int last_full = k_tail ? KT - 2 : KT - 1;  // highest stage loadable without the tail path
+    int kt = 0;
+    for (; kt + 1 <= last_full; ++kt) {
+      al.template gload<false>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
+      wl.template gload<false>(rw, kt + 1, ldsW0 + ((kt + 1) & 1) * W_TILE);
+      stage(kt & 1, std::true_type{});
+      wait_direct();
+      __syncthreads();
+    }
+    if (kt + 1 < KT) {  // the partial last stage
+      al.template gload<true>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
+      wl.template gload<true>(rw, kt + 1, ldsW0 + ((kt + 1) & 1) * W_TILE);
+      stage(kt & 1, std::true_type{});
+      wait_direct();
+      __syncthreads();
+      ++kt;
+    }
   }
   if (KT > 0) stage((KT - 1) & 1, std::false_type{});
 

@@ -9,6 +9,9 @@ namespace tlq {
 template <int ROWS, int NT>
 struct H16KNLoader {
   typedef RowFrag Frag;
+  static constexpr bool DIRECT = false;
+  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
+  static constexpr bool PREFETCH2 = false;
   static constexpr int NBLK = ROWS / 8;            // 8-column blocks per tile
   static constexpr int PASSES = (16 * NBLK) / NT;  // 64 k = 16 blocks of 4 rows
   static constexpr int UNITS = PASSES * 4;
@@ -40,7 +43,7 @@ struct H16KNLoader {
   }
 
   template <bool TAIL>
-  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* /*lds_next*/ = nullptr) const {
     const uint8_t* sb = base + (int64_t)kt * 64 * ld;
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
@@ -86,11 +89,11 @@ template <class Mma, int BM, int BN, int WM, int WN>
 static int run_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int out_dtype, int b_layout,
                    hipStream_t st) {
   constexpr int NT = WM * WN * 64;
-  typedef RowLoader<BM, NT> AL;
+  typedef RowLoaderDirect<BM, NT> AL;
   typename AL::Params pa{(const uint8_t*)A, K * 2, 0, K * 2};
   EpiFloat::Params pe{C, N, 0, out_dtype};
   if (b_layout == TLQ_B_NK) {
-    typedef RowLoader<BN, NT> WL;
+    typedef RowLoaderDirect<BN, NT> WL;
     typename WL::Params pw{(const uint8_t*)B, K * 2, 0, K * 2};
     return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16");
   }

@@ -12,6 +12,9 @@ namespace tlq {
 template <int ROWS, int NT>
 struct W4I8Loader {
   typedef RowFrag Frag;
+  static constexpr bool DIRECT = false;
+  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
+  static constexpr bool PREFETCH2 = false;
   static constexpr int SLOTS = ROWS * 4;
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
@@ -48,7 +51,7 @@ struct W4I8Loader {
   }
 
   template <bool TAIL>
-  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* /*lds_next*/ = nullptr) const {
     const uint8_t* sb = base + (int64_t)kt * 64;
     if (!TAIL) {
 #pragma unroll
@@ -100,7 +103,7 @@ template <class WL, class Epi, int BM, int BN, int WM, int WN>
 static int run_i8(const void* A, const typename WL::Params& pw, const typename Epi::Params& pe, int64_t batch,
                   int64_t M, int64_t N, int64_t K, hipStream_t st, const char* what) {
   constexpr int NT = WM * WN * 64;
-  typedef RowLoader<BM, NT> AL;
+  typedef RowLoaderDirect<BM, NT> AL;  // activations travel global -> LDS without passing through registers
   typename AL::Params pa{(const uint8_t*)A, K, M * K, K};
   return launch_gemm<MmaI8, AL, WL, Epi, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K, st, what);
 }
@@ -137,7 +140,7 @@ static int dispatch_i8(const void* A, const void* B, const typename Epi::Params&
   } else {
 #define TLQ_RUN(BM, BN, WM, WN)                                               \
   {                                                                           \
-    typedef RowLoader<BN, WM * WN * 64> WL;                                   \
+    typedef RowLoaderDirect<BN, WM * WN * 64> WL;                             \
     typename WL::Params pw{(const uint8_t*)B, K, N * K, K};                   \
     return run_i8<WL, Epi, BM, BN, WM, WN>(A, pw, pe, batch, M, N, K, st, what); \
   }

@@ -95,6 +95,9 @@ struct Expand8<bf16_t, FOLD> {
 template <typename T, bool FOLD, int ROWS, int NT>
 struct W4Loader {
   typedef RowFrag Frag;
+  static constexpr bool DIRECT = false;
+  static constexpr int VALU_PER_MFMA = 0;
+  static constexpr bool PREFETCH2 = true;  // convert from registers loaded one stage earlier
   static constexpr int SLOTS = ROWS * 2;  // 16-byte packed loads per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
@@ -149,7 +152,7 @@ struct W4Loader {
   // Group index of element (kt*64 + half*32) = ((kt*64) >> shift) + ((half*32) >> shift) for every
   // power-of-two group >= 32.
   template <bool TAIL>
-  __device__ __forceinline__ void gload(Regs& r, int kt) const {
+  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* /*lds_next*/ = nullptr) const {
     const uint8_t* sb = base + (int64_t)kt * 32;
     const uint32_t gk = (uint32_t)((kt * 64) >> group_shift);
 #pragma unroll
@@ -225,7 +228,9 @@ static typename W4Loader<T, FOLD, ROWS, NT>::Params w4_params(const W4Args& a) {
 template <typename T, bool FOLD, int BM, int BN, int WM, int WN>
 static int run_w4a16(const W4Args& a) {
   constexpr int NT = WM * WN * 64;
-  typedef RowLoader<BM, NT> AL;
+  // activations travel global -> LDS directly whenever the tile splits into whole wavefront loads
+  constexpr bool DIRECT = BM % 8 == 0 && (BM / 8) % (NT / 64) == 0;
+  typedef typename std::conditional<DIRECT, RowLoaderDirect<DIRECT ? BM : 8 * (NT / 64), NT>, RowLoader<BM, NT>>::type AL;
   typedef W4Loader<T, FOLD, BN, NT> WL;
   typename AL::Params pa{(const uint8_t*)a.A, a.K * 2, 0, a.K * 2};
   auto pw = w4_params<T, FOLD, BN, NT>(a);

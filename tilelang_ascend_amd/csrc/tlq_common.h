@@ -86,6 +86,15 @@ __device__ __forceinline__ float ubyte_to_float(uint32_t x) {
 __device__ __forceinline__ float round_to_bf16(float f) { return bitcast<float>(float_to_bf16_bits(f) << 16); }
 
 // Generic load of a 16-bit float T (half_t or bf16_t) as float, and store with RNE.
+// Tells the compiler that a pointer is the same in every lane, so that address = scalar base +
+// 32-bit lane offset stays in that form (one VGPR per access instead of a 64-bit pair).
+__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
+  const uint64_t a = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return (const uint8_t*)(((uint64_t)hi << 32) | lo);
+}
+
 template <typename T>
 __device__ __forceinline__ float to_float(T v);
 template <>
