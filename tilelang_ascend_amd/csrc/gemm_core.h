@@ -338,6 +338,90 @@ struct I8KNLoader {
   __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
 };
 
+// The same [128 k][BN] tile filled by direct global -> LDS loads: one wavefront instruction covers
+// 1024 / BN consecutive k rows; the lane landing on (k, physical chunk pc) fetches logical chunk
+// pc ^ kn_swz(k) of that k row.  A partial last stage (rows past K must read as zero) goes through
+// registers.
+template <int BN, int NT>
+struct I8KNLoaderDirect {
+  typedef KNFrag8<BN> Frag;
+  static constexpr bool DIRECT = true;
+  static constexpr int VALU_PER_MFMA = 0;
+  static constexpr bool PREFETCH2 = false;
+  static constexpr int CH = BN / 16;              // 16-byte chunks per k row
+  static constexpr int KPI = 64 / CH;             // k rows per wavefront instruction
+  static constexpr int WAVES = NT / 64;
+  static constexpr int INSTR = kStageBytes / KPI;  // wavefront instructions per stage
+  static constexpr int PER_WAVE = INSTR / WAVES;
+  static constexpr int UNITS = PER_WAVE;
+  static_assert(INSTR % WAVES == 0 && PER_WAVE >= 1, "tile does not split into whole wavefront loads");
+  typedef typename I8KNLoader<BN, NT>::Params Params;
+  struct Regs {
+    uint4_t v[PER_WAVE];
+    bool pending;
+  };
+  const uint8_t* base;
+  uint32_t voff[PER_WAVE];  // per lane: k * ld + logical chunk * 16
+  uint32_t wave_off, lane_off;
+  int k_lane;  // k row of this lane inside instruction 0 of wavefront 0
+  int wave, k_total;
+
+  __device__ __forceinline__ I8KNLoaderDirect(const Params& p, int batch, int col0, int cols_total, int tid)
+      : base(p.base + batch * p.batch_stride + col0), k_total((int)p.k_total) {
+    const int cols_valid = cols_total - col0;
+    const int lane = tid & 63;
+    wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    wave_off = (uint32_t)wave * 1024u;
+    lane_off = (uint32_t)lane * 16u;
+    k_lane = lane / CH;
+    const int pc = lane % CH;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) {
+      const int k = (j * WAVES + wave) * KPI + k_lane;
+      int col = (pc ^ kn_swz<BN>(k)) * 16;
+      col = col < cols_valid ? col : cols_valid - 16;  // clamp whole chunks; those columns are masked later
+      voff[j] = (uint32_t)k * (uint32_t)p.ld + (uint32_t)col;
+    }
+    ld_ = (uint32_t)p.ld;
+  }
+  uint32_t ld_;
+
+  template <bool TAIL>
+  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* lds_next) const {
+    typedef __attribute__((address_space(3))) uint8_t* lptr_t;
+    if (!TAIL) {
+      r.pending = false;
+      const uint8_t* sb = uniform_ptr(base + (int64_t)kt * kStageBytes * ld_);
+      const uint32_t l0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lptr_t)lds_next + wave_off);
+#pragma unroll
+      for (int j = 0; j < PER_WAVE; ++j)
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0 + (uint32_t)(j * WAVES * 1024)),
+                     "v"(voff[j]), "s"(sb)
+                     : "memory");
+    } else {
+      r.pending = true;
+      const uint8_t* sb = base + (int64_t)kt * kStageBytes * ld_;
+#pragma unroll
+      for (int j = 0; j < PER_WAVE; ++j) {
+        const int k = (j * WAVES + wave) * KPI + k_lane;
+        const bool ok = kt * kStageBytes + k < k_total;
+        uint4_t v = *(const uint4_t*)(ok ? sb + voff[j] : base + (voff[j] - (uint32_t)k * ld_));
+        if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
+        r.v[j] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
+    if (!r.pending) return;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) {
+      if (j * np / UNITS != pc) continue;
+      *(uint4_t*)(lds + wave_off + j * WAVES * 1024 + lane_off) = r.v[j];
+    }
+  }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
+};
+
 // ---- epilogues ----------------------------------------------------------------------------
 // store(m, n, acc): acc holds C[m, n .. n+3]
 struct EpiFloat {  // fp32 accumulators -> f16 / bf16 / f32

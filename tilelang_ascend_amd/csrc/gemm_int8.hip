@@ -124,7 +124,7 @@ static int dispatch_i8(const void* A, const void* B, const typename Epi::Params&
   if (b_layout == TLQ_B_KN) {
 #define TLQ_RUN(BM, BN, WM, WN)                                               \
   {                                                                           \
-    typedef I8KNLoader<BN, WM * WN * 64> WL;                                  \
+    typedef I8KNLoaderDirect<BN, WM * WN * 64> WL;                            \
     typename WL::Params pw{(const uint8_t*)B, N, K * N, K};                   \
     return run_i8<WL, Epi, BM, BN, WM, WN>(A, pw, pe, batch, M, N, K, st, what); \
   }
