@@ -62,7 +62,8 @@ enum {
 enum {
   TLQ_ALGO_AUTO = 0,
   TLQ_ALGO_GEMV = 1, /* split-K wavefront GEMV (M <= 16) */
-  TLQ_ALGO_MFMA = 2  /* LDS-staged MFMA dequant-GEMM */
+  TLQ_ALGO_MFMA = 2, /* LDS-staged MFMA dequant-GEMM */
+  TLQ_ALGO_SKINNY = 3 /* M <= 64: weights stream from HBM through the dequantiser into MFMA operands, no LDS tile */
 };
 
 int tlq_abi_version(void);
@@ -101,7 +102,8 @@ int tlq_decode_i4_interleaved(const void* words, const void* scales, const void*
  *   C[M,N] = rn_out( sum_k f32(A[m,k]) * f32(W[n,k]) ),  W as in tlq_dequant_w4, fp32 accumulate.
  * A: [M,K] in_dtype (TLQ_F16 / TLQ_BF16); C: [M,N] out_dtype (TLQ_F16 / TLQ_BF16 / TLQ_F32).
  * Requires K % 64 == 0 and group % 32 == 0 (group divides K).  The MFMA kernel additionally needs
- * N % 4 == 0 and a power-of-two group (32, 64, 128, ...); the GEMV kernel takes any such group. */
+ * N % 4 == 0 and a power-of-two group (32, 64, 128, ...); the GEMV kernel (M <= 16) takes any such group;
+ * the skinny kernel (M <= 64) needs K % 128 == 0.  TLQ_ALGO_AUTO: M <= 4 GEMV, M <= 64 skinny, else MFMA. */
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                    void* stream);
@@ -153,6 +155,7 @@ int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void*
 void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4, waves 1..4 */
 void tlq_tune_gemv_unroll(int blocks_per_cu);               /* resident blocks per CU the GEMV grid is sized for */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
+void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16, 16-row tiles per wavefront 1|2 */
 void tlq_tune_i8_tile(int block_m);                         /* 32|128|256 */
 
 #ifdef __cplusplus

@@ -64,7 +64,7 @@ def test_enum_codes_match_the_header():
                       ("TLQ_I32", _abi.I32), ("TLQ_U4", _abi.U4), ("TLQ_S4_TWOS", _abi.S4_TWOS),
                       ("TLQ_S4_OFFSET8", _abi.S4_OFFSET8), ("TLQ_S4_OFFSET7", _abi.S4_OFFSET7), ("TLQ_B_KN", _abi.B_KN),
                       ("TLQ_B_NK", _abi.B_NK), ("TLQ_ALGO_AUTO", _abi.ALGO_AUTO), ("TLQ_ALGO_GEMV", _abi.ALGO_GEMV),
-                      ("TLQ_ALGO_MFMA", _abi.ALGO_MFMA)):
+                      ("TLQ_ALGO_MFMA", _abi.ALGO_MFMA), ("TLQ_ALGO_SKINNY", _abi.ALGO_SKINNY)):
         m = re.search(rf"\b{name}\s*=\s*(\d+)", text)
         assert m and int(m.group(1)) == val, name
 

@@ -382,3 +382,51 @@ def test_golden_int8(ops):
     workspace = torch.empty(N, K, dtype=torch.int8, device="cuda")  # a caller-supplied input in the reference
     got = ops.w4a8_gemm_cv(M, N, K)(Ad[0].contiguous(), Wp.cuda(), workspace).cpu()
     assert_bit_equal(got.T.contiguous(), torch.from_numpy(d["w4.C_signed_t"]), "golden s4 x i8")
+
+
+# ------------------------------------------------------------------------------------------
+# skinny kernel (M <= 64, weights streamed from HBM straight into MFMA operands)
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K,group,zeros_kind", [
+    (5, 64, 128, 32, None), (16, 1000, 4096, 128, "int"), (17, 130, 2048, 64, "scalar8"), (32, 512, 1024, 1024, "frac"),
+    (33, 272, 1536, 96, "int"), (64, 4096, 1024, 128, "scalar8"), (48, 14336, 4096, 64, "int"),
+])
+def test_skinny_shapes(ops, in_dtype, M, N, K, group, zeros_kind):
+    dt = DT[in_dtype]
+    A = torch.randn(M, K, generator=gen(40)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=41)
+    want = w4a16_reference(A, Wp, s, z, group)
+    for out_dtype in ("float32", in_dtype):
+        got = _run_w4a16(ops, A, Wp, s, z, group, out_dtype, "skinny", in_dtype)
+        check_float_output(got, want, f"skinny {in_dtype}->{out_dtype}")
+
+
+@pytest.mark.parametrize("waves,row_tiles", [(1, 1), (3, 1), (16, 1), (4, 2), (16, 2)])
+def test_skinny_tunings_and_one_hot(ops, waves, row_tiles):
+    """One-hot activations return dequantised weight columns bit-exactly through the MFMA path, whatever
+    the split of K between wavefronts."""
+    from tilelang_ascend_amd import _abi
+
+    N, K, group = 200, 1024, 128
+    Wp, s, z = make_w4(N, K, group, torch.float16, "int", seed=42)
+    W = ref.dequant_w4(Wp, s, z, group, torch.float16)
+    A = torch.zeros(16, K, dtype=torch.float16)
+    cols = [0, 1, 31, 32, 127, 128, 500, 1023, 640, 77, 900, 255, 256, 511, 512, 1000]
+    for m, k in enumerate(cols):
+        A[m, k] = 1.0
+    _abi.load().tlq_tune_w4a16_skinny(waves, row_tiles)
+    try:
+        got = _run_w4a16(ops, A, Wp, s, z, group, "float16", "skinny", "float16")
+    finally:
+        _abi.load().tlq_tune_w4a16_skinny(0, 0)
+    assert_bit_equal(got, W[:, cols].T.contiguous(), f"skinny one-hot waves={waves} rt={row_tiles}")
+
+
+def test_auto_picks_a_kernel_for_every_m(ops):
+    N, K, group = 256, 1024, 128
+    Wp, s, z = make_w4(N, K, group, torch.float16, "int", seed=43)
+    for M in (1, 4, 5, 16, 64, 65, 200):
+        A = torch.randn(M, K, generator=gen(44)).to(torch.float16)
+        got = _run_w4a16(ops, A, Wp, s, z, group, "float16", "auto", "float16")
+        check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"auto M={M}")

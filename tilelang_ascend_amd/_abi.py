@@ -17,7 +17,7 @@ from . import build as _build
 F16, BF16, F32, I8, I32 = 0, 1, 2, 3, 4
 U4, S4_TWOS, S4_OFFSET8, S4_OFFSET7 = 0, 1, 2, 3
 B_KN, B_NK = 0, 1
-ALGO_AUTO, ALGO_GEMV, ALGO_MFMA = 0, 1, 2
+ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY = 0, 1, 2, 3
 ABI_VERSION = 1
 
 _vp, _i64, _int, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
@@ -39,6 +39,7 @@ SIGNATURES = {
     "tlq_tune_gemv": (None, [_int, _int]),
     "tlq_tune_gemv_unroll": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),
+    "tlq_tune_w4a16_skinny": (None, [_int, _int]),
     "tlq_tune_i8_tile": (None, [_int]),
 }
 

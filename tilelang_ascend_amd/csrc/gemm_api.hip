@@ -7,6 +7,8 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
                int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
+int gemm_w4a16_skinny(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                      int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
                    int b_layout, hipStream_t st);
 int gemm_i8_i32(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,
@@ -38,7 +40,7 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
               in_dtype);
   TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32,
               "tlq_gemm_w4a16: out_dtype must be float16, bfloat16 or float32 (got %d)", out_dtype);
-  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_MFMA, "tlq_gemm_w4a16: bad algo %d", algo);
+  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_SKINNY, "tlq_gemm_w4a16: bad algo %d", algo);
   if (M == 0 || N == 0) return 0;
   TLQ_REQUIRE(K > 0 && K % 64 == 0, "tlq_gemm_w4a16: K=%lld must be a positive multiple of 64", (long long)K);
   TLQ_REQUIRE(group > 0 && K % group == 0 && group % 32 == 0,
@@ -47,7 +49,13 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
   TLQ_REQUIRE(aligned16(A) && aligned16(w_packed) && aligned16(C), "tlq_gemm_w4a16: A, w_packed and C must be 16-byte aligned");
   TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16: scales / zeros misaligned");
   hipStream_t st = (hipStream_t)stream;
-  if (algo == TLQ_ALGO_AUTO) algo = (M <= 4) ? TLQ_ALGO_GEMV : TLQ_ALGO_MFMA;
+  if (algo == TLQ_ALGO_AUTO) algo = (M <= 4) ? TLQ_ALGO_GEMV : ((M <= 64 && K % 128 == 0) ? TLQ_ALGO_SKINNY : TLQ_ALGO_MFMA);
+  if (algo == TLQ_ALGO_SKINNY) {
+    TLQ_REQUIRE(M <= 64, "tlq_gemm_w4a16: the skinny kernel handles M <= 64 (got %lld)", (long long)M);
+    TLQ_REQUIRE(K % 128 == 0, "tlq_gemm_w4a16: the skinny kernel needs K %% 128 == 0 (got %lld)", (long long)K);
+    TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K / 2), "tlq_gemm_w4a16: a matrix spans 4 GiB or more");
+    return gemm_w4a16_skinny(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, st);
+  }
   if (algo == TLQ_ALGO_GEMV) {
     TLQ_REQUIRE(M <= 16, "tlq_gemm_w4a16: the GEMV kernel handles M <= 16 (got %lld)", (long long)M);
     return gemv_w4a16(A, w_packed, scales, zeros, C, 1, M, N, K, group, zero_scalar, in_dtype, out_dtype, st);

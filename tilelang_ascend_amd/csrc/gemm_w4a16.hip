@@ -272,6 +272,205 @@ static int dispatch_w4a16(const W4Args& a) {
   }
 }
 
+// ---- skinny kernel: a few activation rows (M <= 64) against a large weight matrix ---------------
+// HBM bound: every packed weight is read once and goes straight from global memory through the
+// dequantiser into an MFMA operand register; there is no LDS tile.  A wavefront owns RT tiles of 16
+// weight rows and a slice of K; per 128 values of K ("k-block") lane (row r = lane % 16, k-group
+// q = lane / 16) loads the 16 packed bytes of k = 128*kb + 32*q .. +31 of its row (one quantisation
+// group, so one scale / zero per lane and k-block), expands them into four 8-value operands, and
+// feeds four MFMAs whose activation operand holds A[m = lane % 16][the same 8 k] (the MFMA does not
+// care which k a k-group holds as long as both operands agree).  The wavefronts of a work-group
+// split K between them and add their partial tiles through LDS, so no global reduction is needed.
+template <typename T, bool FOLD, int RT, int MT>
+__global__ __launch_bounds__(MT >= 4 ? 512 : 1024) void w4a16_skinny_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
+                                                            const T* __restrict__ scales, const T* __restrict__ zeros,
+                                                            void* __restrict__ C, int M, int N, int K, int group,
+                                                            float zero_scalar, int out_dtype) {
+  typedef typename MmaOf<T>::type Mma;
+  extern __shared__ __align__(16) uint8_t smem[];
+  float4_t* const red = (float4_t*)smem;  // [waves][RT * MT][64 lanes]
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves = blockDim.x >> 6;
+  const int r16 = lane & 15, q = lane >> 4;
+  const int n_base = blockIdx.x * (16 * RT);
+  const int groups = K / group;
+  const int KB = K >> 7;
+  const int kb0 = (int)(((int64_t)wave * KB) / waves), kb1 = (int)(((int64_t)(wave + 1) * KB) / waves);
+  const bool has_s = scales != nullptr, has_z = zeros != nullptr;
+  const T one = from_float<T>(1.0f), zs = from_float<T>(zero_scalar);
+  const NibbleMagic mg = make_nibble_magic();
+
+  uint32_t woff[RT], goff[RT], aoff[MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    int n = n_base + rt * 16 + r16;
+    n = n < N ? n : N - 1;  // clamp: loads stay in bounds, the rows are masked at the store
+    woff[rt] = (uint32_t)n * (uint32_t)(K >> 1) + (uint32_t)(q * 16);
+    goff[rt] = (uint32_t)n * (uint32_t)groups;
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int m = mt * 16 + r16;
+    m = m < M ? m : M - 1;
+    aoff[mt] = ((uint32_t)m * (uint32_t)K + (uint32_t)(q * 32)) * 2u;
+  }
+  const T* const sp = has_s ? scales : A;  // absent tensors: read a valid dummy location, discard the value
+  const T* const zp = has_z ? zeros : A;
+
+  struct Block {
+    uint4_t w[RT];
+    T s[RT], z[RT];
+    uint4_t a[MT][4];
+  };
+  auto load = [&](Block& b, int kb) {
+    const uint32_t gi = (uint32_t)((kb * 128 + q * 32) / group);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      b.w[rt] = *(const uint4_t*)(Wp + woff[rt] + (uint32_t)kb * 64u);
+      const T sv = sp[has_s ? goff[rt] + gi : 0u];
+      const T zv = zp[has_z ? goff[rt] + gi : 0u];
+      b.s[rt] = has_s ? sv : one;
+      b.z[rt] = has_z ? zv : zs;
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b.a[mt][j] = *(const uint4_t*)((const uint8_t*)A + aoff[mt] + (uint32_t)kb * 256u + j * 16);
+  };
+
+  typename Mma::acc_t acc[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = typename Mma::acc_t{0, 0, 0, 0};
+  auto compute = [&](const Block& b) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const Expand8<T, FOLD> ex(b.s[rt], b.z[rt], mg);
+      const uint32_t w[4] = {b.w[rt].x, b.w[rt].y, b.w[rt].z, b.w[rt].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint4_t wf = ex(w[j]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = Mma::mma(wf, b.a[mt][j], acc[rt][mt]);
+      }
+    }
+  };
+
+  // A wavefront's slice of K is only a few k-blocks long, and one k-block of arithmetic is far
+  // shorter than a trip to memory: issue the loads of DEPTH k-blocks at once, then compute them.
+  // (Other wavefronts of the CU cover the time between chunks.)
+  constexpr int DEPTH = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
+  Block b[DEPTH];
+  for (int kb = kb0; kb < kb1; kb += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int k = kb + d < kb1 ? kb + d : kb1 - 1;  // past the slice: reload the last block, skip its arithmetic
+      load(b[d], k);
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (kb + d < kb1) compute(b[d]);
+  }
+
+  // add the partial tiles of the wavefronts (they hold different slices of K)
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[(wave * (RT * MT) + rt * MT + mt) * 64 + lane] = acc[rt][mt];
+  __syncthreads();
+  for (int item = threadIdx.x; item < RT * MT * 64; item += blockDim.x) {
+    float4_t sum = red[item];
+    for (int w = 1; w < waves; ++w) {
+      const float4_t v = red[w * (RT * MT * 64) + item];
+      sum[0] += v[0];
+      sum[1] += v[1];
+      sum[2] += v[2];
+      sum[3] += v[3];
+    }
+    // lane l of a tile holds D[n = 4 * (l / 16) + i][m = l % 16]
+    const int tile = item >> 6, l = item & 63;
+    const int rt = tile / MT, mt = tile - rt * MT;
+    const int m = mt * 16 + (l & 15);
+    const int n = n_base + rt * 16 + 4 * (l >> 4);
+    if (m >= M || n >= N) continue;
+    const int64_t idx = (int64_t)m * N + n;
+    if (n + 3 < N && (N & 3) == 0) {
+      if (out_dtype == TLQ_F32) {
+        *(float4_t*)((float*)C + idx) = sum;
+      } else if (out_dtype == TLQ_F16) {
+        half_t h[4] = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+        *(uint2_t*)((half_t*)C + idx) = bitcast<uint2_t>(h);
+      } else {
+        uint2_t o;
+        o.x = pack_bf16x2(sum[0], sum[1]);
+        o.y = pack_bf16x2(sum[2], sum[3]);
+        *(uint2_t*)((uint16_t*)C + idx) = o;
+      }
+    } else {
+      for (int i = 0; i < 4 && n + i < N; ++i) store_out(C, idx + i, sum[i], out_dtype);
+    }
+  }
+}
+
+static int g_skinny_waves = 0, g_skinny_rt = 0;  // tuning overrides (0 = automatic)
+
+template <typename T, bool FOLD, int RT, int MT>
+static int launch_skinny(const W4Args& a, int waves) {
+  auto kern = w4a16_skinny_kernel<T, FOLD, RT, MT>;
+  const int blocks = (int)ceil_div(a.N, 16 * RT);
+  const size_t lds = (size_t)waves * RT * MT * 64 * sizeof(float4_t);
+  kern<<<blocks, waves * 64, lds, a.st>>>((const T*)a.A, (const uint8_t*)a.Wp, (const T*)a.scales, (const T*)a.zeros, a.C,
+                                          (int)a.M, (int)a.N, (int)a.K, (int)a.group, a.zero_scalar, a.out_dtype);
+  return check_launch("tlq_gemm_w4a16(skinny)") ? 0 : 1;
+}
+
+template <typename T, bool FOLD>
+static int dispatch_skinny(const W4Args& a) {
+  const int64_t row_tiles = ceil_div(a.N, 16);
+  const int KB = (int)(a.K / 128);
+  // enough wavefronts to keep every CU streaming: about 24 per CU over the whole grid, at least two k-blocks each
+  // two row tiles per wavefront halve the activation loads per weight; worth it once there are plenty of rows
+  int rt = g_skinny_rt ? g_skinny_rt : (row_tiles >= 2048 / 4 ? 2 : 1);
+  int waves = g_skinny_waves;
+  if (!waves) {
+    static int cus = 0;  // cached: one attribute query per process
+    if (cus == 0) {
+      int dev = 0;
+      if (hipGetDevice(&dev) != hipSuccess ||
+          hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    }
+    const int64_t want = (int64_t)cus * 24;
+    waves = 1;
+    while (waves < 16 && row_tiles / rt * waves < want && KB / (waves * 2) >= 2) waves *= 2;
+  }
+  if (waves > KB) waves = KB < 1 ? 1 : KB;
+  const int mt = a.M <= 16 ? 1 : (a.M <= 32 ? 2 : 4);
+  const int max_waves = mt >= 4 ? 8 : 16;  // four activation tiles need 256 registers per lane
+  if (waves > max_waves) waves = max_waves;
+#define TLQ_SK(RTT, MTT) return launch_skinny<T, FOLD, RTT, MTT>(a, waves)
+  if (rt == 2) {
+    if (mt == 1) TLQ_SK(2, 1);
+    if (mt == 2) TLQ_SK(2, 2);
+    TLQ_SK(2, 4);
+  }
+  if (mt == 1) TLQ_SK(1, 1);
+  if (mt == 2) TLQ_SK(1, 2);
+  TLQ_SK(1, 4);
+#undef TLQ_SK
+}
+
+int gemm_w4a16_skinny(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                      int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st) {
+  const bool fold = zeros == nullptr && zero_scalar == (float)(int)zero_scalar && zero_scalar >= -256.0f &&
+                    zero_scalar <= 256.0f;
+  const W4Args a{A, Wp, scales, zeros, C, M, N, K, group, zero_scalar, out_dtype, st};
+  if (in_dtype == TLQ_F16) return fold ? dispatch_skinny<half_t, true>(a) : dispatch_skinny<half_t, false>(a);
+  return fold ? dispatch_skinny<bf16_t, true>(a) : dispatch_skinny<bf16_t, false>(a);
+}
+
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st) {
   if ((group & (group - 1)) != 0) {
@@ -292,4 +491,10 @@ extern "C" {
 // Tuning hook used by the benchmark sweeps: forces the activation-tile height (16, 32, 64,
 // 128, 256) of the W4A16 MFMA kernel; 0 restores the automatic choice.
 void tlq_tune_w4a16_tile(int block_m) { tlq::g_w4a16_tile = block_m; }
+// Wavefronts per work-group (1..16, the in-group split of K) and 16-row weight tiles per wavefront
+// (1 | 2) of the skinny W4A16 kernel; 0 restores the automatic choice.
+void tlq_tune_w4a16_skinny(int waves, int row_tiles) {
+  tlq::g_skinny_waves = (waves < 0 || waves > 16) ? 0 : waves;
+  tlq::g_skinny_rt = (row_tiles == 2) ? 2 : (row_tiles == 1 ? 1 : 0);
+}
 }
