@@ -155,7 +155,8 @@ int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void*
 void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4, waves 1..4 */
 void tlq_tune_gemv_unroll(int blocks_per_cu);               /* resident blocks per CU the GEMV grid is sized for */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
-void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16, 16-row tiles per wavefront 1|2 */
+void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,
+                                                               +10 = never stage through LDS, +20 = stage whenever possible */
 void tlq_tune_i8_tile(int block_m);                         /* 32|128|256 */
 
 #ifdef __cplusplus

@@ -414,6 +414,213 @@ __global__ __launch_bounds__(MT >= 4 ? 512 : 1024) void w4a16_skinny_kernel(cons
   }
 }
 
+// ---- skinny kernel for M <= 16, operands staged through wavefront-private LDS -------------------
+// The direct form above asks every lane for 16 bytes of a different row, which the memory pipeline
+// serves one lane per cycle.  Here every global access is a full-width direct global -> LDS load
+// (1 KB per wavefront instruction, adjacent lanes adjacent addresses): per k-block RT loads of a
+// [16 rows][64 B] packed-weight tile and four loads of the [16 rows][256 B] activation tile, into one
+// of two slots of LDS that only this wavefront uses (so there is no barrier, only counters).  The
+// MFMA-shaped fragments are then read back with ds_read_b128; 16-byte pieces are XOR-swizzled on the
+// global side so that those reads are conflict free.  Scales / zeros come in as dword gathers that
+// cover four consecutive groups of the 16 rows at once, i.e. once per four k-blocks at group 128.
+// While k-block i is dequantised and multiplied, the loads of i+1 and i+2 are in flight.
+template <typename T, bool FOLD, int RT>
+__global__ __launch_bounds__(1024) void w4a16_skinny_lds_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
+                                                                const T* __restrict__ scales, const T* __restrict__ zeros,
+                                                                void* __restrict__ C, int M, int N, int K, int gshift,
+                                                                float zero_scalar, int out_dtype) {
+  typedef typename MmaOf<T>::type Mma;
+  typedef __attribute__((address_space(3))) uint8_t* lptr_t;
+  constexpr int SLOT = RT * 1024 + 4096;  // RT weight tiles + one activation tile
+  constexpr int SC = RT * 2 * 256;        // [rt][scale | zero][64 dwords]
+  constexpr int WAVE_LDS = 2 * SLOT + 2 * SC;
+  constexpr int NI = RT + 4;              // direct loads per k-block
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves = blockDim.x >> 6;
+  const int r16 = lane & 15, q = lane >> 4;
+  uint8_t* const mine = smem + wave * WAVE_LDS;
+  const uint32_t mine_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lptr_t)mine);
+  const int n_base = blockIdx.x * (16 * RT);
+  const int groups = K >> gshift;
+  const int KB = K >> 7;
+  const int kb0 = (int)(((int64_t)wave * KB) / waves), kb1 = (int)(((int64_t)(wave + 1) * KB) / waves);
+  const int nkb = kb1 - kb0;
+  const bool has_s = scales != nullptr, has_z = zeros != nullptr;
+  const int NS = RT * ((has_s ? 1 : 0) + (has_z ? 1 : 0));  // gathers per scale period (uniform)
+  const T one = from_float<T>(1.0f), zs = from_float<T>(zero_scalar);
+  const NibbleMagic mg = make_nibble_magic();
+
+  // ---- per-lane source offsets of the direct loads ----
+  uint32_t voff_w[RT], voff_a[4], row_g[RT];
+  {
+    const int rho = lane >> 2, piece = (lane & 3) ^ ((rho >> 1) & 3);  // lands on row lane/4, physical piece lane%4
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      int n = n_base + rt * 16 + rho;
+      n = n < N ? n : N - 1;
+      voff_w[rt] = (uint32_t)n * (uint32_t)(K >> 1) + (uint32_t)(piece * 16);
+      int ng = n_base + rt * 16 + r16;  // the row this lane gathers scales for / dequantises
+      ng = ng < N ? ng : N - 1;
+      row_g[rt] = (uint32_t)ng * (uint32_t)groups;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = i * 4 + (lane >> 4);
+      const int lp = (lane & 15) ^ (row & 7);  // physical piece lane%16 holds logical piece lp
+      const int m = row < M ? row : M - 1;
+      voff_a[i] = ((uint32_t)m * (uint32_t)K) * 2u + (uint32_t)(lp * 16);
+    }
+  }
+  // ---- per-lane LDS offsets of the fragment reads ----
+  const uint32_t fo_w = (uint32_t)(r16 * 64 + ((q ^ ((r16 >> 1) & 3)) << 4));
+  uint32_t fo_a[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) fo_a[j] = (uint32_t)(RT * 1024 + r16 * 256 + (((q * 4 + j) ^ (r16 & 7)) << 4));
+
+  auto dma16 = [&](uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+  };
+  auto issue_kb = [&](int kb, int slot) {
+    const uint8_t* wsb = uniform_ptr(Wp + (int64_t)kb * 64);
+    const uint8_t* asb = uniform_ptr((const uint8_t*)A + (int64_t)kb * 256);
+    const uint32_t l0 = mine_lds + (uint32_t)(slot * SLOT);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) dma16(l0 + rt * 1024, voff_w[rt], wsb);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16(l0 + RT * 1024 + i * 1024, voff_a[i], asb);
+  };
+  // four consecutive groups (base .. base+3) of the 16 rows of every tile: lane (row r16, group q)
+  auto issue_sc = [&](int base, int buf) {
+    int g = base + q;
+    g = g < groups ? g : groups - 1;
+    const uint32_t l0 = mine_lds + (uint32_t)(2 * SLOT + buf * SC);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const uint64_t e2 = ((uint64_t)row_g[rt] + (uint64_t)g) * 2u;
+      if (has_s) {
+        const uint64_t a = ((uint64_t)(uintptr_t)scales + e2) & ~(uint64_t)3;
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(l0 + (rt * 2 + 0) * 256), "v"(a) : "memory");
+      }
+      if (has_z) {
+        const uint64_t a = ((uint64_t)(uintptr_t)zeros + e2) & ~(uint64_t)3;
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(l0 + (rt * 2 + 1) * 256), "v"(a) : "memory");
+      }
+    }
+  };
+  auto sc_base = [&](int kb) { return ((kb << 7) >> gshift) & ~3; };
+  auto new_period = [&](int kb) { return NS > 0 && (kb == kb0 || sc_base(kb) != sc_base(kb - 1)); };
+  auto sc_buf = [&](int kb) { return (sc_base(kb) >> 2) & 1; };
+
+  typename Mma::acc_t acc[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) acc[rt] = typename Mma::acc_t{0, 0, 0, 0};
+
+  if (nkb > 0) {
+    if (new_period(kb0)) issue_sc(sc_base(kb0), sc_buf(kb0));
+    issue_kb(kb0, 0);
+    if (nkb > 1) {
+      if (new_period(kb0 + 1)) issue_sc(sc_base(kb0 + 1), sc_buf(kb0 + 1));
+      issue_kb(kb0 + 1, 1);
+    }
+  }
+  for (int i = 0; i < nkb; ++i) {
+    const int kb = kb0 + i;
+    // everything issued for this k-block has landed once only the next k-block's loads are outstanding
+    if (i + 1 < nkb) {
+      if (new_period(kb + 1)) {
+        if (NS == 1 * RT) {
+          if (RT == 1) asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        } else {
+          if (RT == 1) asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+        }
+      } else {
+        if (RT == 1) asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+      }
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    const uint8_t* slot = mine + (i & 1) * SLOT;
+    uint4_t wf[RT], af[4];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) wf[rt] = *(const uint4_t*)(slot + rt * 1024 + fo_w);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) af[j] = *(const uint4_t*)(slot + fo_a[j]);
+    T sv[RT], zv[RT];
+    {
+      const int g = ((kb << 7) + (q << 5)) >> gshift;
+      const int rel = g - sc_base(kb);
+      const uint8_t* sc = mine + 2 * SLOT + sc_buf(kb) * SC + (r16 + 16 * rel) * 4;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const uint32_t sh = (((uint32_t)row_g[rt] + (uint32_t)g) & 1u) * 16u;
+        const uint32_t sa = (uint32_t)(((uintptr_t)scales >> 1) & 1), za = (uint32_t)(((uintptr_t)zeros >> 1) & 1);
+        sv[rt] = one;
+        zv[rt] = zs;
+        if (has_s) {
+          const uint32_t dw = *(const uint32_t*)(sc + (rt * 2 + 0) * 256);
+          sv[rt] = bitcast<T>((uint16_t)(dw >> (sh ^ (sa * 16u))));
+        }
+        if (has_z) {
+          const uint32_t dw = *(const uint32_t*)(sc + (rt * 2 + 1) * 256);
+          zv[rt] = bitcast<T>((uint16_t)(dw >> (sh ^ (za * 16u))));
+        }
+      }
+    }
+    // the slot may be overwritten once its contents are in registers
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (i + 2 < nkb) {
+      if (new_period(kb + 2)) issue_sc(sc_base(kb + 2), sc_buf(kb + 2));
+      issue_kb(kb + 2, i & 1);
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const Expand8<T, FOLD> ex(sv[rt], zv[rt], mg);
+      const uint32_t w[4] = {wf[rt].x, wf[rt].y, wf[rt].z, wf[rt].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[rt] = Mma::mma(ex(w[j]), af[j], acc[rt]);
+    }
+  }
+
+  // add the partial tiles of the wavefronts (the private regions are dead now)
+  __syncthreads();
+  float4_t* const red = (float4_t*)smem;  // [waves][RT][64 lanes]
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) red[(wave * RT + rt) * 64 + lane] = acc[rt];
+  __syncthreads();
+  for (int item = threadIdx.x; item < RT * 64; item += blockDim.x) {
+    float4_t sum = red[item];
+    for (int w = 1; w < waves; ++w) {
+      const float4_t v = red[w * (RT * 64) + item];
+      sum[0] += v[0];
+      sum[1] += v[1];
+      sum[2] += v[2];
+      sum[3] += v[3];
+    }
+    const int rt = item >> 6, l = item & 63;
+    const int m = l & 15;
+    const int n = n_base + rt * 16 + 4 * (l >> 4);
+    if (m >= M || n >= N) continue;
+    const int64_t idx = (int64_t)m * N + n;
+    if (n + 3 < N && (N & 3) == 0) {
+      if (out_dtype == TLQ_F32) {
+        *(float4_t*)((float*)C + idx) = sum;
+      } else if (out_dtype == TLQ_F16) {
+        half_t h[4] = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+        *(uint2_t*)((half_t*)C + idx) = bitcast<uint2_t>(h);
+      } else {
+        uint2_t o;
+        o.x = pack_bf16x2(sum[0], sum[1]);
+        o.y = pack_bf16x2(sum[2], sum[3]);
+        *(uint2_t*)((uint16_t*)C + idx) = o;
+      }
+    } else {
+      for (int i = 0; i < 4 && n + i < N; ++i) store_out(C, idx + i, sum[i], out_dtype);
+    }
+  }
+}
+
 static int g_skinny_waves = 0, g_skinny_rt = 0;  // tuning overrides (0 = automatic)
 
 template <typename T, bool FOLD, int RT, int MT>
@@ -426,13 +633,51 @@ static int launch_skinny(const W4Args& a, int waves) {
   return check_launch("tlq_gemm_w4a16(skinny)") ? 0 : 1;
 }
 
+template <typename T, bool FOLD, int RT>
+static int launch_skinny_lds(const W4Args& a, int waves, int gshift) {
+  auto kern = w4a16_skinny_lds_kernel<T, FOLD, RT>;
+  constexpr int WAVE_LDS = 2 * (RT * 1024 + 4096) + 2 * (RT * 2 * 256);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      set_error("tlq_gemm_w4a16(skinny): cannot reserve LDS: %s", hipGetErrorString(e));
+      return 1;
+    }
+    attr_set = true;
+  }
+  const int blocks = (int)ceil_div(a.N, 16 * RT);
+  kern<<<blocks, waves * 64, (size_t)waves * WAVE_LDS, a.st>>>((const T*)a.A, (const uint8_t*)a.Wp, (const T*)a.scales,
+                                                                (const T*)a.zeros, a.C, (int)a.M, (int)a.N, (int)a.K,
+                                                                gshift, a.zero_scalar, a.out_dtype);
+  return check_launch("tlq_gemm_w4a16(skinny)") ? 0 : 1;
+}
+
+static int g_skinny_lds = -1;  // tuning override: 0 = never, 1 = whenever possible, -1 = automatic
+
 template <typename T, bool FOLD>
 static int dispatch_skinny(const W4Args& a) {
   const int64_t row_tiles = ceil_div(a.N, 16);
   const int KB = (int)(a.K / 128);
+  // M <= 16 and a power-of-two group: operands staged through wavefront-private LDS
+  const bool pow2 = (a.group & (a.group - 1)) == 0;
+  // (the scale / zero gathers read aligned dwords: the tensors must start and end on a dword boundary)
+  const bool sz_ok = (((uintptr_t)a.scales | (uintptr_t)a.zeros) & 3) == 0 && ((a.N * (a.K / a.group)) & 1) == 0;
+  if (a.M <= 16 && pow2 && sz_ok && g_skinny_lds != 0) {
+    int gshift = 0;
+    while (((int64_t)1 << gshift) < a.group) ++gshift;
+    const int rt = g_skinny_rt ? g_skinny_rt : (row_tiles >= 512 ? 2 : 1);
+    // small work-groups while there are plenty of them (two or more fit on a CU), larger ones to split K further
+    int waves = g_skinny_waves ? g_skinny_waves : (row_tiles / rt >= 400 ? 4 : 8);
+    const int max_waves = rt == 2 ? 11 : 14;  // 160 KB of LDS
+    if (waves > max_waves) waves = max_waves;
+    if (waves > KB) waves = KB;
+    if (rt == 2) return launch_skinny_lds<T, FOLD, 2>(a, waves, gshift);
+    return launch_skinny_lds<T, FOLD, 1>(a, waves, gshift);
+  }
   // enough wavefronts to keep every CU streaming: about 24 per CU over the whole grid, at least two k-blocks each
   // two row tiles per wavefront halve the activation loads per weight; worth it once there are plenty of rows
-  int rt = g_skinny_rt ? g_skinny_rt : (row_tiles >= 2048 / 4 ? 2 : 1);
+  int rt = g_skinny_rt ? g_skinny_rt : (row_tiles >= 512 ? 2 : 1);
   int waves = g_skinny_waves;
   if (!waves) {
     static int cus = 0;  // cached: one attribute query per process
@@ -495,6 +740,7 @@ void tlq_tune_w4a16_tile(int block_m) { tlq::g_w4a16_tile = block_m; }
 // (1 | 2) of the skinny W4A16 kernel; 0 restores the automatic choice.
 void tlq_tune_w4a16_skinny(int waves, int row_tiles) {
   tlq::g_skinny_waves = (waves < 0 || waves > 16) ? 0 : waves;
-  tlq::g_skinny_rt = (row_tiles == 2) ? 2 : (row_tiles == 1 ? 1 : 0);
+  tlq::g_skinny_rt = (row_tiles % 10 == 2) ? 2 : (row_tiles % 10 == 1 ? 1 : 0);
+  tlq::g_skinny_lds = row_tiles >= 20 ? 1 : (row_tiles >= 10 ? 0 : -1);  // +10: registers only, +20: LDS staged
 }
 }
