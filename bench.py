@@ -35,8 +35,9 @@ POOL_BYTES = 576 * 1024 * 1024  # weight pool > 2x the 256 MB last-level cache
 # runs of this script with --calibrate-copy, each scaled by what the counter reads for the 256 MiB
 # copy kernel: x2.000 and x1.000); the summaries are the text files under profiles/.
 TRAFFIC_GEMV_1SET = 24_170_000
-TRAFFIC_PREFILL = 182_200_000
-TRAFFIC_W8A8 = 935_500_000
+TRAFFIC_PREFILL = 162_900_000
+TRAFFIC_W8A8 = 935_200_000
+TRAFFIC_SKINNY = 33_130_000
 
 
 def w4a16_bytes(M, N, K, group, zeros_tensor=True, elem=2):
@@ -125,7 +126,7 @@ def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
         "config": {"workload": f"W4A16 decode GEMV M=1 N=11008 K=4096 group=128 fp16 scales+zeros, {units} weight set(s) per launch, "
                                f"{sets} sets rotating ({sets * unit_bytes >> 20} MiB)",
                    "M": M, "N": N, "K": K, "group": g, "units_per_launch": units},
-        "roofline": {"kernel": "gemv_w4a16_kernel", "bound": "hbm", "achieved": round(step_bytes / ev / 1e9, 1),
+        "roofline": {"kernel": "gemv_w4a16_f16_kernel", "bound": "hbm", "achieved": round(step_bytes / ev / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(step_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": TRAFFIC_GEMV_1SET * units, "bytes_per_launch": step_bytes, "avg_launch_us": round(ev * 1e6, 3)},
         "cpu_baseline": cpu,
@@ -179,9 +180,42 @@ def bench_prefill(args, steps=None):
     flops = 2.0 * M * N * K
     return {"workload": "W4A16 prefill GEMM M=N=K=4096 bf16 group=128 zero=8", "dtype": "bf16",
             "value": round(flops / wall / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": wall * 1e3,
-            "roofline": {"kernel": "gemm_mfma_kernel<MmaBF16,W4Loader>", "bound": "mfma", "achieved": round(flops / ev / 1e12, 1),
+            "roofline": {"kernel": "gemm_mfma_kernel<MmaBF16,RowLoaderDirect,W4Loader>", "bound": "mfma", "achieved": round(flops / ev / 1e12, 1),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": TRAFFIC_PREFILL, "flops_per_launch": flops, "avg_launch_us": round(ev * 1e6, 2)}}
+
+
+def bench_skinny(args, steps=None):
+    """cfg-5 decode batch: M=16 activations against a 14336 x 4096 weight matrix (HBM bound)."""
+    import torch
+
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dev = torch.device("cuda:0")
+    M, N, K, g = 16, 14336, 4096, 128
+    unit_bytes = w4a16_bytes(M, N, K, g)
+    sets = -(-POOL_BYTES // unit_bytes)
+    gen = torch.Generator(device="cpu").manual_seed(3)
+    Wp = torch.randint(0, 256, (sets, N, K // 2), dtype=torch.uint8, generator=gen).to(dev)
+    S = (torch.rand(sets, N, K // g, generator=gen) * 0.015 + 0.005).to(torch.float16).to(dev)
+    Z = torch.randint(6, 10, (sets, N, K // g), generator=gen).to(torch.float16).to(dev)
+    A = torch.randn(M, K, generator=gen).to(torch.float16).to(dev)
+    C = torch.empty(M, N, dtype=torch.float16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    pre = [(P(A), P(Wp[j]), P(S[j]), P(Z[j]), P(C), M, N, K, g, 0.0, _abi.F16, _abi.F16, _abi.ALGO_AUTO, stream)
+           for j in range(sets)]
+
+    def step(i):
+        if lib.tlq_gemm_w4a16(*pre[i % sets]):
+            raise RuntimeError(_abi.last_error())
+
+    wall, ev = timed(step, steps or args.steps, args.warmup)
+    return {"workload": f"W4A16 decode batch M=16 N=14336 K=4096 group=128 fp16 scales+zeros, {sets} weight sets rotating",
+            "dtype": "f16", "value": round(unit_bytes / wall / 1e9, 1), "unit": "GB/s", "ms_per_step": wall * 1e3,
+            "roofline": {"kernel": "w4a16_skinny_lds_kernel", "bound": "hbm", "achieved": round(unit_bytes / ev / 1e9, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(unit_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
+                         "traffic": TRAFFIC_SKINNY, "bytes_per_launch": unit_bytes, "avg_launch_us": round(ev * 1e6, 3)}}
 
 
 def bench_w8a8(args, steps=None):
@@ -209,7 +243,7 @@ def bench_w8a8(args, steps=None):
     ops = 2.0 * B * M * N * K
     return {"workload": "W8A8 quant batch matmul B=8 M=2048 N=K=4096, per-token x per-channel rescale, fp16 out",
             "dtype": "i8", "value": round(ops / wall / 1e12, 1), "unit": "TOP/s", "ms_per_step": wall * 1e3,
-            "roofline": {"kernel": "gemm_mfma_kernel<MmaI8,I8KNLoader,EpiRescale>", "bound": "mfma",
+            "roofline": {"kernel": "gemm_mfma_kernel<MmaI8,RowLoaderDirect,I8KNLoaderDirect,EpiRescale>", "bound": "mfma",
                          "achieved": round(ops / ev / 1e12, 1), "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
                          "frac": round(ops / ev / 1e12 / MFMA_I8_PEAK_TOPS, 4), "traffic": TRAFFIC_W8A8, "ops_per_launch": ops,
                          "avg_launch_us": round(ev * 1e6, 2)}}
@@ -220,7 +254,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=48)
-    ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8"])
+    ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8", "skinny"])
     ap.add_argument("--units", type=int, default=1, help="independent weight sets per GEMV launch")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
@@ -247,9 +281,9 @@ def main():
             line["other_workloads"] = [
                 {"workload": many["config"]["workload"], "dtype": "f16", "value": many["value"], "unit": "GB/s",
                  "ms_per_step": many["ms_per_step"], "roofline": many["roofline"]},
-                bench_prefill(args, steps=20), bench_w8a8(args, steps=10)]
+                bench_skinny(args, steps=60), bench_prefill(args, steps=20), bench_w8a8(args, steps=10)]
     else:
-        res = bench_prefill(args) if args.workload == "prefill" else bench_w8a8(args)
+        res = {"prefill": bench_prefill, "w8a8": bench_w8a8, "skinny": bench_skinny}[args.workload](args)
         line = {"metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
                 "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
                 "config": {"workload": res["workload"]}, "roofline": res["roofline"], "cpu_baseline": None}
