@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|prefill|w8a8] [--units U]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|prefill|w8a8|skinny|actquant] [--units U]
 
 Headline workload (default): the W4A16 decode GEMV -- M=1, N=11008, K=4096, fp16 activations,
 uint4 weights packed low-nibble-first, group 128, fp16 scales U[0.005,0.02] and fp16 zeros U{6..9},
@@ -38,6 +38,7 @@ TRAFFIC_GEMV_1SET = 24_170_000
 TRAFFIC_PREFILL = 162_900_000
 TRAFFIC_W8A8 = 935_200_000
 TRAFFIC_SKINNY = 33_130_000
+TRAFFIC_ACT_QUANT = 201_554_000
 
 
 def w4a16_bytes(M, N, K, group, zeros_tensor=True, elem=2):
@@ -218,6 +219,37 @@ def bench_skinny(args, steps=None):
                          "traffic": TRAFFIC_SKINNY, "bytes_per_launch": unit_bytes, "avg_launch_us": round(ev * 1e6, 3)}}
 
 
+def bench_act_quant(args, steps=None):
+    """Per-token int8 quantiser on the activations of the W8A8 workload: 16384 tokens x 4096, bf16 in."""
+    import torch
+
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dev = torch.device("cuda:0")
+    M, N = 8 * 2048, 4096
+    unit_bytes = M * N * 3 + 4 * M
+    sets = -(-POOL_BYTES // (2 * M * N))
+    gen = torch.Generator(device="cpu").manual_seed(4)
+    X = torch.randn(M, N, generator=gen).to(torch.bfloat16).to(dev).repeat(sets, 1, 1)
+    X *= torch.linspace(0.5, 2.0, sets, device=dev).view(sets, 1, 1).to(torch.bfloat16)
+    Y = torch.empty(M, N, dtype=torch.int8, device=dev)
+    S = torch.empty(M, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    pre = [(P(X[j]), P(Y), P(S), M, N, _abi.BF16, 0, stream) for j in range(sets)]
+
+    def step(i):
+        if lib.tlq_act_quant_i8(*pre[i % sets]):
+            raise RuntimeError(_abi.last_error())
+
+    wall, ev = timed(step, steps or args.steps, args.warmup)
+    return {"workload": f"per-token int8 activation quantiser M=16384 N=4096 bf16 in, {sets} inputs rotating",
+            "dtype": "f32", "value": round(unit_bytes / wall / 1e9, 1), "unit": "GB/s", "ms_per_step": wall * 1e3,
+            "roofline": {"kernel": "act_quant_rows_kernel<bf16,8,1>", "bound": "hbm", "achieved": round(unit_bytes / ev / 1e9, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(unit_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
+                         "traffic": TRAFFIC_ACT_QUANT, "bytes_per_launch": unit_bytes, "avg_launch_us": round(ev * 1e6, 3)}}
+
+
 def bench_w8a8(args, steps=None):
     import torch
 
@@ -254,7 +286,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=48)
-    ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8", "skinny"])
+    ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8", "skinny", "actquant"])
     ap.add_argument("--units", type=int, default=1, help="independent weight sets per GEMV launch")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
@@ -281,9 +313,11 @@ def main():
             line["other_workloads"] = [
                 {"workload": many["config"]["workload"], "dtype": "f16", "value": many["value"], "unit": "GB/s",
                  "ms_per_step": many["ms_per_step"], "roofline": many["roofline"]},
-                bench_skinny(args, steps=60), bench_prefill(args, steps=20), bench_w8a8(args, steps=10)]
+                bench_skinny(args, steps=60), bench_prefill(args, steps=20), bench_w8a8(args, steps=10),
+                bench_act_quant(args, steps=40)]
     else:
-        res = {"prefill": bench_prefill, "w8a8": bench_w8a8, "skinny": bench_skinny}[args.workload](args)
+        res = {"prefill": bench_prefill, "w8a8": bench_w8a8, "skinny": bench_skinny,
+               "actquant": bench_act_quant}[args.workload](args)
         line = {"metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
                 "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
                 "config": {"workload": res["workload"]}, "roofline": res["roofline"], "cpu_baseline": None}

@@ -149,6 +149,14 @@ int tlq_gemm_w4a8(const void* A, const void* w_packed, void* C, int64_t M, int64
 int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
                   int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, void* stream);
 
+/* Per-token int8 activation quantiser, replaces act_quant_kernel_int8_optimized
+ * (examples/deepseek_v4/act_quant.py:25-92) with the arithmetic of its golden function (:112-142):
+ *   amax = max(max_n |x[m,n]|, 1e-4);  scale[m] = amax / 127  (round_scale: 2^ceil(log2(amax / 127)), :95-109)
+ *   y[m,n] = int8( rint( clamp(x[m,n] / scale[m], -127, 127) ) ),  all in fp32, round half to even.
+ * X: [M,N] in_dtype (TLQ_BF16 like the reference, TLQ_F16 or TLQ_F32), Y: int8 [M,N], S: fp32 [M].
+ * Its outputs are the A / scale_a operands of tlq_gemm_w8a8. */
+int tlq_act_quant_i8(const void* X, void* Y, void* S, int64_t M, int64_t N, int in_dtype, int round_scale, void* stream);
+
 /* Tuning hooks for benchmark sweeps (process-global, not thread safe; 0 = automatic choice).
  * They play the role of the reference's block_M / block_N / block_K factory arguments
  * (example_dequant_gemm_fine_grained.py:437,462), which here select among pre-built tilings. */

@@ -95,3 +95,23 @@ def rescale(acc, sa, sb, out_kind) -> np.ndarray:
     lib().orc_rescale(_p(acc), _p(sa), _p(sb), _i64(0 if sb is None else sb.size), _p(out), _i64(M), _i64(N),
                       ctypes.c_int(out_kind))
     return out
+
+
+def act_quant(x: np.ndarray, round_scale: bool = False):
+    """x float32 [M,N] -> (int8 [M,N], float32 [M])."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    M, N = x.shape
+    y = np.empty((M, N), dtype=np.int8)
+    s = np.empty(M, dtype=np.float32)
+    lib().orc_act_quant(_p(x), _p(y), _p(s), _i64(M), _i64(N), ctypes.c_int(int(round_scale)))
+    return y, s
+
+
+def act_quant_quotient_check(n: int, seed: int = 0):
+    """(pairs whose rounded integer differs, pairs whose raw quotient differs) between x / s and
+    the reciprocal-and-two-fma quotient, over n pseudo-random pairs."""
+    f = lib().orc_act_quant_quotient_check
+    f.restype = ctypes.c_int64
+    bad_q = ctypes.c_int64(0)
+    bad_int = f(_i64(n), ctypes.c_uint64(seed), ctypes.byref(bad_q))
+    return int(bad_int), int(bad_q.value)

@@ -156,3 +156,71 @@ void orc_rescale(const int32_t* acc, const float* sa, const float* sb, int64_t n
         ((uint16_t*)out)[m * N + n] = bits_kind(rn_kind(c, out_kind), out_kind);
     }
 }
+
+/* ---- per-token int8 activation quantiser (examples/deepseek_v4/act_quant.py:112-142) ----
+ * x: float32 [M,N] (bf16 / fp16 inputs are widened by the caller, which is exact).
+ * round_scale: smallest power of two >= amax / 127 (:93-105, exponent field plus "mantissa != 0"). */
+void orc_act_quant(const float* x, int8_t* y, float* s, int64_t M, int64_t N, int round_scale) {
+  for (int64_t m = 0; m < M; ++m) {
+    float amax = 0.f;
+    for (int64_t n = 0; n < N; ++n) amax = fmaxf(amax, fabsf(x[m * N + n]));
+    if (amax < 1e-4f) amax = 1e-4f;
+    float sc = amax / 127.0f;
+    if (round_scale) {
+      uint32_t b;
+      memcpy(&b, &sc, 4);
+      uint32_t e = ((b >> 23) & 0xffu) + ((b & 0x7fffffu) != 0);
+      b = e << 23;
+      memcpy(&sc, &b, 4);
+    }
+    s[m] = sc;
+    for (int64_t n = 0; n < N; ++n) {
+      float q = x[m * N + n] / sc;
+      q = q < -127.f ? -127.f : (q > 127.f ? 127.f : q);
+      y[m * N + n] = (int8_t)nearbyintf(q); /* default rounding mode: to nearest, ties to even */
+    }
+  }
+}
+
+/* Checker for the division-free quotient the HIP kernel uses: q0 = x * r, q = fma(fma(-q0, s, x), r, q0)
+ * with r = fl(1 / s).  Draws n pseudo-random (x, s) pairs, a third of them within two ulp of a tie
+ * (k + 1/2) * s, and counts the pairs whose clamped, rounded integer differs from that of x / s.
+ * quotient_mismatches receives the count of raw quotients that differ in any bit. */
+int64_t orc_act_quant_quotient_check(int64_t n, uint64_t seed, int64_t* quotient_mismatches) {
+  uint64_t st = seed ? seed : 88172645463325252ull;
+  int64_t bad_int = 0, bad_q = 0;
+#define ORC_RND() (st ^= st << 13, st ^= st >> 7, st ^= st << 17, st)
+  for (int64_t i = 0; i < n; ++i) {
+    uint32_t ea = 60 + (uint32_t)(ORC_RND() % 190), u = (ea << 23) | (uint32_t)(ORC_RND() & 0x7fffff);
+    float amax, sc, x;
+    memcpy(&amax, &u, 4);
+    if (amax < 1e-4f) amax = 1e-4f;
+    sc = amax / 127.0f;
+    if (i & 1) {
+      memcpy(&u, &sc, 4);
+      u = (((u >> 23) & 0xffu) + ((u & 0x7fffffu) != 0)) << 23;
+      memcpy(&sc, &u, 4);
+    }
+    if (i % 3 == 0) {
+      x = ((float)(ORC_RND() % 128) + 0.5f) * sc;
+      memcpy(&u, &x, 4);
+      u += (uint32_t)(ORC_RND() % 5) - 2u;
+      memcpy(&x, &u, 4);
+    } else {
+      uint32_t xb = (uint32_t)ORC_RND(), ex = (uint32_t)(ORC_RND() % (ea + 1));
+      u = (ex << 23) | (xb & 0x7fffff);
+      memcpy(&x, &u, 4);
+    }
+    if (x > amax) x = amax;
+    if (ORC_RND() & 1) x = -x;
+    const float r = 1.0f / sc, q_ref = x / sc, q0 = x * r;
+    const float q = fmaf(fmaf(-q0, sc, x), r, q0);
+    bad_q += q != q_ref;
+    const float a = q_ref < -127.f ? -127.f : (q_ref > 127.f ? 127.f : q_ref);
+    const float b = q < -127.f ? -127.f : (q > 127.f ? 127.f : q);
+    bad_int += nearbyintf(a) != nearbyintf(b);
+  }
+#undef ORC_RND
+  if (quotient_mismatches) *quotient_mismatches = bad_q;
+  return bad_int;
+}

@@ -26,6 +26,11 @@ operand fails a test):
 * rescale epilogues: pure functions of (acc, scale) -- compared with a float64
   evaluation rounded once.
 * lop3 decoders: closed forms (u-8 for signed, (u-z)*s, fma(u,s,-z), (u-qz)*s).
+* act_quant_torch (per-token int8 quantiser): hand-built rows with known answers (ties at
+  .5 fix round-half-to-even, the row maximum maps to +-127, all-zero rows give the 1e-4 / 127
+  scale), invariants (odd symmetry, exact invariance under power-of-two rescaling,
+  |y * s - x| <= s / 2), and a per-element float32 loop.  pow2_ceil is pinned by a search over
+  all powers of two.
 """
 from __future__ import annotations
 
@@ -379,3 +384,57 @@ def lop3_decode_i4_to_f16(words_u32, signed=False, scale=None, zeros=None, zeros
         else:
             h = (h * np.float16(scale)).astype(np.float16)
     return h
+
+
+# --------------------------------------------------------------------------------------
+# A1: per-token int8 activation quantiser (examples/deepseek_v4/act_quant.py)
+# --------------------------------------------------------------------------------------
+def pow2_ceil(s):
+    """Smallest power of two >= s for positive normal float32 s: the bit arithmetic of
+    fast_log2_ceil / fast_pow2 (examples/deepseek_v4/act_quant.py:93-105) -- the exponent field,
+    plus one when any mantissa bit is set."""
+    s = np.asarray(s, dtype=np.float32)
+    bits = s.view(np.uint32)
+    e = ((bits >> 23) & 0xFF).astype(np.int64) + (bits & 0x7FFFFF != 0)
+    return (e.astype(np.uint32) << 23).view(np.float32)
+
+
+def act_quant_torch(x: torch.Tensor, round_scale: bool = False, exact_log2: bool = False):
+    """Golden of examples/deepseek_v4/act_quant.py:112-142, all in float32 on the CPU.
+    Returns (int8 tensor of x's shape, float32 scales [..., 1]).
+
+    ``exact_log2`` replaces ``2 ** ceil(log2(.))`` by pow2_ceil: torch.log2 rounds its result,
+    so a scale within a few ulp above a power of two 2**k (|k| >= 2) has log2 == k exactly and
+    the literal form returns 2**k instead of 2**(k+1)."""
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1]).float()
+    abs_max = torch.max(torch.abs(x2), dim=1, keepdim=True)[0]
+    abs_max = torch.clamp(abs_max, min=1e-4)
+    if round_scale:
+        if exact_log2:
+            scales = torch.from_numpy(pow2_ceil((abs_max / 127.0).numpy()))
+        else:
+            scales = 2 ** torch.ceil(torch.log2(abs_max / 127.0))
+    else:
+        scales = abs_max / 127.0
+    clipped = torch.clamp(x2 / scales, -127, 127)
+    y = torch.round(clipped).to(torch.float16).to(torch.int8)
+    return y.view(shape), scales.view(*shape[:-1], 1)
+
+
+def act_quant_loop(x: torch.Tensor):
+    """Per-element float32 loop of the same definition (small inputs only)."""
+    x2 = x.float().numpy()
+    M, N = x2.shape
+    y = np.zeros((M, N), dtype=np.int8)
+    s = np.zeros(M, dtype=np.float32)
+    for m in range(M):
+        amax = np.float32(1e-4)
+        for n in range(N):
+            amax = max(amax, np.float32(abs(x2[m, n])))
+        s[m] = np.float32(amax) / np.float32(127.0)
+        for n in range(N):
+            q = np.float32(x2[m, n]) / s[m]
+            q = min(max(q, np.float32(-127.0)), np.float32(127.0))
+            y[m, n] = int(np.rint(q))
+    return y, s

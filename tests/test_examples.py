@@ -35,3 +35,15 @@ def test_quant_matmul_examples(capsys):
     ex2.main(["--m", "256", "--n", "512", "--k", "256"])
     out = capsys.readouterr().out
     assert out.rstrip().splitlines()[-2:] == ["QuantMatmul example passed!", "Kernel Output Match!"]
+
+
+def test_deepseek_v4_examples(caplog):
+    import logging
+
+    from tilelang_ascend_amd.examples.deepseek_v4 import act_quant, int8_gemm
+
+    with caplog.at_level(logging.INFO):
+        act_quant.test()
+        int8_gemm.test()
+    msgs = [r.getMessage() for r in caplog.records]
+    assert msgs.count("init successful!") == 2 and msgs.count("Kernel Output Match!") == 2

@@ -36,6 +36,7 @@ SIGNATURES = {
     "tlq_gemm_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "tlq_gemm_w4a8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "tlq_act_quant_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "tlq_tune_gemv": (None, [_int, _int]),
     "tlq_tune_gemv_unroll": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),

@@ -29,6 +29,7 @@ SOURCES = [
     "abi.hip",
     "unpack_dequant.hip",
     "decode_i4.hip",
+    "act_quant.hip",
     "gemv_w4a16.hip",
     "gemm_w4a16.hip",
     "gemm_int8.hip",

@@ -1,5 +1,7 @@
 """Operator factories with the names, argument order and defaults of the reference's example
-scripts (examples/dequantize_gemm, examples/quant_batch_matmul, examples/deepseek_v4/int8_gemm.py)."""
+scripts (examples/dequantize_gemm, examples/quant_batch_matmul, examples/deepseek_v4/int8_gemm.py,
+examples/deepseek_v4/act_quant.py)."""
+from .act_quant import act_quant_kernel_int8_optimized  # noqa: F401
 from .dequant_gemm import (  # noqa: F401
     dequant_gemm_fp16_wrapper,
     dequant_gemm_int8_wrapper,
