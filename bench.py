@@ -34,7 +34,7 @@ POOL_BYTES = 576 * 1024 * 1024  # weight pool > 2x the 256 MB last-level cache
 # HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in separate
 # runs of this script with --calibrate-copy, each scaled by what the counter reads for the 256 MiB
 # copy kernel: x2.000 and x1.000); the summaries are the text files under profiles/.
-TRAFFIC_GEMV_1SET = 24_170_000
+TRAFFIC_GEMV_1SET = 24_110_000
 TRAFFIC_PREFILL = 162_900_000
 TRAFFIC_W8A8 = 935_200_000
 TRAFFIC_SKINNY = 33_130_000
@@ -127,7 +127,7 @@ def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
         "config": {"workload": f"W4A16 decode GEMV M=1 N=11008 K=4096 group=128 fp16 scales+zeros, {units} weight set(s) per launch, "
                                f"{sets} sets rotating ({sets * unit_bytes >> 20} MiB)",
                    "M": M, "N": N, "K": K, "group": g, "units_per_launch": units},
-        "roofline": {"kernel": "gemv_w4a16_f16_kernel", "bound": "hbm", "achieved": round(step_bytes / ev / 1e9, 1),
+        "roofline": {"kernel": "gemv_w4a16_f16_rows_kernel", "bound": "hbm", "achieved": round(step_bytes / ev / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(step_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": TRAFFIC_GEMV_1SET * units, "bytes_per_launch": step_bytes, "avg_launch_us": round(ev * 1e6, 3)},
         "cpu_baseline": cpu,

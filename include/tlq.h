@@ -160,8 +160,10 @@ int tlq_act_quant_i8(const void* X, void* Y, void* S, int64_t M, int64_t N, int 
 /* Tuning hooks for benchmark sweeps (process-global, not thread safe; 0 = automatic choice).
  * They play the role of the reference's block_M / block_N / block_K factory arguments
  * (example_dequant_gemm_fine_grained.py:437,462), which here select among pre-built tilings. */
-void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4, waves 1..4 */
+void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4 (negative: never the register-resident
+                                                             * M = 1, K <= 4096 kernel), waves 1..4 (that kernel: 1..16) */
 void tlq_tune_gemv_unroll(int blocks_per_cu);               /* resident blocks per CU the GEMV grid is sized for */
+void tlq_tune_gemv_depth(int steps_in_flight);               /* load steps (1 KB per row each) a GEMV wavefront keeps in flight */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,
                                                                +10 = never stage through LDS, +20 = stage whenever possible */

@@ -94,7 +94,7 @@ def _run_w4a16(ops, A, Wp, s, z, group, out_dtype, algo, in_dtype):
     return wrapper(A.cuda(), Wp.cuda(), None if s is None else s.cuda(), zd).cpu()
 
 
-@pytest.mark.parametrize("rows,waves", [(0, 0), (1, 1), (1, 4), (2, 2), (4, 4)])
+@pytest.mark.parametrize("rows,waves", [(0, 0), (1, 1), (1, 4), (2, 2), (4, 4), (-1, 4), (-2, 2), (0, 7), (0, 16)])
 def test_gemv_headline(ops, rows, waves):
     """M=1, N=11008, K=4096, group 128, fp16 scales U[0.005,0.02], fp16 zeros U{6..9}, fp16 out."""
     from tilelang_ascend_amd import _abi
@@ -123,6 +123,54 @@ def test_gemv_shapes(ops, in_dtype, M, N, K, group, zeros_kind):
     for out_dtype in ("float32", in_dtype):
         got = _run_w4a16(ops, A, Wp, s, z, group, out_dtype, "gemv", in_dtype)
         check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"gemv {in_dtype}->{out_dtype}")
+
+
+@pytest.mark.parametrize("N,K,group,zeros_kind", [
+    (11008, 4096, 128, "int"), (1000, 4096, 32, "int"), (250, 2048, 128, "frac"), (77, 1088, 64, "int"),
+    (5, 64, 32, None), (4097, 1024, 1024, "scalar8"), (333, 3136, 64, "frac"), (64, 4096, 4096, "int"),
+])
+@pytest.mark.parametrize("waves,blocks_per_cu,depth", [(0, 0, 0), (16, 1, 3), (5, 3, 2), (2, 8, 6), (16, 2, 1)])
+def test_gemv_register_resident_kernel(ops, N, K, group, zeros_kind, waves, blocks_per_cu, depth):
+    """M = 1, K <= 4096: the kernel that keeps the activations in registers and stages the scales and
+    zero points of a work-group's rows in LDS, over its grid shapes and queue depths."""
+    from tilelang_ascend_amd import _abi
+
+    lib = _abi.load()
+    A = torch.randn(1, K, generator=gen(40)).to(torch.float16)
+    Wp, s, z = make_w4(N, K, group, torch.float16, zeros_kind, seed=41)
+    want = w4a16_reference(A, Wp, s, z, group)
+    lib.tlq_tune_gemv(0, waves)
+    lib.tlq_tune_gemv_unroll(blocks_per_cu)
+    lib.tlq_tune_gemv_depth(depth)
+    try:
+        for out_dtype in ("float16", "float32"):
+            got = _run_w4a16(ops, A, Wp, s, z, group, out_dtype, "gemv", "float16")
+            check_float_output(got, want, f"gemv rows kernel -> {out_dtype}")
+    finally:
+        lib.tlq_tune_gemv(0, 0)
+        lib.tlq_tune_gemv_unroll(0)
+        lib.tlq_tune_gemv_depth(0)
+
+
+@pytest.mark.parametrize("M,N,K,group", [(1, 1000, 4096, 128), (1, 130, 8192, 128), (2, 257, 2048, 64)])
+def test_gemv_batched_entry_point(M, N, K, group):
+    """tlq_gemv_w4a16_batched: several independent problems (own activations, weights, scales, zeros) per launch."""
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    batch = 3
+    sets = [make_w4(N, K, group, torch.float16, "int", seed=50 + b) for b in range(batch)]
+    A = torch.randn(batch, M, K, generator=gen(49)).to(torch.float16)
+    Wp = torch.stack([x[0] for x in sets]).cuda()
+    S = torch.stack([x[1] for x in sets]).cuda()
+    Z = torch.stack([x[2] for x in sets]).cuda()
+    C = torch.empty(batch, M, N, dtype=torch.float16, device="cuda")
+    Ad = A.cuda()
+    rc = lib.tlq_gemv_w4a16_batched(P(Ad), P(Wp), P(S), P(Z), P(C), batch, M, N, K, group, 0.0, _abi.F16, _abi.F16,
+                                    torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _abi.last_error()
+    for b in range(batch):
+        check_float_output(C[b].cpu(), w4a16_reference(A[b], *sets[b], group), f"batched set {b}")
 
 
 def test_gemv_one_hot_reads_back_dequantised_rows(ops):

@@ -39,6 +39,7 @@ SIGNATURES = {
     "tlq_act_quant_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "tlq_tune_gemv": (None, [_int, _int]),
     "tlq_tune_gemv_unroll": (None, [_int]),
+    "tlq_tune_gemv_depth": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),
     "tlq_tune_w4a16_skinny": (None, [_int, _int]),
     "tlq_tune_i8_tile": (None, [_int]),

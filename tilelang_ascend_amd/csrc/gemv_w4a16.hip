@@ -71,6 +71,28 @@ __device__ __forceinline__ void load_act(ActF16& r, const half_t* __restrict__ A
   r.bsum = 1024.0f * se + 64.0f * (s - se);
 }
 
+// the same from four 16-byte words already loaded
+__device__ __forceinline__ void permute_act(ActF16& r, const uint4_t (&p)[4]) {
+  float s = 0.f, se = 0.f;
+  const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint4_t v = p[j];
+    half2_t q0 = bitcast<half2_t>(v.x), q1 = bitcast<half2_t>(v.y);
+    half2_t q2 = bitcast<half2_t>(v.z), q3 = bitcast<half2_t>(v.w);
+    r.a[4 * j + 0] = half2_t{q0.x, q2.x};
+    r.a[4 * j + 1] = half2_t{q0.y, q2.y};
+    r.a[4 * j + 2] = half2_t{q1.x, q3.x};
+    r.a[4 * j + 3] = half2_t{q1.y, q3.y};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s = __builtin_amdgcn_fdot2(r.a[4 * j + i], ones, s, false);
+    se = __builtin_amdgcn_fdot2(r.a[4 * j + 0], ones, se, false);
+    se = __builtin_amdgcn_fdot2(r.a[4 * j + 2], ones, se, false);
+  }
+  r.sum = s;
+  r.bsum = 1024.0f * se + 64.0f * (s - se);
+}
+
 // Sum over the chunk of A[k] * (bias_k + u[k]) with the unpack bias left in (1024 for even k,
 // 64 for odd k); the caller subtracts act.bsum.  fp32 accumulation keeps the cancellation error
 // near 1e-5 relative, far below the fp16 output rounding.
@@ -166,10 +188,11 @@ __device__ __forceinline__ float chunk_term(const uint4_t& w, const ActBF16& act
 // so that consecutive lanes read consecutive 16-byte words (no bank conflicts).
 //
 // A wavefront walks over "steps": step (rg, it) covers R rows (row group rg) x one 16-byte chunk
-// per lane (chunk it*64 + lane).  Row groups are dealt round-robin to all wavefronts of the grid;
-// the loads of the next step are always issued before the current step is computed, so a
-// wavefront keeps 2*R*1 KB in flight from its first instruction to its last.
-template <int R, int MT>
+// per lane (chunk it*64 + lane).  Row groups are dealt round-robin to all wavefronts of the grid.
+// The loads of D steps are in flight per wavefront: a problem of a few tens of MB is latency
+// bound (bytes in flight / memory latency), so every wavefront requests its first D KB before
+// anything else and requests step s + D as soon as step s has been consumed.
+template <int R, int MT, int D>
 __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __restrict__ A,
                                                                 const uint8_t* __restrict__ Wp,
                                                                 const half_t* __restrict__ scales,
@@ -212,14 +235,23 @@ __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __
     uint4_t w[R];
     half_t s[R], z[R];
   };
-  auto issue = [&](Stage& st, int rg, int it) {
-    const int c = (it << 6) + lane;
+  struct Cursor {  // wave-uniform position in this wavefront's sequence of steps
+    int rg, it;
+  };
+  auto advance = [&](Cursor& c) {
+    if (++c.it == iters) {
+      c.it = 0;
+      c.rg += wave_count;
+    }
+  };
+  auto issue = [&](Stage& st, const Cursor& at) {
+    const int c = (at.it << 6) + lane;
     const bool ok = c < chunks;
     const int cc = ok ? c : chunks - 1;
     const int gi = (cc << 5) >> group_shift;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      int row = rg * R + r;
+      int row = at.rg * R + r;
       row = row < N ? row : N - 1;  // clamp: loads stay in bounds
       st.w[r] = *(const uint4_t*)(Wp + (uint32_t)(row * row_bytes + (cc << 4)));
       const uint32_t go = (uint32_t)(row * groups + gi);
@@ -231,10 +263,17 @@ __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __
   };
 
   const NibbleMagic mg = make_nibble_magic();
-  Stage cur, nxt;
-  int rg = wave_id, it = 0;
-  const bool any = rg < row_groups;
-  if (any) issue(cur, rg, it);  // first weight loads go out before the activation staging
+  Stage st[D];
+  Cursor ic = {wave_id, 0};  // next step to request
+  auto fill = [&]() {
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+      if (ic.rg < row_groups) {
+        issue(st[d], ic);
+        advance(ic);
+      }
+  };
+  fill();  // the first weight loads go out before the activation staging
 
   for (int m0 = 0; m0 < m_count; m0 += MT) {
     if (m0 > 0) __syncthreads();  // previous pass has finished reading LDS
@@ -255,9 +294,8 @@ __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __
     __syncthreads();
 
     if (m0 > 0) {
-      rg = wave_id;
-      it = 0;
-      if (any) issue(cur, rg, it);
+      ic = Cursor{wave_id, 0};
+      fill();
     }
     float acc[R][MT];
 #pragma unroll
@@ -265,49 +303,200 @@ __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __
 #pragma unroll
       for (int m = 0; m < MT; ++m) acc[r][m] = 0.f;
 
-    while (rg < row_groups) {
-      // next step of this wavefront
-      int rg2 = rg, it2 = it + 1;
-      if (it2 == iters) {
-        it2 = 0;
-        rg2 = rg + wave_count;
-      }
-      if (rg2 < row_groups) issue(nxt, rg2, it2);
-
-      int c = (it << 6) + lane;
-      c = c < chunks ? c : chunks - 1;
+    Cursor cc = {wave_id, 0};  // step being consumed
+    while (cc.rg < row_groups) {
 #pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        ActF16 act;
+      for (int d = 0; d < D; ++d) {
+        if (cc.rg >= row_groups) break;
+        int c = (cc.it << 6) + lane;
+        c = c < chunks ? c : chunks - 1;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint4_t v = lds_pairs[(m * 4 + j) * chunks + c];
-          act.a[4 * j + 0] = bitcast<half2_t>(v.x);
-          act.a[4 * j + 1] = bitcast<half2_t>(v.y);
-          act.a[4 * j + 2] = bitcast<half2_t>(v.z);
-          act.a[4 * j + 3] = bitcast<half2_t>(v.w);
-        }
-        const float2 sb = lds_sums[m * chunks + c];
-        act.sum = sb.x;
-        act.bsum = sb.y;
+        for (int m = 0; m < MT; ++m) {
+          ActF16 act;
 #pragma unroll
-        for (int r = 0; r < R; ++r) acc[r][m] += chunk_term_biased(cur.w[r], act, cur.s[r], cur.z[r], mg);
-      }
-
-      if (it == iters - 1) {  // row group finished: reduce over the lanes and store
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-          for (int m = 0; m < MT; ++m) {
-            const float v = wave_sum_to_lane63(acc[r][m]);
-            const int row = rg * R + r;
-            if (lane == 63 && row < N && m0 + m < m_count) store_out(C, (int64_t)(m0 + m) * N + row, v, out_dtype);
-            acc[r][m] = 0.f;
+          for (int j = 0; j < 4; ++j) {
+            const uint4_t v = lds_pairs[(m * 4 + j) * chunks + c];
+            act.a[4 * j + 0] = bitcast<half2_t>(v.x);
+            act.a[4 * j + 1] = bitcast<half2_t>(v.y);
+            act.a[4 * j + 2] = bitcast<half2_t>(v.z);
+            act.a[4 * j + 3] = bitcast<half2_t>(v.w);
           }
+          const float2 sb = lds_sums[m * chunks + c];
+          act.sum = sb.x;
+          act.bsum = sb.y;
+#pragma unroll
+          for (int r = 0; r < R; ++r) acc[r][m] += chunk_term_biased(st[d].w[r], act, st[d].s[r], st[d].z[r], mg);
+        }
+
+        if (cc.it == iters - 1) {  // row group finished: reduce over the lanes and store
+#pragma unroll
+          for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+              const float v = wave_sum_to_lane63(acc[r][m]);
+              const int row = cc.rg * R + r;
+              if (lane == 63 && row < N && m0 + m < m_count) store_out(C, (int64_t)(m0 + m) * N + row, v, out_dtype);
+              acc[r][m] = 0.f;
+            }
+        }
+        advance(cc);
+        if (ic.rg < row_groups) {  // the slot just consumed takes the step D ahead
+          issue(st[d], ic);
+          advance(ic);
+        }
       }
-      cur = nxt;
-      rg = rg2;
-      it = it2;
+    }
+  }
+}
+
+// ---- fp16, M = 1, short rows: activations in registers --------------------------------------------
+// For K <= 2048 * ITERS a lane meets the same ITERS chunks of the activation vector in every row, so
+// each wavefront keeps them (permuted, with their sums) in registers.  The work-group is as large as
+// the CU takes (up to 16 wavefronts) and owns a contiguous range of rows: it prepares the activations
+// ONCE and copies the scales and zero points of its rows (contiguous in memory) into LDS with a few
+// wide loads.  The path from L2 to the CUs carries about 15 TB/s on this part: a private copy of the
+// activations per wavefront would put more bytes on it than the weights themselves, and one small
+// gather per row and tensor costs about as much as a 1 KB weight load.
+// A step is a whole row: ITERS 16-byte weight loads per lane.  D rows are in flight per wavefront; the
+// first D are requested before anything else, the staging loads right behind them.  The loop body
+// is free of branches (rows past the end are clamped and their results dropped): the compiler then
+// keeps exact counts of the loads in flight instead of draining them at every control-flow merge.
+template <int ITERS, int D>
+__global__ __launch_bounds__(1024) void gemv_w4a16_f16_rows_kernel(const half_t* __restrict__ A,
+                                                                  const uint8_t* __restrict__ Wp,
+                                                                  const half_t* __restrict__ scales,
+                                                                  const half_t* __restrict__ zeros,
+                                                                  void* __restrict__ C, int N, int K, int group_shift,
+                                                                  float zero_scalar, int out_dtype, int rows_per_block) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int chunks = K >> 5;
+  const int groups = K >> group_shift;
+  uint4_t* const lds_pairs = (uint4_t*)smem;                       // [4][chunks]
+  float2* const lds_sums = (float2*)(smem + (size_t)chunks * 64);  // [chunks]
+  half_t* const lds_s = (half_t*)(smem + (size_t)chunks * 72);     // [rows_per_block][groups]
+  half_t* const lds_z = lds_s + rows_per_block * groups;           // [rows_per_block][groups] (16-byte aligned: see launcher)
+  {
+    const int64_t b = blockIdx.y;
+    const int64_t gsz = (int64_t)N * groups;
+    A += b * K;
+    Wp += b * N * (int64_t)(K >> 1);
+    if (scales) scales += b * gsz;
+    if (zeros) zeros += b * gsz;
+    const int64_t coff = b * N;
+    C = out_dtype == TLQ_F32 ? (void*)((float*)C + coff) : (void*)((uint16_t*)C + coff);
+  }
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nwaves = blockDim.x >> 6;
+  const int r0 = blockIdx.x * rows_per_block;
+  const int r1 = r0 + rows_per_block < N ? r0 + rows_per_block : N;  // rows [r0, r1) belong to this work-group
+  const int row_bytes = K >> 1;
+  const bool has_s = scales != nullptr, has_z = zeros != nullptr;
+
+  int cc[ITERS], gsel[ITERS];
+  bool ok[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = (it << 6) + lane;
+    ok[it] = c < chunks;
+    cc[it] = ok[it] ? c : chunks - 1;
+    gsel[it] = (cc[it] << 5) >> group_shift;
+  }
+
+  struct Stage {
+    uint4_t w[ITERS];
+  };
+  auto issue = [&](Stage& st, int row) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) st.w[it] = *(const uint4_t*)(Wp + (uint32_t)(row * row_bytes + (cc[it] << 4)));
+  };
+  Stage st[D];
+  int irow = r0 + wave;  // next row to request
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    issue(st[d], irow < r1 ? irow : r1 - 1);
+    irow += nwaves;
+  }
+
+  // staging loads, behind the first weight rows (which are the ones that miss every cache and cannot be
+  // consumed before they arrive anyway): thread t < chunks fetches activation chunk t, and all threads
+  // copy the scale / zero rows, 16 bytes (or one value) each
+  const int tchunk = threadIdx.x < chunks ? threadIdx.x : chunks - 1;
+  uint4_t araw[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) araw[j] = ((const uint4_t*)(A + ((int64_t)tchunk << 5)))[j];
+  const int n_sz = (r1 - r0) * groups;  // values per tensor
+  const int64_t sz0 = (int64_t)r0 * groups;
+  const bool wide = (groups & 7) == 0 && (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0;  // r0 * groups is a multiple of 8 too
+  uint4_t s_raw = {0, 0, 0, 0}, z_raw = {0, 0, 0, 0};
+  const int t8 = threadIdx.x << 3;
+  if (wide && t8 < n_sz) {  // a work-group of 1024 threads covers 8192 values per tensor in one go
+    if (has_s) s_raw = *(const uint4_t*)(scales + sz0 + t8);
+    if (has_z) z_raw = *(const uint4_t*)(zeros + sz0 + t8);
+  }
+
+  if (threadIdx.x < chunks) {
+    ActF16 a;
+    permute_act(a, araw);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      lds_pairs[j * chunks + tchunk] = uint4_t{bitcast<uint32_t>(a.a[4 * j + 0]), bitcast<uint32_t>(a.a[4 * j + 1]),
+                                               bitcast<uint32_t>(a.a[4 * j + 2]), bitcast<uint32_t>(a.a[4 * j + 3])};
+    lds_sums[tchunk] = make_float2(a.sum, a.bsum);
+  }
+  if (wide) {
+    if (t8 < n_sz) {
+      if (has_s) *(uint4_t*)(lds_s + t8) = s_raw;
+      if (has_z) *(uint4_t*)(lds_z + t8) = z_raw;
+    }
+    for (int i = t8 + (int)(blockDim.x << 3); i < n_sz; i += (int)(blockDim.x << 3)) {  // more than 8192 values
+      if (has_s) *(uint4_t*)(lds_s + i) = *(const uint4_t*)(scales + sz0 + i);
+      if (has_z) *(uint4_t*)(lds_z + i) = *(const uint4_t*)(zeros + sz0 + i);
+    }
+  } else {
+    for (int i = threadIdx.x; i < n_sz; i += blockDim.x) {
+      if (has_s) lds_s[i] = scales[sz0 + i];
+      if (has_z) lds_z[i] = zeros[sz0 + i];
+    }
+  }
+  __syncthreads();
+  ActF16 act[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint4_t v = lds_pairs[j * chunks + cc[it]];
+      act[it].a[4 * j + 0] = bitcast<half2_t>(v.x);
+      act[it].a[4 * j + 1] = bitcast<half2_t>(v.y);
+      act[it].a[4 * j + 2] = bitcast<half2_t>(v.z);
+      act[it].a[4 * j + 3] = bitcast<half2_t>(v.w);
+    }
+    const float2 sb = lds_sums[cc[it]];
+    act[it].sum = sb.x;
+    act[it].bsum = sb.y;
+  }
+
+  const NibbleMagic mg = make_nibble_magic();
+  const half_t one = (half_t)1.0f, zs = (half_t)zero_scalar;
+  const int my_rows = r0 + wave < r1 ? (r1 - r0 - wave + nwaves - 1) / nwaves : 0;
+  int row = r0 + wave;
+  for (int round = 0; round * D < my_rows; ++round) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int lrow = (row < r1 ? row : r1 - 1) - r0;
+      float acc = 0.f;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const half_t sv = has_s ? lds_s[lrow * groups + gsel[it]] : one;
+        const half_t z = has_z ? lds_z[lrow * groups + gsel[it]] : zs;
+        const half_t s = ok[it] ? sv : (half_t)0.0f;  // a chunk past the end contributes 0
+        acc += chunk_term_biased(st[d].w[it], act[it], s, z, mg);
+      }
+      const float v = wave_sum_to_lane63(acc);
+      if (lane == 63 && row < r1) store_out(C, row, v, out_dtype);
+      row += nwaves;
+      issue(st[d], irow < r1 ? irow : r1 - 1);  // the slot just consumed takes the row D ahead
+      irow += nwaves;
     }
   }
 }
@@ -405,7 +594,7 @@ static void launch_gemv(const void* A, const void* Wp, const void* scales, const
 }
 
 // rows-per-wave / waves-per-block / blocks-per-CU overrides for tuning runs (0 = automatic)
-static int g_gemv_rows = 0, g_gemv_waves = 0, g_gemv_unroll = 0;
+static int g_gemv_rows = 0, g_gemv_waves = 0, g_gemv_waves16 = 0, g_gemv_unroll = 0, g_gemv_depth = 0;
 
 static int cu_count() {
   static int n = 0;
@@ -417,7 +606,7 @@ static int cu_count() {
   return n;
 }
 
-template <int R, int MT>
+template <int R, int MT, int D>
 static int launch_gemv_f16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int batch,
                            int M, int N, int K, int group_shift, float zero_scalar, int out_dtype, int waves_per_block,
                            int blocks_per_cu, hipStream_t st) {
@@ -430,9 +619,31 @@ static int launch_gemv_f16(const void* A, const void* Wp, const void* scales, co
   int blocks = (int)ceil_div(row_groups, waves_per_block);
   const int cap = (int)ceil_div((int64_t)cu_count() * blocks_per_cu, batch);
   if (blocks > cap) blocks = cap < 1 ? 1 : cap;
-  gemv_w4a16_f16_kernel<R, MT><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
+  gemv_w4a16_f16_kernel<R, MT, D><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
       (const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C, M, N, K, group_shift,
       zero_scalar, out_dtype);
+  return 0;
+}
+
+// rows kernel: work-groups of `waves_per_block` wavefronts, each owning a contiguous range of rows whose
+// scales and zero points fit its LDS; at least `blocks_per_cu` work-groups per CU when there are rows enough
+template <int ITERS, int D>
+static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int batch,
+                            int N, int K, int group_shift, float zero_scalar, int out_dtype, int waves_per_block,
+                            int blocks_per_cu, hipStream_t st) {
+  const int groups = K >> group_shift;
+  int blocks = (int)ceil_div((int64_t)cu_count() * blocks_per_cu, batch);
+  if (blocks < 1) blocks = 1;
+  int rpb = (int)ceil_div(N, blocks);
+  if (rpb < waves_per_block) rpb = waves_per_block;
+  const int rpb_max = (48 * 1024) / (4 * groups);  // scales + zeros of a work-group's rows: at most 48 KB of LDS
+  if (rpb > rpb_max) rpb = rpb_max;
+  rpb = (rpb + 3) & ~3;  // keeps the zero-point block of LDS 16-byte aligned for any group count
+  blocks = (int)ceil_div(N, rpb);
+  const size_t lds = (size_t)(K / 32) * 72 + (size_t)rpb * groups * 4;
+  gemv_w4a16_f16_rows_kernel<ITERS, D><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
+      (const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C, N, K, group_shift,
+      zero_scalar, out_dtype, rpb);
   return 0;
 }
 
@@ -448,20 +659,56 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     // blocks per CU (each wavefront then walks ~3 rows with the next row's loads in flight).
     // Large / batched problems stream: two rows per wavefront, one block per 8 rows.
     const bool streaming = batch * N * (K / 2) > ((int64_t)64 << 20);
-    const int R = g_gemv_rows ? g_gemv_rows : (streaming ? 2 : 1);
+    const int R = g_gemv_rows > 0 ? g_gemv_rows : (streaming ? 2 : 1);
     const int bpc = g_gemv_unroll ? g_gemv_unroll : (streaming ? 64 : 8);  // grid size cap, blocks per CU
+    const int depth_req = g_gemv_depth;
+    if (M == 1 && K <= 4096 && g_gemv_rows >= 0) {
+      const int bpc_rows = g_gemv_unroll ? g_gemv_unroll : 1;
+      int wpb_rows = g_gemv_waves16 ? g_gemv_waves16 : 16;
+      if (wpb_rows * 64 < K / 32) wpb_rows = (int)ceil_div(K / 32, (int64_t)64);  // one staging thread per chunk
+      // one problem of a few tens of MB: one row in flight per wavefront (deeper queues delay the staging
+      // loads behind the weights and measured slower); many problems per launch stream with two
+      const int d = depth_req ? depth_req : (batch * N * (K / 2) > ((int64_t)64 << 20) ? 2 : 1);
+#define TLQ_ROWS_CASE(IT, DD)                                                                                      \
+  launch_gemv_rows<IT, DD>(A, Wp, scales, zeros, C, (int)batch, (int)N, (int)K, shift, zero_scalar, out_dtype,      \
+                           wpb_rows, bpc_rows, st)
+      if (K <= 2048) {
+        if (d <= 2) TLQ_ROWS_CASE(1, 2);
+        else if (d <= 4) TLQ_ROWS_CASE(1, 4);
+        else TLQ_ROWS_CASE(1, 8);
+      } else {
+        if (d <= 1) TLQ_ROWS_CASE(2, 1);
+        else if (d == 2) TLQ_ROWS_CASE(2, 2);
+        else if (d == 3) TLQ_ROWS_CASE(2, 3);
+        else if (d == 4) TLQ_ROWS_CASE(2, 4);
+        else TLQ_ROWS_CASE(2, 6);
+      }
+#undef TLQ_ROWS_CASE
+      return check_launch("tlq_gemm_w4a16(gemv)") ? 0 : 1;
+    }
     const bool two_rows = M > 1 && (size_t)2 * (K / 32) * 72 <= 64 * 1024;
-#define TLQ_F16_CASE(RR, MTT)                                                                                       \
-  rc = launch_gemv_f16<RR, MTT>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, shift, zero_scalar,   \
-                                out_dtype, wpb, bpc, st)
+#define TLQ_F16_CASE(RR, MTT, DD)                                                                                  \
+  rc = launch_gemv_f16<RR, MTT, DD>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, shift, zero_scalar, \
+                                    out_dtype, wpb, bpc, st)
+    // steps in flight per wavefront (each R KB)
+    const int depth = g_gemv_depth ? g_gemv_depth : (streaming ? 2 : 6);
     if (two_rows) {
-      TLQ_F16_CASE(2, 2);
+      if (depth <= 1) TLQ_F16_CASE(2, 2, 1);
+      else if (depth == 2) TLQ_F16_CASE(2, 2, 2);
+      else TLQ_F16_CASE(2, 2, 3);
     } else if (R == 1) {
-      TLQ_F16_CASE(1, 1);
+      if (depth <= 1) TLQ_F16_CASE(1, 1, 1);
+      else if (depth == 2) TLQ_F16_CASE(1, 1, 2);
+      else if (depth <= 4) TLQ_F16_CASE(1, 1, 4);
+      else if (depth <= 6) TLQ_F16_CASE(1, 1, 6);
+      else TLQ_F16_CASE(1, 1, 8);
     } else if (R == 4) {
-      TLQ_F16_CASE(4, 1);
+      if (depth <= 1) TLQ_F16_CASE(4, 1, 1);
+      else TLQ_F16_CASE(4, 1, 2);
     } else {
-      TLQ_F16_CASE(2, 1);
+      if (depth <= 1) TLQ_F16_CASE(2, 1, 1);
+      else if (depth == 2) TLQ_F16_CASE(2, 1, 2);
+      else TLQ_F16_CASE(2, 1, 4);
     }
 #undef TLQ_F16_CASE
     if (rc) return rc;
@@ -487,8 +734,10 @@ extern "C" {
 // Tuning hook used by the benchmark sweeps: rows per wavefront (1, 2, 4) and wavefronts per
 // block (1..4) of the GEMV kernel; 0 restores the automatic choice.
 void tlq_tune_gemv(int rows_per_wave, int waves_per_block) {
-  tlq::g_gemv_rows = rows_per_wave;
+  tlq::g_gemv_rows = rows_per_wave;  // negative: never use the register-resident rows kernel
   tlq::g_gemv_waves = (waves_per_block < 0 || waves_per_block > 4) ? 0 : waves_per_block;
+  tlq::g_gemv_waves16 = (waves_per_block < 0 || waves_per_block > 16) ? 0 : waves_per_block;  // register-resident kernel
 }
 void tlq_tune_gemv_unroll(int blocks_per_cu) { tlq::g_gemv_unroll = blocks_per_cu; }
+void tlq_tune_gemv_depth(int steps_in_flight) { tlq::g_gemv_depth = steps_in_flight < 0 ? 0 : steps_in_flight; }
 }
