@@ -367,42 +367,24 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_f16_rows_kernel(const half_t*
                                                                   const half_t* __restrict__ scales,
                                                                   const half_t* __restrict__ zeros,
                                                                   void* __restrict__ C, int N, int K, int group_shift,
-                                                                  float zero_scalar, int out_dtype, int rows_per_block) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  const int chunks = K >> 5;
-  const int groups = K >> group_shift;
-  uint4_t* const lds_pairs = (uint4_t*)smem;                       // [4][chunks]
-  float2* const lds_sums = (float2*)(smem + (size_t)chunks * 64);  // [chunks]
-  half_t* const lds_s = (half_t*)(smem + (size_t)chunks * 72);     // [rows_per_block][groups]
-  half_t* const lds_z = lds_s + rows_per_block * groups;           // [rows_per_block][groups] (16-byte aligned: see launcher)
-  {
-    const int64_t b = blockIdx.y;
-    const int64_t gsz = (int64_t)N * groups;
-    A += b * K;
-    Wp += b * N * (int64_t)(K >> 1);
-    if (scales) scales += b * gsz;
-    if (zeros) zeros += b * gsz;
-    const int64_t coff = b * N;
-    C = out_dtype == TLQ_F32 ? (void*)((float*)C + coff) : (void*)((uint16_t*)C + coff);
-  }
+                                                                  float zero_scalar, int out_dtype, int rows_per_block, int nwaves) {
+  // The first weight rows: as few instructions as possible between the start of a wavefront and its first
+  // loads (everything they need sits in the first 64 bytes of the kernel arguments).
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int nwaves = blockDim.x >> 6;
+  const int chunks = K >> 5;
+  const int row_bytes = K >> 1;
   const int r0 = blockIdx.x * rows_per_block;
   const int r1 = r0 + rows_per_block < N ? r0 + rows_per_block : N;  // rows [r0, r1) belong to this work-group
-  const int row_bytes = K >> 1;
-  const bool has_s = scales != nullptr, has_z = zeros != nullptr;
-
-  int cc[ITERS], gsel[ITERS];
+  Wp += (int64_t)blockIdx.y * N * (int64_t)row_bytes;
+  int cc[ITERS];
   bool ok[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int c = (it << 6) + lane;
     ok[it] = c < chunks;
     cc[it] = ok[it] ? c : chunks - 1;
-    gsel[it] = (cc[it] << 5) >> group_shift;
   }
-
   struct Stage {
     uint4_t w[ITERS];
   };
@@ -417,6 +399,27 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_f16_rows_kernel(const half_t*
     issue(st[d], irow < r1 ? irow : r1 - 1);
     irow += nwaves;
   }
+  __builtin_amdgcn_sched_barrier(0);
+
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int groups = K >> group_shift;
+  uint4_t* const lds_pairs = (uint4_t*)smem;                       // [4][chunks]
+  float2* const lds_sums = (float2*)(smem + (size_t)chunks * 64);  // [chunks]
+  half_t* const lds_s = (half_t*)(smem + (size_t)chunks * 72);     // [rows_per_block][groups]
+  half_t* const lds_z = lds_s + rows_per_block * groups;           // [rows_per_block][groups] (16-byte aligned: see launcher)
+  {
+    const int64_t b = blockIdx.y;
+    const int64_t gsz = (int64_t)N * groups;
+    A += b * K;
+    if (scales) scales += b * gsz;
+    if (zeros) zeros += b * gsz;
+    const int64_t coff = b * N;
+    C = out_dtype == TLQ_F32 ? (void*)((float*)C + coff) : (void*)((uint16_t*)C + coff);
+  }
+  const bool has_s = scales != nullptr, has_z = zeros != nullptr;
+  int gsel[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) gsel[it] = (cc[it] << 5) >> group_shift;
 
   // staging loads, behind the first weight rows (which are the ones that miss every cache and cannot be
   // consumed before they arrive anyway): thread t < chunks fetches activation chunk t, and all threads
@@ -449,12 +452,12 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_f16_rows_kernel(const half_t*
       if (has_s) *(uint4_t*)(lds_s + t8) = s_raw;
       if (has_z) *(uint4_t*)(lds_z + t8) = z_raw;
     }
-    for (int i = t8 + (int)(blockDim.x << 3); i < n_sz; i += (int)(blockDim.x << 3)) {  // more than 8192 values
+    for (int i = t8 + (int)((nwaves << 6) << 3); i < n_sz; i += (int)((nwaves << 6) << 3)) {  // more than 8192 values
       if (has_s) *(uint4_t*)(lds_s + i) = *(const uint4_t*)(scales + sz0 + i);
       if (has_z) *(uint4_t*)(lds_z + i) = *(const uint4_t*)(zeros + sz0 + i);
     }
   } else {
-    for (int i = threadIdx.x; i < n_sz; i += blockDim.x) {
+    for (int i = threadIdx.x; i < n_sz; i += (nwaves << 6)) {
       if (has_s) lds_s[i] = scales[sz0 + i];
       if (has_z) lds_z[i] = zeros[sz0 + i];
     }
@@ -643,7 +646,7 @@ static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, c
   const size_t lds = (size_t)(K / 32) * 72 + (size_t)rpb * groups * 4;
   gemv_w4a16_f16_rows_kernel<ITERS, D><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
       (const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C, N, K, group_shift,
-      zero_scalar, out_dtype, rpb);
+      zero_scalar, out_dtype, rpb, waves_per_block);
   return 0;
 }
 
