@@ -7,6 +7,7 @@ operators raise.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 import threading
@@ -96,3 +97,43 @@ def check(rc: int) -> None:
 
 def ptr(t) -> ctypes.c_void_p:
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+_tuning_lock = threading.RLock()
+
+
+@contextlib.contextmanager
+def tuning(w4a16_tile: int = 0, i8_tile: int = 0, gemv: tuple = None, skinny: tuple = None):
+    """Applies tiling choices to the launches made inside the block, then restores the automatic
+    choice.  The hooks are process-global and only read on the host while a launch is being set up
+    (asynchronous execution is not affected), so holding this lock around the call is enough."""
+    lib = load()
+    active = bool(w4a16_tile or i8_tile or gemv or skinny)
+    if not active:
+        yield
+        return
+    with _tuning_lock:
+        try:
+            if w4a16_tile:
+                lib.tlq_tune_w4a16_tile(int(w4a16_tile))
+            if i8_tile:
+                lib.tlq_tune_i8_tile(int(i8_tile))
+            if gemv:
+                rows, waves, blocks_per_cu, depth = (tuple(gemv) + (0, 0, 0, 0))[:4]
+                lib.tlq_tune_gemv(int(rows), int(waves))
+                lib.tlq_tune_gemv_unroll(int(blocks_per_cu))
+                lib.tlq_tune_gemv_depth(int(depth))
+            if skinny:
+                lib.tlq_tune_w4a16_skinny(int(skinny[0]), int(skinny[1]))
+            yield
+        finally:
+            if w4a16_tile:
+                lib.tlq_tune_w4a16_tile(0)
+            if i8_tile:
+                lib.tlq_tune_i8_tile(0)
+            if gemv:
+                lib.tlq_tune_gemv(0, 0)
+                lib.tlq_tune_gemv_unroll(0)
+                lib.tlq_tune_gemv_depth(0)
+            if skinny:
+                lib.tlq_tune_w4a16_skinny(0, 0)

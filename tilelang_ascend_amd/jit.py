@@ -113,6 +113,7 @@ class JITKernel:
         self.target = target
         self.execution_backend = execution_backend
         self.input_idx = [i for i in range(n) if i not in self.result_idx and i not in self.workspace_idx]
+        self._tuner_result = None
 
     # -- introspection kept for drop-in use ----------------------------------------------
     @property
@@ -121,6 +122,10 @@ class JITKernel:
 
     def get_kernel_source(self) -> str:
         return f"// pre-built HIP kernel '{self.spec.name}' in {_abi.library_path()}"
+
+    def get_tuner_result(self):
+        """The AutotuneResult of the search that produced this kernel, or None (tilelang/jit/kernel.py)."""
+        return self._tuner_result
 
     def get_profiler(self):
         from .profiler import Profiler

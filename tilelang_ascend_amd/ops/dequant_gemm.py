@@ -150,13 +150,21 @@ def int8_gemm(M: int, N: int, K: int, block_M: int, block_N: int, block_K: int):
 @jit(out_idx=[-1], pass_configs=_PASS_CONFIGS)
 def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, block_K: int = 64,
                in_dtype: str = "float16", out_dtype: str = "float16", group_size: int = 128,
-               with_scales: bool = True, zeros: Union[None, float, int, str] = None, algo: str = "auto"):
+               with_scales: bool = True, zeros: Union[None, float, int, str] = None, algo: str = "auto",
+               tile: int = 0, gemv_tuning: tuple = None, skinny_tuning: tuple = None):
     """Device-resident fused kernel: kernel(A, B_packed[, scales][, zeros]) -> C.
 
     A [M,K] in_dtype; B_packed uint8 [N,K/2]; scales [N,K/group_size] in_dtype when with_scales;
     zeros: None (no zero point), a number (one zero point for the whole matrix) or "tensor"
     (a [N,K/group_size] in_dtype input follows).  C [M,N] out_dtype, fp32 accumulate.
-    algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "mfma" (LDS-staged MFMA kernel)."""
+    algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "skinny" (M <= 64) | "mfma" (LDS-staged MFMA kernel).
+    tile: rows of activations per work-group of the MFMA kernel (16, 32, 64, 128, 256; 0 = chosen by the
+    library); gemv_tuning = (rows_per_wave, waves, blocks_per_cu, depth) and skinny_tuning = (waves,
+    row_tiles) select among the pre-built variants of those kernels.  These are the tunable parameters an
+    autotuner searches (the role of block_M / block_N / block_K in the reference, which are accepted and
+    recorded but do not select a tiling here)."""
+    if tile not in (0, 16, 32, 64, 128, 256):
+        raise ValueError(f"tile must be one of 0, 16, 32, 64, 128, 256 (got {tile})")
     if in_dtype not in ("float16", "bfloat16"):
         raise ValueError(f"in_dtype must be float16 or bfloat16, got {in_dtype}")
     if out_dtype not in ("float16", "bfloat16", "float32"):
@@ -186,11 +194,13 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
             Z = t[i]
             i += 1
         C = t[i]
-        _abi.check(_abi.load().tlq_gemm_w4a16(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(S), _abi.ptr(Z), _abi.ptr(C), M, N, K,
-                                              group_size, zero_scalar, tin, tout, algo_code, stream))
+        with _abi.tuning(w4a16_tile=tile, gemv=gemv_tuning, skinny=skinny_tuning):
+            _abi.check(_abi.load().tlq_gemm_w4a16(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(S), _abi.ptr(Z), _abi.ptr(C), M, N,
+                                                  K, group_size, zero_scalar, tin, tout, algo_code, stream))
 
     return KernelSpec("w4a16_gemm", params, launch,
-                      {"block": (block_M, block_N, block_K), "group": group_size, "zeros": zeros, "algo": algo})
+                      {"block": (block_M, block_N, block_K), "group": group_size, "zeros": zeros, "algo": algo,
+                       "tile": tile, "gemv_tuning": gemv_tuning, "skinny_tuning": skinny_tuning})
 
 
 def dequant_gemm_fp16_wrapper(M: int, N: int, K: int, block_M: int, block_N: int, block_K: int,
