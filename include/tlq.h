@@ -124,6 +124,19 @@ int tlq_gemv_w4a16_batched(const void* A, const void* w_packed, const void* scal
 int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
                  int b_layout, void* stream);
 
+/* Split-K form of the same GEMM, replaces gemm_splitk (examples/gemm_splitk/example_tilelang_gemm_splitk.py:16-48):
+ * C (fp32 [M,N], accumulated IN PLACE, the caller zeroes it as the example does) += A[M,K] . B.  K is cut into
+ * split_k slices handled by different work-groups that add their partial tiles with atomic adds, so small-M /
+ * large-K problems fill the chip.  K % split_k == 0 and (K / split_k) % 8 == 0.  The order of the atomic adds is
+ * not fixed: results can differ between runs in the last bits. */
+int tlq_gemm_f16_splitk(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
+                        int in_dtype, int b_layout, void* stream);
+
+/* Plain GEMV y[N] = A[N,K] . x[K] with fp32 accumulate, replaces simple_gemv (examples/gemv/example_gemv_v.py:17-80 on
+ * the vector cores, example_gemv_c.py:16-46 on the cube cores; both y = x @ A.T).  dtype (of x and A): TLQ_F16,
+ * TLQ_BF16 or TLQ_F32; a row must be a multiple of 16 bytes; y in out_dtype. */
+int tlq_gemv(const void* x, const void* A, void* y, int64_t N, int64_t K, int dtype, int out_dtype, void* stream);
+
 /* int8 x int8 -> int32 GEMM (bit exact), replaces int8_gemm
  * (example_dequant_gemm_fine_grained.py:118-173); batched when batch > 1 (A [B,M,K], B [B,K,N] or
  * [B,N,K], C [B,M,N]). */

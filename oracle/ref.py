@@ -438,3 +438,18 @@ def act_quant_loop(x: torch.Tensor):
             q = min(max(q, np.float32(-127.0)), np.float32(127.0))
             y[m, n] = int(np.rint(q))
     return y, s
+
+
+# --------------------------------------------------------------------------------------
+# N1: non-quantised twins (examples/gemv, examples/gemm_splitk)
+# --------------------------------------------------------------------------------------
+def ref_program_gemv(x: torch.Tensor, A: torch.Tensor) -> torch.Tensor:
+    """examples/gemv/example_gemv_v.py:83-84 (``x @ A.T``), evaluated in float64 and rounded once to
+    x's dtype: the kernels accumulate in float32, so this is a tolerance oracle (pinned by the
+    one-hot and constant-row closed forms in the tests)."""
+    return (A.double() @ x.double()).to(x.dtype)
+
+
+def ref_program_splitk(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """examples/gemm_splitk/example_tilelang_gemm_splitk.py:66 (``a @ b`` compared in float32), in float64."""
+    return (a.double() @ b.double()).float()

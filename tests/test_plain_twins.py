@@ -1,0 +1,128 @@
+"""Non-quantised twins: plain GEMV (examples/gemv) and split-K GEMM (examples/gemm_splitk)."""
+import pytest
+import torch
+
+from oracle import ref
+
+DT = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def test_oracles_closed_forms():
+    A = torch.arange(24, dtype=torch.float32).view(4, 6)
+    x = torch.zeros(6)
+    x[2] = 1.0
+    assert torch.equal(ref.ref_program_gemv(x, A), A[:, 2])                  # one-hot picks a column
+    assert torch.equal(ref.ref_program_gemv(torch.ones(6), A), A.sum(dim=1))  # constant vector: row sums
+    a = torch.randn(5, 8, generator=torch.Generator().manual_seed(1)).half()
+    b = torch.eye(8).half()
+    assert torch.equal(ref.ref_program_splitk(a, b), a.float())              # identity
+
+
+def _rel_l2(got, want):
+    return float((got.double() - want.double()).norm() / want.double().norm().clamp_min(1e-30))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32"])
+@pytest.mark.parametrize("N,K", [(1024, 1024), (64, 64), (3, 8), (1, 4096), (257, 11008), (11008, 4096), (77, 40000)])
+def test_gemv_matches_reference(dtype, N, K):
+    from tilelang_ascend_amd.ops import simple_gemv
+
+    g = torch.Generator().manual_seed(N + K)
+    x = torch.randn(K, generator=g).to(DT[dtype])
+    A = torch.randn(N, K, generator=g).to(DT[dtype])
+    y = simple_gemv(N, K, 128, 128, dtype=dtype)(x.cuda(), A.cuda()).cpu()
+    assert y.dtype == DT[dtype] and y.shape == (N,)
+    want = ref.ref_program_gemv(x, A)
+    exact = A.double() @ x.double()
+    # fp32 accumulation: relative L2 <= 1e-3 of the exact product on top of the output rounding; the
+    # reference's own criterion (example_gemv_v.py:97) is assert_close(rtol=atol=1e-2) scaled by sqrt(K) magnitudes
+    assert _rel_l2(y, exact) <= (1e-5 if dtype == "float32" else 3e-3), _rel_l2(y, exact)
+    torch.testing.assert_close(y.float(), want.float(), rtol=1e-2, atol=1e-2 * max(1.0, (K / 1024) ** 0.5))
+
+
+@pytest.mark.gpu
+def test_gemv_one_hot_and_row_sums_are_exact():
+    from tilelang_ascend_amd.ops import simple_gemv
+
+    N, K = 130, 2048
+    A = torch.randint(-8, 8, (N, K), generator=torch.Generator().manual_seed(3)).half()
+    k = simple_gemv(N, K, 64, 64)
+    for j in (0, 7, 8, 1023, 2047):
+        x = torch.zeros(K, dtype=torch.float16)
+        x[j] = 1.0
+        assert torch.equal(k(x.cuda(), A.cuda()).cpu(), A[:, j])
+    ones = torch.ones(K, dtype=torch.float16)
+    assert torch.equal(k(ones.cuda(), A.cuda()).cpu().float(), A.float().sum(dim=1))  # small integers: exact in fp32
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K,split_k", [(128, 128, 128, 2), (1024, 1024, 1024, 4), (16, 4096, 14336, 16), (100, 72, 960, 3),
+                                           (300, 264, 512, 1), (64, 128, 8192, 64)])
+def test_splitk_matches_reference(dtype, M, N, K, split_k):
+    from tilelang_ascend_amd.ops import gemm_splitk
+
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).to(DT[dtype])
+    b = torch.randn(K, N, generator=g).to(DT[dtype])
+    c = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+    out = gemm_splitk(M, N, K, 128, 128, 32, split_k, dtype=dtype)(a.cuda(), b.cuda(), c)
+    assert out == [] or out is None
+    want = ref.ref_program_splitk(a, b)
+    assert _rel_l2(c.cpu(), want) <= 1e-5
+    torch.testing.assert_close(c.cpu(), want, rtol=1e-2, atol=1e-2)
+    # accumulation in place: a second call doubles the result
+    gemm_splitk(M, N, K, 128, 128, 32, split_k, dtype=dtype)(a.cuda(), b.cuda(), c)
+    assert _rel_l2(c.cpu(), 2 * want) <= 1e-5
+
+
+@pytest.mark.gpu
+def test_splitk_integer_inputs_are_exact_for_any_split():
+    """Small-integer operands make every partial sum exact in fp32, so all splits must agree bit for bit."""
+    from tilelang_ascend_amd.ops import gemm_splitk
+
+    M, N, K = 48, 136, 1536
+    g = torch.Generator().manual_seed(9)
+    a = torch.randint(-4, 5, (M, K), generator=g).half()
+    b = torch.randint(-4, 5, (K, N), generator=g).half()
+    want = ref.ref_program_splitk(a, b)
+    for split_k in (1, 2, 3, 6, 12, 24):
+        c = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+        gemm_splitk(M, N, K, 128, 128, 32, split_k)(a.cuda(), b.cuda(), c)
+        assert torch.equal(c.cpu(), want), split_k
+
+
+@pytest.mark.gpu
+def test_plain_twins_reject_bad_arguments():
+    from tilelang_ascend_amd import _abi
+    from tilelang_ascend_amd.ops import gemm_splitk
+
+    lib, P = _abi.load(), _abi.ptr
+    x = torch.zeros(64, device="cuda", dtype=torch.float16)
+    A = torch.zeros(4, 64, device="cuda", dtype=torch.float16)
+    y = torch.zeros(4, device="cuda", dtype=torch.float16)
+    assert lib.tlq_gemv(P(x), P(A), P(y), 4, 60, _abi.F16, _abi.F16, None) != 0 and "16 bytes" in _abi.last_error()
+    assert lib.tlq_gemv(P(x), P(A), P(y), 4, 64, _abi.I8, _abi.F16, None) != 0
+    assert lib.tlq_gemv(P(x), P(A), P(y), 0, 64, _abi.F16, _abi.F16, None) == 0
+    c = torch.zeros(4, 8, device="cuda")
+    assert lib.tlq_gemm_f16_splitk(P(A), P(A), P(c), 4, 8, 64, 3, _abi.F16, _abi.B_KN, None) != 0
+    assert "slices" in _abi.last_error()
+    with pytest.raises(ValueError):
+        gemm_splitk(4, 8, 64, 128, 128, 32, 5)
+
+
+@pytest.mark.gpu
+def test_plain_twin_examples(capsys):
+    from tilelang_ascend_amd.examples.gemm_splitk import example_gemm_splitk as exs
+    from tilelang_ascend_amd.examples.gemv import example_gemv as exg
+
+    exg.main(["--n", "512", "--k", "768"])
+    out = capsys.readouterr().out
+    assert out.rstrip().splitlines()[-2:] == ["GEMV example passed!", "Kernel Output Match!"]
+    exs.main([])
+    out = capsys.readouterr().out
+    assert "Test passed: M=128, N=128, K=128, split_k=2" in out and "Test passed: M=1024, N=1024, K=1024, split_k=4" in out
+    assert out.rstrip().endswith("Kernel Output Match!")
+    exs.main(["--M", "64", "--N", "256", "--K", "2048", "--split-k", "8"])
+    assert "Test passed: M=64, N=256, K=2048, split_k=8" in capsys.readouterr().out

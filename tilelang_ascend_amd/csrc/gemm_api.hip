@@ -11,6 +11,8 @@ int gemm_w4a16_skinny(const void* A, const void* Wp, const void* scales, const v
                       int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
                    int b_layout, hipStream_t st);
+int gemm_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
+                    int in_dtype, int b_layout, hipStream_t st);
 int gemm_i8_i32(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,
                 hipStream_t st);
 int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
@@ -99,6 +101,23 @@ int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, in
   TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_f16: pointers must be 16-byte aligned");
   TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K * 2), "tlq_gemm_f16: a matrix spans 4 GiB or more");
   return gemm_f16_plain(A, B, C, M, N, K, in_dtype, out_dtype, b_layout, (hipStream_t)stream);
+}
+
+int tlq_gemm_f16_splitk(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
+                        int in_dtype, int b_layout, void* stream) {
+  TLQ_CHECK_DIMS("tlq_gemm_f16_splitk");
+  TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16,
+              "tlq_gemm_f16_splitk: in_dtype must be float16 or bfloat16 (got %d)", in_dtype);
+  TLQ_REQUIRE(b_layout == TLQ_B_KN || b_layout == TLQ_B_NK, "tlq_gemm_f16_splitk: bad b_layout %d", b_layout);
+  TLQ_REQUIRE(split_k >= 1 && split_k <= 1024, "tlq_gemm_f16_splitk: split_k=%lld out of range 1..1024", (long long)split_k);
+  if (M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(K > 0 && K % split_k == 0 && (K / split_k) % 8 == 0,
+              "tlq_gemm_f16_splitk: K=%lld must split into %lld slices of a multiple of 8", (long long)K, (long long)split_k);
+  TLQ_REQUIRE(N % 8 == 0, "tlq_gemm_f16_splitk: N=%lld must be a multiple of 8", (long long)N);
+  TLQ_REQUIRE(A && B && C, "tlq_gemm_f16_splitk: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_f16_splitk: pointers must be 16-byte aligned");
+  TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K * 2), "tlq_gemm_f16_splitk: a matrix spans 4 GiB or more");
+  return gemm_f16_splitk(A, B, (float*)C, M, N, K, split_k, in_dtype, b_layout, (hipStream_t)stream);
 }
 
 int tlq_gemm_i8(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,

@@ -455,6 +455,20 @@ struct EpiFloat {  // fp32 accumulators -> f16 / bf16 / f32
   }
 };
 
+struct EpiAtomicAdd {  // fp32 accumulators added into C (split-K: several work-groups share an output tile)
+  struct Params {
+    float* C;
+    int64_t ldc;
+  };
+  Params p;
+  __device__ __forceinline__ EpiAtomicAdd(const Params& pp, int /*split*/) : p(pp) {}
+  __device__ __forceinline__ void store(int m, int n, const float4_t& acc, int M, int N) const {
+    if (m >= M || n >= N) return;
+    float* c = p.C + (int64_t)m * p.ldc + n;
+    for (int i = 0; i < 4 && n + i < N; ++i) unsafeAtomicAdd(c + i, acc[i]);
+  }
+};
+
 struct EpiInt32 {  // raw int32 accumulators
   struct Params {
     int32_t* C;

@@ -102,6 +102,36 @@ static int run_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, 
   return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16");
 }
 
+// Split-K: slice z of K is "batch" z of the loaders (the batch strides step along K), and every slice
+// adds its partial tile into the one fp32 C.
+template <class Mma, int BM, int BN, int WM, int WN>
+static int run_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
+                          int b_layout, hipStream_t st) {
+  constexpr int NT = WM * WN * 64;
+  const int64_t ks = K / split_k;
+  typedef RowLoaderDirect<BM, NT> AL;
+  typename AL::Params pa{(const uint8_t*)A, K * 2, ks * 2, ks * 2};
+  EpiAtomicAdd::Params pe{C, N};
+  if (b_layout == TLQ_B_NK) {
+    typedef RowLoaderDirect<BN, NT> WL;
+    typename WL::Params pw{(const uint8_t*)B, K * 2, ks * 2, ks * 2};
+    return launch_gemm<Mma, AL, WL, EpiAtomicAdd, BM, BN, WM, WN>(pa, pw, pe, split_k, M, N, ks * 2, st, "tlq_gemm_f16_splitk");
+  }
+  typedef H16KNLoader<BN, NT> WL;
+  typename WL::Params pw{(const uint8_t*)B, N * 2, ks * N * 2, ks};
+  return launch_gemm<Mma, AL, WL, EpiAtomicAdd, BM, BN, WM, WN>(pa, pw, pe, split_k, M, N, ks * 2, st, "tlq_gemm_f16_splitk");
+}
+
+int gemm_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
+                    int in_dtype, int b_layout, hipStream_t st) {
+  const bool small = M <= 128 || ceil_div(M, 256) * ceil_div(N, 256) * split_k < 128;
+  if (in_dtype == TLQ_F16)
+    return small ? run_f16_splitk<MmaF16, 128, 128, 2, 2>(A, B, C, M, N, K, split_k, b_layout, st)
+                 : run_f16_splitk<MmaF16, 256, 256, 2, 4>(A, B, C, M, N, K, split_k, b_layout, st);
+  return small ? run_f16_splitk<MmaBF16, 128, 128, 2, 2>(A, B, C, M, N, K, split_k, b_layout, st)
+               : run_f16_splitk<MmaBF16, 256, 256, 2, 4>(A, B, C, M, N, K, split_k, b_layout, st);
+}
+
 template <class Mma>
 static int dispatch_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int out_dtype,
                         int b_layout, hipStream_t st) {
