@@ -162,6 +162,19 @@ int tlq_gemm_w4a8(const void* A, const void* w_packed, void* C, int64_t M, int64
 int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
                   int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, void* stream);
 
+/* Offline weight preparation on the GPU.
+ * tlq_pack_int4 replaces general_compress (tilelang/quantize/utils.py:53-69, 4-bit source) and, with
+ * interleave = 1 (fp16 target) or 2 (int8 target), the interleave_weight that follows it (:73-101):
+ * values int8 [N,K] -> packed bytes [N,K/2], value k of a byte pair at bits 4k (not masked, like the
+ * reference: out-of-range values spill into their neighbours), then the field permutation within each
+ * 32-bit word.  K % 8 == 0.
+ * tlq_quantize_sym4 is the quantiser of gen_quant4 (:5-50) for weights stored [N,K] with groups along K:
+ * s = max|w| / 8 per group, q = clamp(round(w / s) + 8, 0, 16); writes q - 8 (int8 [N,K]) and s
+ * ([N,K/group], dtype of W: TLQ_F16 or TLQ_BF16).  group % 8 == 0. */
+int tlq_pack_int4(const void* values, void* packed, int64_t N, int64_t K, int interleave, void* stream);
+int tlq_quantize_sym4(const void* W, void* q_minus8, void* scales, int64_t N, int64_t K, int64_t group, int dtype,
+                      void* stream);
+
 /* Per-token int8 activation quantiser, replaces act_quant_kernel_int8_optimized
  * (examples/deepseek_v4/act_quant.py:25-92) with the arithmetic of its golden function (:112-142):
  *   amax = max(max_n |x[m,n]|, 1e-4);  scale[m] = amax / 127  (round_scale: 2^ceil(log2(amax / 127)), :95-109)

@@ -453,3 +453,20 @@ def ref_program_gemv(x: torch.Tensor, A: torch.Tensor) -> torch.Tensor:
 def ref_program_splitk(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """examples/gemm_splitk/example_tilelang_gemm_splitk.py:66 (``a @ b`` compared in float32), in float64."""
     return (a.double() @ b.double()).float()
+
+
+# --------------------------------------------------------------------------------------
+# P5: the quantiser inside gen_quant4 for weights stored [N, K], groups along K
+# --------------------------------------------------------------------------------------
+def quantize_sym4(W: torch.Tensor, group: int):
+    """tilelang/quantize/utils.py:20-31 on W [N, K] (the reference holds w [k, n] and groups along k:
+    the same numbers, transposed): s = max|w| * (2 / 16) in W's dtype, q = clamp(round(w / s).int() + 8, 0, 16).
+    Returns (q - 8 as int8, s [N, K/group]).  A group of zeros divides 0 by 0; the int conversion of the
+    NaN is the most negative integer on x86, so q = 0 there (q - 8 = -8)."""
+    N, K = W.shape
+    wg = W.reshape(N, K // group, group)
+    s = wg.abs().amax(dim=2, keepdim=True) * (2 / 16)
+    quot = torch.round(wg / s).float()                      # w / s is rounded to W's dtype before the round
+    quot = torch.where(torch.isnan(quot), torch.full_like(quot, -1e9), quot)
+    q = torch.clamp(quot.to(torch.int64) + 8, 0, 16)
+    return (q - 8).to(torch.int8).reshape(N, K), s.reshape(N, K // group).contiguous()

@@ -39,6 +39,8 @@ SIGNATURES = {
     "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_gemm_f16_splitk": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_gemv": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
+    "tlq_pack_int4": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "tlq_quantize_sym4": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "tlq_act_quant_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "tlq_tune_gemv": (None, [_int, _int]),
     "tlq_tune_gemv_unroll": (None, [_int]),

@@ -30,6 +30,7 @@ SOURCES = [
     "unpack_dequant.hip",
     "decode_i4.hip",
     "act_quant.hip",
+    "repack.hip",
     "gemv_plain.hip",
     "gemv_w4a16.hip",
     "gemm_w4a16.hip",
