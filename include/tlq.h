@@ -63,7 +63,8 @@ enum {
   TLQ_ALGO_AUTO = 0,
   TLQ_ALGO_GEMV = 1, /* split-K wavefront GEMV (M <= 16) */
   TLQ_ALGO_MFMA = 2, /* LDS-staged MFMA dequant-GEMM */
-  TLQ_ALGO_SKINNY = 3 /* M <= 64: weights stream from HBM through the dequantiser into MFMA operands, no LDS tile */
+  TLQ_ALGO_SKINNY = 3, /* M <= 64: weights stream from HBM through the dequantiser into MFMA operands, no LDS tile */
+  TLQ_ALGO_TWO_PASS = 4 /* tlq_gemm_w4a16_ws only: dequantise into the workspace, then the plain GEMM */
 };
 
 int tlq_abi_version(void);
@@ -107,6 +108,17 @@ int tlq_decode_i4_interleaved(const void* words, const void* scales, const void*
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                    void* stream);
+
+/* The same operator with a caller-owned workspace of tlq_w4a16_workspace_bytes(M, N, K) bytes (0 when a
+ * workspace would not be used).  With it, large-M problems (M >= 2048) take two passes -- tlq_dequant_w4 into
+ * the workspace, then tlq_gemm_f16 on it -- which is the structure of the reference's own wrapper
+ * (example_dequant_gemm_fine_grained.py:176-223 unpacks, then calls fp16_gemm) and is faster than converting
+ * the weights again in every row block of the fused kernel.  The workspace holds nothing between calls.
+ * algo: as tlq_gemm_w4a16, or TLQ_ALGO_TWO_PASS to force the two passes (workspace required). */
+int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
+                      int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
+                      void* workspace, int64_t workspace_bytes, void* stream);
 
 /* `batch` independent decode GEMVs in one launch (one grid row per problem): A [batch,M,K],
  * w_packed [batch,N,K/2], scales / zeros [batch,N,K/group], C [batch,M,N], all contiguous.

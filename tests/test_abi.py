@@ -13,7 +13,7 @@ HEADER = os.path.join(ROOT, "include", "tlq.h")
 
 CTYPE = {"const void*": ctypes.c_void_p, "void*": ctypes.c_void_p, "int64_t": ctypes.c_int64, "int": ctypes.c_int,
          "float": ctypes.c_float}
-RESTYPE = {"int": ctypes.c_int, "void": None, "const char*": ctypes.c_char_p}
+RESTYPE = {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "void": None, "const char*": ctypes.c_char_p}
 
 
 def declared():
@@ -21,7 +21,7 @@ def declared():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
     out = {}
-    for m in re.finditer(r"(const char\*|int|void)\s+(tlq_\w+)\s*\(([^)]*)\)\s*;", text):
+    for m in re.finditer(r"(const char\*|int64_t|int|void)\s+(tlq_\w+)\s*\(([^)]*)\)\s*;", text):
         ret, name, args = m.group(1), m.group(2), " ".join(m.group(3).split())
         types = []
         if args != "void":
@@ -64,7 +64,8 @@ def test_enum_codes_match_the_header():
                       ("TLQ_I32", _abi.I32), ("TLQ_U4", _abi.U4), ("TLQ_S4_TWOS", _abi.S4_TWOS),
                       ("TLQ_S4_OFFSET8", _abi.S4_OFFSET8), ("TLQ_S4_OFFSET7", _abi.S4_OFFSET7), ("TLQ_B_KN", _abi.B_KN),
                       ("TLQ_B_NK", _abi.B_NK), ("TLQ_ALGO_AUTO", _abi.ALGO_AUTO), ("TLQ_ALGO_GEMV", _abi.ALGO_GEMV),
-                      ("TLQ_ALGO_MFMA", _abi.ALGO_MFMA), ("TLQ_ALGO_SKINNY", _abi.ALGO_SKINNY)):
+                      ("TLQ_ALGO_MFMA", _abi.ALGO_MFMA), ("TLQ_ALGO_SKINNY", _abi.ALGO_SKINNY),
+                      ("TLQ_ALGO_TWO_PASS", _abi.ALGO_TWO_PASS)):
         m = re.search(rf"\b{name}\s*=\s*(\d+)", text)
         assert m and int(m.group(1)) == val, name
 

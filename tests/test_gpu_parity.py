@@ -173,6 +173,50 @@ def test_gemv_batched_entry_point(M, N, K, group):
         check_float_output(C[b].cpu(), w4a16_reference(A[b], *sets[b], group), f"batched set {b}")
 
 
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K,group,zeros_kind,algo", [
+    (2048, 256, 512, 128, "int", "auto"), (100, 136, 256, 64, "frac", "two_pass"), (2304, 72, 192, 32, None, "auto"),
+    (16, 64, 128, 128, "scalar8", "two_pass"),
+])
+def test_w4a16_two_pass_with_workspace(ops, in_dtype, M, N, K, group, zeros_kind, algo):
+    """Dequantise into the kernel object's workspace, then the plain GEMM: what auto does from M = 2048 up."""
+    dt = DT[in_dtype]
+    A = torch.randn(M, K, generator=gen(60)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=61)
+    want = w4a16_reference(A, Wp, s, z, group)
+    for out_dtype in ("float32", in_dtype):
+        got = _run_w4a16(ops, A, Wp, s, z, group, out_dtype, algo, in_dtype)
+        check_float_output(got, want, f"two-pass {in_dtype}->{out_dtype}")
+
+
+def test_w4a16_workspace_entry_point_rules():
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    assert lib.tlq_w4a16_workspace_bytes(2048, 256, 512) == 256 * 512 * 2
+    assert lib.tlq_w4a16_workspace_bytes(2047, 256, 512) == 0
+    M, N, K, g = 64, 128, 256, 128
+    A = torch.randn(M, K, generator=gen(62)).half()
+    Wp, s, z = make_w4(N, K, g, torch.float16, "int", seed=63)
+    Ad, Wd, sd, zd = A.cuda(), Wp.cuda(), s.cuda(), z.cuda()
+    C = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    args = (P(Ad), P(Wd), P(sd), P(zd), P(C), M, N, K, g, 0.0, _abi.F16, _abi.F16)
+    # forced two-pass without (or with a short) workspace is an error, auto falls back to the fused kernels
+    assert lib.tlq_gemm_w4a16_ws(*args, _abi.ALGO_TWO_PASS, None, 0, st) != 0 and "workspace" in _abi.last_error()
+    ws = torch.empty(N * K * 2, dtype=torch.uint8, device="cuda")
+    assert lib.tlq_gemm_w4a16_ws(*args, _abi.ALGO_TWO_PASS, P(ws), N * K * 2 - 1, st) != 0
+    assert lib.tlq_gemm_w4a16_ws(*args, _abi.ALGO_AUTO, None, 0, st) == 0
+    fused = C.clone()
+    assert lib.tlq_gemm_w4a16_ws(*args, _abi.ALGO_TWO_PASS, P(ws), N * K * 2, st) == 0
+    want = w4a16_reference(A, Wp, s, z, g)
+    check_float_output(fused.cpu(), want, "auto without workspace")
+    check_float_output(C.cpu(), want, "forced two-pass")
+    # the workspace holds the dequantised matrix, bit for bit
+    assert_bit_equal(ws.view(torch.float16).view(N, K).cpu(), ref.dequant_w4(Wp, s, z, g, torch.float16), "workspace")
+    assert lib.tlq_gemm_w4a16(*args, _abi.ALGO_TWO_PASS, st) != 0          # not an algo of the plain entry point
+
+
 def test_gemv_one_hot_reads_back_dequantised_rows(ops):
     """A one-hot activation row makes the output equal one column of the dequantised matrix:
     pins nibble order, group indexing and zero / scale handling inside the fused kernel."""

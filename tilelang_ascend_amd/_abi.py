@@ -18,7 +18,7 @@ from . import build as _build
 F16, BF16, F32, I8, I32 = 0, 1, 2, 3, 4
 U4, S4_TWOS, S4_OFFSET8, S4_OFFSET7 = 0, 1, 2, 3
 B_KN, B_NK = 0, 1
-ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY = 0, 1, 2, 3
+ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY, ALGO_TWO_PASS = 0, 1, 2, 3, 4
 ABI_VERSION = 1
 
 _vp, _i64, _int, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
@@ -37,6 +37,8 @@ SIGNATURES = {
     "tlq_gemm_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "tlq_gemm_w4a8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "tlq_w4a16_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "tlq_gemm_w4a16_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp, _i64, _vp]),
     "tlq_gemm_f16_splitk": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_gemv": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "tlq_pack_int4": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),

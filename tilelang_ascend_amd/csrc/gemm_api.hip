@@ -67,6 +67,40 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
   return gemm_w4a16_mfma(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, st);
 }
 
+// M from which dequantising the whole matrix once and running the plain GEMM on it beats converting the
+// weights again in every 256-row block of the fused kernel (measured: N=14336, K=4096 breaks even near 1500)
+static const int64_t kTwoPassMinM = 2048;
+
+int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M < kTwoPassMinM || N <= 0 || K <= 0) return 0;
+  return N * K * 2;
+}
+
+int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
+                      int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
+                      void* workspace, int64_t workspace_bytes, void* stream) {
+  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_TWO_PASS, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  const int64_t need = (N > 0 && K > 0) ? N * K * 2 : 0;
+  const bool have = workspace != nullptr && workspace_bytes >= need && aligned16(workspace);
+  if (algo == TLQ_ALGO_TWO_PASS)
+    TLQ_REQUIRE(have, "tlq_gemm_w4a16_ws: the two-pass path needs a 16-byte aligned workspace of %lld bytes (got %lld)",
+                (long long)need, (long long)workspace_bytes);
+  const bool two_pass = algo == TLQ_ALGO_TWO_PASS || (algo == TLQ_ALGO_AUTO && have && M >= kTwoPassMinM && N % 8 == 0);
+  if (!two_pass)
+    return tlq_gemm_w4a16(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype,
+                          algo == TLQ_ALGO_TWO_PASS ? TLQ_ALGO_AUTO : algo, stream);
+  TLQ_CHECK_DIMS("tlq_gemm_w4a16_ws");
+  TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_w4a16_ws: in_dtype must be float16 or bfloat16 (got %d)",
+              in_dtype);
+  if (M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(K > 0 && K % 64 == 0, "tlq_gemm_w4a16_ws: K=%lld must be a positive multiple of 64", (long long)K);
+  TLQ_REQUIRE(group > 0 && K % group == 0 && group % 32 == 0,
+              "tlq_gemm_w4a16_ws: group=%lld must divide K=%lld and be a multiple of 32", (long long)group, (long long)K);
+  TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16_ws: scales / zeros misaligned");
+  if (int rc = tlq_dequant_w4(w_packed, scales, zeros, workspace, N, K, group, zero_scalar, in_dtype, stream)) return rc;
+  return tlq_gemm_f16(A, workspace, C, M, N, K, in_dtype, out_dtype, TLQ_B_NK, stream);
+}
+
 int tlq_gemv_w4a16_batched(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C,
                            int64_t batch, int64_t M, int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype,
                            int out_dtype, void* stream) {

@@ -26,7 +26,8 @@ _PASS_CONFIGS = {
     PassConfigKey.TL_ASCEND_AUTO_CV_SYNC: True,
 }
 _SIGN_MODES = {"unsigned": _abi.U4, "twos": _abi.S4_TWOS, "offset8": _abi.S4_OFFSET8, "offset7": _abi.S4_OFFSET7}
-_ALGOS = {"auto": _abi.ALGO_AUTO, "gemv": _abi.ALGO_GEMV, "mfma": _abi.ALGO_MFMA, "skinny": _abi.ALGO_SKINNY}
+_ALGOS = {"auto": _abi.ALGO_AUTO, "gemv": _abi.ALGO_GEMV, "mfma": _abi.ALGO_MFMA, "skinny": _abi.ALGO_SKINNY,
+          "two_pass": _abi.ALGO_TWO_PASS}
 
 
 def _stream() -> int:
@@ -157,7 +158,9 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
     A [M,K] in_dtype; B_packed uint8 [N,K/2]; scales [N,K/group_size] in_dtype when with_scales;
     zeros: None (no zero point), a number (one zero point for the whole matrix) or "tensor"
     (a [N,K/group_size] in_dtype input follows).  C [M,N] out_dtype, fp32 accumulate.
-    algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "skinny" (M <= 64) | "mfma" (LDS-staged MFMA kernel).
+    algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "skinny" (M <= 64) | "mfma" (LDS-staged MFMA kernel)
+    | "two_pass" (dequantise into a workspace, then the plain GEMM: what "auto" does from M = 2048 up; the kernel
+    object then keeps a [N, K] workspace in the activation type on the device of its first call).
     tile: rows of activations per work-group of the MFMA kernel (16, 32, 64, 128, 256; 0 = chosen by the
     library); gemv_tuning = (rows_per_wave, waves, blocks_per_cu, depth) and skinny_tuning = (waves,
     row_tiles) select among the pre-built variants of those kernels.  These are the tunable parameters an
@@ -182,6 +185,7 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
     params.append(Param("C", (M, N), out_dtype))
     tin, tout = ABI_DTYPE[TORCH_DTYPES[in_dtype]], ABI_DTYPE[TORCH_DTYPES[out_dtype]]
     algo_code = _ALGOS[algo]
+    workspace = {}  # device -> uint8 tensor, created on the first launch that needs it
 
     def launch(t, sym, stream):
         A, Bp = t[0], t[1]
@@ -194,9 +198,16 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
             Z = t[i]
             i += 1
         C = t[i]
+        lib = _abi.load()
+        ws = None
+        ws_bytes = N * K * 2 if algo == "two_pass" else (lib.tlq_w4a16_workspace_bytes(M, N, K) if algo == "auto" else 0)
+        if ws_bytes:
+            ws = workspace.get(A.device)
+            if ws is None:
+                ws = workspace[A.device] = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
         with _abi.tuning(w4a16_tile=tile, gemv=gemv_tuning, skinny=skinny_tuning):
-            _abi.check(_abi.load().tlq_gemm_w4a16(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(S), _abi.ptr(Z), _abi.ptr(C), M, N,
-                                                  K, group_size, zero_scalar, tin, tout, algo_code, stream))
+            _abi.check(lib.tlq_gemm_w4a16_ws(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(S), _abi.ptr(Z), _abi.ptr(C), M, N, K,
+                                             group_size, zero_scalar, tin, tout, algo_code, _abi.ptr(ws), ws_bytes, stream))
 
     return KernelSpec("w4a16_gemm", params, launch,
                       {"block": (block_M, block_N, block_K), "group": group_size, "zeros": zeros, "algo": algo,
