@@ -121,7 +121,6 @@ template <int ROWS, int NT>
 struct RowLoader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
-  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
   static constexpr bool PREFETCH2 = false;
   static constexpr int SLOTS = ROWS * 8;  // 16-byte chunks per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
@@ -196,7 +195,6 @@ template <int ROWS, int NT>
 struct RowLoaderDirect {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = true;
-  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
   static constexpr bool PREFETCH2 = false;
   static constexpr int WAVES = NT / 64;
   static constexpr int INSTR = ROWS / 8;          // wavefront-instructions per stage
@@ -273,72 +271,14 @@ struct RowLoaderDirect {
 
 // int8 source stored [K, N] (N contiguous): rows of k are copied unchanged into a [128 k][BN] LDS
 // tile; the transposition happens in the operand read (KNFrag8).
-template <int BN, int NT>
-struct I8KNLoader {
-  typedef KNFrag8<BN> Frag;
-  static constexpr bool DIRECT = false;
-  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
-  static constexpr bool PREFETCH2 = false;
-  static constexpr int CH = BN / 16;            // 16-byte chunks per k row
-  static constexpr int RPP = NT / CH;           // k rows per pass
-  static constexpr int PASSES = kStageBytes / RPP;
-  static constexpr int UNITS = PASSES;
-  static_assert(NT % CH == 0 && RPP % 32 == 0 && kStageBytes % RPP == 0, "pass stride must keep the swizzle phase");
-  struct Params {
-    const uint8_t* base;  // B[0, 0] of batch 0
-    int64_t ld;           // bytes per k row (= N)
-    int64_t batch_stride;
-    int64_t k_total;  // K
-  };
-  struct Regs {
-    uint4_t v[PASSES];
-  };
-  const uint8_t* base;  // uniform
-  uint32_t ld;
-  uint32_t voff;  // per lane: k0 * ld + col
-  uint32_t loff;  // per lane: LDS offset of pass 0
-  int k0;
-  int k_total;
-
-  // cols_total must be a multiple of 16 (checked on the host)
-  __device__ __forceinline__ I8KNLoader(const Params& p, int batch, int col0, int cols_total, int tid)
-      : base(p.base + batch * p.batch_stride + col0), ld((uint32_t)p.ld), k_total((int)p.k_total) {
-    const int cols_valid = cols_total - col0;
-    const int c = tid % CH;
-    k0 = tid / CH;
-    int col = c * 16;
-    col = col < cols_valid ? col : cols_valid - 16;  // clamp whole chunks: loads stay in bounds, results are masked
-    voff = (uint32_t)k0 * ld + (uint32_t)col;
-    loff = (uint32_t)(k0 * BN + ((c ^ kn_swz<BN>(k0)) << 4));
-  }
-
-  template <bool TAIL>
-  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* /*lds_next*/ = nullptr) const {
-    const uint8_t* sb = uniform_ptr(base + (int64_t)kt * kStageBytes * ld);
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-      const uint32_t o = voff + (uint32_t)(ps * RPP) * ld;
-      if (!TAIL) {
-        r.v[ps] = *(const uint4_t*)(sb + o);
-      } else {
-        const bool ok = kt * kStageBytes + ps * RPP + k0 < k_total;
-        uint4_t v = *(const uint4_t*)(ok ? sb + o : base + (voff - (uint32_t)k0 * ld));
-        if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
-        r.v[ps] = v;
-      }
-    }
-  }
-  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-      if (ps * np / UNITS != pc) continue;
-      *(uint4_t*)(lds + loff + ps * RPP * BN) = r.v[ps];
-    }
-  }
-  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
+struct I8KNParams {
+  const uint8_t* base;  // B[0, 0] of batch 0
+  int64_t ld;           // bytes per k row (= N)
+  int64_t batch_stride;
+  int64_t k_total;  // K
 };
 
-// The same [128 k][BN] tile filled by direct global -> LDS loads: one wavefront instruction covers
+// The tile is filled by direct global -> LDS loads: one wavefront instruction covers
 // 1024 / BN consecutive k rows; the lane landing on (k, physical chunk pc) fetches logical chunk
 // pc ^ kn_swz(k) of that k row.  A partial last stage (rows past K must read as zero) goes through
 // registers.
@@ -346,7 +286,6 @@ template <int BN, int NT>
 struct I8KNLoaderDirect {
   typedef KNFrag8<BN> Frag;
   static constexpr bool DIRECT = true;
-  static constexpr int VALU_PER_MFMA = 0;
   static constexpr bool PREFETCH2 = false;
   static constexpr int CH = BN / 16;              // 16-byte chunks per k row
   static constexpr int KPI = 64 / CH;             // k rows per wavefront instruction
@@ -355,7 +294,7 @@ struct I8KNLoaderDirect {
   static constexpr int PER_WAVE = INSTR / WAVES;
   static constexpr int UNITS = PER_WAVE;
   static_assert(INSTR % WAVES == 0 && PER_WAVE >= 1, "tile does not split into whole wavefront loads");
-  typedef typename I8KNLoader<BN, NT>::Params Params;
+  typedef I8KNParams Params;
   struct Regs {
     uint4_t v[PER_WAVE];
     bool pending;
@@ -622,21 +561,6 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
           else
             wl.lstore_piece(rw, nw, pc - NPA, NP - NPA);
           if (NPA == 0 && pc == 0) al.lstore(ra, na);  // direct loader: only a partial last stage stores anything
-        }
-      }
-    }
-    // Scheduling pipeline for the whole stage: left alone, the compiler gathers the conversion
-    // arithmetic of the fill into one long run after the last MFMA, where nothing hides it.
-    constexpr int VPM = WL::VALU_PER_MFMA;
-    if (FILL && VPM > 0) {
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        __builtin_amdgcn_sched_group_barrier(0x100, TN + TM, 0);  // operand fragment reads of this k-step
-#pragma unroll
-        for (int i = 0; i < TN * TM; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);  // VPM conversion instructions in its shadow
-          if (i % 16 == 15) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // an LDS store of converted weights
         }
       }
     }

@@ -10,7 +10,6 @@ template <int ROWS, int NT>
 struct H16KNLoader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
-  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
   static constexpr bool PREFETCH2 = false;
   static constexpr int NBLK = ROWS / 8;            // 8-column blocks per tile
   static constexpr int PASSES = (16 * NBLK) / NT;  // 64 k = 16 blocks of 4 rows

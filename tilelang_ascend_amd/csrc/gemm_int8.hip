@@ -13,7 +13,6 @@ template <int ROWS, int NT>
 struct W4I8Loader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
-  static constexpr int VALU_PER_MFMA = 0;  // no scheduling hint
   static constexpr bool PREFETCH2 = false;
   static constexpr int SLOTS = ROWS * 4;
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;

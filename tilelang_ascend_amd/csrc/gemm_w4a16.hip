@@ -96,7 +96,6 @@ template <typename T, bool FOLD, int ROWS, int NT>
 struct W4Loader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
-  static constexpr int VALU_PER_MFMA = 0;
   static constexpr bool PREFETCH2 = true;  // convert from registers loaded one stage earlier
   static constexpr int SLOTS = ROWS * 2;  // 16-byte packed loads per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
