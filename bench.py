@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|prefill|w8a8|skinny|actquant] [--units U]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|prefill|w8a8|skinny|actquant|mlp-sweep] [--units U]
 
 Headline workload (default): the W4A16 decode GEMV -- M=1, N=11008, K=4096, fp16 activations,
 uint4 weights packed low-nibble-first, group 128, fp16 scales U[0.005,0.02] and fp16 zeros U{6..9},
@@ -266,6 +266,52 @@ def bench_act_quant(args, steps=None):
                          "traffic": TRAFFIC_ACT_QUANT, "bytes_per_launch": unit_bytes, "avg_launch_us": round(ev * 1e6, 3)}}
 
 
+def bench_mlp_sweep(args, steps=None):
+    """cfg-5 sweep: M in {16, 64, 256, 1024, 8192} x (N, K) in {(14336, 4096), (4096, 14336)} x group in {128, 64},
+    fp16, per-group scales and zeros, automatic kernel choice with a workspace (tlq_gemm_w4a16_ws)."""
+    import torch
+
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for (N, K) in ((14336, 4096), (4096, 14336)):
+        for g in (128, 64):
+            sets = 6  # 6 x 29 MB of packed weights rotate: small-M launches always stream from HBM
+            gen = torch.Generator(device="cpu").manual_seed(5)
+            Wp = torch.randint(0, 256, (sets, N, K // 2), dtype=torch.uint8, generator=gen).to(dev)
+            S = (torch.rand(sets, N, K // g, generator=gen) * 0.015 + 0.005).to(torch.float16).to(dev)
+            Z = torch.randint(6, 10, (sets, N, K // g), generator=gen).to(torch.float16).to(dev)
+            for M in (16, 64, 256, 1024, 8192):
+                A = torch.randn(M, K, generator=gen).to(torch.float16).to(dev)
+                C = torch.empty(M, N, dtype=torch.float16, device=dev)
+                ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
+                ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+                pre = [(P(A), P(Wp[j]), P(S[j]), P(Z[j]), P(C), M, N, K, g, 0.0, _abi.F16, _abi.F16, _abi.ALGO_AUTO,
+                        P(ws) if ws_bytes else None, ws_bytes, stream) for j in range(sets)]
+
+                def step(i):
+                    if lib.tlq_gemm_w4a16_ws(*pre[i % sets]):
+                        raise RuntimeError(_abi.last_error())
+
+                _, ev = timed(step, steps or (12 if M < 8192 else 4), 3)
+                flops, nbytes = 2.0 * M * N * K, w4a16_bytes(M, N, K, g)
+                rows.append({"M": M, "N": N, "K": K, "group": g, "us": round(ev * 1e6, 1),
+                             "TFLOP/s": round(flops / ev / 1e12, 1), "frac_mfma": round(flops / ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                             "GB/s": round(nbytes / ev / 1e9), "frac_hbm": round(nbytes / ev / 1e9 / HBM_PEAK_GBS, 4)})
+                del A, C, ws
+            del Wp, S, Z
+    big = max(rows, key=lambda r: r["TFLOP/s"])
+    return {"workload": "W4A16 MLP-shaped sweep, fp16, 20 shapes, automatic kernel choice with workspace", "dtype": "f16",
+            "value": big["TFLOP/s"], "unit": "TFLOP/s", "ms_per_step": big["us"] * 1e-3,
+            "roofline": {"kernel": "best of the sweep (M=%d N=%d K=%d)" % (big["M"], big["N"], big["K"]), "bound": "mfma",
+                         "achieved": big["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": big["frac_mfma"],
+                         "traffic": None},
+            "shapes": rows}
+
+
 def bench_w8a8(args, steps=None):
     import torch
 
@@ -302,7 +348,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=48)
-    ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8", "skinny", "actquant"])
+    ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8", "skinny", "actquant", "mlp-sweep"])
     ap.add_argument("--units", type=int, default=1, help="independent weight sets per GEMV launch")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
@@ -333,10 +379,13 @@ def main():
                 bench_act_quant(args, steps=40)]
     else:
         res = {"prefill": bench_prefill, "w8a8": bench_w8a8, "skinny": bench_skinny,
-               "actquant": bench_act_quant}[args.workload](args)
+               "actquant": bench_act_quant, "mlp-sweep": bench_mlp_sweep}[args.workload](args)
         line = {"metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
                 "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
                 "config": {"workload": res["workload"]}, "roofline": res["roofline"], "cpu_baseline": None}
+        for extra in ("shapes", "with_workspace"):
+            if extra in res:
+                line[extra] = res[extra]
     if args.calibrate_copy:
         src = torch.zeros(64 * 1024 * 1024, dtype=torch.int32, device="cuda:0")
         dst = torch.empty_like(src)

@@ -110,7 +110,7 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
                    void* stream);
 
 /* The same operator with a caller-owned workspace of tlq_w4a16_workspace_bytes(M, N, K) bytes (0 when a
- * workspace would not be used).  With it, large-M problems (M >= 2048) take two passes -- tlq_dequant_w4 into
+ * workspace would not be used).  With it, problems from M = 256 up take two passes -- tlq_dequant_w4 into
  * the workspace, then tlq_gemm_f16 on it -- which is the structure of the reference's own wrapper
  * (example_dequant_gemm_fine_grained.py:176-223 unpacks, then calls fp16_gemm) and is faster than converting
  * the weights again in every row block of the fused kernel.  The workspace holds nothing between calls.

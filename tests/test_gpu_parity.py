@@ -176,10 +176,10 @@ def test_gemv_batched_entry_point(M, N, K, group):
 @pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
 @pytest.mark.parametrize("M,N,K,group,zeros_kind,algo", [
     (2048, 256, 512, 128, "int", "auto"), (100, 136, 256, 64, "frac", "two_pass"), (2304, 72, 192, 32, None, "auto"),
-    (16, 64, 128, 128, "scalar8", "two_pass"),
+    (16, 64, 128, 128, "scalar8", "two_pass"), (256, 264, 8192, 128, "int", "auto"), (300, 72, 14336, 64, "frac", "auto"),
 ])
 def test_w4a16_two_pass_with_workspace(ops, in_dtype, M, N, K, group, zeros_kind, algo):
-    """Dequantise into the kernel object's workspace, then the plain GEMM: what auto does from M = 2048 up."""
+    """Dequantise into the kernel object's workspace, then the plain GEMM: what auto does from M = 256 up."""
     dt = DT[in_dtype]
     A = torch.randn(M, K, generator=gen(60)).to(dt)
     Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=61)
@@ -194,7 +194,8 @@ def test_w4a16_workspace_entry_point_rules():
 
     lib, P = _abi.load(), _abi.ptr
     assert lib.tlq_w4a16_workspace_bytes(2048, 256, 512) == 256 * 512 * 2
-    assert lib.tlq_w4a16_workspace_bytes(2047, 256, 512) == 0
+    assert lib.tlq_w4a16_workspace_bytes(255, 256, 512) == 0
+    assert lib.tlq_w4a16_workspace_bytes(256, 264, 8192) == 264 * 8192 * 2
     M, N, K, g = 64, 128, 256, 128
     A = torch.randn(M, K, generator=gen(62)).half()
     Wp, s, z = make_w4(N, K, g, torch.float16, "int", seed=63)

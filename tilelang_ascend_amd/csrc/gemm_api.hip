@@ -68,8 +68,9 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
 }
 
 // M from which dequantising the whole matrix once and running the plain GEMM on it beats converting the
-// weights again in every 256-row block of the fused kernel (measured: N=14336, K=4096 breaks even near 1500)
-static const int64_t kTwoPassMinM = 2048;
+// weights again in every row block of the fused kernel (measured on the MLP shapes: level at M = 256 for
+// N = 14336, K = 4096 and 20-40 % ahead from there on and for N = 4096, K = 14336)
+static const int64_t kTwoPassMinM = 256;
 
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M < kTwoPassMinM || N <= 0 || K <= 0) return 0;
@@ -92,6 +93,8 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
   TLQ_CHECK_DIMS("tlq_gemm_w4a16_ws");
   TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_w4a16_ws: in_dtype must be float16 or bfloat16 (got %d)",
               in_dtype);
+  TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32,
+              "tlq_gemm_w4a16_ws: out_dtype must be float16, bfloat16 or float32 (got %d)", out_dtype);
   if (M == 0 || N == 0) return 0;
   TLQ_REQUIRE(K > 0 && K % 64 == 0, "tlq_gemm_w4a16_ws: K=%lld must be a positive multiple of 64", (long long)K);
   TLQ_REQUIRE(group > 0 && K % group == 0 && group % 32 == 0,

@@ -159,7 +159,7 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
     zeros: None (no zero point), a number (one zero point for the whole matrix) or "tensor"
     (a [N,K/group_size] in_dtype input follows).  C [M,N] out_dtype, fp32 accumulate.
     algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "skinny" (M <= 64) | "mfma" (LDS-staged MFMA kernel)
-    | "two_pass" (dequantise into a workspace, then the plain GEMM: what "auto" does from M = 2048 up; the kernel
+    | "two_pass" (dequantise into a workspace, then the plain GEMM: what "auto" does from M = 256 up; the kernel
     object then keeps a [N, K] workspace in the activation type on the device of its first call).
     tile: rows of activations per work-group of the MFMA kernel (16, 32, 64, 128, 256; 0 = chosen by the
     library); gemv_tuning = (rows_per_wave, waves, blocks_per_cu, depth) and skinny_tuning = (waves,
@@ -200,7 +200,11 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
         C = t[i]
         lib = _abi.load()
         ws = None
-        ws_bytes = N * K * 2 if algo == "two_pass" else (lib.tlq_w4a16_workspace_bytes(M, N, K) if algo == "auto" else 0)
+        ws_bytes = 0
+        if algo in ("auto", "two_pass"):
+            ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
+            if algo == "two_pass":
+                ws_bytes = max(ws_bytes, N * K * 2)
         if ws_bytes:
             ws = workspace.get(A.device)
             if ws is None:
