@@ -110,8 +110,9 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
                    void* stream);
 
 /* The same operator with a caller-owned workspace of tlq_w4a16_workspace_bytes(M, N, K) bytes (0 when a
- * workspace would not be used).  With it, problems from M = 256 up take two passes -- tlq_dequant_w4 into
- * the workspace, then tlq_gemm_f16 on it -- which is the structure of the reference's own wrapper
+ * workspace would not be used).  With it, 16 < M <= 512 (and up to 2048 while there are few output tiles) runs the
+ * tile kernel over slices of K whose fp32 partial sums live in the workspace and are added in slice order, and larger
+ * problems take two passes -- tlq_dequant_w4 into the workspace, then tlq_gemm_f16 on it -- which is the structure of the reference's own wrapper
  * (example_dequant_gemm_fine_grained.py:176-223 unpacks, then calls fp16_gemm) and is faster than converting
  * the weights again in every row block of the fused kernel.  The workspace holds nothing between calls.
  * algo: as tlq_gemm_w4a16, or TLQ_ALGO_TWO_PASS to force the two passes (workspace required). */
@@ -203,6 +204,7 @@ void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4 (negat
 void tlq_tune_gemv_unroll(int blocks_per_cu);               /* resident blocks per CU the GEMV grid is sized for */
 void tlq_tune_gemv_depth(int steps_in_flight);               /* load steps (1 KB per row each) a GEMV wavefront keeps in flight */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
+void tlq_tune_w4a16_split(int slices);                       /* K slices of the tile kernel, 16 < M < 256 with a workspace */
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,
                                                                +10 = never stage through LDS, +20 = stage whenever possible */
 void tlq_tune_i8_tile(int block_m);                         /* 32|128|256 */

@@ -176,7 +176,7 @@ def test_gemv_batched_entry_point(M, N, K, group):
 @pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
 @pytest.mark.parametrize("M,N,K,group,zeros_kind,algo", [
     (2048, 256, 512, 128, "int", "auto"), (100, 136, 256, 64, "frac", "two_pass"), (2304, 72, 192, 32, None, "auto"),
-    (16, 64, 128, 128, "scalar8", "two_pass"), (256, 264, 8192, 128, "int", "auto"), (300, 72, 14336, 64, "frac", "auto"),
+    (16, 64, 128, 128, "scalar8", "two_pass"), (256, 264, 8192, 128, "int", "two_pass"), (2100, 72, 14336, 64, "frac", "auto"),
 ])
 def test_w4a16_two_pass_with_workspace(ops, in_dtype, M, N, K, group, zeros_kind, algo):
     """Dequantise into the kernel object's workspace, then the plain GEMM: what auto does from M = 256 up."""
@@ -189,13 +189,35 @@ def test_w4a16_two_pass_with_workspace(ops, in_dtype, M, N, K, group, zeros_kind
         check_float_output(got, want, f"two-pass {in_dtype}->{out_dtype}")
 
 
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K,group,zeros_kind", [
+    (64, 4096, 14336, 128, "int"), (17, 136, 2048, 64, "frac"), (255, 520, 4096, 32, None), (48, 14336, 4096, 128, "scalar8"),
+    (130, 64, 8192, 1024, "int"), (32, 4, 1024, 128, "int"), (512, 264, 8192, 128, "int"), (1500, 72, 14336, 64, "frac"),
+])
+def test_w4a16_mid_m_split_k_with_workspace(ops, in_dtype, M, N, K, group, zeros_kind):
+    """Small and middle M with a workspace: the tile kernel over K slices, fp32 partial sums added in slice order."""
+    from tilelang_ascend_amd import _abi
+
+    assert _abi.load().tlq_w4a16_workspace_bytes(M, N, K) > 0
+    dt = DT[in_dtype]
+    A = torch.randn(M, K, generator=gen(70)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=71)
+    want = w4a16_reference(A, Wp, s, z, group)
+    for out_dtype in ("float32", in_dtype):
+        got = _run_w4a16(ops, A, Wp, s, z, group, out_dtype, "auto", in_dtype)
+        check_float_output(got, want, f"mid-M split-K {in_dtype}->{out_dtype}")
+        again = _run_w4a16(ops, A, Wp, s, z, group, out_dtype, "auto", in_dtype)
+        assert torch.equal(got, again), "slice order must make the result reproducible"
+
+
 def test_w4a16_workspace_entry_point_rules():
     from tilelang_ascend_amd import _abi
 
     lib, P = _abi.load(), _abi.ptr
-    assert lib.tlq_w4a16_workspace_bytes(2048, 256, 512) == 256 * 512 * 2
-    assert lib.tlq_w4a16_workspace_bytes(255, 256, 512) == 0
-    assert lib.tlq_w4a16_workspace_bytes(256, 264, 8192) == 264 * 8192 * 2
+    assert lib.tlq_w4a16_workspace_bytes(2048, 256, 512) == 256 * 512 * 2       # two passes: the dequantised matrix
+    assert lib.tlq_w4a16_workspace_bytes(255, 256, 512) == 0                     # K too short to cut, M below the two passes
+    assert lib.tlq_w4a16_workspace_bytes(16, 4096, 4096) == 0                    # decode sizes use no workspace
+    assert lib.tlq_w4a16_workspace_bytes(64, 4096, 14336) == 16 * 64 * 4096 * 4  # 16 K slices of fp32 partial sums
     M, N, K, g = 64, 128, 256, 128
     A = torch.randn(M, K, generator=gen(62)).half()
     Wp, s, z = make_w4(N, K, g, torch.float16, "int", seed=63)

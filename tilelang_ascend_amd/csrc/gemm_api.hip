@@ -7,6 +7,10 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
                int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
+int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group);
+int gemm_w4a16_mfma_splitk(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M,
+                           int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype,
+                           int64_t split, float* partial, hipStream_t st);
 int gemm_w4a16_skinny(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                       int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
@@ -73,8 +77,11 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
 static const int64_t kTwoPassMinM = 256;
 
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  if (M < kTwoPassMinM || N <= 0 || K <= 0) return 0;
-  return N * K * 2;
+  if (N <= 0 || K <= 0) return 0;
+  // small and middle M: fp32 partial sums of the K slices (sized for the smallest group, which allows the most slices)
+  const int64_t split = w4a16_mid_split(M, N, K, 32);
+  if (split > 1) return split * M * N * 4;
+  return M >= kTwoPassMinM ? N * K * 2 : 0;
 }
 
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
@@ -86,7 +93,20 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
   if (algo == TLQ_ALGO_TWO_PASS)
     TLQ_REQUIRE(have, "tlq_gemm_w4a16_ws: the two-pass path needs a 16-byte aligned workspace of %lld bytes (got %lld)",
                 (long long)need, (long long)workspace_bytes);
-  const bool two_pass = algo == TLQ_ALGO_TWO_PASS || (algo == TLQ_ALGO_AUTO && have && M >= kTwoPassMinM && N % 8 == 0);
+  const bool split_region = w4a16_mid_split(M, N, K, group > 0 ? group : 32) > 1;
+  const bool two_pass = algo == TLQ_ALGO_TWO_PASS ||
+                        (algo == TLQ_ALGO_AUTO && have && M >= kTwoPassMinM && N % 8 == 0 && !split_region);
+  if (!two_pass && (algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_MFMA) && M > 16 && workspace && aligned16(workspace) &&
+      K > 0 && K % 64 == 0 && group > 0 && K % group == 0 && group % 32 == 0 && A && w_packed && C && aligned16(A) &&
+      aligned16(w_packed) && aligned16(C) && N % 4 == 0 && (M * N) % 4 == 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim &&
+      (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) && (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) &&
+      fits32(M, K * 2) && fits32(N, K / 2) && ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0) {
+    // small and middle M: the tile kernel over K slices, partial sums in the workspace, one pass to add them up
+    const int64_t split = w4a16_mid_split(M, N, K, group);
+    if (split > 1 && workspace_bytes >= split * M * N * 4)
+      return gemm_w4a16_mfma_splitk(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, split,
+                                    (float*)workspace, (hipStream_t)stream);
+  }
   if (!two_pass)
     return tlq_gemm_w4a16(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype,
                           algo == TLQ_ALGO_TWO_PASS ? TLQ_ALGO_AUTO : algo, stream);

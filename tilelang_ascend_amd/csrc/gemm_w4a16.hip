@@ -111,6 +111,8 @@ struct W4Loader {
     int group_shift;    // log2(group); group is a power of two here
     float zero_scalar;
     int has_scales, has_zeros;
+    int64_t slice_bytes;  // split-K: packed bytes of one K slice within a row (0 without a split) ...
+    int slice_groups;     // ... and its number of quantisation groups; slice z is the kernel's "batch" z
   };
   struct Regs {
     uint4_t v[PASSES];
@@ -127,12 +129,13 @@ struct W4Loader {
   T one, zs;
   NibbleMagic mg;
 
-  __device__ __forceinline__ W4Loader(const Params& p, int /*batch*/, int row0, int rows_total, int tid)
-      : base(p.wp + (int64_t)row0 * p.row_bytes), group_shift(p.group_shift), has_s(p.has_scales != 0),
-        has_z(p.has_zeros != 0), one(from_float<T>(1.0f)), zs(from_float<T>(p.zero_scalar)), mg(make_nibble_magic()) {
+  __device__ __forceinline__ W4Loader(const Params& p, int batch, int row0, int rows_total, int tid)
+      : base(p.wp + (int64_t)row0 * p.row_bytes + batch * p.slice_bytes), group_shift(p.group_shift),
+        has_s(p.has_scales != 0), has_z(p.has_zeros != 0), one(from_float<T>(1.0f)), zs(from_float<T>(p.zero_scalar)),
+        mg(make_nibble_magic()) {
     const int rows_valid = rows_total - row0;
-    sbase = p.scales + (has_s ? (int64_t)row0 * p.groups : 0);
-    zbase = p.zeros + (has_z ? (int64_t)row0 * p.groups : 0);
+    sbase = p.scales + (has_s ? (int64_t)row0 * p.groups + batch * p.slice_groups : 0);
+    zbase = p.zeros + (has_z ? (int64_t)row0 * p.groups + batch * p.slice_groups : 0);
     const int half = tid & 1;
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
@@ -206,6 +209,8 @@ struct W4Args {
   float zero_scalar;
   int out_dtype;
   hipStream_t st;
+  int64_t split = 1;         // K slices handled by different work-groups (the MFMA tile kernel only)
+  float* partial = nullptr;  // [split][M][N] fp32 partial sums when split > 1
 };
 
 template <typename T, bool FOLD, int ROWS, int NT>
@@ -221,7 +226,9 @@ static typename W4Loader<T, FOLD, ROWS, NT>::Params w4_params(const W4Args& a) {
           shift,
           a.zero_scalar,
           a.scales ? 1 : 0,
-          a.zeros ? 1 : 0};
+          a.zeros ? 1 : 0,
+          a.split > 1 ? a.K / a.split / 2 : 0,
+          a.split > 1 ? (int)(a.K / a.split / a.group) : 0};
 }
 
 template <typename T, bool FOLD, int BM, int BN, int WM, int WN>
@@ -231,8 +238,16 @@ static int run_w4a16(const W4Args& a) {
   constexpr bool DIRECT = BM % 8 == 0 && (BM / 8) % (NT / 64) == 0;
   typedef typename std::conditional<DIRECT, RowLoaderDirect<DIRECT ? BM : 8 * (NT / 64), NT>, RowLoader<BM, NT>>::type AL;
   typedef W4Loader<T, FOLD, BN, NT> WL;
-  typename AL::Params pa{(const uint8_t*)a.A, a.K * 2, 0, a.K * 2};
   auto pw = w4_params<T, FOLD, BN, NT>(a);
+  if (a.split > 1) {
+    // slice z of K is "batch" z of the loaders; every slice writes its own fp32 partial matrix
+    const int64_t ks = a.K / a.split;
+    typename AL::Params pa{(const uint8_t*)a.A, a.K * 2, ks * 2, ks * 2};
+    EpiFloat::Params pe{a.partial, a.N, a.M * a.N, TLQ_F32};
+    return launch_gemm<typename MmaOf<T>::type, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, a.split, a.M, a.N, ks * 2, a.st,
+                                                                                 "tlq_gemm_w4a16(mfma, split K)");
+  }
+  typename AL::Params pa{(const uint8_t*)a.A, a.K * 2, 0, a.K * 2};
   EpiFloat::Params pe{a.C, a.N, 0, a.out_dtype};
   return launch_gemm<typename MmaOf<T>::type, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, a.M, a.N, a.K * 2, a.st,
                                                                                "tlq_gemm_w4a16(mfma)");
@@ -252,8 +267,8 @@ static int dispatch_w4a16(const W4Args& a) {
       tile = 32;
     else if (M <= 64)
       tile = 64;
-    else if (M <= 128 || ceil_div(M, 256) * ceil_div(N, 256) < 128)
-      tile = 128;
+    else if (M <= 128 || (a.split <= 1 && ceil_div(M, 256) * ceil_div(N, 256) < 128))
+      tile = 128;  // few large tiles: smaller ones fill more CUs, unless K is being cut for that purpose
     else
       tile = 256;
   }
@@ -737,6 +752,66 @@ int gemm_w4a16_skinny(const void* A, const void* Wp, const void* scales, const v
   return fold ? dispatch_skinny<bf16_t, true>(a) : dispatch_skinny<bf16_t, false>(a);
 }
 
+// C[i] = round(sum over the K slices of partial[z][i]), slices added in index order (so the result does not
+// depend on which work-group finished first)
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4_t* __restrict__ partial, void* __restrict__ C,
+                                                           int64_t n4, int split, int out_dtype) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+    float4_t v = partial[i];
+    for (int z = 1; z < split; ++z) v += partial[(int64_t)z * n4 + i];
+    if (out_dtype == TLQ_F16) {
+      half_t h[4] = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+      ((uint2_t*)C)[i] = bitcast<uint2_t>(h);
+    } else if (out_dtype == TLQ_BF16) {
+      ((uint2_t*)C)[i] = uint2_t{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+    } else {
+      ((float4_t*)C)[i] = v;
+    }
+  }
+}
+
+// K slices for the tile kernel at small M, where the output tiles alone leave most of the chip idle and a
+// work-group's run of stages is latency bound: aim at one to two work-groups per CU (measured best on the
+// MLP shapes), slices of at least 512 values that are whole stages and whole quantisation groups.  1 = no split.
+static int g_w4a16_split = 0;  // forced number of K slices for tuning runs (0 = automatic)
+
+int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group) {
+  // Where cutting K pays (measured against the two passes on the MLP shapes): up to M = 512 always, up to
+  // M = 2048 while the 256 x 256 output tiles would fill at most a quarter of the chip.
+  const bool region = M > 16 && (M <= 512 || (M < 2048 && ceil_div(M, (int64_t)256) * ceil_div(N, (int64_t)256) <= 64));
+  if (!region || (group & (group - 1)) != 0 || N % 4 != 0) return 1;
+  if (g_w4a16_split > 0) {
+    const int64_t s = g_w4a16_split, unit0 = group > 64 ? group : 64;
+    return (s <= 16 && K % s == 0 && (K / s) % unit0 == 0) ? s : 1;
+  }
+  const int64_t bm = M <= 32 ? 32 : (M <= 64 ? 64 : (M <= 128 ? 128 : 256)), bn = (M <= 32 || (M > 64 && M <= 128)) ? 128 : 256;
+  const int64_t tiles = ceil_div(M, bm) * ceil_div(N, bn);
+  const int64_t want = ceil_div((int64_t)(bm == 256 ? 256 : 512), tiles);  // one 256-row work-group fills a CU, two smaller ones do
+  const int64_t unit = group > 64 ? group : 64;
+  for (int64_t s = want < 16 ? want : 16; s >= 2; --s)
+    if (K % s == 0 && (K / s) % unit == 0 && K / s >= 512) return s;
+  return 1;
+}
+
+int gemm_w4a16_mfma_splitk(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M,
+                           int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype,
+                           int64_t split, float* partial, hipStream_t st) {
+  const bool fold = zeros == nullptr && zero_scalar == (float)(int)zero_scalar && zero_scalar >= -256.0f &&
+                    zero_scalar <= 256.0f;
+  W4Args a{A, Wp, scales, zeros, C, M, N, K, group, zero_scalar, out_dtype, st};
+  a.split = split;
+  a.partial = partial;
+  int rc;
+  if (in_dtype == TLQ_F16)
+    rc = fold ? dispatch_w4a16<half_t, true>(a) : dispatch_w4a16<half_t, false>(a);
+  else
+    rc = fold ? dispatch_w4a16<bf16_t, true>(a) : dispatch_w4a16<bf16_t, false>(a);
+  if (rc) return rc;
+  const int64_t n4 = M * N / 4, want = ceil_div(n4, (int64_t)256);
+  splitk_reduce_kernel<<<(int)(want > 65536 ? 65536 : want), 256, 0, st>>>((const float4_t*)partial, C, n4, (int)split, out_dtype);
+  return check_launch("tlq_gemm_w4a16(split-K reduce)") ? 0 : 1;
+}
+
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st) {
   if ((group & (group - 1)) != 0) {
@@ -757,6 +832,9 @@ extern "C" {
 // Tuning hook used by the benchmark sweeps: forces the activation-tile height (16, 32, 64,
 // 128, 256) of the W4A16 MFMA kernel; 0 restores the automatic choice.
 void tlq_tune_w4a16_tile(int block_m) { tlq::g_w4a16_tile = block_m; }
+// K slices of the tile kernel for 16 < M < 256 when a workspace is given (2..16, must divide K into whole
+// stages and groups); 0 restores the automatic choice.
+void tlq_tune_w4a16_split(int slices) { tlq::g_w4a16_split = slices < 0 ? 0 : slices; }
 // Wavefronts per work-group (1..16, the in-group split of K) and 16-row weight tiles per wavefront
 // (1 | 2) of the skinny W4A16 kernel; 0 restores the automatic choice.
 void tlq_tune_w4a16_skinny(int waves, int row_tiles) {
