@@ -311,13 +311,15 @@ def test_gemm_w4a16_config1_reference_loops(ops):
 
 @pytest.mark.parametrize("M", [1024, 4096])
 def test_gemm_w4a16_prefill_bf16(ops, M):
-    """bf16 prefill shape (N=K=4096, group 128, zero = 8, bf16 out)."""
+    """bf16 prefill shape (N=K=4096, group 128, zero = 8, bf16 out): the fused kernel, and what the automatic
+    choice does with a workspace (K slices at M = 1024, two passes at M = 4096)."""
     N = K = 4096
     A = torch.randn(M, K, generator=gen(14)).to(torch.bfloat16)
     Wp, s, _ = make_w4(N, K, 128, torch.bfloat16, None, seed=15)
     want = w4a16_reference(A, Wp, s, 8, 128)
-    got = _run_w4a16(ops, A, Wp, s, 8, 128, "bfloat16", "mfma", "bfloat16")
-    check_float_output(got, want, f"prefill bf16 M={M}")
+    for algo in ("mfma", "auto"):
+        got = _run_w4a16(ops, A, Wp, s, 8, 128, "bfloat16", algo, "bfloat16")
+        check_float_output(got, want, f"prefill bf16 M={M} {algo}")
 
 
 @pytest.mark.parametrize("M,N,K,group", [(16, 14336, 4096, 64), (64, 4096, 14336, 128), (256, 14336, 4096, 128)])
