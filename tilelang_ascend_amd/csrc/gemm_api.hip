@@ -24,6 +24,7 @@ int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const v
 int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
                   hipStream_t st);
 
+int g_gemm_band_rows = 0;
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // the tile loaders address one matrix with 32-bit byte offsets
 static bool fits32(int64_t rows, int64_t row_bytes) { return rows * row_bytes < ((int64_t)1 << 32); }
@@ -37,6 +38,8 @@ using namespace tlq;
               (long long)M, (long long)N, (long long)K)
 
 extern "C" {
+
+void tlq_tune_gemm_band(int tile_rows) { tlq::g_gemm_band_rows = tile_rows < 0 ? 0 : tile_rows; }
 
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,

@@ -471,13 +471,16 @@ struct EpiRescale {
 };
 
 // Work-group -> tile.  Consecutive hardware ids are dealt round-robin to the 8 XCDs; give
-// every XCD a contiguous range of logical tiles so that tiles sharing an activation panel
-// also share an L2.
+// every XCD a contiguous range of logical tiles, and order the tiles of a matrix in bands of four
+// tile rows walked column by column, so that the 32 tiles an XCD runs at a time form a 4 x 8
+// block: they share four activation panels and eight weight panels in that XCD's L2 instead of
+// two and sixteen (a third less traffic past the L2 on square problems).  The band height is a launch
+// parameter.
 struct TileCoord {
   int batch, m0, n0;
 };
 template <int BM, int BN>
-__device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n) {
+__device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n, int GM) {
   const int total = gridDim.x;
   int lid = blockIdx.x;
   if ((total & 7) == 0) lid = (lid & 7) * (total >> 3) + (lid >> 3);
@@ -485,8 +488,11 @@ __device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n) {
   TileCoord t;
   t.batch = lid / per_batch;
   const int rem = lid - t.batch * per_batch;
-  t.m0 = (rem / tiles_n) * BM;
-  t.n0 = (rem % tiles_n) * BN;
+  const int band = rem / (GM * tiles_n);
+  const int r = rem - band * (GM * tiles_n);
+  const int rows = tiles_m - band * GM < GM ? tiles_m - band * GM : GM;  // the last band may be lower
+  t.m0 = (band * GM + r % rows) * BM;
+  t.n0 = (r / rows) * BN;
   return t;
 }
 
@@ -494,7 +500,7 @@ __device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n) {
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma_kernel(
     typename AL::Params pa, typename WL::Params pw, typename Epi::Params pe, int M, int N, int KT, int k_tail,
-    int tiles_m, int tiles_n) {
+    int tiles_m, int tiles_n, int band_rows) {
   constexpr int TM = BM / WM / 16;  // 16-row activation tiles per wave
   constexpr int TN = BN / WN / 16;  // 16-row weight tiles per wave
   constexpr int A_TILE = BM * kStageBytes, W_TILE = BN * kStageBytes;
@@ -509,7 +515,7 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   const int q = lane >> 4;
   const int wave_m0 = (wave % WM) * (BM / WM);
   const int wave_n0 = (wave / WM) * (BN / WN);
-  const TileCoord tc = tile_of_block<BM, BN>(tiles_m, tiles_n);
+  const TileCoord tc = tile_of_block<BM, BN>(tiles_m, tiles_n, band_rows);
   const int m0 = tc.m0, n0 = tc.n0, batch = tc.batch;
 
   AL al(pa, batch, m0, M, tid);
@@ -635,9 +641,13 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
 }
 
 // Host-side launcher: sets the dynamic LDS size and launches one work-group per tile.
+// tile rows per band of the work-group -> tile order, for tuning runs (0 = each launcher's own choice: measured best
+// were 2 for the int8 kernels, 4 for the plain 16-bit GEMM and 8 for the fused W4A16 kernel; 1 = plain row-major)
+extern int g_gemm_band_rows;
+
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,
-                int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what) {
+                int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what, int band_rows = 4) {
   auto kern = gemm_mfma_kernel<Mma, AL, WL, Epi, BM, BN, WM, WN>;
   constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes;
   static bool attr_set = false;  // per instantiation; idempotent, so a race only repeats the call
@@ -659,7 +669,7 @@ int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, co
   const int KT = (int)ceil_div(k_bytes, kStageBytes);
   const int k_tail = (k_bytes % kStageBytes) != 0;
   kern<<<(unsigned)blocks, WM * WN * 64, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, KT, k_tail, (int)tiles_m,
-                                                          (int)tiles_n);
+                                                          (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows);
   return check_launch(what) ? 0 : 1;
 }
 

@@ -104,7 +104,7 @@ static int run_i8(const void* A, const typename WL::Params& pw, const typename E
   constexpr int NT = WM * WN * 64;
   typedef RowLoaderDirect<BM, NT> AL;  // activations travel global -> LDS without passing through registers
   typename AL::Params pa{(const uint8_t*)A, K, M * K, K};
-  return launch_gemm<MmaI8, AL, WL, Epi, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K, st, what);
+  return launch_gemm<MmaI8, AL, WL, Epi, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K, st, what, 2);
 }
 
 static int g_i8_tile = 0;

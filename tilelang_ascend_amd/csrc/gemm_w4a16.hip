@@ -245,12 +245,12 @@ static int run_w4a16(const W4Args& a) {
     typename AL::Params pa{(const uint8_t*)a.A, a.K * 2, ks * 2, ks * 2};
     EpiFloat::Params pe{a.partial, a.N, a.M * a.N, TLQ_F32};
     return launch_gemm<typename MmaOf<T>::type, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, a.split, a.M, a.N, ks * 2, a.st,
-                                                                                 "tlq_gemm_w4a16(mfma, split K)");
+                                                                                 "tlq_gemm_w4a16(mfma, split K)", 8);
   }
   typename AL::Params pa{(const uint8_t*)a.A, a.K * 2, 0, a.K * 2};
   EpiFloat::Params pe{a.C, a.N, 0, a.out_dtype};
   return launch_gemm<typename MmaOf<T>::type, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, a.M, a.N, a.K * 2, a.st,
-                                                                               "tlq_gemm_w4a16(mfma)");
+                                                                               "tlq_gemm_w4a16(mfma)", 8);
 }
 
 // tile override for tuning runs (0 = automatic)
