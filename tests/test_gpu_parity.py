@@ -540,10 +540,13 @@ def test_skinny_tunings_and_one_hot(ops, waves, row_tiles):
     assert_bit_equal(got, W[:, cols].T.contiguous(), f"skinny one-hot waves={waves} rt={row_tiles}")
 
 
-def test_auto_picks_a_kernel_for_every_m(ops):
-    N, K, group = 256, 1024, 128
-    Wp, s, z = make_w4(N, K, group, torch.float16, "int", seed=43)
-    for M in (1, 4, 5, 16, 64, 65, 200):
-        A = torch.randn(M, K, generator=gen(44)).to(torch.float16)
-        got = _run_w4a16(ops, A, Wp, s, z, group, "float16", "auto", "float16")
-        check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"auto M={M}")
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("N,K,group", [(256, 1024, 128), (48, 8192, 64), (40, 448, 64)])
+def test_auto_picks_a_kernel_for_every_m(ops, in_dtype, N, K, group):
+    """The automatic choice (GEMV, skinny or tile kernel by M, K and type; K = 448 admits no skinny kernel)."""
+    dt = DT[in_dtype]
+    Wp, s, z = make_w4(N, K, group, dt, "int", seed=43)
+    for M in (1, 2, 3, 4, 5, 16, 64, 65, 200):
+        A = torch.randn(M, K, generator=gen(44)).to(dt)
+        got = _run_w4a16(ops, A, Wp, s, z, group, in_dtype, "auto", in_dtype)
+        check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"auto {in_dtype} M={M} K={K}")
