@@ -128,10 +128,13 @@ def test_gemv_shapes(ops, in_dtype, M, N, K, group, zeros_kind):
 @pytest.mark.parametrize("N,K,group,zeros_kind", [
     (11008, 4096, 128, "int"), (1000, 4096, 32, "int"), (250, 2048, 128, "frac"), (77, 1088, 64, "int"),
     (5, 64, 32, None), (4097, 1024, 1024, "scalar8"), (333, 3136, 64, "frac"), (64, 4096, 4096, "int"),
+    # long rows: 3 .. 8 chunks per lane, work-groups of 8 wavefronts
+    (4096, 11008, 128, "int"), (520, 14336, 128, "frac"), (300, 6144, 64, "int"), (130, 8192, 32, "scalar8"),
+    (77, 16384, 256, "int"), (1000, 4160, 64, "int"), (64, 9984, 128, None),
 ])
 @pytest.mark.parametrize("waves,blocks_per_cu,depth", [(0, 0, 0), (16, 1, 3), (5, 3, 2), (2, 8, 6), (16, 2, 1)])
 def test_gemv_register_resident_kernel(ops, N, K, group, zeros_kind, waves, blocks_per_cu, depth):
-    """M = 1, K <= 4096: the kernel that keeps the activations in registers and stages the scales and
+    """M = 1, K <= 16384: the kernel that keeps the activations in registers and stages the scales and
     zero points of a work-group's rows in LDS, over its grid shapes and queue depths."""
     from tilelang_ascend_amd import _abi
 

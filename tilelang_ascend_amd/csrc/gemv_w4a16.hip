@@ -361,8 +361,10 @@ __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __
 // first D are requested before anything else, the staging loads right behind them.  The loop body
 // is free of branches (rows past the end are clamped and their results dropped): the compiler then
 // keeps exact counts of the loads in flight instead of draining them at every control-flow merge.
-template <int ITERS, int D>
-__global__ __launch_bounds__(1024) void gemv_w4a16_f16_rows_kernel(const half_t* __restrict__ A,
+// Long rows (ITERS > 2) keep more activations per lane than a 16-wavefront work-group has registers for: those
+// instances are built for work-groups of 8 wavefronts (MAXT = 512 threads, 256 registers per lane).
+template <int ITERS, int D, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_w4a16_f16_rows_kernel(const half_t* __restrict__ A,
                                                                   const uint8_t* __restrict__ Wp,
                                                                   const half_t* __restrict__ scales,
                                                                   const half_t* __restrict__ zeros,
@@ -630,7 +632,7 @@ static int launch_gemv_f16(const void* A, const void* Wp, const void* scales, co
 
 // rows kernel: work-groups of `waves_per_block` wavefronts, each owning a contiguous range of rows whose
 // scales and zero points fit its LDS; at least `blocks_per_cu` work-groups per CU when there are rows enough
-template <int ITERS, int D>
+template <int ITERS, int D, int MAXT>
 static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int batch,
                             int N, int K, int group_shift, float zero_scalar, int out_dtype, int waves_per_block,
                             int blocks_per_cu, hipStream_t st) {
@@ -644,7 +646,7 @@ static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, c
   rpb = (rpb + 3) & ~3;  // keeps the zero-point block of LDS 16-byte aligned for any group count
   blocks = (int)ceil_div(N, rpb);
   const size_t lds = (size_t)(K / 32) * 72 + (size_t)rpb * groups * 4;
-  gemv_w4a16_f16_rows_kernel<ITERS, D><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
+  gemv_w4a16_f16_rows_kernel<ITERS, D, MAXT><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
       (const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C, N, K, group_shift,
       zero_scalar, out_dtype, rpb, waves_per_block);
   return 0;
@@ -665,26 +667,45 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     const int R = g_gemv_rows > 0 ? g_gemv_rows : (streaming ? 2 : 1);
     const int bpc = g_gemv_unroll ? g_gemv_unroll : (streaming ? 64 : 8);  // grid size cap, blocks per CU
     const int depth_req = g_gemv_depth;
-    if (M == 1 && K <= 4096 && g_gemv_rows >= 0) {
+    if (M == 1 && K <= 16384 && g_gemv_rows >= 0) {
       const int bpc_rows = g_gemv_unroll ? g_gemv_unroll : 1;
+      const bool long_rows = K > 4096;  // 8 wavefronts per work-group (see the kernel)
       int wpb_rows = g_gemv_waves16 ? g_gemv_waves16 : 16;
+      if (long_rows && wpb_rows > 8) wpb_rows = 8;
       if (wpb_rows * 64 < K / 32) wpb_rows = (int)ceil_div(K / 32, (int64_t)64);  // one staging thread per chunk
       // one problem of a few tens of MB: one row in flight per wavefront (deeper queues delay the staging
       // loads behind the weights and measured slower); many problems per launch stream with two
       const int d = depth_req ? depth_req : (batch * N * (K / 2) > ((int64_t)64 << 20) ? 2 : 1);
-#define TLQ_ROWS_CASE(IT, DD)                                                                                      \
-  launch_gemv_rows<IT, DD>(A, Wp, scales, zeros, C, (int)batch, (int)N, (int)K, shift, zero_scalar, out_dtype,      \
-                           wpb_rows, bpc_rows, st)
+#define TLQ_ROWS_CASE(IT, DD, MAXT)                                                                                \
+  launch_gemv_rows<IT, DD, MAXT>(A, Wp, scales, zeros, C, (int)batch, (int)N, (int)K, shift, zero_scalar, out_dtype, \
+                                 wpb_rows, bpc_rows, st)
       if (K <= 2048) {
-        if (d <= 2) TLQ_ROWS_CASE(1, 2);
-        else if (d <= 4) TLQ_ROWS_CASE(1, 4);
-        else TLQ_ROWS_CASE(1, 8);
+        if (d <= 2) TLQ_ROWS_CASE(1, 2, 1024);
+        else if (d <= 4) TLQ_ROWS_CASE(1, 4, 1024);
+        else TLQ_ROWS_CASE(1, 8, 1024);
+      } else if (K <= 4096) {
+        if (d <= 1) TLQ_ROWS_CASE(2, 1, 1024);
+        else if (d == 2) TLQ_ROWS_CASE(2, 2, 1024);
+        else if (d == 3) TLQ_ROWS_CASE(2, 3, 1024);
+        else if (d == 4) TLQ_ROWS_CASE(2, 4, 1024);
+        else TLQ_ROWS_CASE(2, 6, 1024);
       } else {
-        if (d <= 1) TLQ_ROWS_CASE(2, 1);
-        else if (d == 2) TLQ_ROWS_CASE(2, 2);
-        else if (d == 3) TLQ_ROWS_CASE(2, 3);
-        else if (d == 4) TLQ_ROWS_CASE(2, 4);
-        else TLQ_ROWS_CASE(2, 6);
+        const int iters = (int)ceil_div(K, (int64_t)2048);  // 3 .. 8
+#define TLQ_LONG_CASE(IT)                    \
+  case IT:                                   \
+    if (d <= 1) TLQ_ROWS_CASE(IT, 1, 512);   \
+    else TLQ_ROWS_CASE(IT, 2, 512);          \
+    break;
+        switch (iters) {
+          TLQ_LONG_CASE(3)
+          TLQ_LONG_CASE(4)
+          TLQ_LONG_CASE(5)
+          TLQ_LONG_CASE(6)
+          TLQ_LONG_CASE(7)
+          default:
+            TLQ_LONG_CASE(8)
+        }
+#undef TLQ_LONG_CASE
       }
 #undef TLQ_ROWS_CASE
       return check_launch("tlq_gemm_w4a16(gemv)") ? 0 : 1;
