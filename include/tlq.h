@@ -104,8 +104,8 @@ int tlq_decode_i4_interleaved(const void* words, const void* scales, const void*
  * A: [M,K] in_dtype (TLQ_F16 / TLQ_BF16); C: [M,N] out_dtype (TLQ_F16 / TLQ_BF16 / TLQ_F32).
  * Requires K % 64 == 0 and group % 32 == 0 (group divides K).  The MFMA kernel additionally needs
  * N % 4 == 0 and a power-of-two group (32, 64, 128, ...); the GEMV kernel (M <= 16) takes any such group;
- * the skinny kernel (M <= 64) needs K % 128 == 0.  TLQ_ALGO_AUTO: fp16 M = 1 (and M = 2 with
- * K <= 4096) GEMV, otherwise M <= 64 skinny where its conditions hold (else GEMV up to M = 4), else MFMA. */
+ * the skinny kernel (M <= 64) needs K % 128 == 0.  TLQ_ALGO_AUTO: M = 1 GEMV (fp16; bf16 up to K = 8192; fp16 also M = 2 with
+ * K <= 4096), otherwise M <= 64 skinny where its conditions hold (else GEMV up to M = 4), else MFMA. */
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                    void* stream);

@@ -133,22 +133,25 @@ def test_gemv_shapes(ops, in_dtype, M, N, K, group, zeros_kind):
     (77, 16384, 256, "int"), (1000, 4160, 64, "int"), (64, 9984, 128, None),
 ])
 @pytest.mark.parametrize("waves,blocks_per_cu,depth", [(0, 0, 0), (16, 1, 3), (5, 3, 2), (2, 8, 6), (16, 2, 1)])
-def test_gemv_register_resident_kernel(ops, N, K, group, zeros_kind, waves, blocks_per_cu, depth):
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+def test_gemv_register_resident_kernel(ops, in_dtype, N, K, group, zeros_kind, waves, blocks_per_cu, depth):
     """M = 1, K <= 16384: the kernel that keeps the activations in registers and stages the scales and
-    zero points of a work-group's rows in LDS, over its grid shapes and queue depths."""
+    zero points of a work-group's rows in LDS, over its grid shapes and queue depths (fp16: biased dot and
+    chunk sums; bf16: element-wise dequantisation and the packed dot)."""
     from tilelang_ascend_amd import _abi
 
     lib = _abi.load()
-    A = torch.randn(1, K, generator=gen(40)).to(torch.float16)
-    Wp, s, z = make_w4(N, K, group, torch.float16, zeros_kind, seed=41)
+    dt = DT[in_dtype]
+    A = torch.randn(1, K, generator=gen(40)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=41)
     want = w4a16_reference(A, Wp, s, z, group)
     lib.tlq_tune_gemv(0, waves)
     lib.tlq_tune_gemv_unroll(blocks_per_cu)
     lib.tlq_tune_gemv_depth(depth)
     try:
-        for out_dtype in ("float16", "float32"):
-            got = _run_w4a16(ops, A, Wp, s, z, group, out_dtype, "gemv", "float16")
-            check_float_output(got, want, f"gemv rows kernel -> {out_dtype}")
+        for out_dtype in (in_dtype, "float32"):
+            got = _run_w4a16(ops, A, Wp, s, z, group, out_dtype, "gemv", in_dtype)
+            check_float_output(got, want, f"gemv rows kernel {in_dtype} -> {out_dtype}")
     finally:
         lib.tlq_tune_gemv(0, 0)
         lib.tlq_tune_gemv_unroll(0)

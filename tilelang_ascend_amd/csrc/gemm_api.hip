@@ -60,15 +60,15 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
   hipStream_t st = (hipStream_t)stream;
   if (algo == TLQ_ALGO_AUTO) {
     // The skinny kernel takes the same time for every M up to 16 (the weights bound it); the GEMV kernels grow with
-    // M.  Measured crossovers: fp16 GEMV wins at M = 1, and at M = 2 while the row fits its register-resident form's
-    // reach (K <= 4096); the bf16 GEMV dequantises element by element and loses to the skinny kernel even at M = 1.
+    // M.  Measured crossovers: fp16 GEMV wins at M = 1, and at M = 2 while K <= 4096; the bf16 GEMV dequantises
+    // element by element and wins only at M = 1 in its register-resident form, for rows of up to 8192 values.
     const bool skinny_ok = M <= 64 && K % 128 == 0 && fits32(M, K * 2) && fits32(N, K / 2);
     if (M > 4)
       algo = skinny_ok ? TLQ_ALGO_SKINNY : TLQ_ALGO_MFMA;
     else if (!skinny_ok)
       algo = TLQ_ALGO_GEMV;
     else if (in_dtype == TLQ_BF16)
-      algo = TLQ_ALGO_SKINNY;
+      algo = (M == 1 && K <= 8192 && (group & (group - 1)) == 0) ? TLQ_ALGO_GEMV : TLQ_ALGO_SKINNY;
     else
       algo = (M == 1 || (M == 2 && K <= 4096)) ? TLQ_ALGO_GEMV : TLQ_ALGO_SKINNY;
   }

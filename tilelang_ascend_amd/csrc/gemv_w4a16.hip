@@ -16,6 +16,7 @@
 // bf16 path: weights are dequantised element-wise with bfloat16 rounding after each step
 // (bf16 keeps only 8 mantissa bits, so skipping those roundings would be visible).
 #include "tlq_common.h"
+#include "expand8.h"
 
 namespace tlq {
 
@@ -177,6 +178,26 @@ __device__ __forceinline__ float chunk_term(const uint4_t& w, const ActBF16& act
       float wv = round_to_bf16(d * sf);
       acc = __builtin_fmaf(act.a[8 * j + i], wv, acc);
     }
+  }
+  return acc;
+}
+
+// the same value with the weights dequantised eight at a time (Expand8: bf16((u - z) * s), exact) and the packed
+// bf16 dot instruction; `a` holds the chunk's 32 activations in memory order
+template <bool FOLD>
+__device__ __forceinline__ float chunk_term_dot2(const uint4_t& w, const uint4_t (&a)[4], bf16_t s, bf16_t z,
+                                                 const NibbleMagic& mg) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const Expand8<bf16_t, FOLD> ex(s, z, mg);
+  const uint32_t x[4] = {w.x, w.y, w.z, w.w};
+  float acc = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint4_t e = ex(x[j]);  // (k0,k1)(k2,k3)(k4,k5)(k6,k7)
+    acc = __builtin_amdgcn_fdot2_f32_bf16(bitcast<bf16x2_t>(e.x), bitcast<bf16x2_t>(a[j].x), acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(bitcast<bf16x2_t>(e.y), bitcast<bf16x2_t>(a[j].y), acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(bitcast<bf16x2_t>(e.z), bitcast<bf16x2_t>(a[j].z), acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(bitcast<bf16x2_t>(e.w), bitcast<bf16x2_t>(a[j].w), acc, false);
   }
   return acc;
 }
@@ -363,13 +384,15 @@ __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __
 // keeps exact counts of the loads in flight instead of draining them at every control-flow merge.
 // Long rows (ITERS > 2) keep more activations per lane than a 16-wavefront work-group has registers for: those
 // instances are built for work-groups of 8 wavefronts (MAXT = 512 threads, 256 registers per lane).
-template <int ITERS, int D, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemv_w4a16_f16_rows_kernel(const half_t* __restrict__ A,
-                                                                  const uint8_t* __restrict__ Wp,
-                                                                  const half_t* __restrict__ scales,
-                                                                  const half_t* __restrict__ zeros,
-                                                                  void* __restrict__ C, int N, int K, int group_shift,
-                                                                  float zero_scalar, int out_dtype, int rows_per_block, int nwaves) {
+// fp16 multiplies the raw nibbles (unpack bias left in, corrected through the chunk sums); bf16 dequantises
+// element by element exactly as the reference does -- bf16((u - z) * s) differs from the exact product in the
+// 8th bit, more than the output tolerance allows -- and multiplies with the packed bf16 dot instruction.
+template <typename T, int ITERS, int D>
+__device__ __forceinline__ void gemv_rows_body(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
+                                               const T* __restrict__ scales, const T* __restrict__ zeros,
+                                               void* __restrict__ C, int N, int K, int group_shift, float zero_scalar,
+                                               int out_dtype, int rows_per_block, int nwaves) {
+  constexpr bool F16 = sizeof(T) == 2 && __is_same(T, half_t);
   // The first weight rows: as few instructions as possible between the start of a wavefront and its first
   // loads (everything they need sits in the first 64 bytes of the kernel arguments).
   const int lane = threadIdx.x & 63;
@@ -407,8 +430,8 @@ __global__ __launch_bounds__(MAXT) void gemv_w4a16_f16_rows_kernel(const half_t*
   const int groups = K >> group_shift;
   uint4_t* const lds_pairs = (uint4_t*)smem;                       // [4][chunks]
   float2* const lds_sums = (float2*)(smem + (size_t)chunks * 64);  // [chunks]
-  half_t* const lds_s = (half_t*)(smem + (size_t)chunks * 72);     // [rows_per_block][groups]
-  half_t* const lds_z = lds_s + rows_per_block * groups;           // [rows_per_block][groups] (16-byte aligned: see launcher)
+  T* const lds_s = (T*)(smem + (size_t)chunks * 72);               // [rows_per_block][groups]
+  T* const lds_z = lds_s + rows_per_block * groups;                // [rows_per_block][groups] (16-byte aligned: see launcher)
   {
     const int64_t b = blockIdx.y;
     const int64_t gsz = (int64_t)N * groups;
@@ -441,13 +464,18 @@ __global__ __launch_bounds__(MAXT) void gemv_w4a16_f16_rows_kernel(const half_t*
   }
 
   if (threadIdx.x < chunks) {
-    ActF16 a;
-    permute_act(a, araw);
+    if constexpr (F16) {
+      ActF16 a;
+      permute_act(a, araw);
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      lds_pairs[j * chunks + tchunk] = uint4_t{bitcast<uint32_t>(a.a[4 * j + 0]), bitcast<uint32_t>(a.a[4 * j + 1]),
-                                               bitcast<uint32_t>(a.a[4 * j + 2]), bitcast<uint32_t>(a.a[4 * j + 3])};
-    lds_sums[tchunk] = make_float2(a.sum, a.bsum);
+      for (int j = 0; j < 4; ++j)
+        lds_pairs[j * chunks + tchunk] = uint4_t{bitcast<uint32_t>(a.a[4 * j + 0]), bitcast<uint32_t>(a.a[4 * j + 1]),
+                                                 bitcast<uint32_t>(a.a[4 * j + 2]), bitcast<uint32_t>(a.a[4 * j + 3])};
+      lds_sums[tchunk] = make_float2(a.sum, a.bsum);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) lds_pairs[j * chunks + tchunk] = araw[j];  // natural order, no sums needed
+    }
   }
   if (wide) {
     if (t8 < n_sz) {
@@ -465,24 +493,30 @@ __global__ __launch_bounds__(MAXT) void gemv_w4a16_f16_rows_kernel(const half_t*
     }
   }
   __syncthreads();
-  ActF16 act[ITERS];
+  ActF16 act[F16 ? ITERS : 1];      // fp16: pairs in unpack order and the chunk sums
+  uint4_t actn[F16 ? 1 : ITERS][4];  // bf16: the 32 activations of a chunk as loaded
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
+    if constexpr (F16) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint4_t v = lds_pairs[j * chunks + cc[it]];
-      act[it].a[4 * j + 0] = bitcast<half2_t>(v.x);
-      act[it].a[4 * j + 1] = bitcast<half2_t>(v.y);
-      act[it].a[4 * j + 2] = bitcast<half2_t>(v.z);
-      act[it].a[4 * j + 3] = bitcast<half2_t>(v.w);
+      for (int j = 0; j < 4; ++j) {
+        const uint4_t v = lds_pairs[j * chunks + cc[it]];
+        act[it].a[4 * j + 0] = bitcast<half2_t>(v.x);
+        act[it].a[4 * j + 1] = bitcast<half2_t>(v.y);
+        act[it].a[4 * j + 2] = bitcast<half2_t>(v.z);
+        act[it].a[4 * j + 3] = bitcast<half2_t>(v.w);
+      }
+      const float2 sb = lds_sums[cc[it]];
+      act[it].sum = sb.x;
+      act[it].bsum = sb.y;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) actn[it][j] = lds_pairs[j * chunks + cc[it]];
     }
-    const float2 sb = lds_sums[cc[it]];
-    act[it].sum = sb.x;
-    act[it].bsum = sb.y;
   }
 
   const NibbleMagic mg = make_nibble_magic();
-  const half_t one = (half_t)1.0f, zs = (half_t)zero_scalar;
+  const T one = from_float<T>(1.0f), zs = from_float<T>(zero_scalar);
   const int my_rows = r0 + wave < r1 ? (r1 - r0 - wave + nwaves - 1) / nwaves : 0;
   int row = r0 + wave;
   for (int round = 0; round * D < my_rows; ++round) {
@@ -490,12 +524,32 @@ __global__ __launch_bounds__(MAXT) void gemv_w4a16_f16_rows_kernel(const half_t*
     for (int d = 0; d < D; ++d) {
       const int lrow = (row < r1 ? row : r1 - 1) - r0;
       float acc = 0.f;
+      if constexpr (F16) {
 #pragma unroll
-      for (int it = 0; it < ITERS; ++it) {
-        const half_t sv = has_s ? lds_s[lrow * groups + gsel[it]] : one;
-        const half_t z = has_z ? lds_z[lrow * groups + gsel[it]] : zs;
-        const half_t s = ok[it] ? sv : (half_t)0.0f;  // a chunk past the end contributes 0
-        acc += chunk_term_biased(st[d].w[it], act[it], s, z, mg);
+        for (int it = 0; it < ITERS; ++it) {
+          const half_t sv = has_s ? lds_s[lrow * groups + gsel[it]] : one;
+          const half_t z = has_z ? lds_z[lrow * groups + gsel[it]] : zs;
+          const half_t s = ok[it] ? sv : (half_t)0.0f;  // a chunk past the end contributes 0
+          acc += chunk_term_biased(st[d].w[it], act[it], s, z, mg);
+        }
+      } else {
+        T sv[ITERS], zv[ITERS];
+        bool integral = true;  // small integer zero points fold exactly into one fused multiply-add per weight
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          const T s0 = has_s ? lds_s[lrow * groups + gsel[it]] : one;
+          zv[it] = has_z ? lds_z[lrow * groups + gsel[it]] : zs;
+          sv[it] = ok[it] ? s0 : from_float<T>(0.0f);
+          const float zf = to_float(zv[it]);
+          integral = integral && zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
+        }
+        if (__builtin_amdgcn_ballot_w64(integral) == ~0ull) {
+#pragma unroll
+          for (int it = 0; it < ITERS; ++it) acc += chunk_term_dot2<true>(st[d].w[it], actn[it], sv[it], zv[it], mg);
+        } else {
+#pragma unroll
+          for (int it = 0; it < ITERS; ++it) acc += chunk_term_dot2<false>(st[d].w[it], actn[it], sv[it], zv[it], mg);
+        }
       }
       const float v = wave_sum_to_lane63(acc);
       if (lane == 63 && row < r1) store_out(C, row, v, out_dtype);
@@ -504,6 +558,28 @@ __global__ __launch_bounds__(MAXT) void gemv_w4a16_f16_rows_kernel(const half_t*
       irow += nwaves;
     }
   }
+}
+
+template <int ITERS, int D, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_w4a16_f16_rows_kernel(const half_t* __restrict__ A,
+                                                                  const uint8_t* __restrict__ Wp,
+                                                                  const half_t* __restrict__ scales,
+                                                                  const half_t* __restrict__ zeros,
+                                                                  void* __restrict__ C, int N, int K, int group_shift,
+                                                                  float zero_scalar, int out_dtype, int rows_per_block,
+                                                                  int nwaves) {
+  gemv_rows_body<half_t, ITERS, D>(A, Wp, scales, zeros, C, N, K, group_shift, zero_scalar, out_dtype, rows_per_block, nwaves);
+}
+
+template <int ITERS, int D, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_w4a16_bf16_rows_kernel(const bf16_t* __restrict__ A,
+                                                                   const uint8_t* __restrict__ Wp,
+                                                                   const bf16_t* __restrict__ scales,
+                                                                   const bf16_t* __restrict__ zeros,
+                                                                   void* __restrict__ C, int N, int K, int group_shift,
+                                                                   float zero_scalar, int out_dtype, int rows_per_block,
+                                                                   int nwaves) {
+  gemv_rows_body<bf16_t, ITERS, D>(A, Wp, scales, zeros, C, N, K, group_shift, zero_scalar, out_dtype, rows_per_block, nwaves);
 }
 
 template <typename T>
@@ -632,7 +708,7 @@ static int launch_gemv_f16(const void* A, const void* Wp, const void* scales, co
 
 // rows kernel: work-groups of `waves_per_block` wavefronts, each owning a contiguous range of rows whose
 // scales and zero points fit its LDS; at least `blocks_per_cu` work-groups per CU when there are rows enough
-template <int ITERS, int D, int MAXT>
+template <typename T, int ITERS, int D, int MAXT>
 static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int batch,
                             int N, int K, int group_shift, float zero_scalar, int out_dtype, int waves_per_block,
                             int blocks_per_cu, hipStream_t st) {
@@ -646,10 +722,63 @@ static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, c
   rpb = (rpb + 3) & ~3;  // keeps the zero-point block of LDS 16-byte aligned for any group count
   blocks = (int)ceil_div(N, rpb);
   const size_t lds = (size_t)(K / 32) * 72 + (size_t)rpb * groups * 4;
-  gemv_w4a16_f16_rows_kernel<ITERS, D, MAXT><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
-      (const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C, N, K, group_shift,
-      zero_scalar, out_dtype, rpb, waves_per_block);
+  if constexpr (__is_same(T, half_t))
+    gemv_w4a16_f16_rows_kernel<ITERS, D, MAXT><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
+        (const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C, N, K, group_shift,
+        zero_scalar, out_dtype, rpb, waves_per_block);
+  else
+    gemv_w4a16_bf16_rows_kernel<ITERS, D, MAXT><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
+        (const bf16_t*)A, (const uint8_t*)Wp, (const bf16_t*)scales, (const bf16_t*)zeros, C, N, K, group_shift,
+        zero_scalar, out_dtype, rpb, waves_per_block);
   return 0;
+}
+
+// M = 1, rows of up to 16384 values: the register-resident kernel (see gemv_rows_body)
+template <typename T>
+static int dispatch_gemv_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch,
+                              int64_t N, int64_t K, int shift, float zero_scalar, int out_dtype, hipStream_t st) {
+  const int depth_req = g_gemv_depth;
+  const int bpc_rows = g_gemv_unroll ? g_gemv_unroll : 1;
+  const bool long_rows = K > 4096;  // 8 wavefronts per work-group (see the kernel)
+  int wpb_rows = g_gemv_waves16 ? g_gemv_waves16 : 16;
+  if (long_rows && wpb_rows > 8) wpb_rows = 8;
+  if (wpb_rows * 64 < K / 32) wpb_rows = (int)ceil_div(K / 32, (int64_t)64);  // one staging thread per chunk
+  // one problem of a few tens of MB: one row in flight per wavefront (deeper queues delay the staging
+  // loads behind the weights and measured slower); many problems per launch stream with two
+  const int d = depth_req ? depth_req : (batch * N * (K / 2) > ((int64_t)64 << 20) ? 2 : 1);
+#define TLQ_ROWS_CASE(IT, DD, MAXT)                                                                                \
+  launch_gemv_rows<T, IT, DD, MAXT>(A, Wp, scales, zeros, C, (int)batch, (int)N, (int)K, shift, zero_scalar, out_dtype, \
+                             wpb_rows, bpc_rows, st)
+  if (K <= 2048) {
+    if (d <= 2) TLQ_ROWS_CASE(1, 2, 1024);
+    else if (d <= 4) TLQ_ROWS_CASE(1, 4, 1024);
+    else TLQ_ROWS_CASE(1, 8, 1024);
+  } else if (K <= 4096) {
+    if (d <= 1) TLQ_ROWS_CASE(2, 1, 1024);
+    else if (d == 2) TLQ_ROWS_CASE(2, 2, 1024);
+    else if (d == 3) TLQ_ROWS_CASE(2, 3, 1024);
+    else if (d == 4) TLQ_ROWS_CASE(2, 4, 1024);
+    else TLQ_ROWS_CASE(2, 6, 1024);
+  } else {
+    const int iters = (int)ceil_div(K, (int64_t)2048);  // 3 .. 8
+#define TLQ_LONG_CASE(IT)                    \
+  case IT:                                   \
+    if (d <= 1) TLQ_ROWS_CASE(IT, 1, 512);   \
+    else TLQ_ROWS_CASE(IT, 2, 512);          \
+    break;
+    switch (iters) {
+      TLQ_LONG_CASE(3)
+      TLQ_LONG_CASE(4)
+      TLQ_LONG_CASE(5)
+      TLQ_LONG_CASE(6)
+      TLQ_LONG_CASE(7)
+      default:
+        TLQ_LONG_CASE(8)
+    }
+#undef TLQ_LONG_CASE
+  }
+#undef TLQ_ROWS_CASE
+  return check_launch("tlq_gemm_w4a16(gemv)") ? 0 : 1;
 }
 
 int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch, int64_t M,
@@ -667,49 +796,8 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     const int R = g_gemv_rows > 0 ? g_gemv_rows : (streaming ? 2 : 1);
     const int bpc = g_gemv_unroll ? g_gemv_unroll : (streaming ? 64 : 8);  // grid size cap, blocks per CU
     const int depth_req = g_gemv_depth;
-    if (M == 1 && K <= 16384 && g_gemv_rows >= 0) {
-      const int bpc_rows = g_gemv_unroll ? g_gemv_unroll : 1;
-      const bool long_rows = K > 4096;  // 8 wavefronts per work-group (see the kernel)
-      int wpb_rows = g_gemv_waves16 ? g_gemv_waves16 : 16;
-      if (long_rows && wpb_rows > 8) wpb_rows = 8;
-      if (wpb_rows * 64 < K / 32) wpb_rows = (int)ceil_div(K / 32, (int64_t)64);  // one staging thread per chunk
-      // one problem of a few tens of MB: one row in flight per wavefront (deeper queues delay the staging
-      // loads behind the weights and measured slower); many problems per launch stream with two
-      const int d = depth_req ? depth_req : (batch * N * (K / 2) > ((int64_t)64 << 20) ? 2 : 1);
-#define TLQ_ROWS_CASE(IT, DD, MAXT)                                                                                \
-  launch_gemv_rows<IT, DD, MAXT>(A, Wp, scales, zeros, C, (int)batch, (int)N, (int)K, shift, zero_scalar, out_dtype, \
-                                 wpb_rows, bpc_rows, st)
-      if (K <= 2048) {
-        if (d <= 2) TLQ_ROWS_CASE(1, 2, 1024);
-        else if (d <= 4) TLQ_ROWS_CASE(1, 4, 1024);
-        else TLQ_ROWS_CASE(1, 8, 1024);
-      } else if (K <= 4096) {
-        if (d <= 1) TLQ_ROWS_CASE(2, 1, 1024);
-        else if (d == 2) TLQ_ROWS_CASE(2, 2, 1024);
-        else if (d == 3) TLQ_ROWS_CASE(2, 3, 1024);
-        else if (d == 4) TLQ_ROWS_CASE(2, 4, 1024);
-        else TLQ_ROWS_CASE(2, 6, 1024);
-      } else {
-        const int iters = (int)ceil_div(K, (int64_t)2048);  // 3 .. 8
-#define TLQ_LONG_CASE(IT)                    \
-  case IT:                                   \
-    if (d <= 1) TLQ_ROWS_CASE(IT, 1, 512);   \
-    else TLQ_ROWS_CASE(IT, 2, 512);          \
-    break;
-        switch (iters) {
-          TLQ_LONG_CASE(3)
-          TLQ_LONG_CASE(4)
-          TLQ_LONG_CASE(5)
-          TLQ_LONG_CASE(6)
-          TLQ_LONG_CASE(7)
-          default:
-            TLQ_LONG_CASE(8)
-        }
-#undef TLQ_LONG_CASE
-      }
-#undef TLQ_ROWS_CASE
-      return check_launch("tlq_gemm_w4a16(gemv)") ? 0 : 1;
-    }
+    if (M == 1 && K <= 16384 && g_gemv_rows >= 0)
+      return dispatch_gemv_rows<half_t>(A, Wp, scales, zeros, C, batch, N, K, shift, zero_scalar, out_dtype, st);
     const bool two_rows = M > 1 && (size_t)2 * (K / 32) * 72 <= 64 * 1024;
 #define TLQ_F16_CASE(RR, MTT, DD)                                                                                  \
   rc = launch_gemv_f16<RR, MTT, DD>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, shift, zero_scalar, \
@@ -741,7 +829,12 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     launch_gemv<half_t, 2, 1>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, (int)group, zero_scalar,
                               out_dtype, wpb, st);
   } else {
-    // bfloat16: element-wise exact dequantisation (generic kernel)
+    if (M == 1 && pow2 && K <= 16384 && g_gemv_rows >= 0) {
+      int shift = 0;
+      while (((int64_t)1 << shift) < group) ++shift;
+      return dispatch_gemv_rows<bf16_t>(A, Wp, scales, zeros, C, batch, N, K, shift, zero_scalar, out_dtype, st);
+    }
+    // bfloat16 otherwise: element-wise exact dequantisation (generic kernel)
     if (M == 1)
       launch_gemv<bf16_t, 2, 1>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, (int)group, zero_scalar,
                                 out_dtype, wpb, st);
