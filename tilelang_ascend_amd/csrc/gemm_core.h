@@ -122,6 +122,7 @@ struct RowLoader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
   static constexpr bool PREFETCH2 = false;
+  static constexpr int TOUCH_LINES = ROWS;  // cache lines per stage (one per row), see touch_ptr
   static constexpr int SLOTS = ROWS * 8;  // 16-byte chunks per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
@@ -136,6 +137,13 @@ struct RowLoader {
   struct Regs {
     uint4_t v[PASSES];
   };
+  // line i of stage 0 of the tile that starts at row0 (the kernel touches the lines of a later stage ahead of time);
+  // the same line of stage kt is touch_step(p) * kt bytes further
+  static __device__ __forceinline__ const uint8_t* touch_ptr(const Params& p, int batch, int row0, int rows_total, int i) {
+    const int row = row0 + i < rows_total ? row0 + i : rows_total - 1;
+    return p.base + batch * p.batch_stride + (int64_t)row * p.ld;
+  }
+  static __device__ __forceinline__ int64_t touch_step(const Params&) { return kStageBytes; }
   const uint8_t* base;    // uniform
   uint32_t voff[PASSES];  // per lane: row * ld + chunk * 16
   uint32_t loff;          // per lane: LDS offset of pass 0
@@ -196,6 +204,12 @@ struct RowLoaderDirect {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = true;
   static constexpr bool PREFETCH2 = false;
+  static constexpr int TOUCH_LINES = ROWS;
+  static __device__ __forceinline__ const uint8_t* touch_ptr(const typename RowLoader<ROWS, NT>::Params& p, int batch, int row0,
+                                                             int rows_total, int i) {
+    return RowLoader<ROWS, NT>::touch_ptr(p, batch, row0, rows_total, i);
+  }
+  static __device__ __forceinline__ int64_t touch_step(const typename RowLoader<ROWS, NT>::Params&) { return kStageBytes; }
   static constexpr int WAVES = NT / 64;
   static constexpr int INSTR = ROWS / 8;          // wavefront-instructions per stage
   static constexpr int PER_WAVE = INSTR / WAVES;  // ... per wavefront
@@ -287,6 +301,12 @@ struct I8KNLoaderDirect {
   typedef KNFrag8<BN> Frag;
   static constexpr bool DIRECT = true;
   static constexpr bool PREFETCH2 = false;
+  static constexpr int TOUCH_LINES = 128 * (BN / 128);  // 128 k rows of BN bytes
+  static __device__ __forceinline__ const uint8_t* touch_ptr(const I8KNParams& p, int batch, int col0, int cols_total, int i) {
+    const int k = i / (BN / 128), c = col0 + (i % (BN / 128)) * 128;
+    return p.base + batch * p.batch_stride + (int64_t)k * p.ld + (c < cols_total ? c : col0);
+  }
+  static __device__ __forceinline__ int64_t touch_step(const I8KNParams& p) { return (int64_t)kStageBytes * p.ld; }
   static constexpr int CH = BN / 16;              // 16-byte chunks per k row
   static constexpr int KPI = 64 / CH;             // k rows per wavefront instruction
   static constexpr int WAVES = NT / 64;
@@ -500,7 +520,7 @@ __device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n, int
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma_kernel(
     typename AL::Params pa, typename WL::Params pw, typename Epi::Params pe, int M, int N, int KT, int k_tail,
-    int tiles_m, int tiles_n, int band_rows) {
+    int tiles_m, int tiles_n, int band_rows, int touch_ahead) {
   constexpr int TM = BM / WM / 16;  // 16-row activation tiles per wave
   constexpr int TN = BN / WN / 16;  // 16-row weight tiles per wave
   constexpr int A_TILE = BM * kStageBytes, W_TILE = BN * kStageBytes;
@@ -539,9 +559,48 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   constexpr int NP = 2 * TN;  // pieces per stage
   // first pieces: activation stores (none when they travel directly), the rest: weight conversion
   constexpr int NPA = AL::DIRECT ? 0 : NP / 2;
+  // Optional (touch_ahead = stages ahead, 0 = off): while stage kt multiplies, every thread asks for four bytes of one
+  // cache line of stage kt + touch_ahead with a direct load into a spare LDS word.  A stage's real loads are issued only
+  // one stage before they are needed; lines that no CU of the XCD has touched yet come from HBM and take longer
+  // than that.  The touch starts that trip earlier, and the real loads then find the line in L2.  Each wavefront
+  // issues exactly one touch per stage (threads beyond the tile's lines repeat line 0), after the stage's other loads,
+  // so "everything but the youngest load has landed" is the wait that leaves the touch in flight.
+  // (Not for the converting weight loader: its 256 x 256 kernels have no registers to spare.)
+  constexpr bool TOUCH_OK = !WL::PREFETCH2 && AL::TOUCH_LINES + WL::TOUCH_LINES > 0;
+  const uint8_t* touch_p = nullptr;
+  int64_t touch_step = 0;
+  if constexpr (TOUCH_OK) {
+    if (touch_ahead > 0) {
+      constexpr int LA = AL::TOUCH_LINES, LW = WL::TOUCH_LINES;
+      if (LA > 0 && (tid < LA || LW == 0)) {
+        if constexpr (LA > 0) {
+          touch_p = AL::touch_ptr(pa, batch, m0, M, tid < LA ? tid : 0);
+          touch_step = AL::touch_step(pa);
+        }
+      } else {
+        if constexpr (LW > 0) {
+          touch_p = WL::touch_ptr(pw, batch, n0, N, tid - LA < LW ? tid - LA : 0);
+          touch_step = WL::touch_step(pw);
+        }
+      }
+    }
+  }
+  const bool touching = TOUCH_OK && touch_ahead > 0;  // then every thread has a line to touch
+  typedef __attribute__((address_space(3))) uint8_t* touch_lptr_t;
+  const uint32_t touch_lds =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(touch_lptr_t)(smem + 2 * (A_TILE + W_TILE)) + (uint32_t)(wave * 256));
+  auto touch = [&](int kt) {  // kt: a full stage inside K
+    const uint64_t a = (uint64_t)(uintptr_t)(touch_p + (int64_t)kt * touch_step);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(touch_lds), "v"(a) : "memory");
+  };
   // hand-issued direct loads are invisible to the compiler's wait insertion
-  auto wait_direct = [&]() {
-    if (AL::DIRECT || WL::DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  auto wait_direct = [&](bool touched = false) {
+    if (AL::DIRECT || WL::DIRECT) {
+      if (touched)
+        asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
   };
   auto stage = [&](int cur, auto fill_tag) {
     constexpr bool FILL = decltype(fill_tag)::value;
@@ -585,6 +644,7 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   wait_direct();
   __syncthreads();
 
+  const int last_full = k_tail ? KT - 2 : KT - 1;  // highest stage that is whole (loadable without the tail path)
   if constexpr (WL::PREFETCH2) {
     // Converting loader: the weights of stage t+1 are converted during stage t from registers that were
     // loaded during stage t-1, so the conversion never waits on a load issued in the same stage and the
@@ -606,19 +666,22 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
         al.template gload<true>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
       else
         al.template gload<false>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
+      const bool touched = touching && kt + touch_ahead <= last_full;
+      if (touched) touch(kt + touch_ahead);
       stage(kt & 1, std::true_type{});
-      wait_direct();
+      wait_direct(touched);
       __syncthreads();
     }
   } else {
     // Stages 0 .. KT-2 compute and fill.  Only the load of stage KT-1 can be a partial stage.
-    const int last_full = k_tail ? KT - 2 : KT - 1;  // highest stage loadable without the tail path
     int kt = 0;
     for (; kt + 1 <= last_full; ++kt) {
       al.template gload<false>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
       wl.template gload<false>(rw, kt + 1, ldsW0 + ((kt + 1) & 1) * W_TILE);
+      const bool touched = touching && kt + touch_ahead <= last_full;
+      if (touched) touch(kt + touch_ahead);
       stage(kt & 1, std::true_type{});
-      wait_direct();
+      wait_direct(touched);
       __syncthreads();
     }
     if (kt + 1 < KT) {  // the partial last stage
@@ -644,12 +707,14 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
 // tile rows per band of the work-group -> tile order, for tuning runs (0 = each launcher's own choice: measured best
 // were 2 for the int8 kernels, 4 for the plain 16-bit GEMM and 8 for the fused W4A16 kernel; 1 = plain row-major)
 extern int g_gemm_band_rows;
+// stages ahead at which the lines of a later stage are touched (0 = off, the default; see the kernel)
+extern int g_gemm_touch_ahead;
 
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,
                 int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what, int band_rows = 4) {
   auto kern = gemm_mfma_kernel<Mma, AL, WL, Epi, BM, BN, WM, WN>;
-  constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes;
+  constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes + WM * WN * 256;  // two stages + one spare word per thread (touches)
   static bool attr_set = false;  // per instantiation; idempotent, so a race only repeats the call
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -669,7 +734,8 @@ int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, co
   const int KT = (int)ceil_div(k_bytes, kStageBytes);
   const int k_tail = (k_bytes % kStageBytes) != 0;
   kern<<<(unsigned)blocks, WM * WN * 64, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, KT, k_tail, (int)tiles_m,
-                                                          (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows);
+                                                          (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows,
+                                                          g_gemm_touch_ahead);
   return check_launch(what) ? 0 : 1;
 }
 
