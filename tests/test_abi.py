@@ -150,3 +150,43 @@ def test_error_string_is_thread_local():
     t.join()
     assert seen["before"] == "" and "tlq_gemm_w4a8" in seen["after"]
     assert "tlq_gemm_i8" in _abi.last_error()
+
+
+def test_rejects_bad_arguments_of_the_widened_entry_points():
+    """Activation quantiser, repacker, plain GEMV / split-K and the workspace entry point validate before any GPU call."""
+    lib = _abi.load()
+    _rejected(lib.tlq_act_quant_i8(FAKE, FAKE, FAKE, 4, 0, _abi.BF16, 0, NULL), "rows are empty")
+    _rejected(lib.tlq_act_quant_i8(FAKE, FAKE, FAKE, 4, 64, _abi.I8, 0, NULL), "in_dtype")
+    _rejected(lib.tlq_act_quant_i8(NULL, FAKE, FAKE, 4, 64, _abi.BF16, 0, NULL), "null pointer")
+    _rejected(lib.tlq_act_quant_i8(FAKE, FAKE, ODD2, 4, 64, _abi.BF16, 0, NULL), "misaligned")
+    _rejected(lib.tlq_pack_int4(FAKE, FAKE, 4, 12, 0, NULL), "K=12")
+    _rejected(lib.tlq_pack_int4(FAKE, FAKE, 4, 16, 3, NULL), "interleave")
+    _rejected(lib.tlq_pack_int4(ODD, FAKE, 4, 16, 0, NULL), "aligned")
+    _rejected(lib.tlq_quantize_sym4(FAKE, FAKE, FAKE, 4, 64, 12, _abi.F16, NULL), "group=12")
+    _rejected(lib.tlq_quantize_sym4(FAKE, FAKE, FAKE, 4, 64, 32, _abi.F32, NULL), "dtype")
+    _rejected(lib.tlq_gemv(FAKE, FAKE, FAKE, 8, 12, _abi.F16, _abi.F16, NULL), "K=12")
+    _rejected(lib.tlq_gemv(FAKE, FAKE, FAKE, 8, 64, _abi.I8, _abi.F16, NULL), "dtype")
+    _rejected(lib.tlq_gemv(ODD, FAKE, FAKE, 8, 64, _abi.F16, _abi.F16, NULL), "16-byte aligned")
+    _rejected(lib.tlq_gemm_w4a16_ws(FAKE, FAKE, NULL, NULL, FAKE, 512, 64, 128, 32, 0.0, _abi.F16, _abi.F16, _abi.ALGO_TWO_PASS,
+                                    NULL, 0, NULL), "two-pass path needs", "workspace")
+    _rejected(lib.tlq_gemm_w4a16_ws(FAKE, FAKE, NULL, NULL, FAKE, 512, 64, 128, 32, 0.0, _abi.F16, _abi.F16, 9, NULL, 0, NULL),
+              "bad algo")
+    # empty problems launch nothing
+    assert lib.tlq_act_quant_i8(NULL, NULL, NULL, 0, 64, _abi.BF16, 0, NULL) == 0
+    assert lib.tlq_gemv(NULL, NULL, NULL, 0, 64, _abi.F16, _abi.F16, NULL) == 0
+
+
+def test_workspace_size_rules():
+    """tlq_w4a16_workspace_bytes: nothing for decode shapes, fp32 partial sums of the K slices for small and middle M,
+    a dequantised copy of the weights (N * K 16-bit values) for large M."""
+    ws = _abi.load().tlq_w4a16_workspace_bytes
+    assert ws(1, 11008, 4096) == 0 and ws(16, 14336, 4096) == 0
+    assert ws(4096, 4096, 4096) == 4096 * 4096 * 2
+    assert ws(8192, 14336, 4096) == 14336 * 4096 * 2
+    for M, N, K in ((64, 14336, 4096), (256, 4096, 14336), (512, 4096, 4096), (1024, 4096, 14336)):
+        b = ws(M, N, K)
+        assert b > 0 and b % (M * N * 4) == 0, (M, N, K, b)
+        split = b // (M * N * 4)
+        assert 2 <= split <= 16 and K % split == 0 and (K // split) % 64 == 0 and K // split >= 512, (M, N, K, split)
+    assert ws(1024, 14336, 4096) == 14336 * 4096 * 2  # many output tiles already: no K slices, two passes
+    assert ws(64, 0, 4096) == 0 and ws(64, 128, 0) == 0
