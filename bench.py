@@ -358,7 +358,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU's share of the path; --gpus {args.gpus} is not supported in this build "
-              "(the path shards over N with no exchange, see DESIGN.md).", file=sys.stderr)
+              "(the path shards over the weight rows N: each GPU holds its rows and all activations, no exchange).",
+              file=sys.stderr)
         sys.exit(2)
 
     import torch
