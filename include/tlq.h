@@ -205,6 +205,8 @@ void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4 (negat
 void tlq_tune_gemv_unroll(int blocks_per_cu);               /* resident blocks per CU the GEMV grid is sized for */
 void tlq_tune_gemv_depth(int steps_in_flight);               /* load steps (1 KB per row each) a GEMV wavefront keeps in flight */
 void tlq_tune_gemm_band(int tile_rows);                       /* tile rows per band of the MFMA kernels' tile order (default 4) */
+void tlq_tune_gemm_slots(int on);                            /* 1: plain 16-bit / int8 GEMM with [N, K] weights on the kernel that cuts LDS
+                                                              * into five operand-tile slots (0 = two stages, the default) */
 void tlq_tune_gemm_touch(int stages_ahead);                  /* MFMA kernels: touch the cache lines of the stage this many stages ahead
                                                               * (0 = off, the default; 2 is the intended setting) */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */

@@ -49,6 +49,7 @@ SIGNATURES = {
     "tlq_tune_gemv_depth": (None, [_int]),
     "tlq_tune_gemm_band": (None, [_int]),
     "tlq_tune_gemm_touch": (None, [_int]),
+    "tlq_tune_gemm_slots": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),
     "tlq_tune_w4a16_split": (None, [_int]),
     "tlq_tune_w4a16_skinny": (None, [_int, _int]),

@@ -1,6 +1,7 @@
 // Plain fp16 / bf16 GEMM with fp32 accumulation: C[M, N] = A[M, K] . B, B stored [K, N]
 // (transposed on the fly) or [N, K].
 #include "gemm_core.h"
+#include "gemm_slots.h"
 
 namespace tlq {
 
@@ -137,6 +138,11 @@ static int dispatch_f16(const void* A, const void* B, void* C, int64_t M, int64_
                         int b_layout, hipStream_t st) {
   if (M <= 128 || ceil_div(M, 256) * ceil_div(N, 256) < 128)
     return run_f16<Mma, 128, 128, 2, 2>(A, B, C, M, N, K, out_dtype, b_layout, st);
+  if (g_gemm_slots && b_layout == TLQ_B_NK && K % 64 == 0) {  // whole 128-byte stages
+    typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K * 2, 0, K * 2}, pw{(const uint8_t*)B, K * 2, 0, K * 2};
+    EpiFloat::Params pe{C, N, 0, out_dtype};
+    return launch_gemm_slots<Mma, EpiFloat>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16", 4);
+  }
   return run_f16<Mma, 256, 256, 2, 4>(A, B, C, M, N, K, out_dtype, b_layout, st);
 }
 

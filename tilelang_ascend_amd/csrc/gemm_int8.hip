@@ -4,6 +4,7 @@
 //   * W4A8: packed int4 weights expanded to int8 on the way into LDS
 // The second operand may be stored [K, N] (transposed on the fly) or [N, K].
 #include "gemm_core.h"
+#include "gemm_slots.h"
 
 namespace tlq {
 
@@ -138,6 +139,10 @@ static int dispatch_i8(const void* A, const void* B, const typename Epi::Params&
     }
 #undef TLQ_RUN
   } else {
+    if (g_gemm_slots && tile == 256 && K % 128 == 0) {  // whole 128-byte stages
+      typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K, M * K, K}, pw{(const uint8_t*)B, K, N * K, K};
+      return launch_gemm_slots<MmaI8, Epi>(pa, pw, pe, batch, M, N, K, st, what, 2);
+    }
 #define TLQ_RUN(BM, BN, WM, WN)                                               \
   {                                                                           \
     typedef RowLoaderDirect<BN, WM * WN * 64> WL;                             \

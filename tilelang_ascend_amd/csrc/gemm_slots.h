@@ -1,0 +1,122 @@
+// 256 x 256 tile, both operands row-major [rows, K] and copied global -> LDS directly, with the 160 KB of LDS cut into
+// FIVE slots of one operand tile (256 rows x 128 bytes of K = 32 KB) instead of two stages of two tiles.
+//
+// With two stages the loads of stage k + 1 can only be issued when stage k - 1 has been consumed and must have landed
+// one stage of MFMA time later; a stage's slowest load takes longer than that, and the loop runs at the pace of the
+// loads.  Here tile t (A of stage s is t = 2s, W of stage s is t = 2s + 1) lives in slot t mod 5.  At the start of
+// stage k the slots of A(k - 1) and W(k - 1) are free, which is where W(k + 1) and A(k + 2) go: one and a half stages
+// of loads are in flight, the A tiles are requested two stages ahead and the W tiles one stage ahead with only half
+// a stage's bytes behind them.  The wait at the end of stage k leaves the youngest tile (A(k + 2), four loads per
+// wavefront) outstanding.  Everything else -- wave tiling, LDS tile layout, fragment reads, epilogue -- is the
+// two-stage kernel's.
+//
+// Selected by tlq_tune_gemm_slots(1); whole stages only (K bytes a multiple of 128).
+#pragma once
+#include "gemm_core.h"
+
+namespace tlq {
+
+template <class Mma, class Epi>
+__global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDirect<256, 512>::Params pa,
+                                                           typename RowLoaderDirect<256, 512>::Params pw,
+                                                           typename Epi::Params pe, int M, int N, int KT, int tiles_m,
+                                                           int tiles_n, int band_rows) {
+  constexpr int BM = 256, BN = 256, WM = 2, WN = 4, TM = 8, TN = 4, SLOTS = 5;
+  constexpr int TILE = 256 * kStageBytes;  // one operand, one stage: 32 KB
+  typedef RowLoaderDirect<256, 512> Loader;
+  static_assert(Loader::PER_WAVE == 4, "the waits below count four loads per wavefront and tile");
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15, q = lane >> 4;
+  const int wave_m0 = (wave % WM) * (BM / WM), wave_n0 = (wave / WM) * (BN / WN);
+  const TileCoord tc = tile_of_block<BM, BN>(tiles_m, tiles_n, band_rows);
+  Loader al(pa, tc.batch, tc.m0, M, tid), wl(pw, tc.batch, tc.n0, N, tid);
+  typename Loader::Regs regs;  // unused by full stages (the data never passes through registers)
+  const RowFrag fragA(lane, wave_m0), fragW(lane, wave_n0);
+  auto slot_of = [&](int t) { return smem + (t % SLOTS) * TILE; };
+  auto issue_a = [&](int s) { al.template gload<false>(regs, s, slot_of(2 * s)); };
+  auto issue_w = [&](int s) { wl.template gload<false>(regs, s, slot_of(2 * s + 1)); };
+
+  typename Mma::acc_t acc[TN][TM];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = typename Mma::acc_t{0, 0, 0, 0};
+
+  // this wavefront's loads of everything but the youngest tile have landed (`keep`: that tile was issued)
+  auto wait_tiles = [&](bool keep) {
+    if (keep)
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+
+  issue_a(0);
+  issue_w(0);
+  if (KT > 1) issue_a(1);
+  wait_tiles(KT > 1);
+  __syncthreads();
+  for (int k = 0; k < KT; ++k) {
+    if (k + 1 < KT) issue_w(k + 1);  // into the slot of A(k - 1)
+    if (k + 2 < KT) issue_a(k + 2);  // into the slot of W(k - 1)
+    const uint8_t* la = slot_of(2 * k);
+    const uint8_t* lw = slot_of(2 * k + 1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      uint4_t wf[TN], af[TM];
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) wf[tn] = fragW.read(lw, ks, tn);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) af[tm] = fragA.read(la, ks, tm);
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = Mma::mma(wf[tn], af[tm], acc[tn][tm]);
+    }
+    if (k + 1 < KT) {
+      wait_tiles(k + 2 < KT);  // A(k + 1) and W(k + 1) are in; A(k + 2) may still be on its way
+      __syncthreads();         // ... for every wavefront, and everyone has read the tiles of stage k
+    }
+  }
+
+  Epi epi(pe, tc.batch);
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+      epi.store(tc.m0 + wave_m0 + tm * 16 + r16, tc.n0 + wave_n0 + tn * 16 + q * 4, acc[tn][tm], M, N);
+}
+
+// tlq_tune_gemm_slots: 0 = the two-stage kernel (default), 1 = this one where it applies
+extern int g_gemm_slots;
+
+// Both matrices [rows, k_bytes] row-major with 16-byte aligned rows; k_bytes a positive multiple of 128.
+template <class Mma, class Epi>
+int launch_gemm_slots(const typename RowLoaderDirect<256, 512>::Params& pa, const typename RowLoaderDirect<256, 512>::Params& pw,
+                      const typename Epi::Params& pe, int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st,
+                      const char* what, int band_rows) {
+  auto kern = gemm_slots_kernel<Mma, Epi>;
+  constexpr int lds_bytes = 5 * 256 * kStageBytes;  // all of the CU's LDS
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) {
+      set_error("%s: cannot reserve %d bytes of LDS: %s", what, lds_bytes, hipGetErrorString(e));
+      return 1;
+    }
+    attr_set = true;
+  }
+  const int64_t tiles_m = ceil_div(M, (int64_t)256), tiles_n = ceil_div(N, (int64_t)256);
+  const int64_t blocks = batch * tiles_m * tiles_n;
+  if (blocks <= 0) return 0;
+  if (blocks > 0x7fffffff) {
+    set_error("%s: too many tiles", what);
+    return 1;
+  }
+  kern<<<(unsigned)blocks, 512, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, (int)(k_bytes / kStageBytes), (int)tiles_m,
+                                                 (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows);
+  return check_launch(what) ? 0 : 1;
+}
+
+}  // namespace tlq
