@@ -141,7 +141,7 @@ static int dispatch_f16(const void* A, const void* B, void* C, int64_t M, int64_
   if (g_gemm_slots && b_layout == TLQ_B_NK && K % 64 == 0) {  // whole 128-byte stages
     typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K * 2, 0, K * 2}, pw{(const uint8_t*)B, K * 2, 0, K * 2};
     EpiFloat::Params pe{C, N, 0, out_dtype};
-    return launch_gemm_slots<Mma, EpiFloat>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16", 4);
+    return launch_gemm_slots<Mma, RowLoaderDirect<256, 512>, EpiFloat>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16", 4);
   }
   return run_f16<Mma, 256, 256, 2, 4>(A, B, C, M, N, K, out_dtype, b_layout, st);
 }

@@ -123,6 +123,12 @@ static int dispatch_i8(const void* A, const void* B, const typename Epi::Params&
                        int64_t N, int64_t K, int b_layout, hipStream_t st, const char* what) {
   const int tile = pick_tile(batch, M, N);
   if (b_layout == TLQ_B_KN) {
+    if (g_gemm_slots && tile == 256 && K % 128 == 0) {  // whole 128-byte stages
+      typedef I8KNLoaderDirect<256, 512> WL;
+      typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K, M * K, K};
+      typename WL::Params pw{(const uint8_t*)B, N, K * N, K};
+      return launch_gemm_slots<MmaI8, WL, Epi>(pa, pw, pe, batch, M, N, K, st, what, 2);
+    }
 #define TLQ_RUN(BM, BN, WM, WN)                                               \
   {                                                                           \
     typedef I8KNLoaderDirect<BN, WM * WN * 64> WL;                            \
@@ -141,7 +147,7 @@ static int dispatch_i8(const void* A, const void* B, const typename Epi::Params&
   } else {
     if (g_gemm_slots && tile == 256 && K % 128 == 0) {  // whole 128-byte stages
       typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K, M * K, K}, pw{(const uint8_t*)B, K, N * K, K};
-      return launch_gemm_slots<MmaI8, Epi>(pa, pw, pe, batch, M, N, K, st, what, 2);
+      return launch_gemm_slots<MmaI8, RowLoaderDirect<256, 512>, Epi>(pa, pw, pe, batch, M, N, K, st, what, 2);
     }
 #define TLQ_RUN(BM, BN, WM, WN)                                               \
   {                                                                           \

@@ -1,5 +1,6 @@
-// 256 x 256 tile, both operands row-major [rows, K] and copied global -> LDS directly, with the 160 KB of LDS cut into
-// FIVE slots of one operand tile (256 rows x 128 bytes of K = 32 KB) instead of two stages of two tiles.
+// 256 x 256 tile, both operands copied global -> LDS directly (activations row-major [M, K]; weights [N, K], or int8
+// [K, N] read transposed), with the 160 KB of LDS cut into FIVE slots of one operand tile (32 KB: 256 rows x 128 bytes
+// of K, or 128 k x 256 bytes of N) instead of two stages of two tiles.
 //
 // With two stages the loads of stage k + 1 can only be issued when stage k - 1 has been consumed and must have landed
 // one stage of MFMA time later; a stage's slowest load takes longer than that, and the loop runs at the pace of the
@@ -16,27 +17,29 @@
 
 namespace tlq {
 
-template <class Mma, class Epi>
+template <class Mma, class WL, class Epi>
 __global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDirect<256, 512>::Params pa,
-                                                           typename RowLoaderDirect<256, 512>::Params pw,
-                                                           typename Epi::Params pe, int M, int N, int KT, int tiles_m,
-                                                           int tiles_n, int band_rows) {
+                                                           typename WL::Params pw, typename Epi::Params pe, int M, int N,
+                                                           int KT, int tiles_m, int tiles_n, int band_rows) {
   constexpr int BM = 256, BN = 256, WM = 2, WN = 4, TM = 8, TN = 4, SLOTS = 5;
   constexpr int TILE = 256 * kStageBytes;  // one operand, one stage: 32 KB
   typedef RowLoaderDirect<256, 512> Loader;
-  static_assert(Loader::PER_WAVE == 4, "the waits below count four loads per wavefront and tile");
+  static_assert(Loader::PER_WAVE == 4 && WL::PER_WAVE == 4 && WL::DIRECT, "the waits below count four direct loads per wavefront and tile");
   extern __shared__ __align__(16) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, q = lane >> 4;
   const int wave_m0 = (wave % WM) * (BM / WM), wave_n0 = (wave / WM) * (BN / WN);
   const TileCoord tc = tile_of_block<BM, BN>(tiles_m, tiles_n, band_rows);
-  Loader al(pa, tc.batch, tc.m0, M, tid), wl(pw, tc.batch, tc.n0, N, tid);
+  Loader al(pa, tc.batch, tc.m0, M, tid);
+  WL wl(pw, tc.batch, tc.n0, N, tid);
   typename Loader::Regs regs;  // unused by full stages (the data never passes through registers)
-  const RowFrag fragA(lane, wave_m0), fragW(lane, wave_n0);
+  typename WL::Regs regs_w;
+  const RowFrag fragA(lane, wave_m0);
+  const typename WL::Frag fragW(lane, wave_n0);
   auto slot_of = [&](int t) { return smem + (t % SLOTS) * TILE; };
   auto issue_a = [&](int s) { al.template gload<false>(regs, s, slot_of(2 * s)); };
-  auto issue_w = [&](int s) { wl.template gload<false>(regs, s, slot_of(2 * s + 1)); };
+  auto issue_w = [&](int s) { wl.template gload<false>(regs_w, s, slot_of(2 * s + 1)); };
 
   typename Mma::acc_t acc[TN][TM];
 #pragma unroll
@@ -91,12 +94,12 @@ __global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDi
 // tlq_tune_gemm_slots: 0 = the two-stage kernel (default), 1 = this one where it applies
 extern int g_gemm_slots;
 
-// Both matrices [rows, k_bytes] row-major with 16-byte aligned rows; k_bytes a positive multiple of 128.
-template <class Mma, class Epi>
-int launch_gemm_slots(const typename RowLoaderDirect<256, 512>::Params& pa, const typename RowLoaderDirect<256, 512>::Params& pw,
+// k_bytes (bytes of K per activation row) a positive multiple of 128: whole stages only.
+template <class Mma, class WL, class Epi>
+int launch_gemm_slots(const typename RowLoaderDirect<256, 512>::Params& pa, const typename WL::Params& pw,
                       const typename Epi::Params& pe, int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st,
                       const char* what, int band_rows) {
-  auto kern = gemm_slots_kernel<Mma, Epi>;
+  auto kern = gemm_slots_kernel<Mma, WL, Epi>;
   constexpr int lds_bytes = 5 * 256 * kStageBytes;  // all of the CU's LDS
   static bool attr_set = false;
   if (!attr_set) {
