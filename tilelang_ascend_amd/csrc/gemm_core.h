@@ -516,6 +516,14 @@ __device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n, int
   return t;
 }
 
+// Which instances can touch a later stage's cache lines (see the kernel): not the converting weight loader (its
+// 256 x 256 kernels have no registers to spare) and not the low tiles (the spare LDS words would cost them a resident
+// work-group).  The launcher reserves the spare words for exactly these instances.
+template <class AL, class WL, int BM>
+constexpr bool gemm_touch_ok() {
+  return !WL::PREFETCH2 && BM >= 128 && AL::TOUCH_LINES + WL::TOUCH_LINES > 0;
+}
+
 // ---- the kernel -----------------------------------------------------------------------------
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma_kernel(
@@ -565,8 +573,7 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   // than that.  The touch starts that trip earlier, and the real loads then find the line in L2.  Each wavefront
   // issues exactly one touch per stage (threads beyond the tile's lines repeat line 0), after the stage's other loads,
   // so "everything but the youngest load has landed" is the wait that leaves the touch in flight.
-  // (Not for the converting weight loader: its 256 x 256 kernels have no registers to spare.)
-  constexpr bool TOUCH_OK = !WL::PREFETCH2 && AL::TOUCH_LINES + WL::TOUCH_LINES > 0;
+  constexpr bool TOUCH_OK = gemm_touch_ok<AL, WL, BM>();
   const uint8_t* touch_p = nullptr;
   int64_t touch_step = 0;
   if constexpr (TOUCH_OK) {
@@ -714,7 +721,8 @@ template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int 
 int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,
                 int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what, int band_rows = 4) {
   auto kern = gemm_mfma_kernel<Mma, AL, WL, Epi, BM, BN, WM, WN>;
-  constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes + WM * WN * 256;  // two stages + one spare word per thread (touches)
+  // two stages, and one spare word per thread where later stages can be touched
+  constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes + (gemm_touch_ok<AL, WL, BM>() ? WM * WN * 256 : 0);
   static bool attr_set = false;  // per instantiation; idempotent, so a race only repeats the call
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
