@@ -352,6 +352,9 @@ def main():
     ap.add_argument("--units", type=int, default=1, help="independent weight sets per GEMV launch")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
+    ap.add_argument("--tune", action="append", default=[], metavar="HOOK=VALUE",
+                    help="call a single-integer tuning hook of the library before measuring, e.g. --tune gemm_slots=1 "
+                         "(tlq_tune_gemm_slots(1)); repeatable; recorded in the output line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain elementwise copy of 256 MiB (int32 x+0 -> y) after the timed region, "
                          "the known-size kernel that hardware traffic counters are scaled by")
@@ -368,6 +371,21 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+
+    tuned = {}
+    if args.tune:
+        from tilelang_ascend_amd import _abi
+
+        lib = _abi.load()
+        for item in args.tune:
+            name, _, value = item.partition("=")
+            hook = "tlq_tune_" + name.strip()
+            sig = _abi.SIGNATURES.get(hook)
+            if sig is None or len(sig[1]) != 1:
+                print(f"bench.py: no single-integer tuning hook {hook}", file=sys.stderr)
+                sys.exit(2)
+            getattr(lib, hook)(int(value))
+            tuned[hook] = int(value)
 
     if args.workload == "gemv":
         line = bench_gemv(args, cpu=not args.no_cpu_baseline)
@@ -406,6 +424,8 @@ def main():
         torch.cuda.synchronize()
     line.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
                  "vs_baseline": None, "data": "synthetic"})
+    if tuned:
+        line["tuning_hooks"] = tuned
     order = ["metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
              "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"]
     out = {k: line[k] for k in order if k in line}
