@@ -30,8 +30,9 @@ def _with_hook(name, value, fn):
 
 # K in 16-bit values: one, two, three stages (64 values each), odd stage counts, a partial last stage (falls back /
 # register tail), long rows; M, N ragged against the 256 x 256 tile
-SHAPES_16 = [(256, 256, 64), (256, 512, 128), (300, 520, 192), (512, 256, 320), (1000, 1288, 4160), (4096, 4096, 4096),
-             (260, 264, 96), (2048, 2304, 72)]
+# (the 256 x 256 kernels, which the slots path replaces, are chosen from 128 output tiles on: M, N around 2900)
+SHAPES_16 = [(256, 256, 64), (300, 520, 192), (1000, 1288, 4160), (4096, 4096, 4096), (260, 264, 96), (2048, 2304, 72),
+             (2900, 2900, 64), (2900, 2824, 128), (3000, 2820, 192), (2816, 3072, 320), (2820, 2900, 72)]
 
 
 @pytest.mark.parametrize("hook,value", HOOKS)
@@ -75,11 +76,15 @@ def test_w8a8_same_bits_as_default(hook, value, layout, B, M, N, K):
     lay = _abi.B_KN if layout == "KN" else _abi.B_NK
 
     def run():
-        C = torch.full((B, M, N), float("nan"), dtype=torch.float16, device="cuda")
-        _abi.check(lib.tlq_gemm_w8a8(P(A), P(W), P(sa), P(sb), P(C), B, M, N, K, N, lay, _abi.F16, st))
-        Ci = torch.full((B, M, N), -1, dtype=torch.int32, device="cuda")
-        _abi.check(lib.tlq_gemm_i8(P(A), P(W), P(Ci), B, M, N, K, lay, st))
-        torch.cuda.synchronize()
+        lib.tlq_tune_i8_tile(256)  # the kernel the slots path replaces, whatever the number of tiles
+        try:
+            C = torch.full((B, M, N), float("nan"), dtype=torch.float16, device="cuda")
+            _abi.check(lib.tlq_gemm_w8a8(P(A), P(W), P(sa), P(sb), P(C), B, M, N, K, N, lay, _abi.F16, st))
+            Ci = torch.full((B, M, N), -1, dtype=torch.int32, device="cuda")
+            _abi.check(lib.tlq_gemm_i8(P(A), P(W), P(Ci), B, M, N, K, lay, st))
+            torch.cuda.synchronize()
+        finally:
+            lib.tlq_tune_i8_tile(0)
         return C.cpu(), Ci.cpu()
 
     want, want_i = run()
