@@ -171,3 +171,71 @@ def test_lds_swizzle_is_a_bijection_and_spreads_banks():
     # tile fill: 8 consecutive lanes write the 8 chunks of one row -> 8 distinct slots as well
     for r in range(rows):
         assert len({(lds_off(r, c) % 128) // 16 for c in range(8)}) == 8
+
+
+def test_five_slot_schedule_keeps_every_tile_until_it_is_read():
+    """Restatement of the issue / wait order of gemm_slots_kernel (csrc/gemm_slots.h) for one wavefront: tile t lives
+    in slot t % 5 (A of stage s is t = 2s, W is t = 2s + 1); loads retire in issue order, `wait(keep)` guarantees all
+    tiles but the youngest when keep is set.  No slot may be reloaded before its tile was multiplied, and every tile
+    must be covered by a wait before its stage."""
+    def run(KT):
+        issued, owner, read = [], {}, set()
+        landed = 0
+
+        def issue(name, t):
+            prev = owner.get(t % 5)
+            assert prev is None or prev in read, (KT, name, "overwrites", prev)
+            owner[t % 5] = name
+            issued.append(name)
+
+        issue("A0", 0)
+        issue("W0", 1)
+        if KT > 1:
+            issue("A1", 2)
+        landed = len(issued) - (1 if KT > 1 else 0)
+        for k in range(KT):
+            if k + 1 < KT:
+                issue(f"W{k + 1}", 2 * k + 3)
+            if k + 2 < KT:
+                issue(f"A{k + 2}", 2 * k + 4)
+            for name, t in ((f"A{k}", 2 * k), (f"W{k}", 2 * k + 1)):
+                assert issued.index(name) < landed, (KT, name, "not waited for")
+                assert owner[t % 5] == name, (KT, name, "slot taken by", owner[t % 5])
+            read.update((f"A{k}", f"W{k}"))
+            if k + 1 < KT:
+                keep = k + 2 < KT
+                assert not keep or issued[-1] == f"A{k + 2}"
+                landed = len(issued) - (1 if keep else 0)
+
+    for KT in range(1, 48):
+        run(KT)
+
+
+def test_touch_addresses_stay_inside_the_matrices():
+    """Restatement of touch_ptr / touch_step (csrc/gemm_core.h): the byte a thread touches for stage kt lies inside
+    its matrix for every whole stage, for row-major operands and for int8 weights stored [K, N]."""
+    rng = np.random.default_rng(5)
+    for _ in range(200):
+        M = int(rng.integers(1, 700))
+        kb = int(rng.integers(1, 40)) * 16 + int(rng.integers(0, 2)) * 128 * int(rng.integers(0, 30))  # bytes of K per row
+        KT = -(-kb // 128)
+        last_full = KT - 2 if kb % 128 else KT - 1
+        m0 = (int(rng.integers(0, -(-M // 256)))) * 256
+        for i in (0, 1, 127, 255):
+            row = m0 + i if m0 + i < M else M - 1
+            for kt in range(0, last_full + 1):
+                off = row * kb + kt * 128
+                assert 0 <= off and off + 4 <= M * kb
+        # [K, N] int8: line i of a stage is k row i // (BN / 128), 128-byte column block i % (BN / 128)
+        N = int(rng.integers(1, 60)) * 16
+        K = int(rng.integers(1, 30)) * 16
+        BN = 256
+        n0 = int(rng.integers(0, -(-N // BN))) * BN
+        KT = -(-K // 128)
+        last_full = KT - 2 if K % 128 else KT - 1
+        for i in (0, 1, 2, 255):
+            k, c = i // (BN // 128), n0 + (i % (BN // 128)) * 128
+            col = c if c < N else n0
+            for kt in range(0, last_full + 1):
+                off = (kt * 128 + k) * N + col
+                assert off + 4 <= K * N, (N, K, i, kt)
