@@ -122,6 +122,21 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose wrapper allocates its
+ * workspace anew on every call (tilelang/jit/adapter/cython/cython_wrapper.pyx:128-129).  The workspace is
+ * a device array built into the library, TLQ_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends; problems whose
+ * tlq_w4a16_workspace_bytes(M, N, K) exceeds it are rejected with an error (use tlq_gemm_w4a16_ws for those).  The call
+ * allocates and frees nothing; results are those of tlq_gemm_w4a16_ws with a sufficient workspace, bit for bit.  All
+ * calls on one GPU share the array: calls that overlap there (other streams, other threads) race.
+ * tlq_gemm_w4a16_noalloc_init looks the array's address up for the current device (otherwise the first call on a
+ * device does it); it allocates nothing either. */
+#define TLQ_NOALLOC_SCRATCH_BYTES (64 << 20)
+int tlq_gemm_w4a16_noalloc_init(void);
+int tlq_gemm_w4a16_noalloc(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
+                           int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
+                           void* stream);
+
 /* `batch` independent decode GEMVs in one launch (one grid row per problem): A [batch,M,K],
  * w_packed [batch,N,K/2], scales / zeros [batch,N,K/group], C [batch,M,N], all contiguous.
  * Same arithmetic as tlq_gemm_w4a16 with TLQ_ALGO_GEMV; M <= 16.  This is the shape of a decode
@@ -196,6 +211,18 @@ int tlq_quantize_sym4(const void* W, void* q_minus8, void* scales, int64_t N, in
  * X: [M,N] in_dtype (TLQ_BF16 like the reference, TLQ_F16 or TLQ_F32), Y: int8 [M,N], S: fp32 [M].
  * Its outputs are the A / scale_a operands of tlq_gemm_w8a8. */
 int tlq_act_quant_i8(const void* X, void* Y, void* S, int64_t M, int64_t N, int in_dtype, int round_scale, void* stream);
+
+/* Self-checks of the MFMA GEMM kernels' address arithmetic, evaluated on the HOST with the functions the kernels
+ * themselves use (no GPU needed; the reference has no counterpart, its tile addressing is generated by TVM).
+ * tlq_debug_check_gemm_addressing walks every tile, thread, load instruction and stage of one operand:
+ * source_kind 0 = row-major [rows, row_bytes] operand copied global -> LDS directly in tiles of `tile` rows by
+ * `threads` threads; 1 = int8 [K = rows, N = row_bytes] weights in tiles of `tile` (128 | 256) columns.  It checks
+ * global extents, LDS extents and coverage, agreement with the operand-fragment reads, and the touch-ahead addresses.
+ * tlq_debug_check_slots_schedule simulates the five-slot kernel's issue / wait / barrier order over `stages` stages
+ * with `loads_per_tile` load instructions per wavefront and tile (the kernel's waits assume 4).
+ * Both return 0 when everything holds, else 1 with tlq_last_error() naming the first violation. */
+int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads, int touch_ahead);
+int tlq_debug_check_slots_schedule(int stages, int loads_per_tile);
 
 /* Tuning hooks for benchmark sweeps (process-global, not thread safe; 0 = automatic choice).
  * They play the role of the reference's block_M / block_N / block_K factory arguments

@@ -1,0 +1,65 @@
+"""Host-side walk of the MFMA GEMM kernels' address arithmetic (csrc/gemm_addr.h through
+tlq_debug_check_gemm_addressing / tlq_debug_check_slots_schedule): the functions the kernels use for their
+global offsets, LDS offsets, touch-ahead addresses and for the five-slot issue / wait order are evaluated on the
+CPU for every tile, thread and stage of a launch and compared with the buffer extents.  The shapes are those of
+the GPU comparison tests of the two opt-in paths plus ragged and very short cases.
+"""
+import pytest
+
+from tilelang_ascend_amd import _abi
+
+
+def _ok(rc):
+    assert rc == 0, _abi.last_error()
+
+
+# (rows, K in 16-bit values): the activation (rows = M) and [N, K] weight (rows = N) operands of the 16-bit GEMMs
+SHAPES_16 = [(256, 256, 64), (300, 520, 192), (1000, 1288, 4160), (4096, 4096, 4096), (260, 264, 96), (2048, 2304, 72),
+             (2900, 2900, 64), (2900, 2824, 128), (3000, 2820, 192), (2816, 3072, 320), (2820, 2900, 72),
+             (1, 8, 8), (7, 16, 24), (255, 257 * 8, 64), (513, 1000, 136)]
+W8A8 = [(1, 256, 256, 128), (2, 300, 528, 384), (1, 2048, 4096, 4096), (3, 512, 272, 640), (1, 260, 512, 144),
+        (1, 1, 16, 16), (1, 33, 48, 272)]
+
+
+@pytest.mark.parametrize("touch", [0, 2, 3])
+@pytest.mark.parametrize("tile,threads", [(256, 512), (128, 256)])
+def test_row_operands_of_the_16_bit_gemms(tile, threads, touch):
+    lib = _abi.load()
+    for M, N, K in SHAPES_16:
+        for rows in (M, N):
+            _ok(lib.tlq_debug_check_gemm_addressing(0, rows, K * 2, tile, threads, touch))
+
+
+@pytest.mark.parametrize("touch", [0, 2, 3])
+def test_int8_operands(touch):
+    lib = _abi.load()
+    for _, M, N, K in W8A8:
+        for tile, threads in ((256, 512), (128, 256), (32, 256)):
+            _ok(lib.tlq_debug_check_gemm_addressing(0, M, K, tile, threads, touch))        # activations [M, K]
+        for tile, threads in ((256, 512), (128, 256)):
+            _ok(lib.tlq_debug_check_gemm_addressing(0, N, K, tile, threads, touch))        # weights [N, K]
+            _ok(lib.tlq_debug_check_gemm_addressing(1, K, N, tile, threads, touch))        # weights [K, N]
+        _ok(lib.tlq_debug_check_gemm_addressing(1, K, N, 128, 256, touch))                 # the 32-row kernel's weights
+
+
+def test_the_walker_rejects_what_it_should():
+    lib = _abi.load()
+    assert lib.tlq_debug_check_gemm_addressing(0, 256, 256, 250, 512, 0) != 0      # tile rows not a multiple of 8
+    assert lib.tlq_debug_check_gemm_addressing(0, 256, 256, 64, 1024, 0) != 0      # fewer load instructions than wavefronts
+    assert lib.tlq_debug_check_gemm_addressing(0, 1 << 20, 1 << 13, 256, 512, 0) != 0  # 8 GiB operand: 32-bit offsets
+    assert lib.tlq_debug_check_gemm_addressing(1, 128, 24, 256, 512, 0) != 0       # N not a multiple of 16
+    assert lib.tlq_debug_check_gemm_addressing(2, 128, 128, 256, 512, 0) != 0
+    assert "bad source kind" in _abi.last_error()
+
+
+def test_five_slot_schedule():
+    """Every tile is waited for and published by a barrier before it is multiplied, and no load overwrites a tile
+    that some wavefront may still read: for 1..64 stages, with the four load instructions per wavefront and tile that
+    the kernel's waits count.  With fewer loads per tile the same waits would leave two tiles in flight, and the check
+    says so; with more they wait for more than they need to."""
+    lib = _abi.load()
+    for stages in range(1, 65):
+        _ok(lib.tlq_debug_check_slots_schedule(stages, 4))
+    assert lib.tlq_debug_check_slots_schedule(8, 2) != 0
+    assert "before its loads were waited for" in _abi.last_error()
+    _ok(lib.tlq_debug_check_slots_schedule(8, 8))

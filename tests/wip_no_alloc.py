@@ -1,0 +1,70 @@
+"""tlq_gemm_w4a16_noalloc (the entry point that allocates nothing: its workspace is a device array built into the
+library) against tlq_gemm_w4a16_ws with a caller-owned workspace, through the C ABI, bit for bit: the same kernels run
+in the same order, only the workspace address differs.  Two calls in a row share the built-in array, the second on a
+smaller problem, so stale contents of the first call lie behind and beside what the second one uses.
+"""
+import pytest
+import torch
+
+from helpers import assert_bit_equal, check_float_output, gen, make_w4, w4a16_reference
+
+pytestmark = pytest.mark.gpu
+
+SCRATCH = 64 << 20
+
+
+def _both(M, N, K, group, dtype, zeros_kind, seed):
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    code = _abi.F16 if dtype == torch.float16 else _abi.BF16
+    A = torch.randn(M, K, generator=gen(seed)).to(dtype)
+    Wp, s, z = make_w4(N, K, group, dtype, zeros_kind, seed + 1)
+    zt = z if torch.is_tensor(z) else None
+    zs = 0.0 if torch.is_tensor(z) or z is None else float(z)
+    dA, dW, dS = A.cuda(), Wp.cuda(), s.cuda()
+    dZ = zt.cuda() if zt is not None else None
+    st = torch.cuda.current_stream().cuda_stream
+    need = lib.tlq_w4a16_workspace_bytes(M, N, K)
+    assert 0 < need <= SCRATCH, f"the case must use scratch memory and fit the built-in array (needs {need})"
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    want = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    _abi.check(lib.tlq_gemm_w4a16_ws(P(dA), P(dW), P(dS), P(dZ), P(want), M, N, K, group, zs, code, code, _abi.ALGO_AUTO,
+                                     P(ws), need, st))
+    got = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    before = torch.cuda.memory_allocated()
+    _abi.check(lib.tlq_gemm_w4a16_noalloc(P(dA), P(dW), P(dS), P(dZ), P(got), M, N, K, group, zs, code, code,
+                                          _abi.ALGO_AUTO, st))
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    return got.cpu(), want.cpu(), (A, Wp, s, z)
+
+
+def test_noalloc_matches_the_workspace_entry_point_twice_in_a_row():
+    from tilelang_ascend_amd import _abi
+
+    lib = _abi.load()
+    assert lib.tlq_gemm_w4a16_noalloc_init() == 0, _abi.last_error()
+    # first call: two passes (the dequantised 4096 x 2048 bf16 matrix, 16 MiB of the array)
+    got, want, _ = _both(2048, 4096, 2048, 128, torch.bfloat16, "scalar8", 11)
+    assert_bit_equal(got, want, "two-pass problem")
+    # second call, smaller: K slices whose fp32 partial sums overlay the start of the first call's matrix
+    got, want, (A, Wp, s, z) = _both(48, 1024, 2048, 64, torch.float16, "int", 21)
+    assert_bit_equal(got, want, "split-K problem after a larger call")
+    check_float_output(got, w4a16_reference(A, Wp, s, z, 64), "split-K problem vs the oracle")
+    # and once more the first shape with other data: nothing of the second call may leak into it
+    got, want, _ = _both(2048, 4096, 2048, 128, torch.bfloat16, "scalar8", 31)
+    assert_bit_equal(got, want, "two-pass problem, third call")
+
+
+def test_noalloc_rejects_what_does_not_fit():
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    M, N, K = 2048, 14336, 4096  # two passes would need 112 MiB
+    assert lib.tlq_w4a16_workspace_bytes(M, N, K) > SCRATCH
+    A = torch.zeros(8, dtype=torch.float16, device="cuda")  # never read: the call is rejected before any launch
+    rc = lib.tlq_gemm_w4a16_noalloc(P(A), P(A), None, None, P(A), M, N, K, 128, 8.0, _abi.F16, _abi.F16, _abi.ALGO_AUTO, None)
+    assert rc != 0
+    msg = _abi.last_error()
+    assert "built-in array holds" in msg and "tlq_gemm_w4a16_ws" in msg

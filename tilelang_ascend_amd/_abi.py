@@ -39,11 +39,15 @@ SIGNATURES = {
     "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_w4a16_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "tlq_gemm_w4a16_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp, _i64, _vp]),
+    "tlq_gemm_w4a16_noalloc_init": (_int, []),
+    "tlq_gemm_w4a16_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp]),
     "tlq_gemm_f16_splitk": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_gemv": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "tlq_pack_int4": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "tlq_quantize_sym4": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "tlq_act_quant_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
+    "tlq_debug_check_gemm_addressing": (_int, [_int, _i64, _i64, _int, _int, _int]),
+    "tlq_debug_check_slots_schedule": (_int, [_int, _int]),
     "tlq_tune_gemv": (None, [_int, _int]),
     "tlq_tune_gemv_unroll": (None, [_int]),
     "tlq_tune_gemv_depth": (None, [_int]),

@@ -37,6 +37,8 @@ SOURCES = [
     "gemm_int8.hip",
     "gemm_f16.hip",
     "gemm_api.hip",
+    "gemm_addr_check.hip",
+    "gemm_w4a16_noalloc.hip",
 ]
 # packed-fp32 VALU forms are disabled on purpose (some have produced silent wrong results on
 # this hardware pool); hipcc's host pass warns that it does not know the feature.

@@ -1,0 +1,247 @@
+// Host-side walkers over the address arithmetic of the MFMA GEMM kernels (gemm_addr.h).  They evaluate, for every
+// work-group, thread, load instruction and stage of a launch, the very functions the kernels use, and check that
+//   * every global byte read lies inside the operand matrix,
+//   * every direct load lands inside its LDS tile, every 16-byte cell of the tile is written exactly once, and holds
+//     the (row, K chunk) that the operand-fragment read of that cell expects,
+//   * every touch-ahead address lies inside the matrix,
+//   * the five-slot schedule never overwrites a tile that has not been multiplied and never multiplies a tile whose
+//     loads were not waited for.
+// No GPU is needed: these run in the CPU-only test suite and can be called before a launch.
+#include <vector>
+
+#include "gemm_addr.h"
+#include "tlq_common.h"
+
+namespace tlq {
+namespace {
+
+#define CHECK_OR_FAIL(cond, ...) \
+  do {                           \
+    if (!(cond)) {               \
+      set_error(__VA_ARGS__);    \
+      return 1;                  \
+    }                            \
+  } while (0)
+
+// Row-major operand [rows_total, k_bytes] (pitch = k_bytes), tiles of `tile_rows` rows loaded by `threads` threads.
+int check_row_direct(int64_t rows_total, int64_t k_bytes, int tile_rows, int threads, int touch_ahead) {
+  CHECK_OR_FAIL(tile_rows % 8 == 0 && threads % 64 == 0, "row loader: tile rows %d / threads %d", tile_rows, threads);
+  const int waves = threads / 64, instr = tile_rows / 8;
+  CHECK_OR_FAIL(instr % waves == 0 && instr >= waves, "row loader: %d load instructions do not split over %d wavefronts", instr, waves);
+  CHECK_OR_FAIL(k_bytes > 0 && k_bytes % 16 == 0 && rows_total > 0, "row loader: bad matrix %lld x %lld bytes",
+                (long long)rows_total, (long long)k_bytes);
+  CHECK_OR_FAIL(rows_total * k_bytes < ((int64_t)1 << 32), "row loader: the matrix spans 4 GiB or more");
+  const int per_wave = instr / waves;
+  const int64_t extent = rows_total * k_bytes;
+  const int KT = (int)((k_bytes + addr::kStage - 1) / addr::kStage);
+  const bool tail = k_bytes % addr::kStage != 0;
+  const int last_full = tail ? KT - 2 : KT - 1;
+  const uint32_t ld = (uint32_t)k_bytes;
+  std::vector<int> cell(tile_rows * 8);
+  for (int64_t row0 = 0; row0 < rows_total; row0 += tile_rows) {
+    const int rows_valid = (int)(rows_total - row0);
+    std::fill(cell.begin(), cell.end(), -1);
+    for (int wave = 0; wave < waves; ++wave)
+      for (int j = 0; j < per_wave; ++j)
+        for (int lane = 0; lane < 64; ++lane) {
+          const uint32_t voff = addr::rd_voff(lane, wave, j, waves, rows_valid, ld);
+          const int kb_lane = addr::rd_chunk(lane) * 16;
+          // whole stages: direct loads of 16 bytes
+          for (int kt = 0; kt <= last_full; ++kt) {
+            const int64_t o = row0 * k_bytes + (int64_t)voff + (int64_t)kt * addr::kStage;
+            CHECK_OR_FAIL(o >= 0 && o + 16 <= extent, "row loader: tile row %lld wave %d instr %d lane %d stage %d reads [%lld, +16) of %lld",
+                          (long long)row0, wave, j, lane, kt, (long long)o, (long long)extent);
+          }
+          if (tail) {  // the partial stage: lanes past the end of the row re-read the row's first bytes and zero them
+            const bool ok = (int64_t)(KT - 1) * addr::kStage + kb_lane < k_bytes;
+            const int64_t o = row0 * k_bytes + (ok ? (int64_t)voff + (int64_t)(KT - 1) * addr::kStage : (int64_t)voff - kb_lane);
+            CHECK_OR_FAIL(o >= 0 && o + 16 <= extent, "row loader: tail stage reads [%lld, +16) of %lld", (long long)o, (long long)extent);
+          }
+          // LDS side
+          const uint32_t l = addr::direct_lds_off(lane, wave, j, waves);
+          CHECK_OR_FAIL(l % 16 == 0 && l + 16 <= (uint32_t)tile_rows * addr::kStage, "row loader: LDS offset %u outside the %d-row tile", l,
+                        tile_rows);
+          CHECK_OR_FAIL(cell[l / 16] == -1, "row loader: LDS cell %u written twice", l / 16);
+          const int row = addr::rd_row(lane, wave, j, waves), chunk = addr::rd_chunk(lane);
+          CHECK_OR_FAIL(row < tile_rows, "row loader: row %d outside the tile", row);
+          CHECK_OR_FAIL((uint32_t)addr::row_lds_off(row, chunk) == l, "row loader: (row %d, chunk %d) lands at %u, the operand read expects %d", row,
+                        chunk, l, addr::row_lds_off(row, chunk));
+          cell[l / 16] = row * 8 + chunk;
+        }
+    for (size_t c = 0; c < cell.size(); ++c) CHECK_OR_FAIL(cell[c] >= 0, "row loader: LDS cell %zu never written", c);
+    // operand reads: every (16-row tile, k-step, lane) reads the cell that holds (its row, its chunk)
+    for (int wave_row0 = 0; wave_row0 < tile_rows; wave_row0 += 16)
+      for (int lane = 0; lane < 64; ++lane) {
+        const uint32_t base = addr::rowfrag_base(lane, wave_row0);
+        for (int ks = 0; ks < 2; ++ks) {
+          const uint32_t off = addr::rowfrag_off(base, ks, 0);
+          CHECK_OR_FAIL(off + 16 <= (uint32_t)tile_rows * addr::kStage, "operand read at %u outside the tile", off);
+          const int want = (wave_row0 + (lane & 15)) * 8 + ks * 4 + (lane >> 4);
+          CHECK_OR_FAIL(cell[off / 16] == want, "operand read (row0 %d lane %d k-step %d) finds cell %d, expects %d", wave_row0, lane, ks,
+                        cell[off / 16], want);
+        }
+      }
+    // touch-ahead: one 4-byte load per cache line of the stage `touch_ahead` stages further on
+    if (touch_ahead > 0)
+      for (int i = 0; i < tile_rows; ++i)
+        for (int kt = 0; kt + touch_ahead <= last_full; ++kt) {
+          const int64_t o = addr::row_touch_off((int)row0, (int)rows_total, i, k_bytes) + (int64_t)(kt + touch_ahead) * addr::kStage;
+          CHECK_OR_FAIL(o >= 0 && o + 4 <= extent, "row touch: line %d stage %d at %lld of %lld", i, kt, (long long)o, (long long)extent);
+        }
+  }
+  return 0;
+}
+
+// int8 operand stored [K, N] (pitch N), tiles of BN columns x 128 k rows.
+template <int BN>
+int check_kn_direct(int64_t K, int64_t N, int threads, int touch_ahead) {
+  CHECK_OR_FAIL(threads % 64 == 0, "[K,N] loader: threads %d", threads);
+  const int waves = threads / 64, kpi = 1024 / BN, instr = addr::kStage / kpi;
+  CHECK_OR_FAIL(instr % waves == 0 && instr >= waves, "[K,N] loader: %d load instructions do not split over %d wavefronts", instr, waves);
+  CHECK_OR_FAIL(K > 0 && N >= 16 && N % 16 == 0, "[K,N] loader: bad matrix K=%lld N=%lld", (long long)K, (long long)N);
+  CHECK_OR_FAIL(K * N < ((int64_t)1 << 32), "[K,N] loader: the matrix spans 4 GiB or more");
+  const int per_wave = instr / waves;
+  const int64_t extent = K * N;
+  const int KT = (int)((K + addr::kStage - 1) / addr::kStage);
+  const bool tail = K % addr::kStage != 0;
+  const int last_full = tail ? KT - 2 : KT - 1;
+  std::vector<int> cell(addr::kStage * BN / 16);
+  for (int64_t col0 = 0; col0 < N; col0 += BN) {
+    const int cols_valid = (int)(N - col0);
+    std::fill(cell.begin(), cell.end(), -1);
+    for (int wave = 0; wave < waves; ++wave)
+      for (int j = 0; j < per_wave; ++j)
+        for (int lane = 0; lane < 64; ++lane) {
+          const uint32_t voff = addr::kn_voff<BN>(lane, wave, j, waves, cols_valid, (uint32_t)N);
+          const int k = addr::kn_k<BN>(lane, wave, j, waves);
+          CHECK_OR_FAIL(k < addr::kStage, "[K,N] loader: k row %d outside the stage", k);
+          for (int kt = 0; kt <= last_full; ++kt) {
+            const int64_t o = col0 + (int64_t)voff + (int64_t)kt * addr::kStage * N;
+            CHECK_OR_FAIL(o >= 0 && o + 16 <= extent, "[K,N] loader: col %lld wave %d instr %d lane %d stage %d reads [%lld, +16) of %lld",
+                          (long long)col0, wave, j, lane, kt, (long long)o, (long long)extent);
+          }
+          if (tail) {  // k rows past K re-read k row 0 of the stage base ... of the matrix (then zeroed)
+            const bool ok = (int64_t)(KT - 1) * addr::kStage + k < K;
+            const int64_t o = col0 + (ok ? (int64_t)voff + (int64_t)(KT - 1) * addr::kStage * N : (int64_t)voff - (int64_t)k * N);
+            CHECK_OR_FAIL(o >= 0 && o + 16 <= extent, "[K,N] loader: tail stage reads [%lld, +16) of %lld", (long long)o, (long long)extent);
+          }
+          const uint32_t l = addr::direct_lds_off(lane, wave, j, waves);
+          CHECK_OR_FAIL(l % 16 == 0 && l + 16 <= (uint32_t)addr::kStage * BN, "[K,N] loader: LDS offset %u outside the tile", l);
+          CHECK_OR_FAIL(cell[l / 16] == -1, "[K,N] loader: LDS cell %u written twice", l / 16);
+          const int pc = lane % (BN / 16);
+          CHECK_OR_FAIL(l == (uint32_t)(k * BN + pc * 16), "[K,N] loader: lane lands at %u, not on (k %d, chunk %d)", l, k, pc);
+          cell[l / 16] = k * (BN / 16) + (pc ^ addr::kn_swz<BN>(k));  // the logical 16-column chunk this cell holds
+        }
+    for (size_t c = 0; c < cell.size(); ++c) CHECK_OR_FAIL(cell[c] >= 0, "[K,N] loader: LDS cell %zu never written", c);
+    // transposing operand reads: lane (r16, q) of column block t supplies the row of k = 16 q + r16 / 2 (+ 8 for the second
+    // read, + 64 for k-step 1) at columns 16 (wave_row0 / 16 + t) + 8 (r16 % 2)
+    for (int wave_row0 = 0; wave_row0 + 64 <= BN; wave_row0 += 64)
+      for (int t = 0; t < 4; ++t)
+        for (int lane = 0; lane < 64; ++lane)
+          for (int ks = 0; ks < 2; ++ks)
+            for (int h = 0; h < 2; ++h) {
+              const uint32_t off = addr::knfrag_off<BN>(lane, wave_row0, t) + (uint32_t)(ks * 64 * BN + h * 8 * BN);
+              CHECK_OR_FAIL(off + 8 <= (uint32_t)addr::kStage * BN, "[K,N] operand read at %u outside the tile", off);
+              const int k = (lane >> 4) * 16 + ((lane & 15) >> 1) + 8 * h + 64 * ks;
+              const int want = k * (BN / 16) + (wave_row0 >> 4) + t;
+              CHECK_OR_FAIL(cell[off / 16] == want && (int)(off % 16) == 8 * (lane & 1), "[K,N] operand read (lane %d t %d) finds cell %d, expects %d",
+                            lane, t, cell[off / 16], want);
+            }
+    if (touch_ahead > 0)
+      for (int i = 0; i < addr::kStage * (BN / 128); ++i)
+        for (int kt = 0; kt + touch_ahead <= last_full; ++kt) {
+          const int64_t o = addr::kn_touch_off<BN>((int)col0, (int)N, i, N) + (int64_t)(kt + touch_ahead) * addr::kStage * N;
+          CHECK_OR_FAIL(o >= 0 && o + 4 <= extent, "[K,N] touch: line %d stage %d at %lld of %lld", i, kt, (long long)o, (long long)extent);
+        }
+  }
+  return 0;
+}
+
+// One wavefront running addr::slots_schedule; every tile is `loads_per_tile` load instructions of that wavefront.
+struct SlotsSim {
+  int loads_per_tile;
+  std::vector<int> in_flight;  // tile ids of the load instructions not yet known to have landed, oldest first
+  int owner[addr::kSlots];     // tile id whose data (or pending load) occupies the slot, -1 = empty
+  bool landed[addr::kSlots];   // the owner's loads have been waited for
+  bool published[addr::kSlots];  // ... and a barrier has passed since (every wavefront's part is in)
+  std::vector<char> multiplied;  // per tile id
+  int error = 0;
+  char msg[160] = "";
+  SlotsSim(int KT, int lpt) : loads_per_tile(lpt), multiplied(2 * KT, 0) {
+    for (int s = 0; s < addr::kSlots; ++s) owner[s] = -1, landed[s] = published[s] = false;
+  }
+  void fail(const char* what, int t) {
+    if (!error) snprintf(msg, sizeof(msg), "five-slot schedule: %s (tile %d)", what, t);
+    error = 1;
+  }
+  void issue(int t) {
+    const int s = addr::slot_of_tile(t);
+    if (owner[s] >= 0 && !multiplied[owner[s]]) fail("a load overwrites a tile that was not multiplied yet", owner[s]);
+    // other wavefronts may still be multiplying the previous owner unless a barrier followed its stage
+    if (owner[s] >= 0 && multiplied[owner[s]] == 2) fail("a load overwrites a tile other wavefronts may still read", owner[s]);
+    owner[s] = t, landed[s] = published[s] = false;
+    for (int i = 0; i < loads_per_tile; ++i) in_flight.push_back(t);
+  }
+  void issue_a(int s) { issue(2 * s); }
+  void issue_w(int s) { issue(2 * s + 1); }
+  void wait_tiles(bool keep) {
+    const size_t leave = keep ? 4 : 0;  // the literal operand of s_waitcnt vmcnt in the kernel
+    while (in_flight.size() > leave) {
+      const int t = in_flight.front();
+      in_flight.erase(in_flight.begin());
+      bool more = false;
+      for (int u : in_flight) more |= (u == t);
+      if (!more && owner[addr::slot_of_tile(t)] == t) landed[addr::slot_of_tile(t)] = true;
+    }
+  }
+  void barrier() {
+    for (int s = 0; s < addr::kSlots; ++s) published[s] = landed[s];
+    for (auto& m : multiplied)
+      if (m == 2) m = 1;  // everyone is past that stage now
+  }
+  void compute(int k) {
+    for (int t = 2 * k; t <= 2 * k + 1; ++t) {
+      const int s = addr::slot_of_tile(t);
+      if (owner[s] != t) fail("the slot of a tile to be multiplied holds another tile", t);
+      else if (!published[s]) fail("a tile is multiplied before its loads were waited for and published by a barrier", t);
+      multiplied[t] = 2;  // 2 = by this wavefront, other wavefronts may lag until the next barrier
+    }
+  }
+};
+
+}  // namespace
+}  // namespace tlq
+
+using namespace tlq;
+
+extern "C" {
+
+int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads, int touch_ahead) {
+  if (source_kind == 0) return check_row_direct(rows, row_bytes, tile, threads, touch_ahead);
+  if (source_kind == 1) {
+    if (tile == 256) return check_kn_direct<256>(rows, row_bytes, threads, touch_ahead);
+    if (tile == 128) return check_kn_direct<128>(rows, row_bytes, threads, touch_ahead);
+    set_error("tlq_debug_check_gemm_addressing: [K,N] tiles are 128 or 256 columns wide (got %d)", tile);
+    return 1;
+  }
+  set_error("tlq_debug_check_gemm_addressing: bad source kind %d", source_kind);
+  return 1;
+}
+
+int tlq_debug_check_slots_schedule(int stages, int loads_per_tile) {
+  if (stages < 1 || loads_per_tile < 1) {
+    set_error("tlq_debug_check_slots_schedule: bad arguments");
+    return 1;
+  }
+  SlotsSim sim(stages, loads_per_tile);
+  addr::slots_schedule(stages, sim);
+  for (int t = 0; t < 2 * stages && !sim.error; ++t)
+    if (!sim.multiplied[t]) sim.fail("a tile was never multiplied", t);
+  if (sim.error) {
+    set_error("%s", sim.msg);
+    return 1;
+  }
+  return 0;
+}
+
+}  // extern "C"

@@ -24,6 +24,7 @@
 
 #include <type_traits>
 
+#include "gemm_addr.h"
 #include "tlq_common.h"
 
 namespace tlq {
@@ -33,8 +34,9 @@ constexpr int kStageBytes = 128;
 // 16-byte chunk swizzle.  Measured on gfx950 with the LDS bank-conflict counter: conflict free
 // for the MFMA operand reads (16 consecutive rows, one logical chunk per 16 lanes), the row-copy
 // stores (8 lanes per row) and the dequantising stores (2 lanes per row, 4 chunks each).
-__device__ __forceinline__ int lds_swz(int row) { return row & 7; }
-__device__ __forceinline__ int lds_off(int row, int chunk) { return row * kStageBytes + ((chunk ^ lds_swz(row)) << 4); }
+static_assert(kStageBytes == addr::kStage, "stage width");
+__device__ __forceinline__ int lds_swz(int row) { return addr::row_swz(row); }
+__device__ __forceinline__ int lds_off(int row, int chunk) { return addr::row_lds_off(row, chunk); }
 
 // ---- MFMA operand fragments ---------------------------------------------------------------
 // A loader names the reader of its LDS tile layout as `Frag`:
@@ -46,9 +48,9 @@ __device__ __forceinline__ int lds_off(int row, int chunk) { return row * kStage
 struct RowFrag {
   uint32_t fo;
   __device__ __forceinline__ RowFrag(int lane, int wave_row0)
-      : fo((uint32_t)lds_off(lane & 15, lane >> 4) + (uint32_t)(wave_row0 * kStageBytes)) {}
+      : fo(addr::rowfrag_base(lane, wave_row0)) {}
   __device__ __forceinline__ uint4_t read(const uint8_t* tile, int ks, int t) const {
-    return *(const uint4_t*)(tile + (fo ^ (uint32_t)(ks << 6)) + t * 16 * kStageBytes);
+    return *(const uint4_t*)(tile + addr::rowfrag_off(fo, ks, t));
   }
 };
 
@@ -62,20 +64,16 @@ struct RowFrag {
 // the row-wise fill stores, spread over all banks.
 template <int BN>
 __device__ __forceinline__ int kn_swz(int k) {
-  static_assert(BN == 128 || BN == 256, "tile width");
-  return BN == 256 ? ((k & 7) | (((k >> 4) & 1) << 3)) : (((k >> 1) & 3) | (((k >> 4) & 1) << 2));
+  return addr::kn_swz<BN>(k);
 }
 template <int BN>
 struct KNFrag8 {
   typedef int v2i_t __attribute__((ext_vector_type(2)));
   uint32_t off[4];
   __device__ __forceinline__ KNFrag8(int lane, int wave_row0) {
-    const int r16 = lane & 15, q = lane >> 4;
-    const int krow = q * 16 + (r16 >> 1);
-    const int sw = kn_swz<BN>(krow);  // unchanged by the +8 (second read) and +64 (k-step) row offsets
-    const uint32_t base = (uint32_t)(krow * BN + 8 * (r16 & 1));
+    // the swizzle of a k row is unchanged by the +8 (second read) and +64 (k-step) row offsets
 #pragma unroll
-    for (int t = 0; t < 4; ++t) off[t] = base + (uint32_t)((((wave_row0 >> 4) + t) ^ sw) << 4);
+    for (int t = 0; t < 4; ++t) off[t] = addr::knfrag_off<BN>(lane, wave_row0, t);
   }
   __device__ __forceinline__ uint4_t read(const uint8_t* tile, int ks, int t) const {
     typedef __attribute__((address_space(3))) v2i_t* lds_ptr;
@@ -140,8 +138,7 @@ struct RowLoader {
   // line i of stage 0 of the tile that starts at row0 (the kernel touches the lines of a later stage ahead of time);
   // the same line of stage kt is touch_step(p) * kt bytes further
   static __device__ __forceinline__ const uint8_t* touch_ptr(const Params& p, int batch, int row0, int rows_total, int i) {
-    const int row = row0 + i < rows_total ? row0 + i : rows_total - 1;
-    return p.base + batch * p.batch_stride + (int64_t)row * p.ld;
+    return p.base + batch * p.batch_stride + addr::row_touch_off(row0, rows_total, i, p.ld);
   }
   static __device__ __forceinline__ int64_t touch_step(const Params&) { return kStageBytes; }
   const uint8_t* base;    // uniform
@@ -231,16 +228,11 @@ struct RowLoaderDirect {
     const int rows_valid = rows_total - row0;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    wave_off = (uint32_t)wave * 1024u;
-    lane_off = (uint32_t)lane * 16u;
-    const int chunk = (lane & 7) ^ ((lane >> 3) & 7);  // rows of one instruction start at a multiple of 8
-    kb_lane = chunk * 16;
+    wave_off = addr::direct_lds_off(0, wave, 0, WAVES);
+    lane_off = addr::direct_lds_off(lane, 0, 0, WAVES);
+    kb_lane = addr::rd_chunk(lane) * 16;  // rows of one instruction start at a multiple of 8
 #pragma unroll
-    for (int j = 0; j < PER_WAVE; ++j) {
-      int row = (j * WAVES + wave) * 8 + (lane >> 3);
-      row = row < rows_valid ? row : rows_valid - 1;
-      voff[j] = (uint32_t)row * (uint32_t)p.ld + (uint32_t)kb_lane;
-    }
+    for (int j = 0; j < PER_WAVE; ++j) voff[j] = addr::rd_voff(lane, wave, j, WAVES, rows_valid, (uint32_t)p.ld);
   }
 
   // The direct loads are written as inline assembly on purpose: while a compiler-visible direct load is
@@ -257,7 +249,7 @@ struct RowLoaderDirect {
       const uint32_t l0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lptr_t)lds_next + wave_off);
 #pragma unroll
       for (int j = 0; j < PER_WAVE; ++j)
-        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0 + (uint32_t)(j * WAVES * 1024)),
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0 + addr::direct_lds_off(0, 0, j, WAVES)),
                      "v"(voff[j]), "s"(sb)
                      : "memory");
     } else {
@@ -277,7 +269,7 @@ struct RowLoaderDirect {
 #pragma unroll
     for (int j = 0; j < PER_WAVE; ++j) {
       if (j * np / UNITS != pc) continue;
-      *(uint4_t*)(lds + wave_off + j * WAVES * 1024 + lane_off) = r.v[j];
+      *(uint4_t*)(lds + wave_off + addr::direct_lds_off(0, 0, j, WAVES) + lane_off) = r.v[j];
     }
   }
   __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
@@ -303,8 +295,7 @@ struct I8KNLoaderDirect {
   static constexpr bool PREFETCH2 = false;
   static constexpr int TOUCH_LINES = 128 * (BN / 128);  // 128 k rows of BN bytes
   static __device__ __forceinline__ const uint8_t* touch_ptr(const I8KNParams& p, int batch, int col0, int cols_total, int i) {
-    const int k = i / (BN / 128), c = col0 + (i % (BN / 128)) * 128;
-    return p.base + batch * p.batch_stride + (int64_t)k * p.ld + (c < cols_total ? c : col0);
+    return p.base + batch * p.batch_stride + addr::kn_touch_off<BN>(col0, cols_total, i, p.ld);
   }
   static __device__ __forceinline__ int64_t touch_step(const I8KNParams& p) { return (int64_t)kStageBytes * p.ld; }
   static constexpr int CH = BN / 16;              // 16-byte chunks per k row
@@ -330,17 +321,11 @@ struct I8KNLoaderDirect {
     const int cols_valid = cols_total - col0;
     const int lane = tid & 63;
     wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    wave_off = (uint32_t)wave * 1024u;
-    lane_off = (uint32_t)lane * 16u;
+    wave_off = addr::direct_lds_off(0, wave, 0, WAVES);
+    lane_off = addr::direct_lds_off(lane, 0, 0, WAVES);
     k_lane = lane / CH;
-    const int pc = lane % CH;
 #pragma unroll
-    for (int j = 0; j < PER_WAVE; ++j) {
-      const int k = (j * WAVES + wave) * KPI + k_lane;
-      int col = (pc ^ kn_swz<BN>(k)) * 16;
-      col = col < cols_valid ? col : cols_valid - 16;  // clamp whole chunks; those columns are masked later
-      voff[j] = (uint32_t)k * (uint32_t)p.ld + (uint32_t)col;
-    }
+    for (int j = 0; j < PER_WAVE; ++j) voff[j] = addr::kn_voff<BN>(lane, wave, j, WAVES, cols_valid, (uint32_t)p.ld);
     ld_ = (uint32_t)p.ld;
   }
   uint32_t ld_;
@@ -354,7 +339,7 @@ struct I8KNLoaderDirect {
       const uint32_t l0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lptr_t)lds_next + wave_off);
 #pragma unroll
       for (int j = 0; j < PER_WAVE; ++j)
-        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0 + (uint32_t)(j * WAVES * 1024)),
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0 + addr::direct_lds_off(0, 0, j, WAVES)),
                      "v"(voff[j]), "s"(sb)
                      : "memory");
     } else {
@@ -362,7 +347,7 @@ struct I8KNLoaderDirect {
       const uint8_t* sb = base + (int64_t)kt * kStageBytes * ld_;
 #pragma unroll
       for (int j = 0; j < PER_WAVE; ++j) {
-        const int k = (j * WAVES + wave) * KPI + k_lane;
+        const int k = addr::kn_k<BN>(0, wave, j, WAVES) + k_lane;
         const bool ok = kt * kStageBytes + k < k_total;
         uint4_t v = *(const uint4_t*)(ok ? sb + voff[j] : base + (voff[j] - (uint32_t)k * ld_));
         if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
@@ -375,7 +360,7 @@ struct I8KNLoaderDirect {
 #pragma unroll
     for (int j = 0; j < PER_WAVE; ++j) {
       if (j * np / UNITS != pc) continue;
-      *(uint4_t*)(lds + wave_off + j * WAVES * 1024 + lane_off) = r.v[j];
+      *(uint4_t*)(lds + wave_off + addr::direct_lds_off(0, 0, j, WAVES) + lane_off) = r.v[j];
     }
   }
   __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }

@@ -37,51 +37,50 @@ __global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDi
   typename WL::Regs regs_w;
   const RowFrag fragA(lane, wave_m0);
   const typename WL::Frag fragW(lane, wave_n0);
-  auto slot_of = [&](int t) { return smem + (t % SLOTS) * TILE; };
-  auto issue_a = [&](int s) { al.template gload<false>(regs, s, slot_of(2 * s)); };
-  auto issue_w = [&](int s) { wl.template gload<false>(regs_w, s, slot_of(2 * s + 1)); };
-
   typename Mma::acc_t acc[TN][TM];
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = typename Mma::acc_t{0, 0, 0, 0};
 
-  // this wavefront's loads of everything but the youngest tile have landed (`keep`: that tile was issued)
-  auto wait_tiles = [&](bool keep) {
-    if (keep)
-      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  };
-
-  issue_a(0);
-  issue_w(0);
-  if (KT > 1) issue_a(1);
-  wait_tiles(KT > 1);
-  __syncthreads();
-  for (int k = 0; k < KT; ++k) {
-    if (k + 1 < KT) issue_w(k + 1);  // into the slot of A(k - 1)
-    if (k + 2 < KT) issue_a(k + 2);  // into the slot of W(k - 1)
-    const uint8_t* la = slot_of(2 * k);
-    const uint8_t* lw = slot_of(2 * k + 1);
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      uint4_t wf[TN], af[TM];
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn) wf[tn] = fragW.read(lw, ks, tn);
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm) af[tm] = fragA.read(la, ks, tm);
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = Mma::mma(wf[tn], af[tm], acc[tn][tm]);
+  auto slot_of = [&](int t) { return smem + addr::slot_of_tile(t) * TILE; };
+  struct Ops {
+    decltype(slot_of)& slot;
+    const Loader& al;
+    const WL& wl;
+    typename Loader::Regs& regs;
+    typename WL::Regs& regs_w;
+    const RowFrag& fragA;
+    const typename WL::Frag& fragW;
+    typename Mma::acc_t (&acc)[TN][TM];
+    __device__ __forceinline__ void issue_a(int s) { al.template gload<false>(regs, s, slot(2 * s)); }
+    __device__ __forceinline__ void issue_w(int s) { wl.template gload<false>(regs_w, s, slot(2 * s + 1)); }
+    // four direct loads per wavefront and tile: vmcnt(4) leaves exactly the youngest tile outstanding
+    __device__ __forceinline__ void wait_tiles(bool keep) {
+      if (keep)
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    if (k + 1 < KT) {
-      wait_tiles(k + 2 < KT);  // A(k + 1) and W(k + 1) are in; A(k + 2) may still be on its way
-      __syncthreads();         // ... for every wavefront, and everyone has read the tiles of stage k
+    __device__ __forceinline__ void barrier() { __syncthreads(); }
+    __device__ __forceinline__ void compute(int k) {
+      const uint8_t* la = slot(2 * k);
+      const uint8_t* lw = slot(2 * k + 1);
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        uint4_t wf[TN], af[TM];
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) wf[tn] = fragW.read(lw, ks, tn);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) af[tm] = fragA.read(la, ks, tm);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+          for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = Mma::mma(wf[tn], af[tm], acc[tn][tm]);
+      }
     }
-  }
+  } ops{slot_of, al, wl, regs, regs_w, fragA, fragW, acc};
+  addr::slots_schedule(KT, ops);
 
   Epi epi(pe, tc.batch);
 #pragma unroll
