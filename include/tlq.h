@@ -217,11 +217,11 @@ int tlq_act_quant_i8(const void* X, void* Y, void* S, int64_t M, int64_t N, int 
  * tlq_debug_check_gemm_addressing walks every tile, thread, load instruction and stage of one operand:
  * source_kind 0 = row-major [rows, row_bytes] operand copied global -> LDS directly in tiles of `tile` rows by
  * `threads` threads; 1 = int8 [K = rows, N = row_bytes] weights in tiles of `tile` (128 | 256) columns.  It checks
- * global extents, LDS extents and coverage, agreement with the operand-fragment reads, and the touch-ahead addresses.
+ * global extents, LDS extents and coverage, and agreement with the operand-fragment reads.
  * tlq_debug_check_slots_schedule simulates the five-slot kernel's issue / wait / barrier order over `stages` stages
  * with `loads_per_tile` load instructions per wavefront and tile (the kernel's waits assume 4).
  * Both return 0 when everything holds, else 1 with tlq_last_error() naming the first violation. */
-int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads, int touch_ahead);
+int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads);
 int tlq_debug_check_slots_schedule(int stages, int loads_per_tile);
 
 /* Tuning hooks for benchmark sweeps (process-global, not thread safe; 0 = automatic choice).
@@ -232,10 +232,9 @@ void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4 (negat
 void tlq_tune_gemv_unroll(int blocks_per_cu);               /* resident blocks per CU the GEMV grid is sized for */
 void tlq_tune_gemv_depth(int steps_in_flight);               /* load steps (1 KB per row each) a GEMV wavefront keeps in flight */
 void tlq_tune_gemm_band(int tile_rows);                       /* tile rows per band of the MFMA kernels' tile order (default 4) */
-void tlq_tune_gemm_slots(int on);                            /* 1: plain 16-bit / int8 GEMM with [N, K] weights on the kernel that cuts LDS
-                                                              * into five operand-tile slots (0 = two stages, the default) */
-void tlq_tune_gemm_touch(int stages_ahead);                  /* MFMA kernels: touch the cache lines of the stage this many stages ahead
-                                                              * (0 = off, the default; 2 is the intended setting) */
+void tlq_tune_gemm_slots(int on);                            /* 1 (default): 256 x 256 tiles of the plain 16-bit GEMM with [N, K] weights and of the
+                                                              * int8 GEMMs run on the kernel that cuts LDS into five operand-tile slots
+                                                              * (whole 128-byte stages of K only); 0: always the two-stage kernel */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
 void tlq_tune_w4a16_split(int slices);                       /* K slices of the tile kernel, 16 < M < 256 with a workspace */
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,

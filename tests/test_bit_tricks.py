@@ -209,33 +209,3 @@ def test_five_slot_schedule_keeps_every_tile_until_it_is_read():
 
     for KT in range(1, 48):
         run(KT)
-
-
-def test_touch_addresses_stay_inside_the_matrices():
-    """Restatement of touch_ptr / touch_step (csrc/gemm_core.h): the byte a thread touches for stage kt lies inside
-    its matrix for every whole stage, for row-major operands and for int8 weights stored [K, N]."""
-    rng = np.random.default_rng(5)
-    for _ in range(200):
-        M = int(rng.integers(1, 700))
-        kb = int(rng.integers(1, 40)) * 16 + int(rng.integers(0, 2)) * 128 * int(rng.integers(0, 30))  # bytes of K per row
-        KT = -(-kb // 128)
-        last_full = KT - 2 if kb % 128 else KT - 1
-        m0 = (int(rng.integers(0, -(-M // 256)))) * 256
-        for i in (0, 1, 127, 255):
-            row = m0 + i if m0 + i < M else M - 1
-            for kt in range(0, last_full + 1):
-                off = row * kb + kt * 128
-                assert 0 <= off and off + 4 <= M * kb
-        # [K, N] int8: line i of a stage is k row i // (BN / 128), 128-byte column block i % (BN / 128)
-        N = int(rng.integers(1, 60)) * 16
-        K = int(rng.integers(1, 30)) * 16
-        BN = 256
-        n0 = int(rng.integers(0, -(-N // BN))) * BN
-        KT = -(-K // 128)
-        last_full = KT - 2 if K % 128 else KT - 1
-        for i in (0, 1, 2, 255):
-            k, c = i // (BN // 128), n0 + (i % (BN // 128)) * 128
-            col = c if c < N else n0
-            for kt in range(0, last_full + 1):
-                off = (kt * 128 + k) * N + col
-                assert off + 4 <= K * N, (N, K, i, kt)

@@ -1,8 +1,8 @@
 """Host-side walk of the MFMA GEMM kernels' address arithmetic (csrc/gemm_addr.h through
 tlq_debug_check_gemm_addressing / tlq_debug_check_slots_schedule): the functions the kernels use for their
-global offsets, LDS offsets, touch-ahead addresses and for the five-slot issue / wait order are evaluated on the
+global offsets, LDS offsets and for the five-slot issue / wait order are evaluated on the
 CPU for every tile, thread and stage of a launch and compared with the buffer extents.  The shapes are those of
-the GPU comparison tests of the two opt-in paths plus ragged and very short cases.
+the GPU comparison test of the two GEMM main loops plus ragged and very short cases.
 """
 import pytest
 
@@ -21,34 +21,32 @@ W8A8 = [(1, 256, 256, 128), (2, 300, 528, 384), (1, 2048, 4096, 4096), (3, 512, 
         (1, 1, 16, 16), (1, 33, 48, 272)]
 
 
-@pytest.mark.parametrize("touch", [0, 2, 3])
 @pytest.mark.parametrize("tile,threads", [(256, 512), (128, 256)])
-def test_row_operands_of_the_16_bit_gemms(tile, threads, touch):
+def test_row_operands_of_the_16_bit_gemms(tile, threads):
     lib = _abi.load()
     for M, N, K in SHAPES_16:
         for rows in (M, N):
-            _ok(lib.tlq_debug_check_gemm_addressing(0, rows, K * 2, tile, threads, touch))
+            _ok(lib.tlq_debug_check_gemm_addressing(0, rows, K * 2, tile, threads))
 
 
-@pytest.mark.parametrize("touch", [0, 2, 3])
-def test_int8_operands(touch):
+def test_int8_operands():
     lib = _abi.load()
     for _, M, N, K in W8A8:
         for tile, threads in ((256, 512), (128, 256), (32, 256)):
-            _ok(lib.tlq_debug_check_gemm_addressing(0, M, K, tile, threads, touch))        # activations [M, K]
+            _ok(lib.tlq_debug_check_gemm_addressing(0, M, K, tile, threads))        # activations [M, K]
         for tile, threads in ((256, 512), (128, 256)):
-            _ok(lib.tlq_debug_check_gemm_addressing(0, N, K, tile, threads, touch))        # weights [N, K]
-            _ok(lib.tlq_debug_check_gemm_addressing(1, K, N, tile, threads, touch))        # weights [K, N]
-        _ok(lib.tlq_debug_check_gemm_addressing(1, K, N, 128, 256, touch))                 # the 32-row kernel's weights
+            _ok(lib.tlq_debug_check_gemm_addressing(0, N, K, tile, threads))        # weights [N, K]
+            _ok(lib.tlq_debug_check_gemm_addressing(1, K, N, tile, threads))        # weights [K, N]
+        _ok(lib.tlq_debug_check_gemm_addressing(1, K, N, 128, 256))                 # the 32-row kernel's weights
 
 
 def test_the_walker_rejects_what_it_should():
     lib = _abi.load()
-    assert lib.tlq_debug_check_gemm_addressing(0, 256, 256, 250, 512, 0) != 0      # tile rows not a multiple of 8
-    assert lib.tlq_debug_check_gemm_addressing(0, 256, 256, 64, 1024, 0) != 0      # fewer load instructions than wavefronts
-    assert lib.tlq_debug_check_gemm_addressing(0, 1 << 20, 1 << 13, 256, 512, 0) != 0  # 8 GiB operand: 32-bit offsets
-    assert lib.tlq_debug_check_gemm_addressing(1, 128, 24, 256, 512, 0) != 0       # N not a multiple of 16
-    assert lib.tlq_debug_check_gemm_addressing(2, 128, 128, 256, 512, 0) != 0
+    assert lib.tlq_debug_check_gemm_addressing(0, 256, 256, 250, 512) != 0      # tile rows not a multiple of 8
+    assert lib.tlq_debug_check_gemm_addressing(0, 256, 256, 64, 1024) != 0      # fewer load instructions than wavefronts
+    assert lib.tlq_debug_check_gemm_addressing(0, 1 << 20, 1 << 13, 256, 512) != 0  # 8 GiB operand: 32-bit offsets
+    assert lib.tlq_debug_check_gemm_addressing(1, 128, 24, 256, 512) != 0       # N not a multiple of 16
+    assert lib.tlq_debug_check_gemm_addressing(2, 128, 128, 256, 512) != 0
     assert "bad source kind" in _abi.last_error()
 
 
@@ -63,3 +61,4 @@ def test_five_slot_schedule():
     assert lib.tlq_debug_check_slots_schedule(8, 2) != 0
     assert "before its loads were waited for" in _abi.last_error()
     _ok(lib.tlq_debug_check_slots_schedule(8, 8))
+

@@ -1,10 +1,8 @@
-"""GPU checks of the two opt-in GEMM paths (tlq_tune_gemm_slots, tlq_tune_gemm_touch).
-
-Not collected by pytest under this name on purpose: both paths were written without access to a GPU and have not run
-on one yet.  Run it by naming the file (`python -m pytest tests/wip_gemm_hooks.py -m gpu -x -v`), and give it a
-collected name once it passes.  Every case compares the hooked path with the default kernel on the same inputs:
-integer GEMMs and the rescaled outputs bit for bit, 16-bit GEMMs bit for bit as well (same tiling, same order of
-accumulation inside a tile; the hooks only change when data is fetched).
+"""The two main loops of the 256 x 256 GEMM tiles against each other: the five-slot kernel (csrc/gemm_slots.h, the
+default for whole 128-byte stages of K) and the two-stage kernel (csrc/gemm_core.h, tlq_tune_gemm_slots(0)).  Every case
+runs the same inputs through both: integer GEMMs and the rescaled outputs must agree bit for bit, and so must the
+16-bit GEMMs (same tiling, same order of accumulation inside a tile; the kernels only differ in when data is fetched).
+The default path is also checked against an exact / fp32 evaluation.
 """
 import pytest
 import torch
@@ -13,7 +11,7 @@ from helpers import assert_bit_equal, gen
 
 pytestmark = pytest.mark.gpu
 
-HOOKS = [("slots", 1), ("touch", 2), ("touch", 3)]
+HOOKS = [("slots", 0)]
 
 
 def _with_hook(name, value, fn):
@@ -25,12 +23,12 @@ def _with_hook(name, value, fn):
     try:
         return fn()
     finally:
-        hook(0)
+        hook(1)  # the default
 
 
 # K in 16-bit values: one, two, three stages (64 values each), odd stage counts, a partial last stage (falls back /
 # register tail), long rows; M, N ragged against the 256 x 256 tile
-# (the 256 x 256 kernels, which the slots path replaces, are chosen from 128 output tiles on: M, N around 2900)
+# (the 256 x 256 kernels are chosen from 128 output tiles on: M, N around 2900)
 SHAPES_16 = [(256, 256, 64), (300, 520, 192), (1000, 1288, 4160), (4096, 4096, 4096), (260, 264, 96), (2048, 2304, 72),
              (2900, 2904, 64), (2900, 2824, 128), (3000, 2824, 192), (2816, 3072, 320), (2820, 2904, 72)]
 
@@ -38,7 +36,7 @@ SHAPES_16 = [(256, 256, 64), (300, 520, 192), (1000, 1288, 4160), (4096, 4096, 4
 @pytest.mark.parametrize("hook,value", HOOKS)
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", SHAPES_16)
-def test_plain_gemm_same_bits_as_default(hook, value, dtype, M, N, K):
+def test_plain_gemm_same_bits_on_both_main_loops(hook, value, dtype, M, N, K):
     from tilelang_ascend_amd import _abi
 
     lib, P = _abi.load(), _abi.ptr
@@ -64,7 +62,7 @@ def test_plain_gemm_same_bits_as_default(hook, value, dtype, M, N, K):
 @pytest.mark.parametrize("layout", ["KN", "NK"])
 @pytest.mark.parametrize("B,M,N,K", [(1, 256, 256, 128), (2, 300, 528, 384), (1, 2048, 4096, 4096), (3, 512, 272, 640),
                                      (1, 260, 512, 144)])
-def test_w8a8_same_bits_as_default(hook, value, layout, B, M, N, K):
+def test_w8a8_same_bits_on_both_main_loops(hook, value, layout, B, M, N, K):
     from tilelang_ascend_amd import _abi
 
     lib, P = _abi.load(), _abi.ptr
@@ -76,7 +74,7 @@ def test_w8a8_same_bits_as_default(hook, value, layout, B, M, N, K):
     lay = _abi.B_KN if layout == "KN" else _abi.B_NK
 
     def run():
-        lib.tlq_tune_i8_tile(256)  # the kernel the slots path replaces, whatever the number of tiles
+        lib.tlq_tune_i8_tile(256)  # the 256 x 256 kernels, whatever the number of tiles
         try:
             C = torch.full((B, M, N), float("nan"), dtype=torch.float16, device="cuda")
             _abi.check(lib.tlq_gemm_w8a8(P(A), P(W), P(sa), P(sb), P(C), B, M, N, K, N, lay, _abi.F16, st))

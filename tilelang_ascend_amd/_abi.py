@@ -46,13 +46,12 @@ SIGNATURES = {
     "tlq_pack_int4": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "tlq_quantize_sym4": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "tlq_act_quant_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
-    "tlq_debug_check_gemm_addressing": (_int, [_int, _i64, _i64, _int, _int, _int]),
+    "tlq_debug_check_gemm_addressing": (_int, [_int, _i64, _i64, _int, _int]),
     "tlq_debug_check_slots_schedule": (_int, [_int, _int]),
     "tlq_tune_gemv": (None, [_int, _int]),
     "tlq_tune_gemv_unroll": (None, [_int]),
     "tlq_tune_gemv_depth": (None, [_int]),
     "tlq_tune_gemm_band": (None, [_int]),
-    "tlq_tune_gemm_touch": (None, [_int]),
     "tlq_tune_gemm_slots": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),
     "tlq_tune_w4a16_split": (None, [_int]),

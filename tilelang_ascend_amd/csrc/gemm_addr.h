@@ -1,6 +1,6 @@
 // Address arithmetic of the MFMA GEMM tile loaders, written as host-callable functions: the kernels
 // (gemm_core.h, gemm_slots.h) take every global byte offset and every LDS offset of a direct
-// global -> LDS load, of a cache-line touch and of an operand-fragment read from here, and the host
+// global -> LDS load and of an operand-fragment read from here, and the host
 // walker in gemm_addr_check.hip evaluates the same functions for every thread, stage and tile of a
 // launch and compares them with the extents of the buffers, without a GPU.
 #pragma once
@@ -41,11 +41,6 @@ __host__ __device__ inline uint32_t rowfrag_base(int lane, int wave_row0) {
 __host__ __device__ inline uint32_t rowfrag_off(uint32_t base, int ks, int t) {
   return (base ^ (uint32_t)(ks << 6)) + (uint32_t)(t * 16 * kStage);
 }
-// cache line i of stage 0 of a row tile (touch-ahead): byte offset from the matrix base
-__host__ __device__ inline int64_t row_touch_off(int row0, int rows_total, int i, int64_t ld) {
-  const int row = row0 + i < rows_total ? row0 + i : rows_total - 1;
-  return (int64_t)row * ld;
-}
 
 // ---- int8 [K, N] source copied unchanged into a [128 k][BN] tile -------------------------------------
 template <int BN>
@@ -73,11 +68,6 @@ __host__ __device__ inline uint32_t knfrag_off(int lane, int wave_row0, int t) {
   const int krow = q * 16 + (r16 >> 1);
   const int sw = kn_swz<BN>(krow);
   return (uint32_t)(krow * BN + 8 * (r16 & 1)) + (uint32_t)((((wave_row0 >> 4) + t) ^ sw) << 4);
-}
-template <int BN>
-__host__ __device__ inline int64_t kn_touch_off(int col0, int cols_total, int i, int64_t ld) {
-  const int k = i / (BN / 128), c = col0 + (i % (BN / 128)) * 128;
-  return (int64_t)k * ld + (c < cols_total ? c : col0);
 }
 
 // ---- five-slot schedule (gemm_slots.h): tile t = 2 * stage (+ 1 for the weights) lives in slot t % 5 ----

@@ -3,7 +3,6 @@
 //   * every global byte read lies inside the operand matrix,
 //   * every direct load lands inside its LDS tile, every 16-byte cell of the tile is written exactly once, and holds
 //     the (row, K chunk) that the operand-fragment read of that cell expects,
-//   * every touch-ahead address lies inside the matrix,
 //   * the five-slot schedule never overwrites a tile that has not been multiplied and never multiplies a tile whose
 //     loads were not waited for.
 // No GPU is needed: these run in the CPU-only test suite and can be called before a launch.
@@ -24,7 +23,7 @@ namespace {
   } while (0)
 
 // Row-major operand [rows_total, k_bytes] (pitch = k_bytes), tiles of `tile_rows` rows loaded by `threads` threads.
-int check_row_direct(int64_t rows_total, int64_t k_bytes, int tile_rows, int threads, int touch_ahead) {
+int check_row_direct(int64_t rows_total, int64_t k_bytes, int tile_rows, int threads) {
   CHECK_OR_FAIL(tile_rows % 8 == 0 && threads % 64 == 0, "row loader: tile rows %d / threads %d", tile_rows, threads);
   const int waves = threads / 64, instr = tile_rows / 8;
   CHECK_OR_FAIL(instr % waves == 0 && instr >= waves, "row loader: %d load instructions do not split over %d wavefronts", instr, waves);
@@ -81,20 +80,13 @@ int check_row_direct(int64_t rows_total, int64_t k_bytes, int tile_rows, int thr
                         cell[off / 16], want);
         }
       }
-    // touch-ahead: one 4-byte load per cache line of the stage `touch_ahead` stages further on
-    if (touch_ahead > 0)
-      for (int i = 0; i < tile_rows; ++i)
-        for (int kt = 0; kt + touch_ahead <= last_full; ++kt) {
-          const int64_t o = addr::row_touch_off((int)row0, (int)rows_total, i, k_bytes) + (int64_t)(kt + touch_ahead) * addr::kStage;
-          CHECK_OR_FAIL(o >= 0 && o + 4 <= extent, "row touch: line %d stage %d at %lld of %lld", i, kt, (long long)o, (long long)extent);
-        }
   }
   return 0;
 }
 
 // int8 operand stored [K, N] (pitch N), tiles of BN columns x 128 k rows.
 template <int BN>
-int check_kn_direct(int64_t K, int64_t N, int threads, int touch_ahead) {
+int check_kn_direct(int64_t K, int64_t N, int threads) {
   CHECK_OR_FAIL(threads % 64 == 0, "[K,N] loader: threads %d", threads);
   const int waves = threads / 64, kpi = 1024 / BN, instr = addr::kStage / kpi;
   CHECK_OR_FAIL(instr % waves == 0 && instr >= waves, "[K,N] loader: %d load instructions do not split over %d wavefronts", instr, waves);
@@ -147,12 +139,6 @@ int check_kn_direct(int64_t K, int64_t N, int threads, int touch_ahead) {
               CHECK_OR_FAIL(cell[off / 16] == want && (int)(off % 16) == 8 * (lane & 1), "[K,N] operand read (lane %d t %d) finds cell %d, expects %d",
                             lane, t, cell[off / 16], want);
             }
-    if (touch_ahead > 0)
-      for (int i = 0; i < addr::kStage * (BN / 128); ++i)
-        for (int kt = 0; kt + touch_ahead <= last_full; ++kt) {
-          const int64_t o = addr::kn_touch_off<BN>((int)col0, (int)N, i, N) + (int64_t)(kt + touch_ahead) * addr::kStage * N;
-          CHECK_OR_FAIL(o >= 0 && o + 4 <= extent, "[K,N] touch: line %d stage %d at %lld of %lld", i, kt, (long long)o, (long long)extent);
-        }
   }
   return 0;
 }
@@ -216,11 +202,11 @@ using namespace tlq;
 
 extern "C" {
 
-int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads, int touch_ahead) {
-  if (source_kind == 0) return check_row_direct(rows, row_bytes, tile, threads, touch_ahead);
+int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads) {
+  if (source_kind == 0) return check_row_direct(rows, row_bytes, tile, threads);
   if (source_kind == 1) {
-    if (tile == 256) return check_kn_direct<256>(rows, row_bytes, threads, touch_ahead);
-    if (tile == 128) return check_kn_direct<128>(rows, row_bytes, threads, touch_ahead);
+    if (tile == 256) return check_kn_direct<256>(rows, row_bytes, threads);
+    if (tile == 128) return check_kn_direct<128>(rows, row_bytes, threads);
     set_error("tlq_debug_check_gemm_addressing: [K,N] tiles are 128 or 256 columns wide (got %d)", tile);
     return 1;
   }

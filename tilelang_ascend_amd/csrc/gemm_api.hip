@@ -25,8 +25,7 @@ int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, 
                   hipStream_t st);
 
 int g_gemm_band_rows = 0;
-int g_gemm_touch_ahead = 0;
-int g_gemm_slots = 0;
+int g_gemm_slots = 1;
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // the tile loaders address one matrix with 32-bit byte offsets
 static bool fits32(int64_t rows, int64_t row_bytes) { return rows * row_bytes < ((int64_t)1 << 32); }
@@ -43,7 +42,6 @@ extern "C" {
 
 void tlq_tune_gemm_band(int tile_rows) { tlq::g_gemm_band_rows = tile_rows < 0 ? 0 : tile_rows; }
 void tlq_tune_gemm_slots(int on) { tlq::g_gemm_slots = on != 0; }
-void tlq_tune_gemm_touch(int stages_ahead) { tlq::g_gemm_touch_ahead = (stages_ahead < 0 || stages_ahead > 8) ? 0 : stages_ahead; }
 
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,

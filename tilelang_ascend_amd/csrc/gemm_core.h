@@ -120,7 +120,6 @@ struct RowLoader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
   static constexpr bool PREFETCH2 = false;
-  static constexpr int TOUCH_LINES = ROWS;  // cache lines per stage (one per row), see touch_ptr
   static constexpr int SLOTS = ROWS * 8;  // 16-byte chunks per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
@@ -135,12 +134,6 @@ struct RowLoader {
   struct Regs {
     uint4_t v[PASSES];
   };
-  // line i of stage 0 of the tile that starts at row0 (the kernel touches the lines of a later stage ahead of time);
-  // the same line of stage kt is touch_step(p) * kt bytes further
-  static __device__ __forceinline__ const uint8_t* touch_ptr(const Params& p, int batch, int row0, int rows_total, int i) {
-    return p.base + batch * p.batch_stride + addr::row_touch_off(row0, rows_total, i, p.ld);
-  }
-  static __device__ __forceinline__ int64_t touch_step(const Params&) { return kStageBytes; }
   const uint8_t* base;    // uniform
   uint32_t voff[PASSES];  // per lane: row * ld + chunk * 16
   uint32_t loff;          // per lane: LDS offset of pass 0
@@ -201,12 +194,6 @@ struct RowLoaderDirect {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = true;
   static constexpr bool PREFETCH2 = false;
-  static constexpr int TOUCH_LINES = ROWS;
-  static __device__ __forceinline__ const uint8_t* touch_ptr(const typename RowLoader<ROWS, NT>::Params& p, int batch, int row0,
-                                                             int rows_total, int i) {
-    return RowLoader<ROWS, NT>::touch_ptr(p, batch, row0, rows_total, i);
-  }
-  static __device__ __forceinline__ int64_t touch_step(const typename RowLoader<ROWS, NT>::Params&) { return kStageBytes; }
   static constexpr int WAVES = NT / 64;
   static constexpr int INSTR = ROWS / 8;          // wavefront-instructions per stage
   static constexpr int PER_WAVE = INSTR / WAVES;  // ... per wavefront
@@ -293,11 +280,6 @@ struct I8KNLoaderDirect {
   typedef KNFrag8<BN> Frag;
   static constexpr bool DIRECT = true;
   static constexpr bool PREFETCH2 = false;
-  static constexpr int TOUCH_LINES = 128 * (BN / 128);  // 128 k rows of BN bytes
-  static __device__ __forceinline__ const uint8_t* touch_ptr(const I8KNParams& p, int batch, int col0, int cols_total, int i) {
-    return p.base + batch * p.batch_stride + addr::kn_touch_off<BN>(col0, cols_total, i, p.ld);
-  }
-  static __device__ __forceinline__ int64_t touch_step(const I8KNParams& p) { return (int64_t)kStageBytes * p.ld; }
   static constexpr int CH = BN / 16;              // 16-byte chunks per k row
   static constexpr int KPI = 64 / CH;             // k rows per wavefront instruction
   static constexpr int WAVES = NT / 64;
@@ -378,6 +360,27 @@ struct EpiFloat {  // fp32 accumulators -> f16 / bf16 / f32
   Params p;
   int64_t boff;
   __device__ __forceinline__ EpiFloat(const Params& pp, int batch) : p(pp), boff(batch * pp.batch_stride) {}
+  // staged epilogue interface: element size of C, the four outputs of one accumulator in C's type (x, y only for
+  // 16-bit types), the byte address of C[m, n], and the row pitch in elements
+  static constexpr bool STAGED = true;
+  __device__ __forceinline__ int out_bytes() const { return p.out_dtype == TLQ_F32 ? 4 : 2; }
+  __device__ __forceinline__ int64_t pitch() const { return p.ldc; }
+  __device__ __forceinline__ uint8_t* addr_of(int m, int n) const {
+    return (uint8_t*)p.C + (boff + (int64_t)m * p.ldc + n) * out_bytes();
+  }
+  __device__ __forceinline__ uint4_t pack(int /*m*/, int /*n*/, const float4_t& acc, int /*M*/, int /*N*/) const {
+    if (p.out_dtype == TLQ_F32) return bitcast<uint4_t>(acc);
+    uint4_t o{0u, 0u, 0u, 0u};
+    if (p.out_dtype == TLQ_F16) {
+      half_t h[4] = {(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
+      const uint2_t u = bitcast<uint2_t>(h);
+      o.x = u.x, o.y = u.y;
+    } else {
+      o.x = pack_bf16x2(acc[0], acc[1]);
+      o.y = pack_bf16x2(acc[2], acc[3]);
+    }
+    return o;
+  }
   __device__ __forceinline__ void store(int m, int n, const float4_t& acc, int M, int N) const {
     if (m >= M || n >= N) return;
     const int64_t idx = boff + (int64_t)m * p.ldc + n;
@@ -406,6 +409,11 @@ struct EpiAtomicAdd {  // fp32 accumulators added into C (split-K: several work-
   };
   Params p;
   __device__ __forceinline__ EpiAtomicAdd(const Params& pp, int /*split*/) : p(pp) {}
+  static constexpr bool STAGED = false;  // atomic adds go out element by element
+  __device__ __forceinline__ int out_bytes() const { return 4; }
+  __device__ __forceinline__ int64_t pitch() const { return p.ldc; }
+  __device__ __forceinline__ uint8_t* addr_of(int, int) const { return nullptr; }
+  __device__ __forceinline__ uint4_t pack(int, int, const float4_t&, int, int) const { return uint4_t{0u, 0u, 0u, 0u}; }
   __device__ __forceinline__ void store(int m, int n, const float4_t& acc, int M, int N) const {
     if (m >= M || n >= N) return;
     float* c = p.C + (int64_t)m * p.ldc + n;
@@ -422,6 +430,11 @@ struct EpiInt32 {  // raw int32 accumulators
   Params p;
   int64_t boff;
   __device__ __forceinline__ EpiInt32(const Params& pp, int batch) : p(pp), boff(batch * pp.batch_stride) {}
+  static constexpr bool STAGED = true;
+  __device__ __forceinline__ int out_bytes() const { return 4; }
+  __device__ __forceinline__ int64_t pitch() const { return p.ldc; }
+  __device__ __forceinline__ uint8_t* addr_of(int m, int n) const { return (uint8_t*)(p.C + boff + (int64_t)m * p.ldc + n); }
+  __device__ __forceinline__ uint4_t pack(int, int, const int4_t& acc, int, int) const { return bitcast<uint4_t>(acc); }
   __device__ __forceinline__ void store(int m, int n, const int4_t& acc, int M, int N) const {
     if (m >= M || n >= N) return;
     const int64_t idx = boff + (int64_t)m * p.ldc + n;
@@ -451,8 +464,8 @@ struct EpiRescale {
   const float* sa;
   __device__ __forceinline__ EpiRescale(const Params& pp, int batch)
       : p(pp), boff(batch * pp.batch_stride), sa(pp.scale_a ? pp.scale_a + batch * pp.scale_a_batch_stride : nullptr) {}
-  __device__ __forceinline__ void store(int m, int n, const int4_t& acc, int M, int N) const {
-    if (m >= M || n >= N) return;
+  // m < M and n < N
+  __device__ __forceinline__ float4_t scaled(int m, int n, const int4_t& acc, int N) const {
     float4_t f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) f[i] = (float)acc[i];
@@ -468,12 +481,89 @@ struct EpiRescale {
         f[i] = f[i] * (p.n_scale_b == 1 ? p.scale_b[0] : p.scale_b[nn]);
       }
     }
+    return f;
+  }
+  __device__ __forceinline__ EpiFloat as_float() const {
     EpiFloat::Params fp{p.C, p.ldc, 0, p.out_dtype};
     EpiFloat ef(fp, 0);
     ef.boff = boff;
-    ef.store(m, n, f, M, N);
+    return ef;
+  }
+  static constexpr bool STAGED = true;
+  __device__ __forceinline__ int out_bytes() const { return p.out_dtype == TLQ_F32 ? 4 : 2; }
+  __device__ __forceinline__ int64_t pitch() const { return p.ldc; }
+  __device__ __forceinline__ uint8_t* addr_of(int m, int n) const { return as_float().addr_of(m, n); }
+  __device__ __forceinline__ uint4_t pack(int m, int n, const int4_t& acc, int M, int N) const {
+    if (m >= M || n >= N) return uint4_t{0u, 0u, 0u, 0u};  // never stored; keeps the scale loads inside their arrays
+    return as_float().pack(m, n, scaled(m, n, acc, N), M, N);
+  }
+  __device__ __forceinline__ void store(int m, int n, const int4_t& acc, int M, int N) const {
+    if (m >= M || n >= N) return;
+    as_float().store(m, n, scaled(m, n, acc, N), M, N);
   }
 };
+
+// Writes a wavefront's accumulators (TN x TM MFMA tiles: lane (r16, q) holds C[m = 16 tm + r16][n = 16 tn + 4 q + 0..3])
+// to C.  Stored straight from the registers a lane would write 8 (16-bit output) or 16 bytes of a row while its 15
+// neighbours write to 15 other rows: 32-byte pieces of 16 different cache lines per instruction, which the memory system
+// does not merge back into whole lines (measured: 1.8-2.5 x the output bytes written, and an epilogue of 17 us for a
+// 32 MB output).  So the tile takes a detour through a wavefront-private piece of LDS (free once the main loop is
+// over): accumulators are written as [row][128 B] with the operand tiles' chunk swizzle, 128 bytes of output per row
+// and pass, and read back row-wise, 16 bytes per lane, eight lanes per row -- every store instruction then writes eight
+// whole 128-byte lines.  Needs 16-byte aligned rows of C (pitch and N multiples of 16 bytes); otherwise, and for
+// tilings whose wavefront rows are shorter than 128 bytes, the direct path is used.
+template <class Epi, int TM, int TN, class Acc>
+__device__ __forceinline__ void write_tile(const Epi& epi, Acc (&acc)[TN][TM], uint8_t* region, int lane, int m_base, int n_base,
+                                           int M, int N) {
+  const int r16 = lane & 15, q = lane >> 4;
+  const int osz = epi.out_bytes();
+  bool staged = false;
+  if constexpr (Epi::STAGED) staged = ((epi.pitch() * osz) & 15) == 0 && ((N * osz) & 15) == 0 && TN * 16 * osz >= 128;
+  if (!staged) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) epi.store(m_base + tm * 16 + r16, n_base + tn * 16 + q * 4, acc[tn][tm], M, N);
+    return;
+  }
+  auto run = [&](auto osz_tag) {
+    constexpr int OSZ = decltype(osz_tag)::value;
+    constexpr int TNP = 128 / (16 * OSZ);  // MFMA tile columns per pass: 128 bytes of output per row
+    if constexpr (TN % TNP == 0) {
+#pragma unroll
+      for (int p0 = 0; p0 < TN; p0 += TNP) {
+#pragma unroll
+        for (int t = 0; t < TNP; ++t)
+#pragma unroll
+          for (int tm = 0; tm < TM; ++tm) {
+            const int row = tm * 16 + r16;
+            const uint4_t v = epi.pack(m_base + row, n_base + (p0 + t) * 16 + q * 4, acc[p0 + t][tm], M, N);
+            const int byte = (t * 16 + q * 4) * OSZ;  // offset inside the 128-byte row of this pass
+            uint8_t* dst = region + lds_off(row, byte >> 4) + (byte & 15);
+            if (OSZ == 2)
+              *(uint2_t*)dst = uint2_t{v.x, v.y};
+            else
+              *(uint4_t*)dst = v;
+          }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 2 * TM; ++j) {
+          const int row = j * 8 + (lane >> 3), chunk = lane & 7;
+          const uint4_t v = *(const uint4_t*)(region + lds_off(row, chunk));
+          const int m = m_base + row, n = n_base + p0 * 16 + chunk * (16 / OSZ);
+          if (m < M && n < N) *(uint4_t*)epi.addr_of(m, n) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();  // the next pass overwrites the rows
+      }
+    }
+  };
+  if (osz == 2)
+    run(std::integral_constant<int, 2>{});
+  else
+    run(std::integral_constant<int, 4>{});
+}
 
 // Work-group -> tile.  Consecutive hardware ids are dealt round-robin to the 8 XCDs; give
 // every XCD a contiguous range of logical tiles, and order the tiles of a matrix in bands of four
@@ -501,19 +591,11 @@ __device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n, int
   return t;
 }
 
-// Which instances can touch a later stage's cache lines (see the kernel): not the converting weight loader (its
-// 256 x 256 kernels have no registers to spare) and not the low tiles (the spare LDS words would cost them a resident
-// work-group).  The launcher reserves the spare words for exactly these instances.
-template <class AL, class WL, int BM>
-constexpr bool gemm_touch_ok() {
-  return !WL::PREFETCH2 && BM >= 128 && AL::TOUCH_LINES + WL::TOUCH_LINES > 0;
-}
-
 // ---- the kernel -----------------------------------------------------------------------------
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma_kernel(
     typename AL::Params pa, typename WL::Params pw, typename Epi::Params pe, int M, int N, int KT, int k_tail,
-    int tiles_m, int tiles_n, int band_rows, int touch_ahead) {
+    int tiles_m, int tiles_n, int band_rows) {
   constexpr int TM = BM / WM / 16;  // 16-row activation tiles per wave
   constexpr int TN = BN / WN / 16;  // 16-row weight tiles per wave
   constexpr int A_TILE = BM * kStageBytes, W_TILE = BN * kStageBytes;
@@ -552,47 +634,9 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   constexpr int NP = 2 * TN;  // pieces per stage
   // first pieces: activation stores (none when they travel directly), the rest: weight conversion
   constexpr int NPA = AL::DIRECT ? 0 : NP / 2;
-  // Optional (touch_ahead = stages ahead, 0 = off): while stage kt multiplies, every thread asks for four bytes of one
-  // cache line of stage kt + touch_ahead with a direct load into a spare LDS word.  A stage's real loads are issued only
-  // one stage before they are needed; lines that no CU of the XCD has touched yet come from HBM and take longer
-  // than that.  The touch starts that trip earlier, and the real loads then find the line in L2.  Each wavefront
-  // issues exactly one touch per stage (threads beyond the tile's lines repeat line 0), after the stage's other loads,
-  // so "everything but the youngest load has landed" is the wait that leaves the touch in flight.
-  constexpr bool TOUCH_OK = gemm_touch_ok<AL, WL, BM>();
-  const uint8_t* touch_p = nullptr;
-  int64_t touch_step = 0;
-  if constexpr (TOUCH_OK) {
-    if (touch_ahead > 0) {
-      constexpr int LA = AL::TOUCH_LINES, LW = WL::TOUCH_LINES;
-      if (LA > 0 && (tid < LA || LW == 0)) {
-        if constexpr (LA > 0) {
-          touch_p = AL::touch_ptr(pa, batch, m0, M, tid < LA ? tid : 0);
-          touch_step = AL::touch_step(pa);
-        }
-      } else {
-        if constexpr (LW > 0) {
-          touch_p = WL::touch_ptr(pw, batch, n0, N, tid - LA < LW ? tid - LA : 0);
-          touch_step = WL::touch_step(pw);
-        }
-      }
-    }
-  }
-  const bool touching = TOUCH_OK && touch_ahead > 0;  // then every thread has a line to touch
-  typedef __attribute__((address_space(3))) uint8_t* touch_lptr_t;
-  const uint32_t touch_lds =
-      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(touch_lptr_t)(smem + 2 * (A_TILE + W_TILE)) + (uint32_t)(wave * 256));
-  auto touch = [&](int kt) {  // kt: a full stage inside K
-    const uint64_t a = (uint64_t)(uintptr_t)(touch_p + (int64_t)kt * touch_step);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(touch_lds), "v"(a) : "memory");
-  };
   // hand-issued direct loads are invisible to the compiler's wait insertion
-  auto wait_direct = [&](bool touched = false) {
-    if (AL::DIRECT || WL::DIRECT) {
-      if (touched)
-        asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-      else
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
+  auto wait_direct = [&]() {
+    if (AL::DIRECT || WL::DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
   auto stage = [&](int cur, auto fill_tag) {
     constexpr bool FILL = decltype(fill_tag)::value;
@@ -658,10 +702,8 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
         al.template gload<true>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
       else
         al.template gload<false>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
-      const bool touched = touching && kt + touch_ahead <= last_full;
-      if (touched) touch(kt + touch_ahead);
       stage(kt & 1, std::true_type{});
-      wait_direct(touched);
+      wait_direct();
       __syncthreads();
     }
   } else {
@@ -670,10 +712,8 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
     for (; kt + 1 <= last_full; ++kt) {
       al.template gload<false>(ra, kt + 1, ldsA0 + ((kt + 1) & 1) * A_TILE);
       wl.template gload<false>(rw, kt + 1, ldsW0 + ((kt + 1) & 1) * W_TILE);
-      const bool touched = touching && kt + touch_ahead <= last_full;
-      if (touched) touch(kt + touch_ahead);
       stage(kt & 1, std::true_type{});
-      wait_direct(touched);
+      wait_direct();
       __syncthreads();
     }
     if (kt + 1 < KT) {  // the partial last stage
@@ -688,26 +728,23 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   if (KT > 0) stage((KT - 1) & 1, std::false_type{});
 
   Epi epi(pe, batch);
-#pragma unroll
-  for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm)
-      epi.store(m0 + wave_m0 + tm * 16 + r16, n0 + wave_n0 + tn * 16 + q * 4, acc[tn][tm], M, N);
+  // the operand tiles are no longer needed once every wavefront is past its last stage: each wavefront then stages its
+  // outputs through its own TM * 16 rows x 128 B of LDS
+  static_assert(WM * WN * TM * 16 * kStageBytes <= 2 * (A_TILE + W_TILE), "staging area exceeds the operand tiles");
+  if constexpr (Epi::STAGED) __syncthreads();
+  write_tile<Epi, TM, TN>(epi, acc, smem + wave * (TM * 16 * kStageBytes), lane, m0 + wave_m0, n0 + wave_n0, M, N);
 }
 
 // Host-side launcher: sets the dynamic LDS size and launches one work-group per tile.
 // tile rows per band of the work-group -> tile order, for tuning runs (0 = each launcher's own choice: measured best
 // were 2 for the int8 kernels, 4 for the plain 16-bit GEMM and 8 for the fused W4A16 kernel; 1 = plain row-major)
 extern int g_gemm_band_rows;
-// stages ahead at which the lines of a later stage are touched (0 = off, the default; see the kernel)
-extern int g_gemm_touch_ahead;
 
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,
                 int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what, int band_rows = 4) {
   auto kern = gemm_mfma_kernel<Mma, AL, WL, Epi, BM, BN, WM, WN>;
-  // two stages, and one spare word per thread where later stages can be touched
-  constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes + (gemm_touch_ok<AL, WL, BM>() ? WM * WN * 256 : 0);
+  constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes;  // two stages
   static bool attr_set = false;  // per instantiation; idempotent, so a race only repeats the call
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -727,8 +764,7 @@ int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, co
   const int KT = (int)ceil_div(k_bytes, kStageBytes);
   const int k_tail = (k_bytes % kStageBytes) != 0;
   kern<<<(unsigned)blocks, WM * WN * 64, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, KT, k_tail, (int)tiles_m,
-                                                          (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows,
-                                                          g_gemm_touch_ahead);
+                                                          (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows);
   return check_launch(what) ? 0 : 1;
 }
 

@@ -12,7 +12,6 @@ struct H16KNLoader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
   static constexpr bool PREFETCH2 = false;
-  static constexpr int TOUCH_LINES = 0;  // no touch-ahead for this source layout
   static constexpr int NBLK = ROWS / 8;            // 8-column blocks per tile
   static constexpr int PASSES = (16 * NBLK) / NT;  // 64 k = 16 blocks of 4 rows
   static constexpr int UNITS = PASSES * 4;

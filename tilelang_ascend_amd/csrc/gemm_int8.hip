@@ -15,7 +15,6 @@ struct W4I8Loader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
   static constexpr bool PREFETCH2 = false;
-  static constexpr int TOUCH_LINES = 0;  // no touch-ahead for this source layout
   static constexpr int SLOTS = ROWS * 4;
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;

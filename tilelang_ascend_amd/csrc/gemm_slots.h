@@ -28,7 +28,6 @@ __global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDi
   extern __shared__ __align__(16) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r16 = lane & 15, q = lane >> 4;
   const int wave_m0 = (wave % WM) * (BM / WM), wave_n0 = (wave / WM) * (BN / WN);
   const TileCoord tc = tile_of_block<BM, BN>(tiles_m, tiles_n, band_rows);
   Loader al(pa, tc.batch, tc.m0, M, tid);
@@ -83,11 +82,8 @@ __global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDi
   addr::slots_schedule(KT, ops);
 
   Epi epi(pe, tc.batch);
-#pragma unroll
-  for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm)
-      epi.store(tc.m0 + wave_m0 + tm * 16 + r16, tc.n0 + wave_n0 + tn * 16 + q * 4, acc[tn][tm], M, N);
+  if constexpr (Epi::STAGED) __syncthreads();  // every wavefront is past its last operand read: LDS becomes the output staging area
+  write_tile<Epi, TM, TN>(epi, acc, smem + wave * (TM * 16 * kStageBytes), lane, tc.m0 + wave_m0, tc.n0 + wave_n0, M, N);
 }
 
 // tlq_tune_gemm_slots: 0 = the two-stage kernel (default), 1 = this one where it applies

@@ -29,7 +29,6 @@ struct W4Loader {
   typedef RowFrag Frag;
   static constexpr bool DIRECT = false;
   static constexpr bool PREFETCH2 = true;  // convert from registers loaded one stage earlier
-  static constexpr int TOUCH_LINES = 0;  // no touch-ahead for this source layout
   static constexpr int SLOTS = ROWS * 2;  // 16-byte packed loads per stage
   static constexpr int PASSES = (SLOTS + NT - 1) / NT;
   static constexpr bool PARTIAL = SLOTS % NT != 0;
