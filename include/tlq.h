@@ -224,6 +224,13 @@ int tlq_act_quant_i8(const void* X, void* Y, void* S, int64_t M, int64_t N, int 
 int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads);
 int tlq_debug_check_slots_schedule(int stages, int loads_per_tile);
 
+/* Launch geometry the register-resident decode GEMV (M = 1, K <= 16384, power-of-two group) would use on a device with
+ * `cus` compute units, computed on the host: plan_out is a HOST array of four int64 that receives rows per work-group,
+ * work-groups, bytes of dynamic LDS and wavefronts per work-group.  Returns 1 when the kernel applies (its LDS stays
+ * within the 64 KB a kernel may use without further set-up), 0 when the launcher falls back to the streaming GEMV,
+ * -1 for bad arguments.  No counterpart in the reference. */
+int tlq_debug_gemv_rows_plan(int64_t batch, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
+
 /* Tuning hooks for benchmark sweeps (process-global, not thread safe; 0 = automatic choice).
  * They play the role of the reference's block_M / block_N / block_K factory arguments
  * (example_dequant_gemm_fine_grained.py:437,462), which here select among pre-built tilings. */

@@ -112,6 +112,23 @@ def test_gemv_headline(ops, rows, waves):
 
 
 @pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("N,K,group", [(49152, 8192, 128), (8192, 16384, 64), (1031, 16384, 32)])
+def test_gemv_long_rows_and_many_rows(ops, in_dtype, N, K, group):
+    """Output-projection-sized decode shapes: rows of 8192 and 16384 values, whose activations alone take 18 - 36 KB of
+    the GEMV's LDS, so that the rows a work-group may own are limited by what is left of 64 KB (or the streaming kernel
+    takes over).  The kernel runs on all rows; 384 seeded rows plus the first and last ones are compared with the oracle."""
+    dt = DT[in_dtype]
+    A = torch.randn(1, K, generator=gen(40)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, "int", seed=41)
+    got = _run_w4a16(ops, A, Wp, s, z, group, in_dtype, "auto", in_dtype)
+    assert torch.isfinite(got.float()).all()
+    rows = torch.cat([torch.arange(0, min(N, 48)), torch.arange(max(0, N - 48), N),
+                      torch.randperm(N, generator=gen(42))[:384]]).unique()
+    want = w4a16_reference(A, Wp[rows], s[rows], z[rows], group)
+    check_float_output(got[:, rows], want, f"gemv {in_dtype} N={N} K={K} g={group}")
+
+
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
 @pytest.mark.parametrize("M,N,K,group,zeros_kind", [
     (1, 64, 64, 32, None), (1, 250, 2048, 128, "frac"), (2, 1000, 4096, 64, "int"), (3, 77, 1024, 1024, "scalar8"),
     (5, 130, 8192, 128, "int"), (16, 512, 14336, 128, "int"),

@@ -48,6 +48,7 @@ SIGNATURES = {
     "tlq_act_quant_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "tlq_debug_check_gemm_addressing": (_int, [_int, _i64, _i64, _int, _int]),
     "tlq_debug_check_slots_schedule": (_int, [_int, _int]),
+    "tlq_debug_gemv_rows_plan": (_int, [_i64, _i64, _i64, _i64, _int, _vp]),
     "tlq_tune_gemv": (None, [_int, _int]),
     "tlq_tune_gemv_unroll": (None, [_int]),
     "tlq_tune_gemv_depth": (None, [_int]),

@@ -379,7 +379,9 @@ __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __
 // activations per wavefront would put more bytes on it than the weights themselves, and one small
 // gather per row and tensor costs about as much as a 1 KB weight load.
 // A step is a whole row: ITERS 16-byte weight loads per lane.  D rows are in flight per wavefront; the
-// first D are requested before anything else, the staging loads right behind them.  The loop body
+// staging loads (a few KB the first multiply waits for) are requested first, the first D rows right behind them
+// (measured: 6.95 against 7.13 us per launch with the rows first; more rows in flight at the start, up to all of a
+// launch's rows, only delay the staging data behind megabytes of weights and were 1 - 2 us slower).  The loop body
 // is free of branches (rows past the end are clamped and their results dropped): the compiler then
 // keeps exact counts of the loads in flight instead of draining them at every control-flow merge.
 // Long rows (ITERS > 2) keep more activations per lane than a 16-wavefront work-group has registers for: those
@@ -393,8 +395,6 @@ __device__ __forceinline__ void gemv_rows_body(const T* __restrict__ A, const ui
                                                void* __restrict__ C, int N, int K, int group_shift, float zero_scalar,
                                                int out_dtype, int rows_per_block, int nwaves) {
   constexpr bool F16 = sizeof(T) == 2 && __is_same(T, half_t);
-  // The first weight rows: as few instructions as possible between the start of a wavefront and its first
-  // loads (everything they need sits in the first 64 bytes of the kernel arguments).
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int chunks = K >> 5;
@@ -419,12 +419,6 @@ __device__ __forceinline__ void gemv_rows_body(const T* __restrict__ A, const ui
   };
   Stage st[D];
   int irow = r0 + wave;  // next row to request
-#pragma unroll
-  for (int d = 0; d < D; ++d) {
-    issue(st[d], irow < r1 ? irow : r1 - 1);
-    irow += nwaves;
-  }
-  __builtin_amdgcn_sched_barrier(0);
 
   extern __shared__ __align__(16) uint8_t smem[];
   const int groups = K >> group_shift;
@@ -446,9 +440,8 @@ __device__ __forceinline__ void gemv_rows_body(const T* __restrict__ A, const ui
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) gsel[it] = (cc[it] << 5) >> group_shift;
 
-  // staging loads, behind the first weight rows (which are the ones that miss every cache and cannot be
-  // consumed before they arrive anyway): thread t < chunks fetches activation chunk t, and all threads
-  // copy the scale / zero rows, 16 bytes (or one value) each
+  // staging loads: thread t < chunks fetches activation chunk t, and all threads copy the scale / zero rows,
+  // 16 bytes (or one value) each
   const int tchunk = threadIdx.x < chunks ? threadIdx.x : chunks - 1;
   uint4_t araw[4];
 #pragma unroll
@@ -462,6 +455,13 @@ __device__ __forceinline__ void gemv_rows_body(const T* __restrict__ A, const ui
     if (has_s) s_raw = *(const uint4_t*)(scales + sz0 + t8);
     if (has_z) z_raw = *(const uint4_t*)(zeros + sz0 + t8);
   }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    issue(st[d], irow < r1 ? irow : r1 - 1);
+    irow += nwaves;
+  }
+  __builtin_amdgcn_sched_barrier(0);
 
   if (threadIdx.x < chunks) {
     if constexpr (F16) {
@@ -706,22 +706,49 @@ static int launch_gemv_f16(const void* A, const void* Wp, const void* scales, co
   return 0;
 }
 
-// rows kernel: work-groups of `waves_per_block` wavefronts, each owning a contiguous range of rows whose
-// scales and zero points fit its LDS; at least `blocks_per_cu` work-groups per CU when there are rows enough
+// Launch geometry of the rows kernel: work-groups of `waves_per_block` wavefronts, each owning `rows_per_block`
+// consecutive rows whose scales and zero points it keeps in LDS next to the prepared activations; at least
+// `blocks_per_cu` work-groups per CU when there are rows enough.  Everything a work-group keeps in LDS must fit the
+// 64 KB a kernel gets without asking for more: 72 bytes per 32 activations, 4 bytes per row and group.
+struct RowsPlan {
+  int rows_per_block, blocks;
+  size_t lds_bytes;
+  bool fits;
+};
+static RowsPlan plan_gemv_rows(int batch, int N, int K, int group_shift, int waves_per_block, int blocks_per_cu, int cus) {
+  RowsPlan p{0, 0, 0, false};
+  const int groups = K >> group_shift;
+  const size_t act_bytes = (size_t)(K / 32) * 72;
+  if (groups < 1 || act_bytes >= 64 * 1024) return p;
+  int blocks = (int)ceil_div((int64_t)cus * blocks_per_cu, batch);
+  if (blocks < 1) blocks = 1;
+  int rpb = (int)ceil_div(N, blocks);
+  if (rpb < waves_per_block) rpb = waves_per_block;
+  int rpb_max = (int)((64 * 1024 - act_bytes) / ((size_t)4 * groups));
+  if (rpb_max > (48 * 1024) / (4 * groups)) rpb_max = (48 * 1024) / (4 * groups);  // at most 48 KB of scales and zero points
+  rpb_max &= ~3;
+  if (rpb_max < waves_per_block) return p;
+  if (rpb > rpb_max) rpb = rpb_max;
+  rpb = (rpb + 3) & ~3;  // keeps the zero-point block of LDS 16-byte aligned for any group count
+  if (rpb > rpb_max) rpb = rpb_max;
+  p.rows_per_block = rpb;
+  p.blocks = (int)ceil_div(N, rpb);
+  p.lds_bytes = act_bytes + (size_t)rpb * groups * 4;
+  p.fits = p.lds_bytes <= 64 * 1024;
+  return p;
+}
+
 template <typename T, int ITERS, int D, int MAXT>
 static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int batch,
                             int N, int K, int group_shift, float zero_scalar, int out_dtype, int waves_per_block,
                             int blocks_per_cu, hipStream_t st) {
-  const int groups = K >> group_shift;
-  int blocks = (int)ceil_div((int64_t)cu_count() * blocks_per_cu, batch);
-  if (blocks < 1) blocks = 1;
-  int rpb = (int)ceil_div(N, blocks);
-  if (rpb < waves_per_block) rpb = waves_per_block;
-  const int rpb_max = (48 * 1024) / (4 * groups);  // scales + zeros of a work-group's rows: at most 48 KB of LDS
-  if (rpb > rpb_max) rpb = rpb_max;
-  rpb = (rpb + 3) & ~3;  // keeps the zero-point block of LDS 16-byte aligned for any group count
-  blocks = (int)ceil_div(N, rpb);
-  const size_t lds = (size_t)(K / 32) * 72 + (size_t)rpb * groups * 4;
+  const RowsPlan plan = plan_gemv_rows(batch, N, K, group_shift, waves_per_block, blocks_per_cu, cu_count());
+  if (!plan.fits) {
+    set_error("tlq_gemm_w4a16(gemv): K=%d with groups of %d does not fit the rows kernel's 64 KB of LDS", K, 1 << group_shift);
+    return 1;
+  }
+  const int rpb = plan.rows_per_block, blocks = plan.blocks;
+  const size_t lds = plan.lds_bytes;
   if constexpr (__is_same(T, half_t))
     gemv_w4a16_f16_rows_kernel<ITERS, D, MAXT><<<dim3(blocks, batch), 64 * waves_per_block, lds, st>>>(
         (const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C, N, K, group_shift,
@@ -733,16 +760,27 @@ static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, c
   return 0;
 }
 
+// wavefronts per work-group and work-groups per CU of the rows kernel for this K
+static void rows_kernel_shape(int64_t K, int& wpb_rows, int& bpc_rows) {
+  bpc_rows = g_gemv_unroll ? g_gemv_unroll : 1;
+  const bool long_rows = K > 4096;  // 8 wavefronts per work-group (see the kernel)
+  wpb_rows = g_gemv_waves16 ? g_gemv_waves16 : 16;
+  if (long_rows && wpb_rows > 8) wpb_rows = 8;
+  if (wpb_rows * 64 < K / 32) wpb_rows = (int)ceil_div(K / 32, (int64_t)64);  // one staging thread per chunk
+}
+static bool rows_kernel_fits(int64_t batch, int64_t N, int64_t K, int shift) {
+  int wpb_rows, bpc_rows;
+  rows_kernel_shape(K, wpb_rows, bpc_rows);
+  return plan_gemv_rows((int)batch, (int)N, (int)K, shift, wpb_rows, bpc_rows, cu_count()).fits;
+}
+
 // M = 1, rows of up to 16384 values: the register-resident kernel (see gemv_rows_body)
 template <typename T>
 static int dispatch_gemv_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch,
                               int64_t N, int64_t K, int shift, float zero_scalar, int out_dtype, hipStream_t st) {
   const int depth_req = g_gemv_depth;
-  const int bpc_rows = g_gemv_unroll ? g_gemv_unroll : 1;
-  const bool long_rows = K > 4096;  // 8 wavefronts per work-group (see the kernel)
-  int wpb_rows = g_gemv_waves16 ? g_gemv_waves16 : 16;
-  if (long_rows && wpb_rows > 8) wpb_rows = 8;
-  if (wpb_rows * 64 < K / 32) wpb_rows = (int)ceil_div(K / 32, (int64_t)64);  // one staging thread per chunk
+  int wpb_rows, bpc_rows;
+  rows_kernel_shape(K, wpb_rows, bpc_rows);
   // one problem of a few tens of MB: one row in flight per wavefront (deeper queues delay the staging
   // loads behind the weights and measured slower); many problems per launch stream with two
   const int d = depth_req ? depth_req : (batch * N * (K / 2) > ((int64_t)64 << 20) ? 2 : 1);
@@ -796,7 +834,7 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     const int R = g_gemv_rows > 0 ? g_gemv_rows : (streaming ? 2 : 1);
     const int bpc = g_gemv_unroll ? g_gemv_unroll : (streaming ? 64 : 8);  // grid size cap, blocks per CU
     const int depth_req = g_gemv_depth;
-    if (M == 1 && K <= 16384 && g_gemv_rows >= 0)
+    if (M == 1 && K <= 16384 && g_gemv_rows >= 0 && rows_kernel_fits(batch, N, K, shift))
       return dispatch_gemv_rows<half_t>(A, Wp, scales, zeros, C, batch, N, K, shift, zero_scalar, out_dtype, st);
     const bool two_rows = M > 1 && (size_t)2 * (K / 32) * 72 <= 64 * 1024;
 #define TLQ_F16_CASE(RR, MTT, DD)                                                                                  \
@@ -829,9 +867,9 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     launch_gemv<half_t, 2, 1>(A, Wp, scales, zeros, C, (int)batch, (int)M, (int)N, (int)K, (int)group, zero_scalar,
                               out_dtype, wpb, st);
   } else {
-    if (M == 1 && pow2 && K <= 16384 && g_gemv_rows >= 0) {
-      int shift = 0;
-      while (((int64_t)1 << shift) < group) ++shift;
+    int shift = 0;
+    while (((int64_t)1 << shift) < group) ++shift;
+    if (M == 1 && pow2 && K <= 16384 && g_gemv_rows >= 0 && rows_kernel_fits(batch, N, K, shift)) {
       return dispatch_gemv_rows<bf16_t>(A, Wp, scales, zeros, C, batch, N, K, shift, zero_scalar, out_dtype, st);
     }
     // bfloat16 otherwise: element-wise exact dequantisation (generic kernel)
@@ -848,6 +886,23 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
 }  // namespace tlq
 
 extern "C" {
+int tlq_debug_gemv_rows_plan(int64_t batch, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
+  int shift = 0;
+  while (((int64_t)1 << shift) < group) ++shift;
+  if (batch < 1 || N < 1 || K < 64 || K > 16384 || K % 64 || ((int64_t)1 << shift) != group || K % group || cus < 1) {
+    tlq::set_error("tlq_debug_gemv_rows_plan: bad arguments");
+    return -1;
+  }
+  int wpb, bpc;
+  tlq::rows_kernel_shape(K, wpb, bpc);
+  const tlq::RowsPlan p = tlq::plan_gemv_rows((int)batch, (int)N, (int)K, shift, wpb, bpc, cus);
+  if (plan_out) {
+    int64_t* out = (int64_t*)plan_out;
+    out[0] = p.rows_per_block, out[1] = p.blocks, out[2] = (int64_t)p.lds_bytes, out[3] = wpb;
+  }
+  return p.fits ? 1 : 0;
+}
+
 // Tuning hook used by the benchmark sweeps: rows per wavefront (1, 2, 4) and wavefronts per
 // block (1..4) of the GEMV kernel; 0 restores the automatic choice.
 void tlq_tune_gemv(int rows_per_wave, int waves_per_block) {
