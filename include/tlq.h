@@ -64,7 +64,9 @@ enum {
   TLQ_ALGO_GEMV = 1, /* split-K wavefront GEMV (M <= 16) */
   TLQ_ALGO_MFMA = 2, /* LDS-staged MFMA dequant-GEMM */
   TLQ_ALGO_SKINNY = 3, /* M <= 64: weights stream from HBM through the dequantiser into MFMA operands, no LDS tile */
-  TLQ_ALGO_TWO_PASS = 4 /* tlq_gemm_w4a16_ws only: dequantise into the workspace, then the plain GEMM */
+  TLQ_ALGO_TWO_PASS = 4, /* tlq_gemm_w4a16_ws only: dequantise into the workspace, then the plain GEMM */
+  TLQ_ALGO_STREAM = 5 /* tlq_gemm_w4a16_ws only: 17 <= M <= 512, weights streamed once per 128 activation rows through a deep
+                       * ring of direct loads, dequantised in registers; K slices add up through the workspace */
 };
 
 int tlq_abi_version(void);
@@ -111,8 +113,9 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
                    void* stream);
 
 /* The same operator with a caller-owned workspace of tlq_w4a16_workspace_bytes(M, N, K) bytes (0 when a
- * workspace would not be used).  With it, 16 < M <= 512 (and up to 2048 while there are few output tiles) runs the
- * tile kernel over slices of K whose fp32 partial sums live in the workspace and are added in slice order, and larger
+ * workspace would not be used).  With it, 16 < M <= 512 runs the streaming kernel (TLQ_ALGO_STREAM; K % 128 == 0,
+ * power-of-two group, N % 4 == 0) or, where that does not apply and up to M = 2048 while there are few output tiles, the
+ * tile kernel, both over slices of K whose fp32 partial sums live in the workspace and are added in slice order, and larger
  * problems take two passes -- tlq_dequant_w4 into the workspace, then tlq_gemm_f16 on it -- which is the structure of the reference's own wrapper
  * (example_dequant_gemm_fine_grained.py:176-223 unpacks, then calls fp16_gemm) and is faster than converting
  * the weights again in every row block of the fused kernel.  The workspace holds nothing between calls.
@@ -223,6 +226,9 @@ int tlq_act_quant_i8(const void* X, void* Y, void* S, int64_t M, int64_t N, int 
  * Both return 0 when everything holds, else 1 with tlq_last_error() naming the first violation. */
 int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads);
 int tlq_debug_check_slots_schedule(int stages, int loads_per_tile);
+/* The same walk for the streaming W4A16 kernel (TLQ_ALGO_STREAM): packed weights [N, K / 2] and 2-byte activations [M, K]
+ * with 16 * activation_tiles rows per work-group (2 | 4 | 8), and its ring of `ring_depth` steps for 1 .. 40 steps. */
+int tlq_debug_check_stream_addressing(int64_t M, int64_t N, int64_t K, int activation_tiles, int ring_depth);
 
 /* Launch geometry the register-resident decode GEMV (M = 1, K <= 16384, power-of-two group) would use on a device with
  * `cus` compute units, computed on the host: plan_out is a HOST array of four int64 that receives rows per work-group,
@@ -242,6 +248,7 @@ void tlq_tune_gemm_band(int tile_rows);                       /* tile rows per b
 void tlq_tune_gemm_slots(int on);                            /* 1 (default): 256 x 256 tiles of the plain 16-bit GEMM with [N, K] weights and of the
                                                               * int8 GEMMs run on the kernel that cuts LDS into five operand-tile slots
                                                               * (whole 128-byte stages of K only); 0: always the two-stage kernel */
+void tlq_tune_w4a16_stream(int on);                          /* 0: tlq_gemm_w4a16_ws never picks the streaming kernel by itself */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
 void tlq_tune_w4a16_split(int slices);                       /* K slices of the tile kernel, 16 < M < 256 with a workspace */
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,

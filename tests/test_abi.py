@@ -187,6 +187,6 @@ def test_workspace_size_rules():
         b = ws(M, N, K)
         assert b > 0 and b % (M * N * 4) == 0, (M, N, K, b)
         split = b // (M * N * 4)
-        assert 2 <= split <= 16 and K % split == 0 and (K // split) % 64 == 0 and K // split >= 512, (M, N, K, split)
+        assert 2 <= split <= 16, (M, N, K, split)  # room for the most K slices any kernel and group size may cut
     assert ws(1024, 14336, 4096) == 14336 * 4096 * 2  # many output tiles already: no K slices, two passes
     assert ws(64, 0, 4096) == 0 and ws(64, 128, 0) == 0

@@ -62,3 +62,15 @@ def test_five_slot_schedule():
     assert "before its loads were waited for" in _abi.last_error()
     _ok(lib.tlq_debug_check_slots_schedule(8, 8))
 
+
+
+@pytest.mark.parametrize("tm,depth", [(2, 5), (4, 4), (8, 3)])
+def test_streaming_kernel_addressing(tm, depth):
+    """Streaming W4A16 kernel: every direct load stays inside the packed weights / the activations (rows past the
+    matrices are clamped), lands on the LDS cell its operand read expects, and the ring never multiplies a step before
+    its loads were waited for nor reloads a slot that may still be read."""
+    lib = _abi.load()
+    for M, N, K in [(17, 256, 128), (64, 14336, 4096), (100, 4096, 14336), (33, 1000, 256), (512, 260, 1152), (128, 8, 128)]:
+        _ok(lib.tlq_debug_check_stream_addressing(M, N, K, tm, depth))
+    assert lib.tlq_debug_check_stream_addressing(64, 256, 100, tm, depth) != 0   # K not a multiple of 128
+    assert lib.tlq_debug_check_stream_addressing(64, 1 << 22, 4096, tm, depth) != 0  # packed weights of 8 GiB

@@ -18,7 +18,7 @@ from . import build as _build
 F16, BF16, F32, I8, I32 = 0, 1, 2, 3, 4
 U4, S4_TWOS, S4_OFFSET8, S4_OFFSET7 = 0, 1, 2, 3
 B_KN, B_NK = 0, 1
-ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY, ALGO_TWO_PASS = 0, 1, 2, 3, 4
+ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY, ALGO_TWO_PASS, ALGO_STREAM = 0, 1, 2, 3, 4, 5
 ABI_VERSION = 1
 
 _vp, _i64, _int, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
@@ -48,12 +48,14 @@ SIGNATURES = {
     "tlq_act_quant_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "tlq_debug_check_gemm_addressing": (_int, [_int, _i64, _i64, _int, _int]),
     "tlq_debug_check_slots_schedule": (_int, [_int, _int]),
+    "tlq_debug_check_stream_addressing": (_int, [_i64, _i64, _i64, _int, _int]),
     "tlq_debug_gemv_rows_plan": (_int, [_i64, _i64, _i64, _i64, _int, _vp]),
     "tlq_tune_gemv": (None, [_int, _int]),
     "tlq_tune_gemv_unroll": (None, [_int]),
     "tlq_tune_gemv_depth": (None, [_int]),
     "tlq_tune_gemm_band": (None, [_int]),
     "tlq_tune_gemm_slots": (None, [_int]),
+    "tlq_tune_w4a16_stream": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),
     "tlq_tune_w4a16_split": (None, [_int]),
     "tlq_tune_w4a16_skinny": (None, [_int, _int]),

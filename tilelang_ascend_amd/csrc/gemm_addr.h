@@ -94,5 +94,35 @@ __host__ __device__ inline void slots_schedule(int KT, Ops& ops) {
   }
 }
 
+// ---- streaming W4A16 kernel for small and middle M (gemm_w4a16_stream.hip) ---------------------------------------
+// One step is 128 values of K.  A work-group of 8 wavefronts owns 256 weight rows (wavefront w: rows 32 w .. 32 w + 31,
+// two 16-row MFMA tiles) and 16 * TM activation rows.
+// Packed weights: [16 rows][64 B] per MFMA tile, private to the wavefront.  One direct load covers a tile (lane l lands
+// on row l / 4, 16-byte piece l % 4 and fetches logical piece (l % 4) ^ ((row >> 2) & 3)); the operand read of lane
+// (row r16, k-group q) takes logical piece q: the four 32-bit words 4 q .. 4 q + 3 = values 32 q .. 32 q + 31 of the step.
+__host__ __device__ inline int sw_row(int lane) { return lane >> 2; }
+__host__ __device__ inline int sw_piece(int lane) { return (lane & 3) ^ ((sw_row(lane) >> 2) & 3); }
+__host__ __device__ inline uint32_t sw_frag_off(int lane) {  // inside the 1 KB tile
+  const int r16 = lane & 15, q = lane >> 4;
+  return (uint32_t)(r16 * 64 + ((q ^ ((r16 >> 2) & 3)) << 4));
+}
+// Activations: [16 TM rows][256 B], shared by the work-group.  Direct load I (of 4 TM) covers rows 4 I .. 4 I + 3 (lane
+// l: row 4 I + l / 16, physical chunk l % 16, logical chunk (l % 16) ^ (row & 15)); lane (m = r16, k-group q) reads
+// logical chunk 4 q + ks for MFMA k-step ks, i.e. the eight values that word 4 q + ks of the weights holds.
+__host__ __device__ inline int sa_row(int lane, int I) { return 4 * I + (lane >> 4); }
+__host__ __device__ inline int sa_chunk(int lane, int I) { return (lane & 15) ^ (sa_row(lane, I) & 15); }
+__host__ __device__ inline uint32_t sa_frag_off(int lane, int tm, int ks) {
+  const int r16 = lane & 15, q = lane >> 4;
+  return (uint32_t)((tm * 16 + r16) * 256 + (((4 * q + ks) ^ r16) << 4));
+}
+// Ring of D steps: step s lives in slot s % D.  Every wavefront issues `per_step` load instructions per step, in
+// step order, and loads retire in issue order: this wavefront's loads of step s have landed once at most the
+// loads of the younger steps that were already issued are outstanding.  At the top of step s (before the loads of
+// step s + D - 1 are issued) those are the steps s + 1 .. min(s + D - 2, last).
+__host__ __device__ inline int stream_younger_steps(int s, int steps, int D) {
+  const int last_issued = s + D - 2 < steps - 1 ? s + D - 2 : steps - 1;
+  return last_issued - s > 0 ? last_issued - s : 0;
+}
+
 }  // namespace addr
 }  // namespace tlq

@@ -195,6 +195,95 @@ struct SlotsSim {
   }
 };
 
+// Streaming W4A16 kernel: packed weights [N, K / 2], activations [M, K] of 2-byte values, 16 * tm activation rows and
+// 256 weight rows per work-group, steps of 128 values of K.
+int check_stream(int64_t M, int64_t N, int64_t K, int tm) {
+  CHECK_OR_FAIL(tm == 2 || tm == 4 || tm == 8, "stream: %d activation tiles", tm);
+  CHECK_OR_FAIL(M > 0 && N > 0 && K >= 128 && K % 128 == 0, "stream: bad shape");
+  CHECK_OR_FAIL(N * (K / 2) < ((int64_t)1 << 32) && M * K * 2 < ((int64_t)1 << 32), "stream: a matrix spans 4 GiB or more");
+  const int64_t w_extent = N * (K / 2), a_extent = M * K * 2;
+  const int steps = (int)(K / 128), la = tm / 2;
+  std::vector<int> cell(1024 / 16), acell(tm * 16 * 16);
+  for (int64_t n0 = 0; n0 < N; n0 += 256)
+    for (int wave = 0; wave < 8; ++wave)
+      for (int tn = 0; tn < 2; ++tn) {
+        std::fill(cell.begin(), cell.end(), -1);
+        for (int lane = 0; lane < 64; ++lane) {
+          int64_t n = n0 + wave * 32 + tn * 16 + addr::sw_row(lane);
+          n = n < N ? n : N - 1;
+          const int64_t voff = n * (K / 2) + addr::sw_piece(lane) * 16;
+          for (int st = 0; st < steps; ++st) {
+            const int64_t o = voff + (int64_t)st * 64;
+            CHECK_OR_FAIL(o >= 0 && o + 16 <= w_extent, "stream: weight load at [%lld, +16) of %lld", (long long)o, (long long)w_extent);
+          }
+          cell[lane] = addr::sw_row(lane) * 4 + addr::sw_piece(lane);  // the lane lands on 16-byte cell `lane` of the 1 KB tile
+        }
+        for (int lane = 0; lane < 64; ++lane) {
+          const uint32_t off = addr::sw_frag_off(lane);
+          CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= 1024, "stream: weight operand read at %u", off);
+          CHECK_OR_FAIL(cell[off / 16] == (lane & 15) * 4 + (lane >> 4), "stream: weight operand read of lane %d finds cell %d", lane, cell[off / 16]);
+        }
+      }
+  for (int64_t m0 = 0; m0 < M; m0 += 16 * tm) {
+    std::fill(acell.begin(), acell.end(), -1);
+    for (int wave = 0; wave < 8; ++wave)
+      for (int j = 0; j < la; ++j) {
+        const int I = j * 8 + wave;
+        CHECK_OR_FAIL(I < 4 * tm, "stream: activation load instruction %d of %d", I, 4 * tm);
+        for (int lane = 0; lane < 64; ++lane) {
+          const int row = addr::sa_row(lane, I), chunk = addr::sa_chunk(lane, I);
+          CHECK_OR_FAIL(row < 16 * tm && chunk >= 0 && chunk < 16, "stream: activation row %d chunk %d", row, chunk);
+          int64_t m = m0 + row;
+          m = m < M ? m : M - 1;
+          const int64_t voff = m * K * 2 + chunk * 16;
+          for (int st = 0; st < steps; ++st) {
+            const int64_t o = voff + (int64_t)st * 256;
+            CHECK_OR_FAIL(o >= 0 && o + 16 <= a_extent, "stream: activation load at [%lld, +16) of %lld", (long long)o, (long long)a_extent);
+          }
+          const int at = I * 64 + lane;  // 16-byte cell inside the activation tile
+          CHECK_OR_FAIL(at < (int)acell.size() && acell[at] == -1, "stream: activation cell %d written twice", at);
+          CHECK_OR_FAIL(at == row * 16 + (lane & 15), "stream: activation lane lands on cell %d, not on its row", at);
+          acell[at] = row * 16 + chunk;
+        }
+      }
+    for (size_t c = 0; c < acell.size(); ++c) CHECK_OR_FAIL(acell[c] >= 0, "stream: activation cell %zu never written", c);
+    for (int t = 0; t < tm; ++t)
+      for (int ks = 0; ks < 4; ++ks)
+        for (int lane = 0; lane < 64; ++lane) {
+          const uint32_t off = addr::sa_frag_off(lane, t, ks);
+          CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= (uint32_t)tm * 4096, "stream: activation operand read at %u", off);
+          const int want = (t * 16 + (lane & 15)) * 16 + 4 * (lane >> 4) + ks;
+          CHECK_OR_FAIL(acell[off / 16] == want, "stream: activation operand read (lane %d, k-step %d) finds cell %d, expects %d", lane, ks,
+                        acell[off / 16], want);
+        }
+  }
+  return 0;
+}
+
+// The ring: step s occupies slot s % D; at the top of step s the wavefront waits until only `younger` steps' loads are
+// outstanding, passes the barrier, and then issues step s + D - 1 into the slot of step s - 1.
+int check_stream_ring(int steps, int D) {
+  CHECK_OR_FAIL(steps >= 1 && D >= 2 && D <= 8, "stream ring: bad arguments");
+  std::vector<int> slot(D, -1), queue;  // slot owner; issued and not yet known to have landed (oldest first)
+  std::vector<char> landed(steps, 0), done(steps, 0);
+  for (int s = 0; s < D - 1 && s < steps; ++s) slot[s % D] = s, queue.push_back(s);
+  for (int s = 0; s < steps; ++s) {
+    const int younger = addr::stream_younger_steps(s, steps, D);
+    while ((int)queue.size() > younger) landed[queue.front()] = 1, queue.erase(queue.begin());
+    CHECK_OR_FAIL(landed[s], "stream ring: step %d multiplied before its loads were waited for", s);
+    // barrier: every wavefront is past step s - 1
+    if (s >= 1) done[s - 1] = 1;
+    if (s + D - 1 < steps) {
+      const int t = s + D - 1, sl = t % D;
+      CHECK_OR_FAIL(slot[sl] < 0 || done[slot[sl]], "stream ring: step %d overwrites step %d which may still be read", t, slot[sl]);
+      slot[sl] = t, queue.push_back(t);
+    }
+    CHECK_OR_FAIL(slot[s % D] == s, "stream ring: the slot of step %d holds step %d", s, slot[s % D]);
+  }
+  CHECK_OR_FAIL(queue.empty() || queue.back() <= steps - 1, "stream ring: bookkeeping");
+  return 0;
+}
+
 }  // namespace
 }  // namespace tlq
 
@@ -212,6 +301,13 @@ int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_b
   }
   set_error("tlq_debug_check_gemm_addressing: bad source kind %d", source_kind);
   return 1;
+}
+
+int tlq_debug_check_stream_addressing(int64_t M, int64_t N, int64_t K, int activation_tiles, int ring_depth) {
+  if (int rc = check_stream(M, N, K, activation_tiles)) return rc;
+  for (int steps = 1; steps <= 40; ++steps)
+    if (int rc = check_stream_ring(steps, ring_depth)) return rc;
+  return 0;
 }
 
 int tlq_debug_check_slots_schedule(int stages, int loads_per_tile) {

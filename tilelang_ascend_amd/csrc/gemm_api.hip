@@ -11,6 +11,14 @@ int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group);
 int gemm_w4a16_mfma_splitk(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M,
                            int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype,
                            int64_t split, float* partial, hipStream_t st);
+struct StreamPlan {
+  bool ok;
+  int tm, m_blocks, n_blocks, split, slice_steps;
+};
+StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus);
+int gemm_w4a16_stream(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                      int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, const StreamPlan& p,
+                      float* partial, hipStream_t st);
 int gemm_w4a16_skinny(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                       int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
@@ -27,6 +35,12 @@ int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, 
 int g_gemm_band_rows = 0;
 int g_gemm_slots = 1;
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+// compute units of the current device (256 when it cannot be asked, e.g. without a GPU)
+static int cu_count_or_default() {
+  const int n = tlq_device_cu_count();
+  return n > 0 ? n : 256;
+}
+int g_w4a16_stream = 1;  // 0: never pick the streaming kernel automatically (tuning runs)
 // the tile loaders address one matrix with 32-bit byte offsets
 static bool fits32(int64_t rows, int64_t row_bytes) { return rows * row_bytes < ((int64_t)1 << 32); }
 static const int64_t kMaxDim = (int64_t)1 << 30;
@@ -42,6 +56,7 @@ extern "C" {
 
 void tlq_tune_gemm_band(int tile_rows) { tlq::g_gemm_band_rows = tile_rows < 0 ? 0 : tile_rows; }
 void tlq_tune_gemm_slots(int on) { tlq::g_gemm_slots = on != 0; }
+void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
 
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
@@ -94,10 +109,23 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
 // N = 14336, K = 4096 and 20-40 % ahead from there on and for N = 4096, K = 14336)
 static const int64_t kTwoPassMinM = 256;
 
+// most K slices the streaming kernel may cut for any group size (the smallest group allows the shortest slices)
+static int64_t stream_max_split(int64_t M, int64_t N, int64_t K) {
+  int64_t most = 0;
+  for (int64_t group = 32; group <= K; group *= 2) {
+    if (K % group) continue;
+    const StreamPlan p = w4a16_stream_plan(M, N, K, group, 256);
+    if (p.ok && p.split > most) most = p.split;
+  }
+  return most;
+}
+
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
   // small and middle M: fp32 partial sums of the K slices (sized for the smallest group, which allows the most slices)
-  const int64_t split = w4a16_mid_split(M, N, K, 32);
+  int64_t split = w4a16_mid_split(M, N, K, 32);
+  const int64_t ssplit = stream_max_split(M, N, K);
+  if (ssplit > split) split = ssplit;
   if (split > 1) return split * M * N * 4;
   return M >= kTwoPassMinM ? N * K * 2 : 0;
 }
@@ -105,12 +133,34 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
-  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_TWO_PASS, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_STREAM, "tlq_gemm_w4a16_ws: bad algo %d", algo);
   const int64_t need = (N > 0 && K > 0) ? N * K * 2 : 0;
   const bool have = workspace != nullptr && workspace_bytes >= need && aligned16(workspace);
   if (algo == TLQ_ALGO_TWO_PASS)
     TLQ_REQUIRE(have, "tlq_gemm_w4a16_ws: the two-pass path needs a 16-byte aligned workspace of %lld bytes (got %lld)",
                 (long long)need, (long long)workspace_bytes);
+  // 17 .. 512 activation rows: the streaming kernel (weights once per 128 rows, deep ring of direct loads)
+  if ((algo == TLQ_ALGO_AUTO && g_w4a16_stream) || algo == TLQ_ALGO_STREAM) {
+    const StreamPlan sp = (K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)
+                              ? w4a16_stream_plan(M, N, K, group, cu_count_or_default())
+                              : StreamPlan{false, 0, 0, 0, 0, 0};
+    const bool args_ok = A && w_packed && C && aligned16(A) && aligned16(w_packed) && aligned16(C) &&
+                         (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) &&
+                         (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) && (M * N) % 4 == 0 &&
+                         ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0 && K > 0 && fits32(M, K * 2) && fits32(N, K / 2);
+    const bool ws_ok = sp.ok && (sp.split == 1 || (workspace && aligned16(workspace) && workspace_bytes >= (int64_t)sp.split * M * N * 4));
+    // measured on the MLP shapes: 20 - 35 % ahead of the tile kernel up to 256 rows, level with it at 512
+    if (sp.ok && args_ok && ws_ok && (algo == TLQ_ALGO_STREAM || M <= 256))
+      return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, sp, (float*)workspace,
+                               (hipStream_t)stream);
+    if (algo == TLQ_ALGO_STREAM) {
+      set_error("tlq_gemm_w4a16_ws: the streaming kernel needs 17 <= M <= 512, K %% 128 == 0, a power-of-two group >= 32, N %% 4 == 0, "
+                "16-byte aligned operands and a workspace of %lld bytes (M=%lld N=%lld K=%lld group=%lld, workspace %lld)",
+                (long long)(sp.ok ? (int64_t)sp.split * M * N * 4 : 0), (long long)M, (long long)N, (long long)K, (long long)group,
+                (long long)workspace_bytes);
+      return 1;
+    }
+  }
   const bool split_region = w4a16_mid_split(M, N, K, group > 0 ? group : 32) > 1;
   const bool two_pass = algo == TLQ_ALGO_TWO_PASS ||
                         (algo == TLQ_ALGO_AUTO && have && M >= kTwoPassMinM && N % 8 == 0 && !split_region);

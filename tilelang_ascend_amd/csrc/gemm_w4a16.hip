@@ -725,6 +725,11 @@ int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group) {
   return 1;
 }
 
+void launch_splitk_reduce(const float* partial, void* C, int64_t M, int64_t N, int split, int out_dtype, hipStream_t st) {
+  const int64_t n4 = M * N / 4, want = ceil_div(n4, (int64_t)256);
+  splitk_reduce_kernel<<<(int)(want > 65536 ? 65536 : want), 256, 0, st>>>((const float4_t*)partial, C, n4, split, out_dtype);
+}
+
 int gemm_w4a16_mfma_splitk(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M,
                            int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype,
                            int64_t split, float* partial, hipStream_t st) {
