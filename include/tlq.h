@@ -58,6 +58,13 @@ enum {
   TLQ_B_NK = 1  /* B[N, K] row-major, i.e. transpose_B (examples/deepseek_v4/int8_gemm.py:58,77) */
 };
 
+/* arrangement of the eight 4-bit fields inside each 32-bit word of packed weights */
+enum {
+  TLQ_W_PLAIN = 0,           /* field k = element k: general_compress (tilelang/quantize/utils.py:53-69) */
+  TLQ_W_INTERLEAVED_F16 = 1  /* fields hold elements 0, 2, 4, 6, 1, 3, 5, 7: interleave_weight for the fp16 target
+                              * (utils.py:73-101), the layout the reference's fast decoders read (lop3.py:17-24) */
+};
+
 /* kernel selection for tlq_gemm_w4a16 */
 enum {
   TLQ_ALGO_AUTO = 0,
@@ -88,6 +95,11 @@ int tlq_unpack_int4(const void* w_packed, void* out, int64_t N, int64_t K, int o
  * group must divide K and be even. */
 int tlq_dequant_w4(const void* w_packed, const void* scales, const void* zeros, void* out, int64_t N, int64_t K,
                    int64_t group, float zero_scalar, int dtype, void* stream);
+
+/* tlq_dequant_w4 for either arrangement of the packed words (w_layout: TLQ_W_PLAIN | TLQ_W_INTERLEAVED_F16).  Interleaved
+ * words need K % 8 == 0 and group % 8 == 0. */
+int tlq_dequant_w4_layout(const void* w_packed, const void* scales, const void* zeros, void* out, int64_t N, int64_t K,
+                          int64_t group, float zero_scalar, int dtype, int w_layout, void* stream);
 
 /* Fast decode of INTERLEAVED 4-bit weights, the gfx950 counterpart of the CUDA decoders that
  * get_lop3_intrin_group returns (tilelang/quantize/lop3.py:5-421, 998-1046, 1090-1202).  `words` are
@@ -124,6 +136,15 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream);
+
+/* tlq_gemm_w4a16_ws for weights whose words were repacked by interleave_weight (w_layout TLQ_W_INTERLEAVED_F16, e.g. by
+ * tlq_pack_int4(interleave = 1)); TLQ_W_PLAIN is tlq_gemm_w4a16_ws itself.  Consumers of the repacked layout: the
+ * streaming kernel (17 <= M <= 512; the fp16 decode saves the four byte permutes per word that only undo the plain layout)
+ * and the two passes (M >= 256 with a workspace of N * K 16-bit values).  Other shapes are rejected: decode-sized problems
+ * read the plain layout.  Results are bit-identical to the plain layout on the same logical weights. */
+int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
+                             int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
+                             int w_layout, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose wrapper allocates its

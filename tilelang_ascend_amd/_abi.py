@@ -18,6 +18,7 @@ from . import build as _build
 F16, BF16, F32, I8, I32 = 0, 1, 2, 3, 4
 U4, S4_TWOS, S4_OFFSET8, S4_OFFSET7 = 0, 1, 2, 3
 B_KN, B_NK = 0, 1
+W_PLAIN, W_INTERLEAVED_F16 = 0, 1
 ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY, ALGO_TWO_PASS, ALGO_STREAM = 0, 1, 2, 3, 4, 5
 ABI_VERSION = 1
 
@@ -39,6 +40,8 @@ SIGNATURES = {
     "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_w4a16_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "tlq_gemm_w4a16_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp, _i64, _vp]),
+    "tlq_gemm_w4a16_layout_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _int, _vp, _i64, _vp]),
+    "tlq_dequant_w4_layout": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _int, _int, _vp]),
     "tlq_gemm_w4a16_noalloc_init": (_int, []),
     "tlq_gemm_w4a16_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp]),
     "tlq_gemm_f16_splitk": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),

@@ -17,7 +17,7 @@ struct StreamPlan {
 };
 StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus);
 int gemm_w4a16_stream(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
-                      int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, const StreamPlan& p,
+                      int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const StreamPlan& p,
                       float* partial, hipStream_t st);
 int gemm_w4a16_skinny(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                       int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
@@ -151,7 +151,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const bool ws_ok = sp.ok && (sp.split == 1 || (workspace && aligned16(workspace) && workspace_bytes >= (int64_t)sp.split * M * N * 4));
     // measured on the MLP shapes: 20 - 35 % ahead of the tile kernel up to 256 rows, level with it at 512
     if (sp.ok && args_ok && ws_ok && (algo == TLQ_ALGO_STREAM || M <= 256))
-      return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, sp, (float*)workspace,
+      return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
     if (algo == TLQ_ALGO_STREAM) {
       set_error("tlq_gemm_w4a16_ws: the streaming kernel needs 17 <= M <= 512, K %% 128 == 0, a power-of-two group >= 32, N %% 4 == 0, "
@@ -189,6 +189,44 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
               "tlq_gemm_w4a16_ws: group=%lld must divide K=%lld and be a multiple of 32", (long long)group, (long long)K);
   TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16_ws: scales / zeros misaligned");
   if (int rc = tlq_dequant_w4(w_packed, scales, zeros, workspace, N, K, group, zero_scalar, in_dtype, stream)) return rc;
+  return tlq_gemm_f16(A, workspace, C, M, N, K, in_dtype, out_dtype, TLQ_B_NK, stream);
+}
+
+int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
+                             int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
+                             int w_layout, void* workspace, int64_t workspace_bytes, void* stream) {
+  TLQ_REQUIRE(w_layout == TLQ_W_PLAIN || w_layout == TLQ_W_INTERLEAVED_F16, "tlq_gemm_w4a16_layout_ws: bad weight layout %d", w_layout);
+  if (w_layout == TLQ_W_PLAIN)
+    return tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, algo, workspace,
+                             workspace_bytes, stream);
+  TLQ_CHECK_DIMS("tlq_gemm_w4a16_layout_ws");
+  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS,
+              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the streaming kernel and the two passes (algo %d)", algo);
+  TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_w4a16_layout_ws: in_dtype must be float16 or bfloat16 (got %d)", in_dtype);
+  TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_w4a16_layout_ws: bad out_dtype %d", out_dtype);
+  if (M == 0 || N == 0) return 0;
+  TLQ_REQUIRE(K > 0 && K % 64 == 0, "tlq_gemm_w4a16_layout_ws: K=%lld must be a positive multiple of 64", (long long)K);
+  TLQ_REQUIRE(group > 0 && K % group == 0 && group % 32 == 0, "tlq_gemm_w4a16_layout_ws: group=%lld must divide K=%lld and be a multiple of 32",
+              (long long)group, (long long)K);
+  TLQ_REQUIRE(A && w_packed && C, "tlq_gemm_w4a16_layout_ws: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(w_packed) && aligned16(C), "tlq_gemm_w4a16_layout_ws: A, w_packed and C must be 16-byte aligned");
+  TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16_layout_ws: scales / zeros misaligned");
+  TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K / 2), "tlq_gemm_w4a16_layout_ws: a matrix spans 4 GiB or more");
+  const bool ws_aligned = workspace && aligned16(workspace);
+  if (algo != TLQ_ALGO_TWO_PASS) {
+    const StreamPlan sp = w4a16_stream_plan(M, N, K, group, cu_count_or_default());
+    const bool ws_ok = sp.ok && (M * N) % 4 == 0 && (sp.split == 1 || (ws_aligned && workspace_bytes >= (int64_t)sp.split * M * N * 4));
+    if (ws_ok && (algo == TLQ_ALGO_STREAM || M <= 256 || !(ws_aligned && workspace_bytes >= N * K * 2)))
+      return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, sp,
+                               (float*)workspace, (hipStream_t)stream);
+    TLQ_REQUIRE(algo != TLQ_ALGO_STREAM, "tlq_gemm_w4a16_layout_ws: the streaming kernel does not take M=%lld N=%lld K=%lld group=%lld "
+                "with a workspace of %lld bytes", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
+  }
+  TLQ_REQUIRE(M >= 17, "tlq_gemm_w4a16_layout_ws: decode-sized problems (M=%lld) read the plain layout", (long long)M);
+  TLQ_REQUIRE(ws_aligned && workspace_bytes >= N * K * 2 && N % 8 == 0,
+              "tlq_gemm_w4a16_layout_ws: M=%lld N=%lld K=%lld needs a 16-byte aligned workspace of %lld bytes (got %lld) and N %% 8 == 0",
+              (long long)M, (long long)N, (long long)K, (long long)(N * K * 2), (long long)workspace_bytes);
+  if (int rc = tlq_dequant_w4_layout(w_packed, scales, zeros, workspace, N, K, group, zero_scalar, in_dtype, w_layout, stream)) return rc;
   return tlq_gemm_f16(A, workspace, C, M, N, K, in_dtype, out_dtype, TLQ_B_NK, stream);
 }
 

@@ -21,6 +21,8 @@
 // k assignment inside a step: lane (row r16, k-group q) holds, at MFMA k-step ks, the eight values of packed word
 // 4 q + ks of its row, i.e. k = 32 q + 8 ks .. + 7; its four words are 16 contiguous bytes (one LDS read), all in one
 // quantisation group (groups are >= 32 values), and the activation operand reads the matching 16-byte chunk 4 q + ks.
+// Weights whose 32-bit words went through interleave_weight (tilelang/quantize/utils.py:73-101, fp16 target) are taken
+// as they are (LAYOUT 1): the word is still the same eight consecutive k, only the decode differs.
 #include "expand8.h"
 #include "gemm_core.h"
 
@@ -60,7 +62,7 @@ struct StreamCfg {
 };
 constexpr int kStreamMaxGroups = 16;  // quantisation groups per K slice whose scales fit the private LDS area
 
-template <typename T, int TM>
+template <typename T, int TM, int LAYOUT>
 __global__ __launch_bounds__(512, 2) void w4a16_stream_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
                                                              const T* __restrict__ scales, const T* __restrict__ zeros,
                                                              void* __restrict__ C, float* __restrict__ partial, int M, int N, int K,
@@ -197,7 +199,7 @@ __global__ __launch_bounds__(512, 2) void w4a16_stream_kernel(const T* __restric
       for (int ks = 0; ks < 4; ++ks) af[tm][ks] = *(const uint4_t*)(slot + fo_a[ks] + tm * 16 * 256);
 #pragma unroll
     for (int tn = 0; tn < 2; ++tn) {
-      const Expand8<T, FOLD> ex(sv[tn], zv[tn], mg);
+      const Expand8<T, FOLD, LAYOUT> ex(sv[tn], zv[tn], mg);
       const uint32_t w[4] = {wq[tn].x, wq[tn].y, wq[tn].z, wq[tn].w};
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
@@ -269,11 +271,11 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   return p;
 }
 
-template <typename T, int TM>
+template <typename T, int TM, int LAYOUT>
 static int launch_stream(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, float* partial,
                          int64_t M, int64_t N, int64_t K, int gshift, float zero_scalar, int out_dtype, const StreamPlan& p,
                          hipStream_t st) {
-  auto kern = w4a16_stream_kernel<T, TM>;
+  auto kern = w4a16_stream_kernel<T, TM, LAYOUT>;
   constexpr int lds_bytes = StreamCfg<TM>::LDS;
   static bool attr_set = false;
   if (!attr_set) {
@@ -292,16 +294,18 @@ static int launch_stream(const void* A, const void* Wp, const void* scales, cons
 
 // partial: fp32 [split][M][N] workspace, needed when the plan has more than one K slice
 int gemm_w4a16_stream(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
-                      int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, const StreamPlan& p,
+                      int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const StreamPlan& p,
                       float* partial, hipStream_t st) {
   int gshift = 0;
   while (((int64_t)1 << gshift) < group) ++gshift;
   int rc;
-#define TLQ_STREAM(T, TM) launch_stream<T, TM>(A, Wp, scales, zeros, C, partial, M, N, K, gshift, zero_scalar, out_dtype, p, st)
+#define TLQ_STREAM3(T, TM, LAY) launch_stream<T, TM, LAY>(A, Wp, scales, zeros, C, partial, M, N, K, gshift, zero_scalar, out_dtype, p, st)
+#define TLQ_STREAM(T, TM) (w_layout == TLQ_W_INTERLEAVED_F16 ? TLQ_STREAM3(T, TM, 1) : TLQ_STREAM3(T, TM, 0))
   if (in_dtype == TLQ_F16)
     rc = p.tm == 2 ? TLQ_STREAM(half_t, 2) : (p.tm == 4 ? TLQ_STREAM(half_t, 4) : TLQ_STREAM(half_t, 8));
   else
     rc = p.tm == 2 ? TLQ_STREAM(bf16_t, 2) : (p.tm == 4 ? TLQ_STREAM(bf16_t, 4) : TLQ_STREAM(bf16_t, 8));
+#undef TLQ_STREAM3
 #undef TLQ_STREAM
   if (rc) return rc;
   if (p.split > 1) launch_splitk_reduce(partial, C, M, N, p.split, out_dtype, st);

@@ -4,6 +4,7 @@
 // (int8) per step, so a wavefront reads 256 contiguous bytes and writes 1024 (512)
 // contiguous bytes per instruction.  Shapes that do not fit (K % 8 != 0, group % 8 != 0)
 // take a one-element-per-lane kernel.
+#include "expand8.h"
 #include "tlq_common.h"
 
 namespace tlq {
@@ -49,27 +50,31 @@ __global__ __launch_bounds__(256) void unpack_int4_scalar(const uint8_t* __restr
 }
 
 // ---- per-group dequantisation -----------------------------------------------------------
-template <typename T>
+// One lane dequantises a 32-bit word (8 weights) with the expander the GEMM kernels use (bit-identical to the
+// element-wise Dequant<T>::apply, a third of its instructions); a zero point that is a small integer folds into
+// the unpack bias.  LAYOUT as in expand8.h (0 plain, 1 words permuted by interleave_weight for the fp16 target).
+template <typename T, int LAYOUT>
 __global__ __launch_bounds__(256) void dequant_w4_vec8(const uint32_t* __restrict__ wp, const T* __restrict__ scales,
                                                        const T* __restrict__ zeros, T* __restrict__ out,
                                                        int64_t n_words, int words_per_row, int group, int groups_per_row,
                                                        float zero_scalar) {
-  struct alignas(16) Vec {
-    T v[8];
-  };
   const T one = from_float<T>(1.0f);
   const T zs = from_float<T>(zero_scalar);
+  const NibbleMagic mg = make_nibble_magic();
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += (int64_t)gridDim.x * blockDim.x) {
     int64_t row = i / words_per_row;
     int k = (int)(i - row * words_per_row) * 8;
     int64_t gi = row * groups_per_row + k / group;
     T s = scales ? scales[gi] : one;
     T z = zeros ? zeros[gi] : zs;
-    uint32_t x = wp[i];
-    Vec r;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) r.v[j] = Dequant<T>::apply((x >> (4 * j)) & 0xF, s, z);
-    ((Vec*)out)[i] = r;
+    const uint32_t x = wp[i];
+    const float zf = to_float(z);
+    uint4_t r;
+    if (zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f)
+      r = Expand8<T, true, LAYOUT>(s, z, mg)(x);
+    else
+      r = Expand8<T, false, LAYOUT>(s, z, mg)(x);
+    ((uint4_t*)out)[i] = r;
   }
 }
 
@@ -113,15 +118,22 @@ static int launch_unpack(const void* wp, void* out, int64_t N, int64_t K, int si
 
 template <typename T>
 static int launch_dequant(const void* wp, const void* scales, const void* zeros, void* out, int64_t N, int64_t K,
-                          int64_t group, float zero_scalar, hipStream_t st) {
+                          int64_t group, float zero_scalar, int w_layout, hipStream_t st) {
   if (N * K == 0) return 0;
   const bool aligned = ((uintptr_t)wp % 4 == 0) && ((uintptr_t)out % 16 == 0);
   if (K % 8 == 0 && group % 8 == 0 && aligned) {
     int64_t n_words = N * K / 8;
-    dequant_w4_vec8<T><<<grid_for(n_words), 256, 0, st>>>((const uint32_t*)wp, (const T*)scales, (const T*)zeros,
-                                                         (T*)out, n_words, (int)(K / 8), (int)group, (int)(K / group),
-                                                         zero_scalar);
+    if (w_layout == TLQ_W_INTERLEAVED_F16)
+      dequant_w4_vec8<T, 1><<<grid_for(n_words), 256, 0, st>>>((const uint32_t*)wp, (const T*)scales, (const T*)zeros, (T*)out, n_words,
+                                                              (int)(K / 8), (int)group, (int)(K / group), zero_scalar);
+    else
+      dequant_w4_vec8<T, 0><<<grid_for(n_words), 256, 0, st>>>((const uint32_t*)wp, (const T*)scales, (const T*)zeros, (T*)out, n_words,
+                                                              (int)(K / 8), (int)group, (int)(K / group), zero_scalar);
   } else {
+    if (w_layout != TLQ_W_PLAIN) {
+      set_error("tlq_dequant_w4_layout: interleaved weights need K %% 8 == 0, group %% 8 == 0, 4-byte aligned words and a 16-byte aligned output");
+      return 1;
+    }
     dequant_w4_scalar<T><<<grid_for(N * K), 256, 0, st>>>((const uint8_t*)wp, (const T*)scales, (const T*)zeros, (T*)out,
                                                          N, K, (int)group, zero_scalar);
   }
@@ -153,21 +165,27 @@ int tlq_unpack_int4(const void* w_packed, void* out, int64_t N, int64_t K, int o
   }
 }
 
-int tlq_dequant_w4(const void* w_packed, const void* scales, const void* zeros, void* out, int64_t N, int64_t K,
-                   int64_t group, float zero_scalar, int dtype, void* stream) {
+int tlq_dequant_w4_layout(const void* w_packed, const void* scales, const void* zeros, void* out, int64_t N, int64_t K,
+                          int64_t group, float zero_scalar, int dtype, int w_layout, void* stream) {
   using namespace tlq;
   TLQ_REQUIRE(N >= 0 && K >= 0, "tlq_dequant_w4: negative shape");
   TLQ_REQUIRE(K % 2 == 0, "tlq_dequant_w4: K=%lld must be even", (long long)K);
+  TLQ_REQUIRE(w_layout == TLQ_W_PLAIN || w_layout == TLQ_W_INTERLEAVED_F16, "tlq_dequant_w4: bad weight layout %d", w_layout);
   if (N * K == 0) return 0;
   TLQ_REQUIRE(group > 0 && K % group == 0, "tlq_dequant_w4: group=%lld must divide K=%lld", (long long)group,
               (long long)K);
   TLQ_REQUIRE(w_packed && out, "tlq_dequant_w4: null pointer");
   TLQ_REQUIRE(N * K < (int64_t)1 << 40, "tlq_dequant_w4: shape too large");
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TLQ_F16) return launch_dequant<half_t>(w_packed, scales, zeros, out, N, K, group, zero_scalar, st);
-  if (dtype == TLQ_BF16) return launch_dequant<bf16_t>(w_packed, scales, zeros, out, N, K, group, zero_scalar, st);
+  if (dtype == TLQ_F16) return launch_dequant<half_t>(w_packed, scales, zeros, out, N, K, group, zero_scalar, w_layout, st);
+  if (dtype == TLQ_BF16) return launch_dequant<bf16_t>(w_packed, scales, zeros, out, N, K, group, zero_scalar, w_layout, st);
   set_error("tlq_dequant_w4: unsupported dtype %d", dtype);
   return 1;
+}
+
+int tlq_dequant_w4(const void* w_packed, const void* scales, const void* zeros, void* out, int64_t N, int64_t K,
+                   int64_t group, float zero_scalar, int dtype, void* stream) {
+  return tlq_dequant_w4_layout(w_packed, scales, zeros, out, N, K, group, zero_scalar, dtype, TLQ_W_PLAIN, stream);
 }
 
 }  // extern "C"

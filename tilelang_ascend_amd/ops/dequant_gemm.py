@@ -27,7 +27,9 @@ _PASS_CONFIGS = {
 }
 _SIGN_MODES = {"unsigned": _abi.U4, "twos": _abi.S4_TWOS, "offset8": _abi.S4_OFFSET8, "offset7": _abi.S4_OFFSET7}
 _ALGOS = {"auto": _abi.ALGO_AUTO, "gemv": _abi.ALGO_GEMV, "mfma": _abi.ALGO_MFMA, "skinny": _abi.ALGO_SKINNY,
-          "two_pass": _abi.ALGO_TWO_PASS}
+          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM}
+# arrangement of the 4-bit fields in each 32-bit word: general_compress order, or interleave_weight(target float16)
+_LAYOUTS = {"plain": _abi.W_PLAIN, "interleaved": _abi.W_INTERLEAVED_F16}
 
 
 def _stream() -> int:
@@ -78,9 +80,10 @@ def torch_unpack_uint4_to_int8(tensor: torch.Tensor) -> torch.Tensor:
 
 def dequantize_w4(B_packed: torch.Tensor, scales: Optional[torch.Tensor] = None,
                   zeros: Union[None, float, int, torch.Tensor] = None, group_size: int = 128,
-                  dtype: torch.dtype = torch.float16) -> torch.Tensor:
+                  dtype: torch.dtype = torch.float16, weight_layout: str = "plain") -> torch.Tensor:
     """W[n, k] = rn( rn(T(u[n,k]) - z[n, k//g]) * s[n, k//g] ), T = dtype, as a [N, K] tensor.
-    scales: [N, K/g] of dtype or None (=1).  zeros: None (=0), a number, or [N, K/g] of dtype."""
+    scales: [N, K/g] of dtype or None (=1).  zeros: None (=0), a number, or [N, K/g] of dtype.
+    weight_layout: "plain", or "interleaved" for words repacked by interleave_weight(target float16)."""
     _require_cuda(B_packed, "B_packed")
     N, Kp = B_packed.shape
     K = Kp * 2
@@ -89,8 +92,9 @@ def dequantize_w4(B_packed: torch.Tensor, scales: Optional[torch.Tensor] = None,
     _check_group_tensor(z_t, "zeros", N, K, group_size, dtype)
     out = torch.empty(N, K, dtype=dtype, device=B_packed.device)
     with torch.cuda.device(B_packed.device):
-        _abi.check(_abi.load().tlq_dequant_w4(_abi.ptr(B_packed), _abi.ptr(scales), _abi.ptr(z_t), _abi.ptr(out), N, K,
-                                              group_size, float(z_s), ABI_DTYPE[dtype], _stream()))
+        _abi.check(_abi.load().tlq_dequant_w4_layout(_abi.ptr(B_packed), _abi.ptr(scales), _abi.ptr(z_t), _abi.ptr(out), N, K,
+                                                     group_size, float(z_s), ABI_DTYPE[dtype], _LAYOUTS[weight_layout],
+                                                     _stream()))
     return out
 
 
@@ -152,15 +156,20 @@ def int8_gemm(M: int, N: int, K: int, block_M: int, block_N: int, block_K: int):
 def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, block_K: int = 64,
                in_dtype: str = "float16", out_dtype: str = "float16", group_size: int = 128,
                with_scales: bool = True, zeros: Union[None, float, int, str] = None, algo: str = "auto",
-               tile: int = 0, gemv_tuning: tuple = None, skinny_tuning: tuple = None):
+               tile: int = 0, gemv_tuning: tuple = None, skinny_tuning: tuple = None, weight_layout: str = "plain"):
     """Device-resident fused kernel: kernel(A, B_packed[, scales][, zeros]) -> C.
 
     A [M,K] in_dtype; B_packed uint8 [N,K/2]; scales [N,K/group_size] in_dtype when with_scales;
     zeros: None (no zero point), a number (one zero point for the whole matrix) or "tensor"
     (a [N,K/group_size] in_dtype input follows).  C [M,N] out_dtype, fp32 accumulate.
     algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "skinny" (M <= 64) | "mfma" (LDS-staged MFMA kernel)
-    | "two_pass" (dequantise into a workspace, then the plain GEMM: what "auto" does from M = 256 up; the kernel
-    object then keeps a [N, K] workspace in the activation type on the device of its first call).
+    | "stream" (wavefront-private packed weights dequantised in registers, 17 <= M <= 512: what "auto" does up to
+    M = 256) | "two_pass" (dequantise into a workspace, then the plain GEMM: what "auto" does above).  A workspace
+    (split-K partial sums or the [N, K] dequantised weights) is taken from torch's stream-ordered allocator on every
+    call, as the reference allocates its workspace_idx buffers per call, so launches on different streams do not share one.
+    weight_layout: "plain" (general_compress order) or "interleaved" (B_packed went through interleave_weight for the
+    float16 target, e.g. quantize.gpu.pack_int4(..., interleave="float16")); interleaved weights are read by the "stream"
+    kernel and the two passes only (M >= 17), with results bit-identical to the plain layout.
     tile: rows of activations per work-group of the MFMA kernel (16, 32, 64, 128, 256; 0 = chosen by the
     library); gemv_tuning = (rows_per_wave, waves, blocks_per_cu, depth) and skinny_tuning = (waves,
     row_tiles) select among the pre-built variants of those kernels.  These are the tunable parameters an
@@ -185,7 +194,7 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
     params.append(Param("C", (M, N), out_dtype))
     tin, tout = ABI_DTYPE[TORCH_DTYPES[in_dtype]], ABI_DTYPE[TORCH_DTYPES[out_dtype]]
     algo_code = _ALGOS[algo]
-    workspace = {}  # device -> uint8 tensor, created on the first launch that needs it
+    layout_code = _LAYOUTS[weight_layout]
 
     def launch(t, sym, stream):
         A, Bp = t[0], t[1]
@@ -201,26 +210,26 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
         lib = _abi.load()
         ws = None
         ws_bytes = 0
-        if algo in ("auto", "two_pass"):
+        if algo in ("auto", "two_pass", "stream"):
             ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
-            if algo == "two_pass":
+            if algo == "two_pass" or (layout_code != _abi.W_PLAIN and algo == "auto" and M > 256):
                 ws_bytes = max(ws_bytes, N * K * 2)
         if ws_bytes:
-            ws = workspace.get(A.device)
-            if ws is None:
-                ws = workspace[A.device] = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
         with _abi.tuning(w4a16_tile=tile, gemv=gemv_tuning, skinny=skinny_tuning):
-            _abi.check(lib.tlq_gemm_w4a16_ws(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(S), _abi.ptr(Z), _abi.ptr(C), M, N, K,
-                                             group_size, zero_scalar, tin, tout, algo_code, _abi.ptr(ws), ws_bytes, stream))
+            _abi.check(lib.tlq_gemm_w4a16_layout_ws(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(S), _abi.ptr(Z), _abi.ptr(C), M, N, K,
+                                                    group_size, zero_scalar, tin, tout, algo_code, layout_code, _abi.ptr(ws),
+                                                    ws_bytes, stream))
 
     return KernelSpec("w4a16_gemm", params, launch,
                       {"block": (block_M, block_N, block_K), "group": group_size, "zeros": zeros, "algo": algo,
-                       "tile": tile, "gemv_tuning": gemv_tuning, "skinny_tuning": skinny_tuning})
+                       "tile": tile, "gemv_tuning": gemv_tuning, "skinny_tuning": skinny_tuning,
+                       "weight_layout": weight_layout})
 
 
 def dequant_gemm_fp16_wrapper(M: int, N: int, K: int, block_M: int, block_N: int, block_K: int,
                               input_dtype: str = "float16", output_dtype: str = "float16",
-                              group_size: int = 128, algo: str = "auto"):
+                              group_size: int = 128, algo: str = "auto", weight_layout: str = "plain"):
     """fine_grained.py:176-223: returns wrapper(A, B_packed) -> C = A @ unpack(B_packed).T.
 
     As in the reference the wrapper takes CPU tensors and returns a CPU tensor (it moves data to
@@ -240,7 +249,7 @@ def dequant_gemm_fp16_wrapper(M: int, N: int, K: int, block_M: int, block_N: int
         key = (scales is not None, "tensor" if z_is_tensor else zeros)
         if key not in kernels:
             kernels[key] = w4a16_gemm(M, N, K, block_M, block_N, block_K, input_dtype, output_dtype, group_size,
-                                      scales is not None, key[1], algo)
+                                      scales is not None, key[1], algo, weight_layout=weight_layout)
         args = [A, B_packed] + ([scales] if scales is not None else []) + ([zeros] if z_is_tensor else [])
         if on_cpu:
             args = [a.cuda() for a in args]
