@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|prefill|w8a8|skinny|actquant|mlp-sweep] [--units U]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|small|prefill|w8a8|skinny|actquant|mlp-sweep] [--units U]
 
 Headline workload (default): the W4A16 decode GEMV -- M=1, N=11008, K=4096, fp16 activations,
 uint4 weights packed low-nibble-first, group 128, fp16 scales U[0.005,0.02] and fp16 zeros U{6..9},
@@ -10,16 +10,25 @@ independent weight sets (default 1).  The weight sets rotate through a pool larg
 256 MB last-level cache, so every step streams its weights from HBM.  Inputs are resident in
 HBM before the timed region starts.
 
-Prints ONE JSON line.  `value` is algorithmic bytes / wall time (GB/s); `roofline` describes the
-dominant kernel from HIP events recorded on the launch stream around the timed region;
-`cpu_baseline` is the CPU oracle (the reference's torch ref_program arithmetic) timed on the
-host cores on a bounded sample; `other_workloads` carries the prefill GEMM and W8A8 figures.
+Prints ONE JSON line.
+  * `value` is algorithmic bytes / WALL-CLOCK time per step of the K timed steps: it includes the host side of every
+    launch (the ctypes call into the C ABI, about 2 us, which a microsecond kernel does not hide).
+  * `roofline.achieved` is algorithmic bytes (or operations) / the average step time between two HIP events recorded on the
+    launch stream around the same K steps.  After the timed region the same step runs again with one event pair per
+    step; `roofline.median_us` and `roofline.min_us` come from those pairs (each pair adds the event markers' own cost,
+    about a microsecond, so they bound the kernel from above and are not comparable with the back-to-back average).
+  * `roofline.traffic` is read from the counter summary under profiles/ for that kernel and workload (a line
+    "traffic_bytes_per_launch: N"), null when the file does not carry one.
+  * `cpu_baseline` is the CPU oracle (the reference's torch ref_program arithmetic) timed on the host cores on a bounded
+    sample; every entry of `other_workloads` (the other configurations) carries its own.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -31,14 +40,19 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_I8_PEAK_TOPS = 5000.0
 POOL_BYTES = 576 * 1024 * 1024  # weight pool > 2x the 256 MB last-level cache
-# HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in separate
-# runs of this script with --calibrate-copy, each scaled by what the counter reads for the 256 MiB
-# copy kernel: x2.000 and x1.000); the summaries are the text files under profiles/.
-TRAFFIC_GEMV_1SET = 24_110_000
-TRAFFIC_PREFILL = 162_900_000
-TRAFFIC_W8A8 = 935_200_000
-TRAFFIC_SKINNY = 33_130_000
-TRAFFIC_ACT_QUANT = 201_554_000
+METRIC = "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)"
+WALL_NOTE = "value = algorithmic bytes / wall-clock per step incl. the host-side launch call; roofline.* from HIP events"
+
+
+def traffic_from_profile(name):
+    """HBM bytes per launch as measured with hardware counters: the line 'traffic_bytes_per_launch: N' of
+    profiles/<name> (FETCH_SIZE + WRITE_SIZE, each scaled by a copy kernel of known size); None without one."""
+    try:
+        with open(os.path.join(ROOT, "profiles", name)) as f:
+            m = re.search(r"^traffic_bytes_per_launch\s*:\s*(\d+)", f.read(), re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def w4a16_bytes(M, N, K, group, zeros_tensor=True, elem=2):
@@ -50,8 +64,30 @@ def w8a8_bytes(B, M, N, K):
     return B * M * K + B * K * N + 2 * B * M * N + 4 * B * M + 4 * N
 
 
-def timed(fn, steps, warmup):
-    """Returns (wall seconds per step, event-measured seconds per step)."""
+class Timing:
+    """wall / ev: seconds per step of the timed region (host clock / HIP events around the whole loop);
+    median / best: seconds per step from one event pair per step, taken after the timed region."""
+
+    def __init__(self, wall, ev, per_step):
+        self.wall, self.ev = wall, ev
+        self.median = statistics.median(per_step) if per_step else None
+        self.best = min(per_step) if per_step else None
+        self.pairs = len(per_step)
+
+    def roofline(self, work, peak, unit, scale):
+        """work per step (bytes or operations), peak in `unit`, scale = 1e9 for GB/s, 1e12 for T.../s."""
+        ach = work / self.ev / scale
+        out = {"achieved": round(ach, 1), "peak": peak, "unit": unit, "frac": round(ach / peak, 4),
+               "avg_launch_us": round(self.ev * 1e6, 3)}
+        if self.pairs:
+            out.update({"median_us": round(self.median * 1e6, 3), "min_us": round(self.best * 1e6, 3),
+                        "per_step_event_pairs": self.pairs})
+        return out
+
+
+def timed(fn, steps, warmup, pairs=None):
+    """warmup untimed steps, then exactly `steps` timed ones between two synchronisations; then `pairs` more
+    (default min(steps, 200)) with one event pair each."""
     import torch
 
     for i in range(warmup):
@@ -65,7 +101,27 @@ def timed(fn, steps, warmup):
     e1.record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
+    n = min(steps, 200) if pairs is None else pairs
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for i, (a, b) in enumerate(evs):
+        a.record()
+        fn(steps + i)
+        b.record()
+    torch.cuda.synchronize()
+    per_step = [a.elapsed_time(b) * 1e-3 for a, b in evs]
+    return Timing((t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps, per_step)
+
+
+def cpu_time(fn, budget_s, max_reps=200):
+    """Seconds per evaluation of fn on the host: one warm-up, then repeats until budget_s has passed."""
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or reps >= max_reps:
+            return dt / reps, reps, dt
 
 
 def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
@@ -106,7 +162,8 @@ def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
         if entry(*pre[i % groups]):
             raise RuntimeError(_abi.last_error())
 
-    wall, ev = timed(step, steps, warmup)
+    tm = timed(step, steps, warmup)
+    wall = tm.wall
     step_bytes = unit_bytes * units
     # spot check of the last result against the oracle (outside the timed region)
     from oracle import ref
@@ -119,17 +176,17 @@ def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
 
     cpu = cpu_baseline_gemv(A[0].cpu(), Wp[0].cpu(), S[0].cpu(), Z[0].cpu(), g, unit_bytes) if cpu else None
     return {
-        "metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
+        "metric": METRIC,
         "value": round(step_bytes / wall / 1e9, 1),
         "unit": "GB/s",
         "ms_per_step": wall * 1e3,
         "dtype": "f16",
         "config": {"workload": f"W4A16 decode GEMV M=1 N=11008 K=4096 group=128 fp16 scales+zeros, {units} weight set(s) per launch, "
-                               f"{sets} sets rotating ({sets * unit_bytes >> 20} MiB)",
+                               f"{sets} sets rotating ({sets * unit_bytes >> 20} MiB); " + WALL_NOTE,
                    "M": M, "N": N, "K": K, "group": g, "units_per_launch": units},
-        "roofline": {"kernel": "gemv_w4a16_f16_rows_kernel", "bound": "hbm", "achieved": round(step_bytes / ev / 1e9, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(step_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": TRAFFIC_GEMV_1SET * units, "bytes_per_launch": step_bytes, "avg_launch_us": round(ev * 1e6, 3)},
+        "roofline": dict({"kernel": "gemv_w4a16_f16_rows_kernel", "bound": "hbm"}, **tm.roofline(step_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
+                         traffic=(traffic_from_profile("gemv_w4a16_f16_M1_N11008_K4096_g128.txt") if units == 1 else None),
+                         bytes_per_launch=step_bytes),
         "cpu_baseline": cpu,
         "parity_rel_l2": rel,
     }
@@ -142,21 +199,64 @@ def cpu_baseline_gemv(A, Wp, S, Z, g, unit_bytes, budget_s=10.0):
 
     from oracle import ref
 
-    ref.ref_program_w4a16(A, Wp, S, Z, g, "float16")  # warm-up
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        ref.ref_program_w4a16(A, Wp, S, Z, g, "float16")
-        reps += 1
-        dt = time.perf_counter() - t0
-        if dt >= budget_s and reps >= 3 or reps >= 200:
-            break
-    per = dt / reps
+    per, reps, dt = cpu_time(lambda: ref.ref_program_w4a16(A, Wp, S, Z, g, "float16"), budget_s)
     return {"value": round(unit_bytes / per / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"{reps} evaluations of the same M=1 N=11008 K=4096 GEMV (unpack + dequant + fp32 matmul) in {dt:.1f} s",
             "ms_per_eval": round(per * 1e3, 2), "host_cpus": os.cpu_count()}
 
 
-def bench_prefill(args, steps=None):
+def bench_small(args, steps=None, cpu=True):
+    """The reference's own CPU-runnable case: W4A16 dequant-GEMM M=N=K=256, fp16, group 128, zero point 8."""
+    import torch
+
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dev = torch.device("cuda:0")
+    M = N = K = 256
+    g = 128
+    gen = torch.Generator(device="cpu").manual_seed(6)
+    Wp_c = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=gen)
+    S_c = (torch.rand(N, K // g, generator=gen) * 0.015 + 0.005).to(torch.float16)
+    A_c = torch.randn(M, K, generator=gen).to(torch.float16)
+    Wp, S, A = Wp_c.to(dev), S_c.to(dev), A_c.to(dev)
+    C = torch.empty(M, N, dtype=torch.float16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    pre = (P(A), P(Wp), P(S), None, P(C), M, N, K, g, 8.0, _abi.F16, _abi.F16, _abi.ALGO_AUTO, P(ws), ws_bytes, stream)
+
+    def step(i):
+        if lib.tlq_gemm_w4a16_ws(*pre):
+            raise RuntimeError(_abi.last_error())
+
+    tm = timed(step, steps or args.steps, args.warmup)
+    flops, nbytes = 2.0 * M * N * K, w4a16_bytes(M, N, K, g, zeros_tensor=False)
+    out = {"workload": "W4A16 dequant-GEMM M=N=K=256 fp16 group=128 zero=8 (launch bound: 0.03 GFLOP, 0.3 MB)", "dtype": "f16",
+           "value": round(flops / tm.wall / 1e12, 3), "unit": "TFLOP/s", "ms_per_step": tm.wall * 1e3,
+           "roofline": dict({"kernel": "automatic choice of tlq_gemm_w4a16_ws", "bound": "hbm"},
+                            **tm.roofline(nbytes, HBM_PEAK_GBS, "GB/s", 1e9), traffic=None, bytes_per_launch=nbytes)}
+    if cpu:
+        from oracle import ref
+
+        def literal():  # the reference's own per-element unpack loop, then (u - 8) * s in fp16 and the fp32 matmul
+            U = ref.unpack_uint4_loop(Wp_c, torch.float16)
+            W = (U - 8) * S_c.repeat_interleave(g, dim=1)
+            return (A_c.float() @ W.float().T).to(torch.float16)
+
+        want = ref.ref_program_w4a16(A_c, Wp_c, S_c, 8, g, "float32")
+        rel = ((C.float().cpu() - want).norm() / want.norm()).item()
+        if rel > 1e-3:
+            raise RuntimeError(f"M=N=K=256 result differs from the oracle: relative L2 {rel}")
+        per, reps, dt = cpu_time(literal, 3.0, 20)
+        out["cpu_baseline"] = {"value": round(flops / per / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                               "sample": f"{reps} evaluations with the literal per-element unpack loop "
+                                         f"(example_dequant_gemm_fine_grained.py:10-32) in {dt:.1f} s",
+                               "ms_per_eval": round(per * 1e3, 2)}
+    return out
+
+
+def bench_prefill(args, steps=None, cpu=True):
     import torch
 
     from tilelang_ascend_amd import _abi
@@ -166,16 +266,17 @@ def bench_prefill(args, steps=None):
     M = N = K = 4096
     g = 128
     gen = torch.Generator(device="cpu").manual_seed(1)
-    Wp = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=gen).to(dev)
-    S = (torch.rand(N, K // g, generator=gen) * 0.015 + 0.005).to(torch.bfloat16).to(dev)
-    A = torch.randn(M, K, generator=gen).to(torch.bfloat16).to(dev)
+    Wp_c = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=gen)
+    S_c = (torch.rand(N, K // g, generator=gen) * 0.015 + 0.005).to(torch.bfloat16)
+    A_c = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    Wp, S, A = Wp_c.to(dev), S_c.to(dev), A_c.to(dev)
     C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
 
     ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
 
-    def step(i):  # dequantise into the workspace, then the plain MFMA GEMM (two launches)
+    def step(i):  # what the library chooses with a workspace: dequantise into it, then the plain MFMA GEMM (two launches)
         rc = lib.tlq_gemm_w4a16_ws(P(A), P(Wp), P(S), None, P(C), M, N, K, g, 8.0, _abi.BF16, _abi.BF16, _abi.ALGO_AUTO,
                                    P(ws), ws_bytes, stream)
         if rc:
@@ -186,24 +287,30 @@ def bench_prefill(args, steps=None):
         if rc:
             raise RuntimeError(_abi.last_error())
 
-    wall, ev = timed(step_fused, steps or args.steps, args.warmup)
-    wall2, ev2 = timed(step, steps or args.steps, min(args.warmup, 4))
+    tm = timed(step, steps or args.steps, args.warmup)
+    fused = timed(step_fused, steps or args.steps, min(args.warmup, 4), pairs=0)
     flops = 2.0 * M * N * K
-    # primary figure: the fused kernel (dequantised weight tiles staged through LDS into MFMA); alongside, the two
-    # launches that a caller-owned workspace allows (whole step priced against the MFMA peak)
-    return {"workload": "W4A16 prefill GEMM M=N=K=4096 bf16 group=128 zero=8", "dtype": "bf16",
-            "value": round(flops / wall / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": wall * 1e3,
-            "roofline": {"kernel": "gemm_mfma_kernel<MmaBF16,RowLoaderDirect,W4Loader>", "bound": "mfma", "achieved": round(flops / ev / 1e12, 1),
-                         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                         "traffic": TRAFFIC_PREFILL, "flops_per_launch": flops, "avg_launch_us": round(ev * 1e6, 2)},
-            "with_workspace": {"path": "tlq_gemm_w4a16_ws: dequant_w4_vec8 into a caller-owned workspace, then "
-                                       "gemm_mfma_kernel<MmaBF16,RowLoaderDirect,RowLoaderDirect>",
-                               "value": round(flops / wall2 / 1e12, 1), "unit": "TFLOP/s", "us_per_step": round(ev2 * 1e6, 2),
-                               "frac_of_mfma_peak": round(flops / ev2 / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}}
+    out = {"workload": "W4A16 prefill GEMM M=N=K=4096 bf16 group=128 zero=8, automatic choice with a caller-owned workspace "
+                       "(dequantisation pass + plain MFMA GEMM; the whole step is priced against the MFMA peak)", "dtype": "bf16",
+           "value": round(flops / tm.wall / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": tm.wall * 1e3,
+           "roofline": dict({"kernel": "dequant_w4_vec8<bf16> + gemm_slots_kernel<MmaBF16,RowLoaderDirect,EpiFloat>", "bound": "mfma"},
+                            **tm.roofline(flops, MFMA_F16_PEAK_TFLOPS, "TFLOP/s", 1e12),
+                            traffic=traffic_from_profile("gemm_w4a16_bf16_M4096_N4096_K4096_g128.txt"), flops_per_launch=flops),
+           "fused_kernel": {"path": "tlq_gemm_w4a16(algo=mfma): gemm_mfma_kernel<MmaBF16,RowLoaderDirect,W4Loader>, one launch, no workspace",
+                            "value": round(flops / fused.wall / 1e12, 1), "unit": "TFLOP/s", "us_per_step": round(fused.ev * 1e6, 2),
+                            "frac_of_mfma_peak": round(flops / fused.ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}}
+    if cpu:
+        from oracle import ref
+
+        per, reps, dt = cpu_time(lambda: ref.ref_program_w4a16(A_c, Wp_c, S_c, 8, g, "bfloat16"), 5.0, 20)
+        out["cpu_baseline"] = {"value": round(flops / per / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{reps} evaluations of the same 4096^3 problem (unpack + dequant in bf16 + fp32 matmul) in {dt:.1f} s",
+                               "ms_per_eval": round(per * 1e3, 1)}
+    return out
 
 
-def bench_skinny(args, steps=None):
-    """cfg-5 decode batch: M=16 activations against a 14336 x 4096 weight matrix (HBM bound)."""
+def bench_skinny(args, steps=None, cpu=True):
+    """Decode batch of the MLP-shaped sweep: M=16 activations against a 14336 x 4096 weight matrix (HBM bound)."""
     import torch
 
     from tilelang_ascend_amd import _abi
@@ -227,12 +334,20 @@ def bench_skinny(args, steps=None):
         if lib.tlq_gemm_w4a16(*pre[i % sets]):
             raise RuntimeError(_abi.last_error())
 
-    wall, ev = timed(step, steps or args.steps, args.warmup)
-    return {"workload": f"W4A16 decode batch M=16 N=14336 K=4096 group=128 fp16 scales+zeros, {sets} weight sets rotating",
-            "dtype": "f16", "value": round(unit_bytes / wall / 1e9, 1), "unit": "GB/s", "ms_per_step": wall * 1e3,
-            "roofline": {"kernel": "w4a16_skinny_lds_kernel", "bound": "hbm", "achieved": round(unit_bytes / ev / 1e9, 1),
-                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(unit_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
-                         "traffic": TRAFFIC_SKINNY, "bytes_per_launch": unit_bytes, "avg_launch_us": round(ev * 1e6, 3)}}
+    tm = timed(step, steps or args.steps, args.warmup)
+    out = {"workload": f"W4A16 decode batch M=16 N=14336 K=4096 group=128 fp16 scales+zeros, {sets} weight sets rotating",
+           "dtype": "f16", "value": round(unit_bytes / tm.wall / 1e9, 1), "unit": "GB/s", "ms_per_step": tm.wall * 1e3,
+           "roofline": dict({"kernel": "w4a16_skinny_lds_kernel", "bound": "hbm"}, **tm.roofline(unit_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
+                            traffic=traffic_from_profile("skinny_w4a16_f16_M16_N14336_K4096_g128.txt"), bytes_per_launch=unit_bytes)}
+    if cpu:
+        from oracle import ref
+
+        a, w, sc, z = A.cpu(), Wp[0].cpu(), S[0].cpu(), Z[0].cpu()
+        per, reps, dt = cpu_time(lambda: ref.ref_program_w4a16(a, w, sc, z, g, "float16"), 4.0, 50)
+        out["cpu_baseline"] = {"value": round(unit_bytes / per / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{reps} evaluations of the same M=16 problem (unpack + dequant + fp32 matmul) in {dt:.1f} s",
+                               "ms_per_eval": round(per * 1e3, 1)}
+    return out
 
 
 def bench_act_quant(args, steps=None):
@@ -258,17 +373,17 @@ def bench_act_quant(args, steps=None):
         if lib.tlq_act_quant_i8(*pre[i % sets]):
             raise RuntimeError(_abi.last_error())
 
-    wall, ev = timed(step, steps or args.steps, args.warmup)
+    tm = timed(step, steps or args.steps, args.warmup)
     return {"workload": f"per-token int8 activation quantiser M=16384 N=4096 bf16 in, {sets} inputs rotating",
-            "dtype": "f32", "value": round(unit_bytes / wall / 1e9, 1), "unit": "GB/s", "ms_per_step": wall * 1e3,
-            "roofline": {"kernel": "act_quant_rows_kernel<bf16,8,1>", "bound": "hbm", "achieved": round(unit_bytes / ev / 1e9, 1),
-                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(unit_bytes / ev / 1e9 / HBM_PEAK_GBS, 4),
-                         "traffic": TRAFFIC_ACT_QUANT, "bytes_per_launch": unit_bytes, "avg_launch_us": round(ev * 1e6, 3)}}
+            "dtype": "f32", "value": round(unit_bytes / tm.wall / 1e9, 1), "unit": "GB/s", "ms_per_step": tm.wall * 1e3,
+            "roofline": dict({"kernel": "act_quant_rows_kernel<bf16,8,1>", "bound": "hbm"}, **tm.roofline(unit_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
+                             traffic=traffic_from_profile("act_quant_bf16_M16384_N4096.txt"), bytes_per_launch=unit_bytes)}
 
 
 def bench_mlp_sweep(args, steps=None):
-    """cfg-5 sweep: M in {16, 64, 256, 1024, 8192} x (N, K) in {(14336, 4096), (4096, 14336)} x group in {128, 64},
-    fp16, per-group scales and zeros, automatic kernel choice with a workspace (tlq_gemm_w4a16_ws)."""
+    """MLP-shaped sweep: M in {16, 64, 256, 1024, 8192} x (N, K) in {(14336, 4096), (4096, 14336)} x group in {128, 64},
+    fp16, per-group scales and zeros, automatic kernel choice with a workspace (tlq_gemm_w4a16_ws).  Inputs are drawn
+    on the device (timing only; every shape is checked against the oracle by the GPU tests)."""
     import torch
 
     from tilelang_ascend_amd import _abi
@@ -277,15 +392,15 @@ def bench_mlp_sweep(args, steps=None):
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream().cuda_stream
     rows = []
+    gen = torch.Generator(device=dev).manual_seed(5)
     for (N, K) in ((14336, 4096), (4096, 14336)):
         for g in (128, 64):
             sets = 6  # 6 x 29 MB of packed weights rotate: small-M launches always stream from HBM
-            gen = torch.Generator(device="cpu").manual_seed(5)
-            Wp = torch.randint(0, 256, (sets, N, K // 2), dtype=torch.uint8, generator=gen).to(dev)
-            S = (torch.rand(sets, N, K // g, generator=gen) * 0.015 + 0.005).to(torch.float16).to(dev)
-            Z = torch.randint(6, 10, (sets, N, K // g), generator=gen).to(torch.float16).to(dev)
+            Wp = torch.randint(0, 256, (sets, N, K // 2), dtype=torch.uint8, generator=gen, device=dev)
+            S = (torch.rand(sets, N, K // g, generator=gen, device=dev) * 0.015 + 0.005).to(torch.float16)
+            Z = torch.randint(6, 10, (sets, N, K // g), generator=gen, device=dev).to(torch.float16)
             for M in (16, 64, 256, 1024, 8192):
-                A = torch.randn(M, K, generator=gen).to(torch.float16).to(dev)
+                A = torch.randn(M, K, generator=gen, device=dev).to(torch.float16)
                 C = torch.empty(M, N, dtype=torch.float16, device=dev)
                 ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
                 ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
@@ -296,9 +411,12 @@ def bench_mlp_sweep(args, steps=None):
                     if lib.tlq_gemm_w4a16_ws(*pre[i % sets]):
                         raise RuntimeError(_abi.last_error())
 
-                _, ev = timed(step, steps or (12 if M < 8192 else 4), 3)
+                n = steps or (12 if M < 8192 else 4)
+                tm = timed(step, n, 3, pairs=n)
+                ev = tm.ev
                 flops, nbytes = 2.0 * M * N * K, w4a16_bytes(M, N, K, g)
-                rows.append({"M": M, "N": N, "K": K, "group": g, "us": round(ev * 1e6, 1),
+                rows.append({"M": M, "N": N, "K": K, "group": g, "us": round(ev * 1e6, 1), "median_us": round(tm.median * 1e6, 1),
+                             "min_us": round(tm.best * 1e6, 1),
                              "TFLOP/s": round(flops / ev / 1e12, 1), "frac_mfma": round(flops / ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                              "GB/s": round(nbytes / ev / 1e9), "frac_hbm": round(nbytes / ev / 1e9 / HBM_PEAK_GBS, 4)})
                 del A, C, ws
@@ -312,7 +430,7 @@ def bench_mlp_sweep(args, steps=None):
             "shapes": rows}
 
 
-def bench_w8a8(args, steps=None):
+def bench_w8a8(args, steps=None, cpu=True):
     import torch
 
     from tilelang_ascend_amd import _abi
@@ -333,14 +451,23 @@ def bench_w8a8(args, steps=None):
         if rc:
             raise RuntimeError(_abi.last_error())
 
-    wall, ev = timed(step, steps or args.steps, args.warmup)
+    tm = timed(step, steps or args.steps, args.warmup)
     ops = 2.0 * B * M * N * K
-    return {"workload": "W8A8 quant batch matmul B=8 M=2048 N=K=4096, per-token x per-channel rescale, fp16 out",
-            "dtype": "i8", "value": round(ops / wall / 1e12, 1), "unit": "TOP/s", "ms_per_step": wall * 1e3,
-            "roofline": {"kernel": "gemm_mfma_kernel<MmaI8,RowLoaderDirect,I8KNLoaderDirect,EpiRescale>", "bound": "mfma",
-                         "achieved": round(ops / ev / 1e12, 1), "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
-                         "frac": round(ops / ev / 1e12 / MFMA_I8_PEAK_TOPS, 4), "traffic": TRAFFIC_W8A8, "ops_per_launch": ops,
-                         "avg_launch_us": round(ev * 1e6, 2)}}
+    out = {"workload": "W8A8 quant batch matmul B=8 M=2048 N=K=4096, per-token x per-channel rescale, fp16 out",
+           "dtype": "i8", "value": round(ops / tm.wall / 1e12, 1), "unit": "TOP/s", "ms_per_step": tm.wall * 1e3,
+           "roofline": dict({"kernel": "gemm_slots_kernel<MmaI8,I8KNLoaderDirect,EpiRescale>", "bound": "mfma"},
+                            **tm.roofline(ops, MFMA_I8_PEAK_TOPS, "TOP/s", 1e12),
+                            traffic=traffic_from_profile("gemm_w8a8_B8_M2048_N4096_K4096.txt"), ops_per_launch=ops)}
+    if cpu:
+        from oracle import ref
+
+        a, w, s_a, s_b = A[0].cpu(), W[0].cpu().T.contiguous(), sa[0].cpu(), sb.cpu()
+        per, reps, dt = cpu_time(lambda: ref.ref_int8_gemm_sequential(a, w, s_a, s_b, torch.float16), 4.0, 10)
+        out["cpu_baseline"] = {"value": round(ops / B / per / 1e12, 4), "unit": "TOP/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{reps} evaluations of ONE of the 8 batch elements (exact integer matmul through float64, "
+                                         f"two fp32 rescales) in {dt:.1f} s; the whole batch takes 8 x ms_per_eval",
+                               "ms_per_eval": round(per * 1e3, 1)}
+    return out
 
 
 def main():
@@ -348,13 +475,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=48)
-    ap.add_argument("--workload", default="gemv", choices=["gemv", "prefill", "w8a8", "skinny", "actquant", "mlp-sweep"])
+    ap.add_argument("--workload", default="gemv", choices=["gemv", "small", "prefill", "w8a8", "skinny", "actquant", "mlp-sweep"])
     ap.add_argument("--units", type=int, default=1, help="independent weight sets per GEMV launch")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
     ap.add_argument("--tune", action="append", default=[], metavar="HOOK=VALUE",
-                    help="call a single-integer tuning hook of the library before measuring, e.g. --tune gemm_slots=1 "
-                         "(tlq_tune_gemm_slots(1)); repeatable; recorded in the output line")
+                    help="call a single-integer tuning hook of the library before measuring, e.g. --tune gemm_slots=0 "
+                         "(tlq_tune_gemm_slots(0): the two-stage main loop instead of the five-slot one); repeatable; "
+                         "recorded in the output line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain elementwise copy of 256 MiB (int32 x+0 -> y) after the timed region, "
                          "the known-size kernel that hardware traffic counters are scaled by")
@@ -397,23 +525,28 @@ def main():
                         "ms_per_step": many["ms_per_step"], "roofline": many["roofline"]}
 
             others = []
+            cpu = not args.no_cpu_baseline
             for name, fn in (("gemv, 24 weight sets per launch", many_sets),
-                             ("skinny", lambda: bench_skinny(args, steps=60)),
-                             ("prefill", lambda: bench_prefill(args, steps=20)),
-                             ("w8a8", lambda: bench_w8a8(args, steps=10)),
-                             ("actquant", lambda: bench_act_quant(args, steps=40))):
+                             ("small", lambda: bench_small(args, steps=100, cpu=cpu)),
+                             ("skinny", lambda: bench_skinny(args, steps=60, cpu=cpu)),
+                             ("prefill", lambda: bench_prefill(args, steps=20, cpu=cpu)),
+                             ("w8a8", lambda: bench_w8a8(args, steps=10, cpu=cpu)),
+                             ("actquant", lambda: bench_act_quant(args, steps=40)),
+                             ("mlp-sweep", lambda: bench_mlp_sweep(args))):
                 try:
                     others.append(fn())
                 except Exception as e:  # noqa: BLE001
                     others.append({"workload": name, "error": f"{type(e).__name__}: {e}"})
             line["other_workloads"] = others
     else:
-        res = {"prefill": bench_prefill, "w8a8": bench_w8a8, "skinny": bench_skinny,
+        cpu = not args.no_cpu_baseline
+        res = {"prefill": lambda a: bench_prefill(a, cpu=cpu), "w8a8": lambda a: bench_w8a8(a, cpu=cpu),
+               "skinny": lambda a: bench_skinny(a, cpu=cpu), "small": lambda a: bench_small(a, cpu=cpu),
                "actquant": bench_act_quant, "mlp-sweep": bench_mlp_sweep}[args.workload](args)
-        line = {"metric": "W4A16 GEMV GB/s (%HBM peak) at M=1; W4A16/W8A8 GEMM TFLOP/s (%MFMA peak)",
-                "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
-                "config": {"workload": res["workload"]}, "roofline": res["roofline"], "cpu_baseline": None}
-        for extra in ("shapes", "with_workspace"):
+        line = {"metric": METRIC, "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
+                "config": {"workload": res["workload"] + ("; every figure from HIP events" if args.workload == "mlp-sweep" else "; " + WALL_NOTE)}, "roofline": res["roofline"],
+                "cpu_baseline": res.get("cpu_baseline")}
+        for extra in ("shapes", "fused_kernel"):
             if extra in res:
                 line[extra] = res[extra]
     if args.calibrate_copy:
