@@ -14,9 +14,10 @@ operand fails a test):
   generate_quantized_weight; C restatement.
 * general_compress: inverse of the unpackers; brute force on tiny shapes.
 * interleave_weight (nbits=4): explicit permutation tables e0,e2,e4,e6,e1,e3,e5,e7
-  (fp16) and e0,e4,e1,e5,e2,e6,e3,e7 (int8).  The 1-bit / 2-bit special branches call
-  ``torch.int32(...)`` in the reference, which raises; they are restated by intent and
-  are PARITY UNPINNED.
+  (fp16) and e0,e4,e1,e5,e2,e6,e3,e7 (int8); the general placement formula bit by bit for
+  2-bit sources with the int8 target.  The 1-bit and the 2-bit/float16 special branches call
+  ``torch.int32(...)`` in the reference, which raises TypeError; so does this restatement
+  (the reference's behaviour is the exception, and a test pins it).
 * gen_quant4: invariants only (ref == (q-8).half()*s, shapes, ranges, seed
   reproducibility) -- the random stream itself is torch's.
 * dequant_w4 (per-group scale / zero): float64 evaluation followed by one correctly
@@ -203,25 +204,12 @@ def interleave_weight(qweight: torch.Tensor, nbits=4, target_dtype="float16") ->
             shift = (off % G) * stride + (off // G) * nbits
             new |= ((q >> np.uint32(nbits * off)) & mask) << np.uint32(shift)
 
-    def mv(x, m, down, up):
-        return ((x & np.uint32(m)) >> np.uint32(down)) << np.uint32(up)
-
-    # The three special branches below are restated by intent (utils.py:103-124); the
-    # reference text calls torch.int32(...) there, which is not callable.  PARITY UNPINNED.
-    if nbits == 1 and target_dtype == "int8":
-        r = new & np.uint32(0xF0F00F0F)
-        r |= mv(new, 0x000000F0, 4, 16) | mv(new, 0x0000F000, 12, 24)
-        r |= mv(new, 0x000F0000, 16, 4) | mv(new, 0x0F000000, 24, 12)
-        new = r
-    elif nbits == 2 and target_dtype == "float16":
-        r = new & np.uint32(0xFF0000FF)
-        r |= mv(new, 0x0000FF00, 8, 16) | mv(new, 0x00FF0000, 16, 8)
-        new = r
-    elif nbits == 1 and target_dtype == "float16":
-        r = new & np.uint32(0xF000000F)
-        r |= mv(new, 0x000000F0, 4, 8) | mv(new, 0x00000F00, 8, 16) | mv(new, 0x0000F000, 12, 24)
-        r |= mv(new, 0x000F0000, 16, 4) | mv(new, 0x00F00000, 20, 12) | mv(new, 0x0F000000, 24, 20)
-        new = r
+    # For 1-bit sources and for 2-bit sources with the float16 target the reference goes on to regroup nibbles /
+    # bytes with masks written torch.int32(0x...) (utils.py:103-124); torch.int32 is a dtype object and calling it
+    # raises TypeError, so those three branches never return a value in the reference.  Same behaviour here.
+    if nbits == 1 or (nbits == 2 and target_dtype == "float16"):
+        raise TypeError("'torch.dtype' object is not callable (interleave_weight of %d-bit weights for %s: the reference "
+                        "raises here, tilelang/quantize/utils.py:103-124)" % (nbits, target_dtype))
     return torch.from_numpy(new.view(np.int32).copy()).view(torch.int8)
 
 

@@ -154,3 +154,31 @@ def test_profiler_module_surface():
     assert [q.name for q in p._get_params()] == ["A", "B"]
     assert [q.name for q in p._get_params(with_output=True)] == ["A", "B", "C"]
     assert profiler.TensorSupplyType.Auto.value == 7 and callable(profiler.do_bench)
+
+
+def test_build_lock_is_exclusive_and_stale_libraries_are_detected(tmp_path, monkeypatch):
+    """Two builders never run at once (advisory file lock), and a library whose build record names other sources
+    than those on disk counts as stale; one without a record is taken as it is."""
+    import fcntl
+    import subprocess
+    import sys
+
+    from tilelang_ascend_amd import build
+
+    monkeypatch.setattr(build, "LIB_DIR", str(tmp_path))
+    monkeypatch.setattr(build, "LIB_PATH", str(tmp_path / "libtlq.so"))
+    monkeypatch.setattr(build, "STAMP_PATH", str(tmp_path / "libtlq.fingerprint"))
+    with build.build_lock():
+        probe = ("import fcntl,sys\nf=open(sys.argv[1],'w')\n"
+                 "try:\n fcntl.flock(f, fcntl.LOCK_EX|fcntl.LOCK_NB); print('free')\nexcept BlockingIOError:\n print('held')\n")
+        out = subprocess.run([sys.executable, "-c", probe, str(tmp_path / ".build.lock")], capture_output=True, text=True)
+        assert out.stdout.strip() == "held"
+    with open(tmp_path / ".build.lock", "w") as f:
+        fcntl.flock(f, fcntl.LOCK_EX | fcntl.LOCK_NB)  # released on leaving the context
+    assert build.is_stale() and not build.is_current()  # no library
+    (tmp_path / "libtlq.so").write_bytes(b"")
+    assert not build.is_stale() and not build.is_current()  # no record: cannot be judged
+    (tmp_path / "libtlq.fingerprint").write_text("0" * 64 + "\n")
+    assert build.is_stale()
+    (tmp_path / "libtlq.fingerprint").write_text(build.source_fingerprint() + "\n")
+    assert not build.is_stale() and build.is_current()

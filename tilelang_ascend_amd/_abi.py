@@ -75,8 +75,9 @@ def library_path() -> str:
 
 def load():
     """Load libtlq.so once per process (mutex; the reference guards its library cache the same
-    way, tilelang/jit/adapter/cython/adapter.py:79-98).  Builds it when it is absent and hipcc
-    is available; otherwise raises -- there is no other implementation to fall back to."""
+    way, tilelang/jit/adapter/cython/adapter.py:79-98).  Builds it when it is absent or was built from other
+    sources than those on disk (fingerprint record next to the library) and hipcc is available; otherwise raises --
+    there is no other implementation to fall back to."""
     global _lib
     if _lib is not None:
         return _lib
@@ -84,14 +85,19 @@ def load():
         if _lib is not None:
             return _lib
         path = library_path()
-        if not os.path.exists(path):
+        # a library built from other sources than the ones on disk is never loaded: rebuild it (under the build
+        # lock, so concurrent processes compile once), or say so when that is impossible
+        if path == _build.LIB_PATH and _build.is_stale():
+            state = "not found" if not os.path.exists(path) else "older than the kernel sources"
             try:
-                path = _build.build_library(force=True)
+                path = _build.build_library(force=False)
             except Exception as e:  # noqa: BLE001
                 raise RuntimeError(
-                    f"libtlq.so not found at {path} and could not be built ({e}); "
+                    f"libtlq.so at {path} is {state} and could not be built ({e}); "
                     "run `python -m tilelang_ascend_amd.build`"
                 ) from e
+        elif not os.path.exists(path):
+            raise RuntimeError(f"libtlq.so not found at {path}")
         lib = ctypes.CDLL(path)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)

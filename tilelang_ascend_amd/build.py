@@ -9,6 +9,8 @@ generated ones, so there is one library for all operators.
 """
 from __future__ import annotations
 
+import contextlib
+import fcntl
 import hashlib
 import os
 import shutil
@@ -94,13 +96,58 @@ def _compile_one(src: str, verbose: bool) -> str:
     return obj
 
 
+STAMP_PATH = os.path.join(LIB_DIR, "libtlq.fingerprint")
+
+
+def built_fingerprint():
+    """Fingerprint the library on disk was built from (None when there is no record)."""
+    try:
+        with open(STAMP_PATH) as f:
+            return f.read().strip() or None
+    except OSError:
+        return None
+
+
+def is_current() -> bool:
+    return os.path.exists(LIB_PATH) and built_fingerprint() == source_fingerprint()
+
+
+def is_stale() -> bool:
+    """True when the library is absent, or carries a build record that names other sources than those on disk.
+    A library without a record (copied on its own) cannot be judged and is taken as it is."""
+    if not os.path.exists(LIB_PATH):
+        return True
+    fp = built_fingerprint()
+    return fp is not None and fp != source_fingerprint()
+
+
+@contextlib.contextmanager
+def build_lock():
+    """Exclusive advisory lock on lib/.build.lock: two processes (pytest workers, a test run next to a benchmark)
+    never compile into the same object directory or replace the library under each other.  The reference
+    serialises its kernel cache the same way (tilelang/cache/kernel_cache.py:119-160, a lock around save / load)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    with open(os.path.join(LIB_DIR, ".build.lock"), "w") as f:
+        fcntl.flock(f, fcntl.LOCK_EX)
+        try:
+            yield
+        finally:
+            fcntl.flock(f, fcntl.LOCK_UN)
+
+
 def build_library(force: bool = True, verbose: bool = False, jobs: int = 6) -> str:
     """Compile every kernel source for gfx950 and link libtlq.so.  With force=False an
-    up-to-date library (matching fingerprint) is reused."""
+    up-to-date library (matching fingerprint) is reused.  Holds the build lock throughout; a process that waited
+    for another one's build finds the library current and (force=False) returns at once."""
+    with build_lock():
+        return _build_locked(force, verbose, jobs)
+
+
+def _build_locked(force: bool, verbose: bool, jobs: int) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
-    stamp = os.path.join(LIB_DIR, "libtlq.fingerprint")
+    stamp = STAMP_PATH
     fp = source_fingerprint()
-    if not force and os.path.exists(LIB_PATH) and os.path.exists(stamp) and open(stamp).read().strip() == fp:
+    if not force and is_current():
         return LIB_PATH
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC_DIR, s))]
     missing = sorted(set(SOURCES) - set(srcs))
