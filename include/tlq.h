@@ -177,6 +177,12 @@ int tlq_gemv_w4a16_batched(const void* A, const void* w_packed, const void* scal
 int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
                  int b_layout, void* stream);
 
+/* Batched form, replaces batch_matmul (examples/batch_gemm/batch_gemm.py:28-60): C[b] = A[b] . B[b] for b < batch,
+ * A [batch, M, K], B [batch, K, N] (or [batch, N, K] per b_layout), C [batch, M, N], dense.  One launch covers the
+ * batch (the reference flattens batch x row tiles x column tiles into one grid the same way, :38-43). */
+int tlq_gemm_f16_batched(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype,
+                         int out_dtype, int b_layout, void* stream);
+
 /* Split-K form of the same GEMM, replaces gemm_splitk (examples/gemm_splitk/example_tilelang_gemm_splitk.py:16-48):
  * C (fp32 [M,N], accumulated IN PLACE, the caller zeroes it as the example does) += A[M,K] . B.  K is cut into
  * split_k slices handled by different work-groups that add their partial tiles with atomic adds, so small-M /

@@ -1,4 +1,5 @@
-"""Non-quantised twins: plain GEMV (examples/gemv) and split-K GEMM (examples/gemm_splitk)."""
+"""Non-quantised twins: plain GEMV (examples/gemv), split-K GEMM (examples/gemm_splitk), batched GEMM
+(examples/batch_gemm) and the plain fp16 GEMM of the dequant example with the second operand stored [K, N]."""
 import pytest
 import torch
 
@@ -126,3 +127,65 @@ def test_plain_twin_examples(capsys):
     assert out.rstrip().endswith("Kernel Output Match!")
     exs.main(["--M", "64", "--N", "256", "--K", "2048", "--split-k", "8"])
     assert "Test passed: M=64, N=256, K=2048, split_k=8" in capsys.readouterr().out
+
+
+def _ternary(shape, seed):
+    return torch.randint(-1, 2, shape, generator=torch.Generator().manual_seed(seed)).to(torch.float16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(2300, 4104, 328), (4096, 2048, 72), (130, 264, 200), (2048, 4096, 1024)])
+def test_fp16_gemm_kn_operand_large_tiles_and_k_tails(M, N, K):
+    """B stored [K, N] is transposed on the way into LDS: shapes that take the 256 x 256 instance (ragged M and N, K not a
+    multiple of the 64-element stage) and the 128 x 128 one.  Ternary inputs make every sum an exact small integer, so the
+    comparison with the integer product is bit for bit; random inputs are checked at the float-output bar."""
+    from helpers import check_float_output
+    from tilelang_ascend_amd.ops import fp16_gemm
+
+    kernel = fp16_gemm(M, N, K, 128, 256, 64)
+    A, B = _ternary((M, K), 60), _ternary((K, N), 61)
+    got = kernel(A.cuda(), B.cuda()).cpu()
+    assert torch.equal(got, (A.float() @ B.float()).half())
+    g = torch.Generator().manual_seed(62)
+    A, B = torch.randn(M, K, generator=g).half(), torch.randn(K, N, generator=g).half()
+    check_float_output(kernel(A.cuda(), B.cuda()).cpu(), A.float() @ B.float(), f"fp16_gemm [K,N] {M}x{N}x{K}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("B,M,N,K", [(8, 1024, 1024, 1024), (3, 100, 72, 40), (2, 520, 264, 136), (20, 256, 512, 64), (1, 64, 64, 64)])
+def test_batch_matmul_matches_reference(dtype, B, M, N, K):
+    from helpers import check_float_output
+    from tilelang_ascend_amd.ops import batch_matmul
+
+    kernel = batch_matmul(B, M, N, K, 128, 256, 64, dtype=dtype)
+    a, b = _ternary((B, M, K), 63).to(DT[dtype]), _ternary((B, K, N), 64).to(DT[dtype])
+    got = kernel(a.cuda(), b.cuda()).cpu()
+    assert got.shape == (B, M, N) and got.dtype == DT[dtype]
+    assert torch.equal(got, torch.matmul(a.float(), b.float()).to(DT[dtype]))  # exact small integers, batch by batch
+    g = torch.Generator().manual_seed(65)
+    a, b = torch.randn(B, M, K, generator=g).to(DT[dtype]), torch.randn(B, K, N, generator=g).to(DT[dtype])
+    got = kernel(a.cuda(), b.cuda()).cpu()
+    want = torch.matmul(a.float(), b.float())
+    for i in range(B):
+        check_float_output(got[i], want[i], f"batch_matmul {dtype} batch {i}")
+    torch.testing.assert_close(got, want.to(DT[dtype]), rtol=1e-2, atol=1e-2)  # the example's own criterion (batch_gemm.py:77)
+
+
+@pytest.mark.gpu
+def test_batch_matmul_example_and_bad_arguments(capsys):
+    from tilelang_ascend_amd import _abi
+    from tilelang_ascend_amd.examples.batch_gemm import batch_gemm as ex
+    from tilelang_ascend_amd.ops import batch_matmul
+
+    ex.main(["--b", "4", "--m", "256", "--n", "512", "--k", "128"])
+    assert capsys.readouterr().out.rstrip().splitlines()[-2:] == ["init successful!", "Batch Kernel Output Match!"]
+    with pytest.raises(ValueError):
+        batch_matmul(2, 64, 64, 64, 128, 256, 64, dtype="float32")
+    lib, P = _abi.load(), _abi.ptr
+    t = torch.zeros(4096, device="cuda", dtype=torch.float16)
+    assert lib.tlq_gemm_f16_batched(P(t), P(t), P(t), 2, 3, 8, 8, _abi.F16, _abi.F16, _abi.B_KN, None) == 0  # 3*8 % 8 == 0
+    assert lib.tlq_gemm_f16_batched(P(t), P(t), P(t), 2, 3, 8, 12, _abi.F16, _abi.F16, _abi.B_KN, None) != 0
+    assert lib.tlq_gemm_f16_batched(P(t), P(t), P(t), -1, 8, 8, 8, _abi.F16, _abi.F16, _abi.B_KN, None) != 0
+    assert "batch" in _abi.last_error()
+    assert lib.tlq_gemm_f16_batched(P(t), P(t), P(t), 0, 8, 8, 8, _abi.F16, _abi.F16, _abi.B_KN, None) == 0

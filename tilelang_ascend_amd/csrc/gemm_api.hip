@@ -21,8 +21,8 @@ int gemm_w4a16_stream(const void* A, const void* Wp, const void* scales, const v
                       float* partial, hipStream_t st);
 int gemm_w4a16_skinny(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                       int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
-int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
-                   int b_layout, hipStream_t st);
+int gemm_f16_plain(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype,
+                   int out_dtype, int b_layout, hipStream_t st);
 int gemm_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
                     int in_dtype, int b_layout, hipStream_t st);
 int gemm_i8_i32(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,
@@ -249,21 +249,29 @@ int tlq_gemv_w4a16_batched(const void* A, const void* w_packed, const void* scal
                     (hipStream_t)stream);
 }
 
-int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
-                 int b_layout, void* stream) {
+int tlq_gemm_f16_batched(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype,
+                         int out_dtype, int b_layout, void* stream) {
   TLQ_CHECK_DIMS("tlq_gemm_f16");
+  TLQ_REQUIRE(batch >= 0 && batch < kMaxDim, "tlq_gemm_f16: bad batch %lld", (long long)batch);
   TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_f16: in_dtype must be float16 or bfloat16 (got %d)",
               in_dtype);
   TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_f16: bad out_dtype %d",
               out_dtype);
   TLQ_REQUIRE(b_layout == TLQ_B_KN || b_layout == TLQ_B_NK, "tlq_gemm_f16: bad b_layout %d", b_layout);
-  if (M == 0 || N == 0) return 0;
+  if (batch == 0 || M == 0 || N == 0) return 0;
   TLQ_REQUIRE(K > 0 && K % 8 == 0, "tlq_gemm_f16: K=%lld must be a positive multiple of 8", (long long)K);
   TLQ_REQUIRE(N % 8 == 0, "tlq_gemm_f16: N=%lld must be a multiple of 8", (long long)N);
   TLQ_REQUIRE(A && B && C, "tlq_gemm_f16: null pointer");
   TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_f16: pointers must be 16-byte aligned");
   TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K * 2), "tlq_gemm_f16: a matrix spans 4 GiB or more");
-  return gemm_f16_plain(A, B, C, M, N, K, in_dtype, out_dtype, b_layout, (hipStream_t)stream);
+  TLQ_REQUIRE(batch == 1 || (((M * K) % 8 == 0) && ((M * N) % 8 == 0)),
+              "tlq_gemm_f16: every matrix of a batch must start on a 16-byte boundary (M*K and M*N multiples of 8)");
+  return gemm_f16_plain(A, B, C, batch, M, N, K, in_dtype, out_dtype, b_layout, (hipStream_t)stream);
+}
+
+int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
+                 int b_layout, void* stream) {
+  return tlq_gemm_f16_batched(A, B, C, 1, M, N, K, in_dtype, out_dtype, b_layout, stream);
 }
 
 int tlq_gemm_f16_splitk(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t split_k,

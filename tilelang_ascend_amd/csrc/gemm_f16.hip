@@ -1,5 +1,5 @@
-// Plain fp16 / bf16 GEMM with fp32 accumulation: C[M, N] = A[M, K] . B, B stored [K, N]
-// (transposed on the fly) or [N, K].
+// Plain fp16 / bf16 GEMM with fp32 accumulation: C[b, M, N] = A[b, M, K] . B[b], B[b] stored [K, N]
+// (transposed on the fly) or [N, K]; the matrices of a batch follow each other densely.
 #include "gemm_core.h"
 #include "gemm_slots.h"
 
@@ -86,20 +86,20 @@ struct H16KNLoader {
 };
 
 template <class Mma, int BM, int BN, int WM, int WN>
-static int run_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int out_dtype, int b_layout,
-                   hipStream_t st) {
+static int run_f16(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int out_dtype,
+                   int b_layout, hipStream_t st) {
   constexpr int NT = WM * WN * 64;
   typedef RowLoaderDirect<BM, NT> AL;
-  typename AL::Params pa{(const uint8_t*)A, K * 2, 0, K * 2};
-  EpiFloat::Params pe{C, N, 0, out_dtype};
+  typename AL::Params pa{(const uint8_t*)A, K * 2, M * K * 2, K * 2};
+  EpiFloat::Params pe{C, N, M * N, out_dtype};
   if (b_layout == TLQ_B_NK) {
     typedef RowLoaderDirect<BN, NT> WL;
-    typename WL::Params pw{(const uint8_t*)B, K * 2, 0, K * 2};
-    return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16");
+    typename WL::Params pw{(const uint8_t*)B, K * 2, N * K * 2, K * 2};
+    return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16");
   }
   typedef H16KNLoader<BN, NT> WL;
-  typename WL::Params pw{(const uint8_t*)B, N * 2, 0, K};
-  return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16");
+  typename WL::Params pw{(const uint8_t*)B, N * 2, K * N * 2, K};
+  return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16");
 }
 
 // Split-K: slice z of K is "batch" z of the loaders (the batch strides step along K), and every slice
@@ -133,22 +133,23 @@ int gemm_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N
 }
 
 template <class Mma>
-static int dispatch_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int out_dtype,
+static int dispatch_f16(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int out_dtype,
                         int b_layout, hipStream_t st) {
-  if (M <= 128 || ceil_div(M, 256) * ceil_div(N, 256) < 128)
-    return run_f16<Mma, 128, 128, 2, 2>(A, B, C, M, N, K, out_dtype, b_layout, st);
+  if (M <= 128 || batch * ceil_div(M, 256) * ceil_div(N, 256) < 128)
+    return run_f16<Mma, 128, 128, 2, 2>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);
   if (g_gemm_slots && b_layout == TLQ_B_NK && K % 64 == 0) {  // whole 128-byte stages
-    typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K * 2, 0, K * 2}, pw{(const uint8_t*)B, K * 2, 0, K * 2};
-    EpiFloat::Params pe{C, N, 0, out_dtype};
-    return launch_gemm_slots<Mma, RowLoaderDirect<256, 512>, EpiFloat>(pa, pw, pe, 1, M, N, K * 2, st, "tlq_gemm_f16", 4);
+    typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K * 2, M * K * 2, K * 2},
+        pw{(const uint8_t*)B, K * 2, N * K * 2, K * 2};
+    EpiFloat::Params pe{C, N, M * N, out_dtype};
+    return launch_gemm_slots<Mma, RowLoaderDirect<256, 512>, EpiFloat>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16", 4);
   }
-  return run_f16<Mma, 256, 256, 2, 4>(A, B, C, M, N, K, out_dtype, b_layout, st);
+  return run_f16<Mma, 256, 256, 2, 4>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);
 }
 
-int gemm_f16_plain(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
-                   int b_layout, hipStream_t st) {
-  if (in_dtype == TLQ_F16) return dispatch_f16<MmaF16>(A, B, C, M, N, K, out_dtype, b_layout, st);
-  return dispatch_f16<MmaBF16>(A, B, C, M, N, K, out_dtype, b_layout, st);
+int gemm_f16_plain(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype,
+                   int out_dtype, int b_layout, hipStream_t st) {
+  if (in_dtype == TLQ_F16) return dispatch_f16<MmaF16>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);
+  return dispatch_f16<MmaBF16>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);
 }
 
 }  // namespace tlq

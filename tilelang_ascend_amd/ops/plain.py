@@ -1,4 +1,7 @@
-"""Non-quantised twins of the quantised operators: plain GEMV and split-K GEMM.
+"""Non-quantised twins of the quantised operators: plain GEMV, split-K GEMM and batched GEMM.
+
+``batch_matmul(B, M, N, K, block_M, block_N, K_L1, dtype="float16", accum_dtype="float")`` ->
+``kernel(A [B, M, K], B [B, K, N]) -> C [B, M, N]`` (examples/batch_gemm/batch_gemm.py:28-60, ``out_idx=[-1]``).
 
 ``simple_gemv(N, K, block_N, block_K, dtype="float16", accum_dtype="float32")`` ->
 ``kernel(x [K], A [N, K]) -> y [N]`` (examples/gemv/example_gemv_v.py:17-80 and example_gemv_c.py:16-46,
@@ -47,3 +50,22 @@ def gemm_splitk(M: int, N: int, K: int, block_M: int, block_N: int, block_K: int
 
     return KernelSpec("gemm_splitk", [Param("A", (M, K), dtype), Param("B", (K, N), dtype), Param("C", (M, N), "float32")],
                       launch, {"block": (block_M, block_N, block_K), "split_k": split_k})
+
+
+@jit(out_idx=[-1], pass_configs={PassConfigKey.TL_ASCEND_AUTO_CV_COMBINE: True, PassConfigKey.TL_ASCEND_AUTO_SYNC: True,
+                                 PassConfigKey.TL_ASCEND_MEMORY_PLANNING: True})
+def batch_matmul(B: int, M: int, N: int, K: int, block_M: int, block_N: int, K_L1: int, dtype: str = "float16",
+                 accum_dtype: str = "float"):
+    """examples/batch_gemm/batch_gemm.py:28-60: C[b] = A[b] @ B[b] in `dtype`, accumulated in float32, one launch for
+    the whole batch.  The block sizes are accepted and recorded; tiling is chosen by the library."""
+    if dtype not in ("float16", "bfloat16") or _DT[accum_dtype] != "float32":
+        raise ValueError("dtype must be float16 or bfloat16 and accum_dtype float")
+    code = ABI_DTYPE[TORCH_DTYPES[dtype]]
+
+    def launch(t, sym, stream):
+        A, Bm, C = t
+        _abi.check(_abi.load().tlq_gemm_f16_batched(_abi.ptr(A), _abi.ptr(Bm), _abi.ptr(C), B, M, N, K, code, code, _abi.B_KN,
+                                                    stream))
+
+    return KernelSpec("batch_matmul", [Param("A_mat", (B, M, K), dtype), Param("B_mat", (B, K, N), dtype),
+                                       Param("C_mat", (B, M, N), dtype)], launch, {"block": (block_M, block_N, K_L1)})
