@@ -107,10 +107,21 @@ int tlq_dequant_w4_layout(const void* w_packed, const void* scales, const void* 
  * for the fp16 target (out_dtype TLQ_F16: 8 fp16 per word) or the int8 target (TLQ_I8: 16 int8 per
  * word pair).  is_signed subtracts 8 (fp16) / 7 (int8), as the reference's decoders do.
  * scales (fp16, one per `words_per_group` words) or NULL; zeros_mode 0 none | 1 original (u - z) * s |
- * 2 rescale fma(u, s, -z) | 3 quantized (u - qz) * s with zeros an int16 array; zeros fp16 otherwise.
+ * 2 rescale fma(u, s, -|z|) | 3 quantized (u - qz) * s with zeros an int16 array; zeros fp16 otherwise.
  * The device functions themselves are in tilelang_ascend_amd/csrc/decode_i4.h. */
 int tlq_decode_i4_interleaved(const void* words, const void* scales, const void* zeros, void* out, int64_t n_words,
                               int64_t words_per_group, int out_dtype, int is_signed, int zeros_mode, void* stream);
+
+/* The "_offset" decoders of the same family (tilelang/quantize/lop3.py:82-131, 177-230, 272-322, 364-421; chosen by
+ * get_lop3_intrin_group for storage_scope "warp" with scaling, :1178-1180): the eight weights of a word belong to two
+ * groups.  Word i has group g = i / words_per_group; outputs 0..3 use scales[g] / zeros[g], outputs 4..7 use
+ * scales[g + offset] / zeros[g + offset].  fp16 output only.  zeros_mode as above, except 3 (quantized): zeros are
+ * 32-bit words of eight 4-bit zero points, the first half takes field group_offset of zeros[g], the second field
+ * group_offset of zeros[g + zero_offset].  n_scales / n_zeros are the lengths of the two arrays (elements / words);
+ * every index is checked against them before the launch. */
+int tlq_decode_i4_interleaved_offset(const void* words, const void* scales, const void* zeros, void* out, int64_t n_words,
+                                     int64_t words_per_group, int64_t n_scales, int64_t n_zeros, int offset, int zero_offset,
+                                     int group_offset, int is_signed, int zeros_mode, void* stream);
 
 /* Fused weight-only GEMM / GEMV, replaces dequant_gemm_fp16_wrapper + fp16_gemm
  * (example_dequant_gemm_fine_grained.py:60-115,176-223) extended with per-group scale / zero:

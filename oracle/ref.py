@@ -351,26 +351,33 @@ def int8_gemm_torch_optimized(a_int8, a_scales, b_int8, b_scales, out_dtype=torc
 LOP3_F16_ORDER = (0, 4, 1, 5, 2, 6, 3, 7)  # output slot j holds field LOP3_F16_ORDER[j] of the u32
 
 
-def lop3_decode_i4_to_f16(words_u32, signed=False, scale=None, zeros=None, zeros_mode=None):
+def lop3_decode_i4_to_f16(words_u32, signed=False, scale=None, zeros=None, zeros_mode=None, scale_r=None, zeros_r=None):
     """One u32 -> 8 fp16.  h[i] (a half2) = fields (i, i+4) of the word (lop3.py:17-24), so the
     flat output order is field 0,4,1,5,2,6,3,7: the weights must have been passed through
     interleave_weight for the flat order to be the logical one.  signed subtracts 8 (:14).
-    zeros_mode: None | 'original' (u - z) * s (:165-166) | 'rescale' fma(u, s, -z) (:247,260) |
-    'quantized' (u - qz) * s with integer qz (:340,351-353)."""
+    zeros_mode: None | 'original' (u - z) * s (:165-166) | 'rescale' fma(u, s, -|z|) (:247,260: the addend is the
+    zero point with its sign bit forced) | 'quantized' (u - qz) * s with integer qz (:340,351-353).
+    scale_r / zeros_r: the "_offset" forms (:82-131, 177-230, 272-322, 364-421) -- h[0], h[1] (flat outputs 0..3) use
+    scale / zeros, h[2], h[3] (flat outputs 4..7) use scale_r / zeros_r."""
     w = np.asarray(words_u32, dtype=np.uint32).reshape(-1)
     f = np.stack([(w >> np.uint32(4 * i)) & np.uint32(0xF) for i in LOP3_F16_ORDER], axis=1)
     h = f.astype(np.float16)
     if signed:
         h = h - np.float16(8)
+
+    def half(a):  # one value per output column: first four from the left parameter, last four from the right one
+        l, r = a
+        return np.array([l] * 4 + [l if r is None else r] * 4)
+
     if zeros_mode in ("original", "quantized"):
-        h = (h - np.float16(zeros)).astype(np.float16)
+        h = (h - half((zeros, zeros_r)).astype(np.float16)).astype(np.float16)
     if scale is not None:
+        sc = half((scale, scale_r)).astype(np.float16)
         if zeros_mode == "rescale":
-            h = (h.astype(np.float64) * np.float64(np.float16(scale)) - np.float64(np.float16(zeros))).astype(
-                np.float16
-            )
+            z = np.abs(half((zeros, zeros_r)).astype(np.float16))
+            h = (h.astype(np.float64) * sc.astype(np.float64) - z.astype(np.float64)).astype(np.float16)
         else:
-            h = (h * np.float16(scale)).astype(np.float16)
+            h = (h * sc).astype(np.float16)
     return h
 
 

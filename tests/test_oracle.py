@@ -166,6 +166,40 @@ def test_lop3_decode_of_interleaved_weights_is_the_plain_unpack():
     resc = ref.lop3_decode_i4_to_f16(words, scale=s, zeros=z, zeros_mode="rescale")
     exact = plain.astype(np.float64) * float(s16) - float(z16)  # single rounding (fma)
     assert np.array_equal(resc, exact.astype(np.float16))
+    # a negative zero point enters the fused form with its sign bit forced (0x80008000 | zeros, lop3.py:247): -|z| again
+    assert np.array_equal(ref.lop3_decode_i4_to_f16(words, scale=s, zeros=-z, zeros_mode="rescale"), resc)
+
+
+def test_lop3_offset_forms_use_one_group_per_half():
+    """The "_offset" decoders (lop3.py:82-131, 177-230, 272-322, 364-421): outputs 0..3 of a word take the first
+    scale / zero point, outputs 4..7 the one `offset` further on.  Checked element by element with scalar arithmetic,
+    and against the one-group forms when both halves get the same parameters."""
+    q = torch.randint(0, 256, (6, 4), dtype=torch.uint8, generator=_rng(18))
+    words = ref.interleave_weight(q.view(torch.int8), 4, "float16").contiguous().view(torch.int32).numpy().view(np.uint32).reshape(-1)
+    plain = ref.unpack_uint4(q).reshape(-1, 8)
+    sl, sr, zl, zr = 0.011, 0.019, 6.5, 9.0
+    for mode in (None, "original", "rescale", "quantized"):
+        zl_, zr_ = (7, 12) if mode == "quantized" else (zl, zr)
+        kw = {} if mode is None else dict(zeros=zl_, zeros_r=zr_, zeros_mode=mode)
+        got = ref.lop3_decode_i4_to_f16(words, scale=sl, scale_r=sr, **kw)
+        same = ref.lop3_decode_i4_to_f16(words, scale=sl, scale_r=sl, **dict(kw, zeros_r=zl_) if kw else {})
+        one = ref.lop3_decode_i4_to_f16(words, scale=sl, **({} if mode is None else dict(zeros=zl_, zeros_mode=mode)))
+        assert np.array_equal(same, one), mode
+        for w in range(plain.shape[0]):
+            for j in range(8):
+                s16 = np.float16(sl if j < 4 else sr)
+                z16 = np.float16(zl_ if j < 4 else zr_)
+                u = np.float16(plain[w, j])
+                if mode is None:
+                    want = np.float16(u * s16)
+                elif mode == "rescale":
+                    want = np.float16(float(u) * float(s16) - float(z16))
+                else:
+                    want = np.float16(np.float16(u - z16) * s16)
+                assert got[w, j] == want, (mode, w, j)
+    signed = ref.lop3_decode_i4_to_f16(words, signed=True, scale=sl, scale_r=sr)
+    assert np.array_equal(signed[:, :4], ((plain[:, :4].astype(np.float16) - np.float16(8)) * np.float16(sl)).astype(np.float16))
+    assert np.array_equal(signed[:, 4:], ((plain[:, 4:].astype(np.float16) - np.float16(8)) * np.float16(sr)).astype(np.float16))
 
 
 def test_gen_quant4_invariants():

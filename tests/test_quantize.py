@@ -110,8 +110,17 @@ def test_lop3_group_naming_grammar():
         Q.get_lop3_intrin_group("float32")
     with pytest.raises(NotImplementedError):
         Q.get_lop3_intrin_group("float16", source_bit=2)
+    # storage_scope "warp" with scaling selects the two-group forms (lop3.py:1178-1180, 1196-1197)
+    for kw, name in ((dict(), "decode_i4u_to_f16_scale_offset"),
+                     (dict(source_format="int"), "decode_i4s_to_f16_scale_offset"),
+                     (dict(with_zeros=True, zeros_mode="original"), "decode_i4u_to_f16_scale_zeros_original_offset"),
+                     (dict(with_zeros=True, zeros_mode="rescale"), "decode_i4u_to_f16_scale_zeros_rescale_offset"),
+                     (dict(with_zeros=True, zeros_mode="quantized"), "decode_i4u_to_f16_scale_zeros_quantized_offset")):
+        g = Q.get_lop3_intrin_group("float16", with_scaling=True, storage_scope="warp", **kw)
+        assert g["func_name"] == name and f" {name}(" in g["c_source"]
+    assert Q.get_lop3_intrin_group("float16", storage_scope="warp")["func_name"] == "decode_i4u_to_f16"  # no scaling: no suffix
     with pytest.raises(NotImplementedError):
-        Q.get_lop3_intrin_group("float16", with_scaling=True, storage_scope="warp")
+        Q.get_lop3_intrin_group("int4", source_bit=2)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -173,3 +182,55 @@ def test_gpu_quantize_utils_run_on_device_tensors():
     assert packed.is_cuda and torch.equal(packed.cpu(), ref.general_compress(w, 4, torch.int8))
     inter = Q.interleave_weight(packed, 4, "float16")
     assert inter.is_cuda and torch.equal(inter.cpu(), ref.interleave_weight(packed.cpu(), 4, "float16"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", [None, "original", "rescale", "quantized"])
+@pytest.mark.parametrize("offset", [0, 1, 5])
+def test_gpu_decode_offset_forms(mode, offset):
+    """The two-group decoders on the GPU against the oracle's word-level closed form, word by word: the first four
+    weights of a word use group g, the last four group g + offset (zero points: field group_offset of the packed words
+    g and g + zero_offset for the quantized mode)."""
+    from tilelang_ascend_amd.quantize import lop3
+
+    g_size, groups = 32, 12
+    wpg = g_size // 8
+    gen = _rng(21 + offset)
+    q = torch.randint(0, 256, (groups * g_size // 2,), dtype=torch.uint8, generator=gen).reshape(1, -1)
+    s = (torch.rand(groups + offset, generator=gen) * 0.015 + 0.005).half()
+    zf = (torch.rand(groups + offset, generator=gen) * 3 + 6).half()
+    zero_offset, group_offset = 2, 3
+    qz_fields = torch.randint(0, 16, (groups + zero_offset, 8), generator=gen)
+    qz_words = sum(qz_fields[:, j].to(torch.int64) << (4 * j) for j in range(8))
+    qz_words = torch.where(qz_words >= (1 << 31), qz_words - (1 << 32), qz_words).to(torch.int32)
+    inter = Q.interleave_weight(q.view(torch.int8), 4, "float16")
+    zeros = None if mode is None else (qz_words if mode == "quantized" else zf)
+    for signed in ((False, True) if mode is None else (False,)):
+        got = lop3.decode_offset(inter.cuda(), s.cuda(), offset, "int" if signed else "uint",
+                                 zeros=None if zeros is None else zeros.cuda(), zeros_mode=mode, group_size=g_size,
+                                 zero_offset=zero_offset, group_offset=group_offset).cpu().numpy().reshape(-1, 8)
+        words = inter.contiguous().view(torch.int32).numpy().view(np.uint32).reshape(-1)
+        for i, word in enumerate(words):
+            grp = i // wpg
+            kw = {}
+            if mode == "quantized":
+                kw = dict(zeros=int(qz_fields[grp, group_offset]), zeros_r=int(qz_fields[grp + zero_offset, group_offset]), zeros_mode=mode)
+            elif mode is not None:
+                kw = dict(zeros=float(zf[grp]), zeros_r=float(zf[grp + offset]), zeros_mode=mode)
+            want = ref.lop3_decode_i4_to_f16([word], signed=signed, scale=float(s[grp]), scale_r=float(s[grp + offset]), **kw)
+            assert np.array_equal(got[i], want[0]), (mode, offset, signed, i)
+
+
+@pytest.mark.gpu
+def test_gpu_decode_offset_rejects_short_parameter_arrays():
+    from tilelang_ascend_amd.quantize import lop3
+
+    w = torch.zeros(1, 64, dtype=torch.uint8, device="cuda")  # 16 words = 4 groups of 32 weights
+    s = torch.ones(4, dtype=torch.float16, device="cuda")
+    assert lop3.decode_offset(w, s, 0, group_size=32).shape == (1, 128)
+    with pytest.raises(RuntimeError, match="need 5 scales"):
+        lop3.decode_offset(w, s, 1, group_size=32)
+    with pytest.raises(RuntimeError, match="zeros"):
+        lop3.decode_offset(w, torch.ones(5, dtype=torch.float16), 1, zeros=s, zeros_mode="original", group_size=32)
+    with pytest.raises(RuntimeError, match="group_offset"):
+        lop3.decode_offset(w, s, 0, zeros=torch.zeros(4, dtype=torch.int32), zeros_mode="quantized", group_size=32, group_offset=8)

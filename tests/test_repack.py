@@ -115,3 +115,33 @@ def test_repack_rejects_bad_arguments():
         gpu.pack_int4(v.cpu())
     with pytest.raises(ValueError):
         gpu.quantize_sym4(w.float())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_gen_quant4_results_feed_the_w4a16_operands(groupsize):
+    """gen_quant4 -> pack_gen_quant4 -> dequantize_w4(zero point 8) gives gen_quant4's own dequantised weight (the
+    nn.Linear it returns), except where q = 16 was stored as 15; scales travel from [K/g, N] to [N, K/g]."""
+    from tilelang_ascend_amd import quantize as Q
+    from tilelang_ascend_amd.ops import dequantize_w4
+    from tilelang_ascend_amd.quantize import gpu
+
+    torch.manual_seed(11)
+    k, n = 256, 72
+    _, linear, s, q8 = Q.gen_quant4(k, n, groupsize)
+    g = k if groupsize == -1 else groupsize
+    assert s.shape == (k // g, n)
+    assert torch.equal(gpu.scales_kn_to_nk(s), s.t())
+    Bp, S = gpu.pack_gen_quant4(q8, s)
+    assert Bp.shape == (n, k // 2) and Bp.dtype == torch.uint8 and S.shape == (n, k // g) and S.is_contiguous()
+    W = dequantize_w4(Bp, S, 8, g, torch.float16).cpu()
+    want = linear.weight.data  # [n, k] = ((q - 8).half() * s).T
+    top = (q8.t() == 8)
+    assert top.any()  # the positive maximum of a group always quantises to 16
+    assert torch.equal(W[~top], want[~top])
+    s_full = s.repeat_interleave(g, dim=0).t()
+    assert torch.equal(W[top], (7 * s_full[top].float()).half())
+    with pytest.raises(ValueError, match="four bits"):
+        gpu.pack_gen_quant4(q8, s, saturate=False)
+    with pytest.raises(ValueError):
+        gpu.pack_gen_quant4(q8 + 5, s)

@@ -8,6 +8,9 @@
 //   decode_i4u_to_f16_scale_zeros_rescale(src, dst, scale, z)    fma(u, s, -z)    one rounding
 //   decode_i4u_to_f16_scale_zeros_quantized(src, dst, scale, qz) (u - qz) * s     qz an integer 0..15
 //   decode_i4{u,s}_to_i8s(src, dst)                              16 nibbles (two words) -> 16 int8
+//   ..._offset(src, dst, scale[, zeros], offset)                 the forms for fragments whose two halves belong to
+//       different groups (lop3.py:82-131, :177-230, :272-322, :364-421): outputs 0..3 use scale[0] / zeros[0],
+//       outputs 4..7 use scale[offset] / zeros[offset]
 // The source words hold the nibbles in the order tilelang/quantize/utils.py:73-126
 // (interleave_weight) produces, so that one shift + one AND-OR yields two neighbouring weights:
 // word >> 4i has logical elements (2i, 2i+1) at bits 0..3 and 16..19 (fp16 target) and logical
@@ -35,6 +38,7 @@ __device__ __forceinline__ uint32_t as_u32(h2 x) {
   return r;
 }
 __device__ __forceinline__ h2 splat(_Float16 v) { return h2{v, v}; }
+__device__ __forceinline__ h2 neg_abs(h2 v) { return as_h2(as_u32(v) | 0x80008000u); }
 // (1024 + u_lo, 1024 + u_hi) from the two nibbles at bits 4i and 16 + 4i
 __device__ __forceinline__ h2 biased_pair(uint32_t word, int i) {
   return as_h2(((word >> (4 * i)) & 0x000f000fu) | 0x64006400u);
@@ -90,7 +94,8 @@ __device__ __forceinline__ void decode_i4u_to_f16_scale_zeros_rescale(T1* src, T
                                                                       T4* zeros = nullptr, const int N = 8) {
   const uint32_t w = *reinterpret_cast<const uint32_t*>(src);
   uint32_t* h = reinterpret_cast<uint32_t*>(dst);
-  const h2 k1024 = splat((_Float16)1024.0f), s = splat((_Float16)*scale), nz = splat(-(_Float16)*zeros);
+  // the addend is the zero point with its sign bit forced (0x80008000 | zeros, lop3.py:247): -|z|
+  const h2 k1024 = splat((_Float16)1024.0f), s = splat((_Float16)*scale), nz = neg_abs(splat((_Float16)*zeros));
 #pragma unroll
   for (int i = 0; i < N / 2; ++i) h[i] = as_u32(__builtin_elementwise_fma(biased_pair(w, i) - k1024, s, nz));
 }
@@ -105,6 +110,72 @@ __device__ __forceinline__ void decode_i4u_to_f16_scale_zeros_quantized(T1* src,
   const h2 median = as_h2(((0xe400u | qz) << 16) | (0xe400u | qz)), s = splat((_Float16)*scale);
 #pragma unroll
   for (int i = 0; i < N / 2; ++i) h[i] = as_u32((biased_pair(w, i) + median) * s);
+}
+
+// ---- forms with two groups per word: outputs 0..3 (h[0], h[1]) use *scale / *zeros, outputs 4..7 (h[2], h[3]) use
+// *(scale + offset) / *(zeros + offset) ----------------------------------------------------------------------
+template <typename T1, typename T2, typename T3, bool isSigned>
+__device__ __forceinline__ void decode_i4b_to_f16_scale_offset(T1* src, T2* dst, const T3* scale, const int offset,
+                                                               const int N = 8) {
+  const uint32_t w = *reinterpret_cast<const uint32_t*>(src);
+  uint32_t* h = reinterpret_cast<uint32_t*>(dst);
+  const h2 median = splat((_Float16)(isSigned ? 1032.0f : 1024.0f));
+  const h2 sl = splat((_Float16)*scale), sr = splat((_Float16) * (scale + offset));
+#pragma unroll
+  for (int i = 0; i < N / 2; ++i) h[i] = as_u32((biased_pair(w, i) - median) * (i < N / 4 ? sl : sr));
+}
+template <typename T1, typename T2, typename T3>
+__device__ __forceinline__ void decode_i4u_to_f16_scale_offset(T1* src, T2* dst, T3* scale = nullptr, const int offset = 0,
+                                                               const int N = 8) {
+  decode_i4b_to_f16_scale_offset<T1, T2, T3, false>(src, dst, scale, offset, N);
+}
+template <typename T1, typename T2, typename T3>
+__device__ __forceinline__ void decode_i4s_to_f16_scale_offset(T1* src, T2* dst, T3* scale = nullptr, const int offset = 0,
+                                                               const int N = 8) {
+  decode_i4b_to_f16_scale_offset<T1, T2, T3, true>(src, dst, scale, offset, N);
+}
+
+template <typename T1, typename T2, typename T3, typename T4>
+__device__ __forceinline__ void decode_i4u_to_f16_scale_zeros_original_offset(T1* src, T2* dst, T3* scale = nullptr,
+                                                                              T4* zeros = nullptr, const int offset = 0,
+                                                                              const int N = 8) {
+  const uint32_t w = *reinterpret_cast<const uint32_t*>(src);
+  uint32_t* h = reinterpret_cast<uint32_t*>(dst);
+  const h2 k1024 = splat((_Float16)1024.0f);
+  const h2 sl = splat((_Float16)*scale), sr = splat((_Float16) * (scale + offset));
+  const h2 zl = splat((_Float16)*zeros), zr = splat((_Float16) * (zeros + offset));
+#pragma unroll
+  for (int i = 0; i < N / 2; ++i) h[i] = as_u32(((biased_pair(w, i) - k1024) - (i < N / 4 ? zl : zr)) * (i < N / 4 ? sl : sr));
+}
+
+template <typename T1, typename T2, typename T3, typename T4>
+__device__ __forceinline__ void decode_i4u_to_f16_scale_zeros_rescale_offset(T1* src, T2* dst, T3* scale = nullptr,
+                                                                             T4* zeros = nullptr, const int offset = 0,
+                                                                             const int N = 8) {
+  const uint32_t w = *reinterpret_cast<const uint32_t*>(src);
+  uint32_t* h = reinterpret_cast<uint32_t*>(dst);
+  const h2 k1024 = splat((_Float16)1024.0f);
+  const h2 sl = splat((_Float16)*scale), sr = splat((_Float16) * (scale + offset));
+  const h2 zl = neg_abs(splat((_Float16)*zeros)), zr = neg_abs(splat((_Float16) * (zeros + offset)));
+#pragma unroll
+  for (int i = 0; i < N / 2; ++i)
+    h[i] = as_u32(__builtin_elementwise_fma(biased_pair(w, i) - k1024, i < N / 4 ? sl : sr, i < N / 4 ? zl : zr));
+}
+
+// qzeros holds packed 4-bit zero points in words of the weights' storage type T1: the zero point of the first half
+// is field group_offset of qzeros[0], that of the second half field group_offset of qzeros[zero_offset]
+template <typename T1, typename T2, typename T3>
+__device__ __forceinline__ void decode_i4u_to_f16_scale_zeros_quantized_offset(T1* src, T2* dst, T3* scale = nullptr,
+                                                                               T1* qzeros = nullptr, const int scale_offset = 0,
+                                                                               const int zero_offset = 0,
+                                                                               const int group_offset = 0, const int N = 8) {
+  const uint32_t w = *reinterpret_cast<const uint32_t*>(src);
+  uint32_t* h = reinterpret_cast<uint32_t*>(dst);
+  const h2 sl = splat((_Float16)*scale), sr = splat((_Float16) * (scale + scale_offset));
+  const uint32_t ql = (uint32_t)(*qzeros >> (group_offset * 4)) & 0xfu, qr = (uint32_t)(*(qzeros + zero_offset) >> (group_offset * 4)) & 0xfu;
+  const h2 ml = as_h2(((0xe400u | ql) << 16) | (0xe400u | ql)), mr = as_h2(((0xe400u | qr) << 16) | (0xe400u | qr));
+#pragma unroll
+  for (int i = 0; i < N / 2; ++i) h[i] = as_u32((biased_pair(w, i) + (i < N / 4 ? ml : mr)) * (i < N / 4 ? sl : sr));
 }
 
 // 16 nibbles -> 16 int8: output word i (i = 0, 1) holds nibbles 4i.. of src word 0 in byte lanes,

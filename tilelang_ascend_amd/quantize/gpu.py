@@ -50,3 +50,35 @@ def quantize_sym4(W: torch.Tensor, group_size: int = -1) -> Tuple[torch.Tensor, 
     with torch.cuda.device(W.device):
         _abi.check(_abi.load().tlq_quantize_sym4(_abi.ptr(W), _abi.ptr(q), _abi.ptr(s), N, K, g, _DT[W.dtype], _stream()))
     return q, s
+
+
+def scales_kn_to_nk(scales: torch.Tensor) -> torch.Tensor:
+    """gen_quant4 (tilelang/quantize/utils.py:5-50) returns its scales as [K / groupsize, N], one row per group of
+    input features; the kernels read [N, K / groupsize], a row per output feature next to that feature's packed
+    weights.  Returns the transposed copy (works on any device)."""
+    if scales.dim() != 2:
+        raise ValueError("scales must be 2-D [K / groupsize, N]")
+    return scales.t().contiguous()
+
+
+def pack_gen_quant4(q_minus8: torch.Tensor, scales: torch.Tensor, interleave: Optional[str] = None,
+                    saturate: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Outputs of gen_quant4 -> operands of the W4A16 kernels with zero point 8.
+
+    q_minus8: [K, N] integer tensor in [-8, 8] (gen_quant4's fourth result); scales: [K / groupsize, N] (its third).
+    Returns (B_packed uint8 [N, K // 2], scales [N, K / groupsize]) on the GPU, so that
+    dequantize_w4(B_packed, scales, 8, groupsize) is gen_quant4's dequantised weight, transposed to [N, K].
+    gen_quant4 clamps q to [0, 16] (maxq = 16, utils.py:8 and :30), and 16 does not fit four bits: with saturate=True
+    such elements (the positive maximum of a group) are stored as 15, i.e. 7 * s instead of 8 * s; with
+    saturate=False their presence raises ValueError."""
+    if q_minus8.dim() != 2 or scales.dim() != 2 or scales.shape[1] != q_minus8.shape[1]:
+        raise ValueError("expected q_minus8 [K, N] and scales [K / groupsize, N]")
+    u = q_minus8.to(torch.int16) + 8
+    if int(u.min()) < 0 or int(u.max()) > 16:
+        raise ValueError("q_minus8 must lie in [-8, 8]")
+    if int(u.max()) == 16:
+        if not saturate:
+            raise ValueError("q_minus8 holds the value 8 (q = 16), which does not fit four bits")
+        u = u.clamp(max=15)
+    vals = u.to(torch.uint8).t().contiguous().cuda()
+    return pack_int4(vals, interleave, torch.uint8), scales_kn_to_nk(scales).cuda()

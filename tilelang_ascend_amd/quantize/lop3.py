@@ -8,7 +8,9 @@ under the reference's naming grammar, and ``decode`` runs the same device functi
 through the C ABI (``tlq_decode_i4_interleaved``).
 
 Only the 4-bit source width is built (the quantized-matmul path uses nothing else); asking for
-1- or 2-bit sources raises NotImplementedError rather than handing back untested code.
+1- or 2-bit sources raises NotImplementedError rather than handing back untested code.  The "_offset"
+decoders (storage_scope "warp" with scaling: the two halves of a word belong to different groups) are
+built for 4-bit sources as well; ``decode_offset`` runs them on a tensor.
 """
 from __future__ import annotations
 
@@ -48,9 +50,8 @@ def get_lop3_intrin_group(
         func_name += f"_zeros_{zeros_mode}"
     if storage_scope == "warp" and with_scaling:
         func_name += "_offset"
-    if source_bit != 4 or out_dtype == "int4" or func_name.endswith("_offset"):
-        raise NotImplementedError(f"{func_name}: only 4-bit sources decoded to float16 / int8 in thread-local "
-                                  "storage are built for gfx950")
+    if source_bit != 4 or out_dtype == "int4":
+        raise NotImplementedError(f"{func_name}: only 4-bit sources decoded to float16 / int8 are built for gfx950")
     if out_dtype == "int8" and (with_scaling or with_zeros):
         raise KeyError(f"i{source_bit}_to_i8" + ("_scale" if with_scaling else "") + " has no decoder")
     if with_zeros and not with_scaling:
@@ -96,4 +97,35 @@ def decode(words, out_dtype: str = "float16", source_format: str = "uint", scale
         _abi.check(lib.tlq_decode_i4_interleaved(_abi.ptr(w), _abi.ptr(s), _abi.ptr(z), _abi.ptr(out), n_words, max(wpg, 1),
                                                  _abi.F16 if out_dtype == "float16" else _abi.I8,
                                                  1 if source_format == "int" else 0, mode, stream))
+    return out
+
+
+def decode_offset(words, scale, offset: int, source_format: str = "uint", zeros=None, zeros_mode: Optional[str] = None,
+                  group_size: int = -1, zero_offset: int = 0, group_offset: int = 0):
+    """Run the "_offset" decoder named by the arguments (lop3.py:82-131, 177-230, 272-322, 364-421) on a device tensor
+    of interleaved weights: word i belongs to group g = i // (group_size // 8); its first four weights use scale[g] /
+    zeros[g], the last four scale[g + offset] / zeros[g + offset].  For zeros_mode='quantized', zeros is an int32
+    tensor of packed 4-bit zero points: the halves take field `group_offset` of zeros[g] and of zeros[g + zero_offset].
+    Returns float16, last dimension expanded to one element per nibble."""
+    import torch
+
+    from .. import _abi
+
+    lib = _abi.load()
+    w = words.contiguous()
+    n_bytes = w.numel() * w.element_size()
+    assert n_bytes % 4 == 0, "the weights must be whole 32-bit words"
+    n_words = n_bytes // 4
+    out = torch.empty(*w.shape[:-1], w.shape[-1] * w.element_size() * 2, dtype=torch.float16, device=w.device)
+    mode = 0 if zeros_mode is None else ZEROS_MODES[zeros_mode]
+    wpg = max(n_words, 1) if group_size in (-1, None) else group_size // 8
+    s = scale.to(device=w.device, dtype=torch.float16).contiguous()
+    z = None
+    if zeros is not None:
+        z = zeros.to(device=w.device, dtype=torch.int32 if mode == 3 else torch.float16).contiguous()
+    stream = torch.cuda.current_stream().cuda_stream
+    with torch.cuda.device(w.device):
+        _abi.check(lib.tlq_decode_i4_interleaved_offset(_abi.ptr(w), _abi.ptr(s), _abi.ptr(z), _abi.ptr(out), n_words, wpg,
+                                                        s.numel(), 0 if z is None else z.numel(), offset, zero_offset,
+                                                        group_offset, 1 if source_format == "int" else 0, mode, stream))
     return out
