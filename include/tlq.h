@@ -72,8 +72,10 @@ enum {
   TLQ_ALGO_MFMA = 2, /* LDS-staged MFMA dequant-GEMM */
   TLQ_ALGO_SKINNY = 3, /* M <= 64: weights stream from HBM through the dequantiser into MFMA operands, no LDS tile */
   TLQ_ALGO_TWO_PASS = 4, /* tlq_gemm_w4a16_ws only: dequantise into the workspace, then the plain GEMM */
-  TLQ_ALGO_STREAM = 5 /* tlq_gemm_w4a16_ws only: 17 <= M <= 512, weights streamed once per 128 activation rows through a deep
+  TLQ_ALGO_STREAM = 5, /* tlq_gemm_w4a16_ws only: 17 <= M <= 512, weights streamed once per 128 activation rows through a deep
                        * ring of direct loads, dequantised in registers; K slices add up through the workspace */
+  TLQ_ALGO_DECODE = 6 /* 1 <= M <= 32, K % 256 == 0, power-of-two group: persistent work-groups, activations resident in registers, every
+                       * weight read once through deep wavefront-private rings (rows longer than 4096 values need the workspace) */
 };
 
 int tlq_abi_version(void);
@@ -130,7 +132,8 @@ int tlq_decode_i4_interleaved_offset(const void* words, const void* scales, cons
  * Requires K % 64 == 0 and group % 32 == 0 (group divides K).  The MFMA kernel additionally needs
  * N % 4 == 0 and a power-of-two group (32, 64, 128, ...); the GEMV kernel (M <= 16) takes any such group;
  * the skinny kernel (M <= 64) needs K % 128 == 0.  TLQ_ALGO_AUTO: M = 1 GEMV (fp16; bf16 up to K = 8192; fp16 also M = 2 with
- * K <= 4096), otherwise M <= 64 skinny where its conditions hold (else GEMV up to M = 4), else MFMA. */
+ * K <= 4096), otherwise the decode kernel (TLQ_ALGO_DECODE) where M <= 32, K % 256 == 0, K <= 4096, the group is a power of two and the
+ * scale / zero tensors are dword aligned, else M <= 64 skinny where its conditions hold (else GEMV up to M = 4), else MFMA. */
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                    void* stream);
@@ -268,6 +271,14 @@ int tlq_debug_check_slots_schedule(int stages, int loads_per_tile);
  * with 16 * activation_tiles rows per work-group (2 | 4 | 8), and its ring of `ring_depth` steps for 1 .. 40 steps. */
 int tlq_debug_check_stream_addressing(int64_t M, int64_t N, int64_t K, int activation_tiles, int ring_depth);
 
+/* The same walk for the decode kernel (TLQ_ALGO_DECODE) launched as grid_x x chunks work-groups of `waves` wavefronts
+ * with 16 * activation_tiles activation rows, and its ring for 2 .. 24 items; tlq_debug_decode_plan gives the geometry
+ * the library would choose on a device with `cus` compute units: plan_out is a HOST array of five int64 that receives
+ * activation tiles, chunks, wavefronts per work-group, grid_x and bytes of dynamic LDS; returns 1 when the kernel applies. */
+int tlq_debug_check_decode_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int activation_tiles, int chunks, int waves,
+                                      int grid_x);
+int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
+
 /* Launch geometry the register-resident decode GEMV (M = 1, K <= 16384, power-of-two group) would use on a device with
  * `cus` compute units, computed on the host: plan_out is a HOST array of four int64 that receives rows per work-group,
  * work-groups, bytes of dynamic LDS and wavefronts per work-group.  Returns 1 when the kernel applies (its LDS stays
@@ -286,6 +297,7 @@ void tlq_tune_gemm_band(int tile_rows);                       /* tile rows per b
 void tlq_tune_gemm_slots(int on);                            /* 1 (default): 256 x 256 tiles of the plain 16-bit GEMM with [N, K] weights and of the
                                                               * int8 GEMMs run on the kernel that cuts LDS into five operand-tile slots
                                                               * (whole 128-byte stages of K only); 0: always the two-stage kernel */
+void tlq_tune_w4a16_decode(int on);                          /* 0: the decode kernel is never picked automatically */
 void tlq_tune_w4a16_stream(int on);                          /* 0: tlq_gemm_w4a16_ws never picks the streaming kernel by itself */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
 void tlq_tune_w4a16_split(int slices);                       /* K slices of the tile kernel, 16 < M < 256 with a workspace */

@@ -124,5 +124,67 @@ __host__ __device__ inline int stream_younger_steps(int s, int steps, int D) {
   return last_issued - s > 0 ? last_issued - s : 0;
 }
 
+// ---- decode kernel (1 .. 32 activation rows): wavefront w of a work-group owns values 256 s .. 256 s + 255 of K
+// (s = chunk * waves + w) for every weight row.  A work item is one 16-row weight tile: two [16 rows][64 B] packed
+// pieces (k-blocks kb = 0, 1 of the slice, 128 values each) plus the scales / zero points of the 16 rows for the
+// slice.  Work-group b handles tiles b, b + grid, ...; the ts-th of them lives in ring slot ts % 3.
+constexpr int kDecSlice = 256;
+constexpr int kDecTileSlots = 3;
+constexpr uint32_t kDecSlotBytes = 2048 + 512;  // packed piece kb 0 | kb 1 | scale dwords (256 B) | zero dwords (256 B)
+__host__ __device__ inline int dec_red_buffers(int mt) { return mt == 1 ? 2 : 1; }
+__host__ __device__ inline uint32_t dec_red_base() { return kDecTileSlots * kDecSlotBytes; }
+__host__ __device__ inline uint32_t dec_wave_bytes(int mt) { return dec_red_base() + (uint32_t)(dec_red_buffers(mt) * mt) * 1024u; }
+// Packed weights: the lane's byte offset from the first byte of (tile t, slice, kb = 0); kb = 1 is 64 bytes further.
+// In the last tile the rows past N repeat row N - 1.
+__host__ __device__ inline uint32_t dec_w_lane(int lane, int64_t t, int64_t N, int64_t K) {
+  int64_t n = t * 16 + sw_row(lane);
+  n = n < N ? n : N - 1;
+  return (uint32_t)((n - t * 16) * (K / 2) + sw_piece(lane) * 16);
+}
+__host__ __device__ inline int64_t dec_w_base(int64_t t, int64_t K, int64_t k0) { return t * 16 * (K / 2) + k0 / 2; }
+// Activations of a slice: per k-block kb and 16-row tile mt a [16 rows][256 B] block, fetched by four direct loads of
+// 1 KB (load i: rows 4 i .. 4 i + 3, lane l on row 4 i + l / 16, physical 16-byte piece l % 16, which receives logical
+// piece (l % 16) ^ (row % 8)) into 4 KB of the wavefront's LDS, and read back as MFMA operands: lane (m = r16, k-group q)
+// takes logical piece 4 q + j for k-step j, the eight values 32 q + 8 j .. of the k-block.  Rows past M repeat the last.
+// dec_a_off: byte offset of the lane's 16 bytes inside A.
+__host__ __device__ inline int64_t dec_a_off(int lane, int mt, int kb, int i, int64_t M, int64_t K, int64_t k0) {
+  const int row = 4 * i + (lane >> 4);
+  int64_t m = mt * 16 + row;
+  m = m < M ? m : M - 1;
+  return (m * K + k0 + kb * 128) * 2 + (((lane & 15) ^ (row & 7)) << 4);
+}
+__host__ __device__ inline uint32_t dec_a_frag(int lane, int j) {  // inside the 4 KB block
+  const int r16 = lane & 15, q = lane >> 4;
+  return (uint32_t)(r16 * 256 + (((4 * q + j) ^ (r16 & 7)) << 4));
+}
+// Scales / zero points of a tile and slice: 256 / group values per row, fetched as dwords (two values).  Lane l of the
+// first 16 nd lanes (nd dwords per row: 1, 2, 4 for groups of >= 128, 64, 32) gathers dword l / 16 of row l % 16 and
+// lands on cell l of the 256-byte area.  dec_sc_elem: the first of the (up to) two values of that dword, for tile 0.
+__host__ __device__ inline int dec_sc_dwords(int gshift) { return gshift >= 7 ? 1 : (gshift == 6 ? 2 : 4); }
+__host__ __device__ inline int64_t dec_sc_elem(int lane, int64_t t, int64_t N, int64_t groups, int64_t k0, int gshift) {
+  int64_t n = t * 16 + (lane & 15);
+  n = n < N ? n : N - 1;
+  return n * groups + (k0 >> gshift) + 2 * (lane >> 4);
+}
+// byte offset of the aligned dword that holds value `elem`
+__host__ __device__ inline uint32_t dec_sc_off(int64_t elem) { return (uint32_t)((elem * 2) & ~(int64_t)3); }
+// where lane (row r16, k-group q) finds the scale of its k-block kb: cell and half of the dword.  With groups of 256
+// values or more one value serves the whole slice, and it is the low or high half according to its index in the tensor.
+__host__ __device__ inline uint32_t dec_sc_cell(int lane, int kb, int gshift) {
+  const int gi = gshift >= 8 ? 0 : ((kb * 128 + 32 * (lane >> 4)) >> gshift);
+  return (uint32_t)(((gi >> 1) * 16 + (lane & 15)) * 4);
+}
+__host__ __device__ inline uint32_t dec_sc_half(int lane, int kb, int64_t groups, int64_t k0, int gshift) {
+  if (gshift >= 8) return (uint32_t)((((int64_t)(lane & 15) * groups + (k0 >> gshift)) & 1) * 16);
+  return (uint32_t)((((kb * 128 + 32 * (lane >> 4)) >> gshift) & 1) * 16);
+}
+// Loads still allowed in flight when k-block kb of the ts-th tile is read.  Per tile four loads are issued, in the order
+// scale gather, zero gather, piece 0, piece 1; tile ts + 2 is issued at the top of iteration ts.
+__host__ __device__ inline int dec_wait_count(int ts, int kb, int my_tiles) {
+  int younger = my_tiles - 1 - ts;
+  younger = younger > 2 ? 2 : younger;
+  return 4 * younger + (kb == 0 ? 1 : 0);
+}
+
 }  // namespace addr
 }  // namespace tlq

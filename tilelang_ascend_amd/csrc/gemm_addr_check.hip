@@ -6,6 +6,7 @@
 //   * the five-slot schedule never overwrites a tile that has not been multiplied and never multiplies a tile whose
 //     loads were not waited for.
 // No GPU is needed: these run in the CPU-only test suite and can be called before a launch.
+#include <utility>
 #include <vector>
 
 #include "gemm_addr.h"
@@ -284,6 +285,147 @@ int check_stream_ring(int steps, int D) {
   return 0;
 }
 
+// Decode kernel (1 .. 32 activation rows): every global access of every work-group, wavefront, item and lane of a
+// launch with `grid_x` x `chunks` work-groups of `waves` wavefronts, and the LDS cells the operands are read from.
+int check_decode(int64_t M, int64_t N, int64_t K, int64_t group, int mt, int chunks, int waves, int grid_x) {
+  CHECK_OR_FAIL(M >= 1 && M <= 16 * mt && (mt == 1 || mt == 2), "decode: %lld activation rows in %d tiles", (long long)M, mt);
+  CHECK_OR_FAIL(N >= 1 && K >= addr::kDecSlice && K % addr::kDecSlice == 0, "decode: bad shape");
+  CHECK_OR_FAIL(group >= 32 && (group & (group - 1)) == 0 && K % group == 0, "decode: bad group %lld", (long long)group);
+  CHECK_OR_FAIL(N * (K / 2) < ((int64_t)1 << 32) && M * K * 2 < ((int64_t)1 << 32), "decode: a matrix spans 4 GiB or more");
+  const int64_t slices = K / addr::kDecSlice, groups = K / group, tiles = (N + 15) / 16;
+  CHECK_OR_FAIL(chunks >= 1 && waves >= 1 && waves <= 16 && (int64_t)chunks * waves >= slices && (int64_t)(chunks - 1) * waves < slices,
+                "decode: %d chunks of %d wavefronts do not cover %lld slices", chunks, waves, (long long)slices);
+  CHECK_OR_FAIL(grid_x >= 1 && grid_x <= tiles, "decode: %d work-groups for %lld tiles", grid_x, (long long)tiles);
+  CHECK_OR_FAIL(((N * groups) & 1) == 0, "decode: scale tensors of an odd number of values");
+  CHECK_OR_FAIL((int64_t)waves * addr::dec_wave_bytes(mt) <= 160 * 1024, "decode: LDS");
+  int gshift = 0;
+  while (((int64_t)1 << gshift) < group) ++gshift;
+  const int64_t w_extent = N * (K / 2), a_extent = M * K * 2, sc_extent = N * groups * 2;
+  // operand cells of the 1 KB weight tile: lane l lands on cell l = (row l / 4, logical piece sw_piece)
+  for (int lane = 0; lane < 64; ++lane) {
+    const uint32_t off = addr::sw_frag_off(lane);
+    CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= 1024, "decode: weight operand read at %u", off);
+    const int src = off / 16;  // the lane that wrote this cell
+    CHECK_OR_FAIL(addr::sw_row(src) == (lane & 15) && addr::sw_piece(src) == (lane >> 4), "decode: weight operand read of lane %d finds row %d piece %d",
+                  lane, addr::sw_row(src), addr::sw_piece(src));
+  }
+  std::vector<char> tile_seen(tiles, 0);
+  for (int bx = 0; bx < grid_x; ++bx)
+    for (int64_t t = bx; t < tiles; t += grid_x) {
+      CHECK_OR_FAIL(!tile_seen[t], "decode: tile %lld handled twice", (long long)t);
+      tile_seen[t] = 1;
+    }
+  for (int64_t t = 0; t < tiles; ++t) CHECK_OR_FAIL(tile_seen[t], "decode: tile %lld never handled", (long long)t);
+  std::vector<char> k_seen(K / 8, 0);  // 16-byte pieces of one activation row
+  const int nd = addr::dec_sc_dwords(gshift);
+  for (int chunk = 0; chunk < chunks; ++chunk)
+    for (int wave = 0; wave < waves; ++wave) {
+      const int64_t slice = (int64_t)chunk * waves + wave;
+      if (slice >= slices) continue;
+      const int64_t k0 = slice * addr::kDecSlice;
+      for (int kb = 0; kb < 2; ++kb)
+        for (int m_t = 0; m_t < mt; ++m_t) {
+          int64_t cell[256];  // 16-byte cells of the 4 KB block: the offset inside A of what landed there
+          for (int i = 0; i < 4; ++i)
+            for (int lane = 0; lane < 64; ++lane) {
+              const int64_t o = addr::dec_a_off(lane, m_t, kb, i, M, K, k0);
+              CHECK_OR_FAIL(o >= 0 && o % 16 == 0 && o + 16 <= a_extent, "decode: activation load at [%lld, +16) of %lld", (long long)o,
+                            (long long)a_extent);
+              const int64_t base = (k0 + kb * 128) * 2;
+              CHECK_OR_FAIL(o - base >= 0 && o - base < ((int64_t)1 << 32), "decode: activation offset does not fit 32 bits");
+              cell[i * 64 + lane] = o;
+            }
+          for (int lane = 0; lane < 64; ++lane)
+            for (int j = 0; j < 4; ++j) {
+              const uint32_t off = addr::dec_a_frag(lane, j);
+              CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= 4096, "decode: activation operand read at %u", off);
+              int64_t m = m_t * 16 + (lane & 15);
+              m = m < M ? m : M - 1;
+              const int64_t k = k0 + kb * 128 + 32 * (lane >> 4) + 8 * j;  // the eight values that word 4 q + j of the weights holds
+              CHECK_OR_FAIL(cell[off / 16] == (m * K + k) * 2, "decode: activation operand of lane %d, k-step %d holds other values", lane, j);
+              if (m_t == 0 && (lane & 15) == 0) k_seen[k / 8] = 1;
+            }
+        }
+      for (int64_t t = 0; t < tiles; ++t) {
+        const int64_t base = addr::dec_w_base(t, K, k0);
+        for (int lane = 0; lane < 64; ++lane) {
+          // the kernel keeps the lane parts of tile 0 and of the last tile only
+          const uint32_t wl = t == tiles - 1 ? addr::dec_w_lane(lane, t, N, K) : addr::dec_w_lane(lane, 0, 16, K);
+          int64_t n = t * 16 + addr::sw_row(lane);
+          n = n < N ? n : N - 1;
+          for (int kb = 0; kb < 2; ++kb) {
+            const int64_t o = base + wl + kb * 64;
+            CHECK_OR_FAIL(o >= 0 && o % 16 == 0 && o + 16 <= w_extent, "decode: weight load at [%lld, +16) of %lld", (long long)o, (long long)w_extent);
+            CHECK_OR_FAIL(o == n * (K / 2) + (k0 + kb * 128) / 2 + addr::sw_piece(lane) * 16, "decode: weight load of lane %d reads another row or piece", lane);
+          }
+          if (lane < 16 * nd) {
+            const int64_t e = t == tiles - 1 ? addr::dec_sc_elem(lane, t, N, groups, k0, gshift)
+                                             : addr::dec_sc_elem(lane, 0, 16, groups, k0, gshift) + t * 16 * groups;
+            const int64_t d = addr::dec_sc_off(e);
+            CHECK_OR_FAIL(e >= 0 && d % 4 == 0 && d + 4 <= sc_extent, "decode: scale gather at [%lld, +4) of %lld", (long long)d, (long long)sc_extent);
+            CHECK_OR_FAIL(e == addr::dec_sc_elem(lane, t, N, groups, k0, gshift), "decode: scale gather of lane %d in tile %lld", lane, (long long)t);
+          }
+        }
+        // every lane finds the scale of its row and group: cell c of the area was written by gather lane c
+        for (int lane = 0; lane < 64; ++lane)
+          for (int kb = 0; kb < 2; ++kb) {
+            const uint32_t cell = addr::dec_sc_cell(lane, kb, gshift);
+            CHECK_OR_FAIL(cell % 4 == 0 && cell / 4 < (uint32_t)(16 * nd), "decode: scale read at %u outside the gathered cells", cell);
+            const int src = (int)(cell / 4);
+            const int64_t e = addr::dec_sc_elem(src, t, N, groups, k0, gshift);
+            const int64_t value = (addr::dec_sc_off(e) >> 1) + (addr::dec_sc_half(lane, kb, groups, k0, gshift) >> 4);
+            int64_t n = t * 16 + (lane & 15);
+            const bool real_row = n < N;
+            n = real_row ? n : N - 1;
+            const int64_t want = n * groups + (k0 + kb * 128 + 32 * (lane >> 4)) / group;
+            // rows past N are never stored: only their reads have to stay inside the area
+            CHECK_OR_FAIL(!real_row || value == want, "decode: lane %d reads scale %lld instead of %lld (tile %lld, k-block %d)", lane,
+                          (long long)value, (long long)want, (long long)t, kb);
+          }
+      }
+    }
+  for (int64_t c = 0; c < K / 8; ++c) CHECK_OR_FAIL(k_seen[c], "decode: values %lld .. of K are never multiplied", (long long)(c * 8));
+  return 0;
+}
+
+// The ring of the decode kernel: the ts-th tile of a wavefront lives in slot ts % 3; tiles 0 and 1 are issued up front
+// (slot 2 is scratch meanwhile); iteration ts issues tile ts + 2, then waits, before each k-block, until at most
+// dec_wait_count loads are in flight.  A tile's loads, in issue order: scale gather, zero gather, piece 0, piece 1.
+int check_decode_ring(int my_tiles) {
+  CHECK_OR_FAIL(my_tiles >= 1, "decode ring: bad arguments");
+  const int TS = addr::kDecTileSlots;
+  std::vector<int> slot(TS, -1);
+  std::vector<std::pair<int, int>> queue;  // (tile, load 0 .. 3), oldest first
+  std::vector<char> read(my_tiles, 0);
+  auto issue = [&](int ts) {
+    for (int l = 0; l < 4; ++l) queue.push_back({ts, l});
+    slot[ts % TS] = ts;
+  };
+  issue(0);
+  if (my_tiles > 1) issue(1);
+  CHECK_OR_FAIL(slot[2] < 0, "decode ring: the scratch slot is in use during the prologue");
+  for (int ts = 0; ts < my_tiles; ++ts) {
+    if (ts + 2 < my_tiles) {
+      const int sl = (ts + 2) % TS;
+      CHECK_OR_FAIL(slot[sl] < 0 || read[slot[sl]], "decode ring: tile %d overwrites tile %d before it was read", ts + 2, slot[sl]);
+      issue(ts + 2);
+    }
+    for (int kb = 0; kb < 2; ++kb) {
+      const int allowed = addr::dec_wait_count(ts, kb, my_tiles);
+      CHECK_OR_FAIL(allowed == 0 || allowed == 1 || allowed == 4 || allowed == 5 || allowed == 8 || allowed == 9,
+                    "decode ring: wait count %d has no s_waitcnt case", allowed);
+      while ((int)queue.size() > allowed) queue.erase(queue.begin());
+      for (auto& e : queue)
+        CHECK_OR_FAIL(!(e.first == ts && (e.second <= 2 || kb == 1)),  // k-block 0 needs the gathers and piece 0, k-block 1 all four
+                      "decode ring: k-block %d of tile %d read while load %d of it may be in flight", kb, ts, e.second);
+    }
+    CHECK_OR_FAIL(slot[ts % TS] == ts, "decode ring: the slot of tile %d holds tile %d", ts, slot[ts % TS]);
+    read[ts] = 1;
+  }
+  CHECK_OR_FAIL(queue.empty(), "decode ring: loads in flight at the end");
+  return 0;
+}
+
 }  // namespace
 }  // namespace tlq
 
@@ -307,6 +449,14 @@ int tlq_debug_check_stream_addressing(int64_t M, int64_t N, int64_t K, int activ
   if (int rc = check_stream(M, N, K, activation_tiles)) return rc;
   for (int steps = 1; steps <= 40; ++steps)
     if (int rc = check_stream_ring(steps, ring_depth)) return rc;
+  return 0;
+}
+
+int tlq_debug_check_decode_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int activation_tiles, int chunks, int waves,
+                                      int grid_x) {
+  if (int rc = check_decode(M, N, K, group, activation_tiles, chunks, waves, grid_x)) return rc;
+  for (int my_tiles = 1; my_tiles <= 16; ++my_tiles)
+    if (int rc = check_decode_ring(my_tiles)) return rc;
   return 0;
 }
 

@@ -32,6 +32,16 @@ int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const v
 int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
                   hipStream_t st);
 
+struct DecodePlan {
+  bool ok;
+  int mt, chunks, waves, grid_x;
+  int64_t lds_bytes;
+};
+DecodePlan w4a16_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus);
+int gemm_w4a16_decode(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N, int64_t K,
+                      int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const DecodePlan& p, float* partial,
+                      hipStream_t st);
+
 int g_gemm_band_rows = 0;
 int g_gemm_slots = 1;
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
@@ -41,6 +51,7 @@ static int cu_count_or_default() {
   return n > 0 ? n : 256;
 }
 int g_w4a16_stream = 1;  // 0: never pick the streaming kernel automatically (tuning runs)
+int g_w4a16_decode = 1;  // 0: never pick the decode kernel automatically
 // the tile loaders address one matrix with 32-bit byte offsets
 static bool fits32(int64_t rows, int64_t row_bytes) { return rows * row_bytes < ((int64_t)1 << 32); }
 static const int64_t kMaxDim = (int64_t)1 << 30;
@@ -57,6 +68,16 @@ extern "C" {
 void tlq_tune_gemm_band(int tile_rows) { tlq::g_gemm_band_rows = tile_rows < 0 ? 0 : tile_rows; }
 void tlq_tune_gemm_slots(int on) { tlq::g_gemm_slots = on != 0; }
 void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
+void tlq_tune_w4a16_decode(int on) { tlq::g_w4a16_decode = on != 0; }
+
+int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
+  const DecodePlan p = w4a16_decode_plan(M, N, K, group, cus);
+  if (plan_out) {
+    int64_t* o = (int64_t*)plan_out;
+    o[0] = p.mt, o[1] = p.chunks, o[2] = p.waves, o[3] = p.grid_x, o[4] = p.lds_bytes;
+  }
+  return p.ok ? 1 : 0;
+}
 
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
@@ -66,7 +87,7 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
               in_dtype);
   TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32,
               "tlq_gemm_w4a16: out_dtype must be float16, bfloat16 or float32 (got %d)", out_dtype);
-  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_SKINNY, "tlq_gemm_w4a16: bad algo %d", algo);
+  TLQ_REQUIRE((algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_SKINNY) || algo == TLQ_ALGO_DECODE, "tlq_gemm_w4a16: bad algo %d", algo);
   if (M == 0 || N == 0) return 0;
   TLQ_REQUIRE(K > 0 && K % 64 == 0, "tlq_gemm_w4a16: K=%lld must be a positive multiple of 64", (long long)K);
   TLQ_REQUIRE(group > 0 && K % group == 0 && group % 32 == 0,
@@ -75,11 +96,23 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
   TLQ_REQUIRE(aligned16(A) && aligned16(w_packed) && aligned16(C), "tlq_gemm_w4a16: A, w_packed and C must be 16-byte aligned");
   TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16: scales / zeros misaligned");
   hipStream_t st = (hipStream_t)stream;
+  // The decode kernel (M <= 32): without a workspace only rows of up to 4096 values (one chunk of K).  Its scale / zero
+  // gathers read aligned dwords: the tensors must start on a dword boundary (their length is checked by the plan).
+  const DecodePlan dp = M <= 32 ? w4a16_decode_plan(M, N, K, group, cu_count_or_default()) : DecodePlan{false, 0, 0, 0, 0, 0};
+  const bool decode_ok = dp.ok && dp.chunks == 1 && (((uintptr_t)scales | (uintptr_t)zeros) & 3) == 0;
+  if (algo == TLQ_ALGO_DECODE) {
+    TLQ_REQUIRE(decode_ok, "tlq_gemm_w4a16: the decode kernel needs 1 <= M <= 32, K %% 256 == 0, K <= 4096 without a workspace, a power-of-two "
+                "group and dword-aligned scale / zero tensors (M=%lld N=%lld K=%lld group=%lld)", (long long)M, (long long)N, (long long)K,
+                (long long)group);
+    return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, dp, nullptr, st);
+  }
   if (algo == TLQ_ALGO_AUTO) {
     // The skinny kernel takes the same time for every M up to 16 (the weights bound it); the GEMV kernels grow with
     // M.  Measured crossovers: fp16 GEMV wins at M = 1, and at M = 2 while K <= 4096; the bf16 GEMV dequantises
     // element by element and wins only at M = 1 in its register-resident form, for rows of up to 8192 values.
     const bool skinny_ok = M <= 64 && K % 128 == 0 && fits32(M, K * 2) && fits32(N, K / 2);
+    if (M > 2 && decode_ok && g_w4a16_decode)
+      return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, dp, nullptr, st);
     if (M > 4)
       algo = skinny_ok ? TLQ_ALGO_SKINNY : TLQ_ALGO_MFMA;
     else if (!skinny_ok)
@@ -126,6 +159,10 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   int64_t split = w4a16_mid_split(M, N, K, 32);
   const int64_t ssplit = stream_max_split(M, N, K);
   if (ssplit > split) split = ssplit;
+  if (M <= 32) {  // the decode kernel cuts rows longer than 4096 values into chunks
+    const DecodePlan dp = w4a16_decode_plan(M, N, K, 32, 256);
+    if (dp.ok && dp.chunks > split) split = dp.chunks;
+  }
   if (split > 1) return split * M * N * 4;
   return M >= kTwoPassMinM ? N * K * 2 : 0;
 }
@@ -133,7 +170,29 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
-  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_STREAM, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_DECODE, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  // decode batches: rows longer than 4096 values run as chunks of K whose fp32 partial sums live in the workspace
+  if (((algo == TLQ_ALGO_AUTO && g_w4a16_decode && M > 2) || algo == TLQ_ALGO_DECODE) && M <= 32 && M >= 1 && N >= 1 && K > 0 && group > 0 &&
+      N < kMaxDim && K < kMaxDim) {
+    const DecodePlan dp = w4a16_decode_plan(M, N, K, group, cu_count_or_default());
+    const bool args_ok = A && w_packed && C && aligned16(A) && aligned16(w_packed) && aligned16(C) &&
+                         (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) &&
+                         (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) &&
+                         (((uintptr_t)scales | (uintptr_t)zeros) & 3) == 0;
+    // measured on rows of 14336 values: with up to 16 activation rows the skinny kernel is level or ahead (no second
+    // launch for the partial sums), from 17 rows on the decode kernel is 10 - 15 % ahead of the streaming kernel
+    if (dp.ok && dp.chunks > 1 && (algo == TLQ_ALGO_DECODE || M > 16) && args_ok && (M * N) % 4 == 0 && workspace && aligned16(workspace) &&
+        workspace_bytes >= (int64_t)dp.chunks * M * N * 4)
+      return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, dp,
+                               (float*)workspace, (hipStream_t)stream);
+    if (algo == TLQ_ALGO_DECODE && !(dp.ok && dp.chunks == 1)) {
+      set_error("tlq_gemm_w4a16_ws: the decode kernel needs 1 <= M <= 32, K %% 256 == 0, a power-of-two group, dword-aligned scale / zero "
+                "tensors, M * N %% 4 == 0 and a workspace of %lld bytes (M=%lld N=%lld K=%lld group=%lld, workspace %lld)",
+                (long long)(dp.ok ? (int64_t)dp.chunks * M * N * 4 : 0), (long long)M, (long long)N, (long long)K, (long long)group,
+                (long long)workspace_bytes);
+      return 1;
+    }
+  }
   const int64_t need = (N > 0 && K > 0) ? N * K * 2 : 0;
   const bool have = workspace != nullptr && workspace_bytes >= need && aligned16(workspace);
   if (algo == TLQ_ALGO_TWO_PASS)

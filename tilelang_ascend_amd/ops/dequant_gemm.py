@@ -27,7 +27,7 @@ _PASS_CONFIGS = {
 }
 _SIGN_MODES = {"unsigned": _abi.U4, "twos": _abi.S4_TWOS, "offset8": _abi.S4_OFFSET8, "offset7": _abi.S4_OFFSET7}
 _ALGOS = {"auto": _abi.ALGO_AUTO, "gemv": _abi.ALGO_GEMV, "mfma": _abi.ALGO_MFMA, "skinny": _abi.ALGO_SKINNY,
-          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM}
+          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM, "decode": _abi.ALGO_DECODE}
 # arrangement of the 4-bit fields in each 32-bit word: general_compress order, or interleave_weight(target float16)
 _LAYOUTS = {"plain": _abi.W_PLAIN, "interleaved": _abi.W_INTERLEAVED_F16}
 
@@ -162,7 +162,8 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
     A [M,K] in_dtype; B_packed uint8 [N,K/2]; scales [N,K/group_size] in_dtype when with_scales;
     zeros: None (no zero point), a number (one zero point for the whole matrix) or "tensor"
     (a [N,K/group_size] in_dtype input follows).  C [M,N] out_dtype, fp32 accumulate.
-    algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "skinny" (M <= 64) | "mfma" (LDS-staged MFMA kernel)
+    algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "decode" (M <= 32, K % 256 == 0: persistent work-groups with the
+    activations in registers: what "auto" does for 3 <= M <= 16) | "skinny" (M <= 64) | "mfma" (LDS-staged MFMA kernel)
     | "stream" (wavefront-private packed weights dequantised in registers, 17 <= M <= 512: what "auto" does up to
     M = 256) | "two_pass" (dequantise into a workspace, then the plain GEMM: what "auto" does above).  A workspace
     (split-K partial sums or the [N, K] dequantised weights) is taken from torch's stream-ordered allocator on every
@@ -210,7 +211,7 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
         lib = _abi.load()
         ws = None
         ws_bytes = 0
-        if algo in ("auto", "two_pass", "stream"):
+        if algo in ("auto", "two_pass", "stream", "decode"):
             ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
             if algo == "two_pass" or (layout_code != _abi.W_PLAIN and algo == "auto" and M > 256):
                 ws_bytes = max(ws_bytes, N * K * 2)
