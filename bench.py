@@ -337,8 +337,8 @@ def bench_skinny(args, steps=None, cpu=True):
     tm = timed(step, steps or args.steps, args.warmup)
     out = {"workload": f"W4A16 decode batch M=16 N=14336 K=4096 group=128 fp16 scales+zeros, {sets} weight sets rotating",
            "dtype": "f16", "value": round(unit_bytes / tm.wall / 1e9, 1), "unit": "GB/s", "ms_per_step": tm.wall * 1e3,
-           "roofline": dict({"kernel": "w4a16_skinny_lds_kernel", "bound": "hbm"}, **tm.roofline(unit_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
-                            traffic=traffic_from_profile("skinny_w4a16_f16_M16_N14336_K4096_g128.txt"), bytes_per_launch=unit_bytes)}
+           "roofline": dict({"kernel": "w4a16_decode_kernel<f16,1>", "bound": "hbm"}, **tm.roofline(unit_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
+                            traffic=traffic_from_profile("decode_w4a16_f16_M16_N14336_K4096_g128.txt"), bytes_per_launch=unit_bytes)}
     if cpu:
         from oracle import ref
 
