@@ -403,7 +403,7 @@ int check_decode_ring(int my_tiles) {
   };
   issue(0);
   if (my_tiles > 1) issue(1);
-  CHECK_OR_FAIL(slot[2] < 0, "decode ring: the scratch slot is in use during the prologue");
+  CHECK_OR_FAIL(slot[2] < 0, "decode ring: the slot that stages the activations is in use during the prologue");
   for (int ts = 0; ts < my_tiles; ++ts) {
     if (ts + 2 < my_tiles) {
       const int sl = (ts + 2) % TS;

@@ -118,46 +118,52 @@ __global__ __launch_bounds__(1024) void w4a16_decode_kernel(const T* __restrict_
   };
 
   // ---- activations of this wavefront's K slice -> MFMA operands in registers ----
-  // Direct loads of 1 KB into the wavefront's own LDS (ring and partial-sum area, both idle yet), 8 KB at a time: they
-  // move twice as many bytes per clock as loads into registers, and every work-group has to pull all of A through its CU.
+  // Direct loads of 1 KB into the wavefront's own LDS, one [16 rows][256 B] block (4 KB) at a time, staged in the third
+  // ring slot plus the partial-sum area (both idle yet): direct loads move twice as many bytes per clock as loads into
+  // registers, and every work-group has to pull all of A through its CU.  The first two tiles of weights are requested
+  // right behind the first block, so that HBM is busy while the activations (L2 hits) are rearranged.
   uint4_t af[2][4][MT];
   if (active) {
-    static_assert(8192 <= WAVE, "staging area of the activations");
-    constexpr int ROUNDS = MT;  // 8 KB = two [16 rows][256 B] blocks per round
+    constexpr uint32_t STG = 2 * SLOT;
+    static_assert(STG + 4096 <= WAVE, "staging area of the activations");
+    auto issue_block = [&](int kb, int mt) {
+      const uint8_t* asb = uniform_ptr((const uint8_t*)A + (k0 + kb * 128) * 2);
 #pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int kb = MT == 1 ? b : r, mt = MT == 1 ? 0 : b;
-        const uint8_t* asb = uniform_ptr((const uint8_t*)A + (k0 + kb * 128) * 2);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t voff = (uint32_t)(addr::dec_a_off(lane, mt, kb, i, M, K, k0) - (k0 + kb * 128) * 2);
-          asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(mine_lds + (uint32_t)(b * 4096 + i * 1024)), "v"(voff), "s"(asb)
-                       : "memory");
-        }
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t voff = (uint32_t)(addr::dec_a_off(lane, mt, kb, i, M, K, k0) - (k0 + kb * 128) * 2);
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(mine_lds + STG + (uint32_t)(i * 1024)), "v"(voff), "s"(asb)
+                     : "memory");
       }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int kb = MT == 1 ? b : r, mt = MT == 1 ? 0 : b;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint4_t v = *(const uint4_t*)(mine + b * 4096 + addr::dec_a_frag(lane, j));
-          if (LAYOUT == 0) {
-            // plain words are decoded without the byte permutes that would restore k order, i.e. as values
-            // k0, k4, k1, k5, k2, k6, k3, k7 of the word: the activations take the same order, once, here
-            af[kb][j][mt] = uint4_t{__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
-                                    __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u)};
-          } else {
-            af[kb][j][mt] = v;
-          }
-        }
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the area is free again: next round, or the ring
-    }
+    };
+    issue_block(0, 0);
     issue_tile(0);
     if (my_tiles > 1) issue_tile(1);
+#pragma unroll
+    for (int b = 0; b < 2 * MT; ++b) {
+      const int kb = b / MT, mt = b % MT;
+      // loads return in issue order: the first block is followed by at most two tiles (eight loads), every later block
+      // is the youngest load there is
+      if (b == 0) {
+        if (my_tiles > 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint4_t v = *(const uint4_t*)(mine + STG + addr::dec_a_frag(lane, j));
+        if (LAYOUT == 0) {
+          // plain words are decoded without the byte permutes that would restore k order, i.e. as values
+          // k0, k4, k1, k5, k2, k6, k3, k7 of the word: the activations take the same order, once, here
+          af[kb][j][mt] = uint4_t{__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                                  __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u)};
+        } else {
+          af[kb][j][mt] = v;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging area is free again: next block, or the third tile
+      if (b + 1 < 2 * MT) issue_block((b + 1) / MT, (b + 1) % MT);
+    }
+    if (my_tiles > 2) issue_tile(2);
   }
 
   typename Mma::acc_t acc[MT];
@@ -167,38 +173,59 @@ __global__ __launch_bounds__(1024) void w4a16_decode_kernel(const T* __restrict_
   for (int ts = 0; ts < my_tiles; ++ts) {
     const int t = first + ts * stride;
     if (active) {
-      if (ts + 2 < my_tiles) issue_tile(ts + 2);  // into the slot that tile ts - 1 was read from
+      if (ts > 0 && ts + 2 < my_tiles) issue_tile(ts + 2);  // into the slot that tile ts - 1 was read from (tile 2: issued above)
       const uint8_t* const slotp = mine + (ts % TS) * SLOT;
+      // one wait and one round of LDS reads per tile: both k-blocks, their scales and zero points
+      wait_vm(addr::dec_wait_count(ts, 1, my_tiles));
+      uint4_t wf[2];
+      uint32_t sdw[2], zdw[2];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
-        wait_vm(addr::dec_wait_count(ts, kb, my_tiles));
-        const uint4_t wf = *(const uint4_t*)(slotp + kb * 1024 + fo_w);
-        const uint32_t sdw = *(const uint32_t*)(slotp + 2048 + rd_cell[kb]);
-        const uint32_t zdw = *(const uint32_t*)(slotp + 2304 + rd_cell[kb]);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const T sv = has_s ? bitcast<T>((uint16_t)(sdw >> rd_half[kb])) : one;
-        const T zv = has_z ? bitcast<T>((uint16_t)(zdw >> rd_half[kb])) : zs;
-        const float zf = to_float(zv);
-        const bool ok = zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
-        const uint32_t w[4] = {wf.x, wf.y, wf.z, wf.w};
-        if (__builtin_amdgcn_ballot_w64(ok) == ~0ull) {  // integer zero points fold into the unpack bias (exact)
-          const Expand8<T, true, 1> ex(sv, zv, mg);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const uint4_t b = ex(w[j]);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[mt] = Mma::mma(b, af[kb][j][mt], acc[mt]);
-          }
-        } else {
-          const Expand8<T, false, 1> ex(sv, zv, mg);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const uint4_t b = ex(w[j]);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[mt] = Mma::mma(b, af[kb][j][mt], acc[mt]);
-          }
-        }
+        wf[kb] = *(const uint4_t*)(slotp + kb * 1024 + fo_w);
+        sdw[kb] = *(const uint32_t*)(slotp + 2048 + rd_cell[kb]);
+        zdw[kb] = *(const uint32_t*)(slotp + 2304 + rd_cell[kb]);
       }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      T sv[2], zv[2];
+      bool ok = true;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        sv[kb] = has_s ? bitcast<T>((uint16_t)(sdw[kb] >> rd_half[kb])) : one;
+        zv[kb] = has_z ? bitcast<T>((uint16_t)(zdw[kb] >> rd_half[kb])) : zs;
+        const float zf = to_float(zv[kb]);
+        ok = ok && zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
+      }
+      // the two k-blocks accumulate separately (two independent MFMA chains), added when the tile is handed over
+      typename Mma::acc_t acc2[2][MT];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc2[kb][mt] = typename Mma::acc_t{0, 0, 0, 0};
+      if (__builtin_amdgcn_ballot_w64(ok) == ~0ull) {  // integer zero points fold into the unpack bias (exact)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb) {
+            const Expand8<T, true, 1> ex(sv[kb], zv[kb], mg);
+            const uint32_t w[4] = {wf[kb].x, wf[kb].y, wf[kb].z, wf[kb].w};
+            const uint4_t b = ex(w[j]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc2[kb][mt] = Mma::mma(b, af[kb][j][mt], acc2[kb][mt]);
+          }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb) {
+            const Expand8<T, false, 1> ex(sv[kb], zv[kb], mg);
+            const uint32_t w[4] = {wf[kb].x, wf[kb].y, wf[kb].z, wf[kb].w};
+            const uint4_t b = ex(w[j]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc2[kb][mt] = Mma::mma(b, af[kb][j][mt], acc2[kb][mt]);
+          }
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = acc2[0][mt] + acc2[1][mt];
     }
     if (RB == 1 && ts > 0) __syncthreads();  // the single buffer: the wavefronts that added up tile ts - 1 have read it
     if (active) {
@@ -206,7 +233,6 @@ __global__ __launch_bounds__(1024) void w4a16_decode_kernel(const T* __restrict_
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         *(float4_t*)(mine + RED + ((ts % RB) * MT + mt) * 1024 + lane * 16) = acc[mt];
-        acc[mt] = typename Mma::acc_t{0, 0, 0, 0};
       }
     }
     __syncthreads();  // all partial tiles of tile t are in LDS (two buffers: the other one was read before the previous barrier)
