@@ -286,7 +286,8 @@ int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cu
  * -1 for bad arguments.  No counterpart in the reference. */
 int tlq_debug_gemv_rows_plan(int64_t batch, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
 
-/* Tuning hooks for benchmark sweeps (process-global, not thread safe; 0 = automatic choice).
+/* Tuning hooks for benchmark sweeps and the autotuner (each sets a value of the CALLING THREAD, read by that thread's
+ * later launches; other threads keep the automatic choice; 0 = automatic choice).
  * They play the role of the reference's block_M / block_N / block_K factory arguments
  * (example_dequant_gemm_fine_grained.py:437,462), which here select among pre-built tilings. */
 void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4 (negative: never the register-resident

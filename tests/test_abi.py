@@ -190,3 +190,29 @@ def test_workspace_size_rules():
         assert 2 <= split <= 16, (M, N, K, split)  # room for the most K slices any kernel and group size may cut
     assert ws(1024, 14336, 4096) == 14336 * 4096 * 2  # many output tiles already: no K slices, two passes
     assert ws(64, 0, 4096) == 0 and ws(64, 128, 0) == 0
+
+
+def test_tuning_hooks_are_per_thread():
+    """A value set through a tlq_tune_* hook belongs to the calling thread: launches prepared on another thread keep the
+    automatic choice.  Observed through the workspace rule, which follows the number of K slices that
+    tlq_tune_w4a16_split forces."""
+    import threading
+
+    from tilelang_ascend_amd import _abi
+
+    lib = _abi.load()
+    M, N, K = 600, 4096, 4096
+    auto = lib.tlq_w4a16_workspace_bytes(M, N, K)
+    assert auto == 4 * M * N * 4
+    lib.tlq_tune_w4a16_split(16)
+    try:
+        here = lib.tlq_w4a16_workspace_bytes(M, N, K)
+        seen = []
+        t = threading.Thread(target=lambda: seen.append(lib.tlq_w4a16_workspace_bytes(M, N, K)))
+        t.start()
+        t.join()
+    finally:
+        lib.tlq_tune_w4a16_split(0)
+    assert here == 16 * M * N * 4, "the override is not seen on the thread that set it"
+    assert seen == [auto], "another thread saw this thread's override"
+    assert lib.tlq_w4a16_workspace_bytes(M, N, K) == auto

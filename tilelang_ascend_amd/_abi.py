@@ -135,8 +135,9 @@ _tuning_lock = threading.RLock()
 @contextlib.contextmanager
 def tuning(w4a16_tile: int = 0, i8_tile: int = 0, gemv: tuple = None, skinny: tuple = None):
     """Applies tiling choices to the launches made inside the block, then restores the automatic
-    choice.  The hooks are process-global and only read on the host while a launch is being set up
-    (asynchronous execution is not affected), so holding this lock around the call is enough."""
+    choice.  The hooks set thread-local values that are only read on the host while a launch is being set up
+    (asynchronous execution is not affected): another thread that launches at the same time keeps the automatic
+    choice.  The lock only keeps nested uses on one thread orderly."""
     lib = load()
     active = bool(w4a16_tile or i8_tile or gemv or skinny)
     if not active:

@@ -42,16 +42,16 @@ int gemm_w4a16_decode(const void* A, const void* Wp, const void* scales, const v
                       int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const DecodePlan& p, float* partial,
                       hipStream_t st);
 
-int g_gemm_band_rows = 0;
-int g_gemm_slots = 1;
+thread_local int g_gemm_band_rows = 0;
+thread_local int g_gemm_slots = 1;
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // compute units of the current device (256 when it cannot be asked, e.g. without a GPU)
 static int cu_count_or_default() {
   const int n = tlq_device_cu_count();
   return n > 0 ? n : 256;
 }
-int g_w4a16_stream = 1;  // 0: never pick the streaming kernel automatically (tuning runs)
-int g_w4a16_decode = 1;  // 0: never pick the decode kernel automatically
+thread_local int g_w4a16_stream = 1;  // 0: never pick the streaming kernel automatically (tuning runs)
+thread_local int g_w4a16_decode = 1;  // 0: never pick the decode kernel automatically
 // the tile loaders address one matrix with 32-bit byte offsets
 static bool fits32(int64_t rows, int64_t row_bytes) { return rows * row_bytes < ((int64_t)1 << 32); }
 static const int64_t kMaxDim = (int64_t)1 << 30;

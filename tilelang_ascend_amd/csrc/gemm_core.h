@@ -738,7 +738,7 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
 // Host-side launcher: sets the dynamic LDS size and launches one work-group per tile.
 // tile rows per band of the work-group -> tile order, for tuning runs (0 = each launcher's own choice: measured best
 // were 2 for the int8 kernels, 4 for the plain 16-bit GEMM and 8 for the fused W4A16 kernel; 1 = plain row-major)
-extern int g_gemm_band_rows;
+extern thread_local int g_gemm_band_rows;
 
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,

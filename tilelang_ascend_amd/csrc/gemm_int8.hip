@@ -108,7 +108,7 @@ static int run_i8(const void* A, const typename WL::Params& pw, const typename E
   return launch_gemm<MmaI8, AL, WL, Epi, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K, st, what, 2);
 }
 
-static int g_i8_tile = 0;
+static thread_local int g_i8_tile = 0;
 
 static int pick_tile(int64_t batch, int64_t M, int64_t N) {
   if (g_i8_tile) return g_i8_tile;

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDi
 }
 
 // tlq_tune_gemm_slots: 0 = the two-stage kernel (default), 1 = this one where it applies
-extern int g_gemm_slots;
+extern thread_local int g_gemm_slots;
 
 // k_bytes (bytes of K per activation row) a positive multiple of 128: whole stages only.
 template <class Mma, class WL, class Epi>

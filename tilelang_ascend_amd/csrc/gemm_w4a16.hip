@@ -186,7 +186,7 @@ static int run_w4a16(const W4Args& a) {
 }
 
 // tile override for tuning runs (0 = automatic)
-static int g_w4a16_tile = 0;
+static thread_local int g_w4a16_tile = 0;
 
 template <typename T, bool FOLD>
 static int dispatch_w4a16(const W4Args& a) {
@@ -589,7 +589,7 @@ __global__ __launch_bounds__(1024) void w4a16_skinny_lds_kernel(const T* __restr
   }
 }
 
-static int g_skinny_waves = 0, g_skinny_rt = 0;  // tuning overrides (0 = automatic)
+static thread_local int g_skinny_waves = 0, g_skinny_rt = 0;  // tuning overrides (0 = automatic)
 
 template <typename T, bool FOLD, int RT, int MT>
 static int launch_skinny(const W4Args& a, int waves) {
@@ -621,7 +621,7 @@ static int launch_skinny_lds(const W4Args& a, int waves, int gshift) {
   return check_launch("tlq_gemm_w4a16(skinny)") ? 0 : 1;
 }
 
-static int g_skinny_lds = -1;  // tuning override: 0 = never, 1 = whenever possible, -1 = automatic
+static thread_local int g_skinny_lds = -1;  // tuning override: 0 = never, 1 = whenever possible, -1 = automatic
 
 template <typename T, bool FOLD>
 static int dispatch_skinny(const W4Args& a) {
@@ -705,7 +705,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4_t* __re
 // K slices for the tile kernel at small M, where the output tiles alone leave most of the chip idle and a
 // work-group's run of stages is latency bound: aim at one to two work-groups per CU (measured best on the
 // MLP shapes), slices of at least 512 values that are whole stages and whole quantisation groups.  1 = no split.
-static int g_w4a16_split = 0;  // forced number of K slices for tuning runs (0 = automatic)
+static thread_local int g_w4a16_split = 0;  // forced number of K slices for tuning runs (0 = automatic)
 
 int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group) {
   // Where cutting K pays (measured against the two passes on the MLP shapes): up to M = 512 always, up to

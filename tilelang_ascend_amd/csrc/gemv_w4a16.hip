@@ -675,7 +675,7 @@ static void launch_gemv(const void* A, const void* Wp, const void* scales, const
 }
 
 // rows-per-wave / waves-per-block / blocks-per-CU overrides for tuning runs (0 = automatic)
-static int g_gemv_rows = 0, g_gemv_waves = 0, g_gemv_waves16 = 0, g_gemv_unroll = 0, g_gemv_depth = 0;
+static thread_local int g_gemv_rows = 0, g_gemv_waves = 0, g_gemv_waves16 = 0, g_gemv_unroll = 0, g_gemv_depth = 0;
 
 static int cu_count() {
   static int n = 0;
