@@ -53,14 +53,15 @@ struct StreamCfg {
   static constexpr int A_TILE = TM * 16 * 256;                // bytes of activations per step
   static constexpr int W_TILE = 8 * 2 * 1024;                 // packed weights per step: 8 wavefronts x 2 tiles x 1 KB
   static constexpr int SLOT = A_TILE + W_TILE;
-  static constexpr int SZ_WAVE = 2048;                        // scales [2][16][16] + zero points [2][16][16], 2 bytes each
+  static constexpr int SZ_WAVE = 2048;                        // scales [32 rows][16 groups] + zero points [32 rows][16 groups], 2 bytes each
   static constexpr int LDS = D * SLOT + 8 * SZ_WAVE;
   static constexpr int LA = TM / 2;                           // activation load instructions per wavefront and step (4 TM / 8)
   static constexpr int L = LA + 2;                            // load instructions per wavefront and step
   static_assert(LDS * PER_CU <= 160 * 1024, "rings do not fit the CU's LDS");
   static_assert((D - 2) * L <= 63, "vmcnt range");
 };
-constexpr int kStreamMaxGroups = 16;  // quantisation groups per K slice whose scales fit the private LDS area
+constexpr int kStreamMaxGroups = 16;
+static_assert(kStreamMaxGroups * 2 == 32, "a row of the scale area is two 16-byte pieces");  // quantisation groups per K slice whose scales fit the private LDS area
 
 template <typename T, int TM, int LAYOUT>
 __global__ __launch_bounds__(512, 2) void w4a16_stream_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
@@ -112,49 +113,93 @@ __global__ __launch_bounds__(512, 2) void w4a16_stream_kernel(const T* __restric
     for (int tn = 0; tn < 2; ++tn) dma16(l0 + (uint32_t)(Cfg::A_TILE + wave * 2048 + tn * 1024), voff_w[tn], wsb);
   };
 
-  // ---- prime the ring, then fetch the scales / zero points of this wavefront's 32 rows for the slice ----
-  // (2-byte gathers over 16 rows keep the address unit busy for about a cycle per lane: only the groups the slice has
-  // are fetched, four per instruction, and behind the weight loads, whose trip to HBM they overlap)
-#pragma unroll
-  for (int s = 0; s < D - 1; ++s)
-    if (s < steps) issue(s, s);
-  __builtin_amdgcn_sched_barrier(0);
+  // ---- scales / zero points of this wavefront's 32 rows for the slice, and the first D - 1 steps ----
+  // Area of the wavefront: [s | z][32 rows][16 groups], 2 bytes each.  A row's groups of the slice are contiguous in
+  // memory (32 bytes): when they are 16-byte aligned and wholly inside the row, ONE direct load per tensor fetches all of
+  // them (lane l: row l / 2, half l % 2), issued ahead of the ring so that the first step's wait covers it.  Otherwise
+  // 2-byte gathers, four groups per instruction (they keep the address unit busy for about a cycle per lane, so they go
+  // behind the weight loads, whose trip to HBM they overlap).
   const bool has_s = scales != nullptr, has_z = zeros != nullptr;
   const T one = from_float<T>(1.0f), zs = from_float<T>(zero_scalar);
   const int G = (steps << 7) >> gshift;  // groups in this slice (>= 1: a slice is a whole number of groups)
   const int g0 = (step0 << 7) >> gshift;
-  T pre_s[2][kStreamMaxGroups / 4], pre_z[2][kStreamMaxGroups / 4];
-#pragma unroll
-  for (int tn = 0; tn < 2; ++tn) {
-    int n = n0 + wave * 32 + tn * 16 + r16;
-    n = n < N ? n : N - 1;
-#pragma unroll
-    for (int i = 0; i < kStreamMaxGroups / 4; ++i) {
-      pre_s[tn][i] = one;
-      pre_z[tn][i] = zs;
-      if (4 * i < G) {  // uniform
-        int g = q + 4 * i;
-        g = g < G ? g : G - 1;
-        const int64_t at = (int64_t)n * groups + g0 + g;
-        if (has_s) pre_s[tn][i] = scales[at];
-        if (has_z) pre_z[tn][i] = zeros[at];
-      }
-    }
-  }
-  uint8_t* const sz = smem + D * Cfg::SLOT + wave * Cfg::SZ_WAVE;  // [s | z][tn][g][r16]
+  uint8_t* const sz = smem + D * Cfg::SLOT + wave * Cfg::SZ_WAVE;
+  const bool wide = (groups & 7) == 0 && (g0 & 7) == 0 && g0 + kStreamMaxGroups <= groups &&
+                    (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0;  // uniform
   bool integral = true;
+  if (wide) {
+    int n = n0 + wave * 32 + (lane >> 1);
+    n = n < N ? n : N - 1;
+    const uint32_t voff = ((uint32_t)n * (uint32_t)groups + (uint32_t)g0) * 2u + (uint32_t)((lane & 1) * 16);
+    const uint32_t l0 = lds0 + (uint32_t)(D * Cfg::SLOT + wave * Cfg::SZ_WAVE);
+    if (has_s) asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0), "v"(voff), "s"(scales) : "memory");
+    if (has_z) asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0 + 1024u), "v"(voff), "s"(zeros) : "memory");
+  }
 #pragma unroll
-  for (int tn = 0; tn < 2; ++tn)
+  for (int s = 0; s < D - 1; ++s)
+    if (s < steps) issue(s, s);
+  __builtin_amdgcn_sched_barrier(0);
+  if (wide) {
+    // loads return in issue order: with the ring's loads still in flight the two above have landed
+    if (steps >= D - 1)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((D - 1) * Cfg::L) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (!has_s || !has_z) {  // an absent tensor is the constant 1 / the scalar zero point
+      const uint32_t ws = (uint32_t)bitcast<uint16_t>(one) * 0x10001u, wz = (uint32_t)bitcast<uint16_t>(zs) * 0x10001u;
+      const uint4_t cs{ws, ws, ws, ws}, cz{wz, wz, wz, wz};
+      if (!has_s) *(uint4_t*)(sz + lane * 16) = cs;
+      if (!has_z) *(uint4_t*)(sz + 1024 + lane * 16) = cz;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-    for (int i = 0; i < kStreamMaxGroups / 4; ++i) {
-      const int g = q + 4 * i;
-      const float zf = to_float(pre_z[tn][i]);
-      integral = integral && zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
-      if (g < kStreamMaxGroups) {
-        *(T*)(sz + ((tn * kStreamMaxGroups + g) * 16 + r16) * 2) = pre_s[tn][i];
-        *(T*)(sz + Cfg::SZ_WAVE / 2 + ((tn * kStreamMaxGroups + g) * 16 + r16) * 2) = pre_z[tn][i];
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint4_t v = *(const uint4_t*)(sz + 1024 + ((tn * 16 + r16) * 2 + h) * 16);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const float zf = to_float(bitcast<T>((uint16_t)(w[i] >> (16 * e))));
+            integral = integral && zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
+          }
+      }
+  } else {
+    T pre_s[2][kStreamMaxGroups / 4], pre_z[2][kStreamMaxGroups / 4];
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn) {
+      int n = n0 + wave * 32 + tn * 16 + r16;
+      n = n < N ? n : N - 1;
+#pragma unroll
+      for (int i = 0; i < kStreamMaxGroups / 4; ++i) {
+        pre_s[tn][i] = one;
+        pre_z[tn][i] = zs;
+        if (4 * i < G) {  // uniform
+          int g = q + 4 * i;
+          g = g < G ? g : G - 1;
+          const int64_t at = (int64_t)n * groups + g0 + g;
+          if (has_s) pre_s[tn][i] = scales[at];
+          if (has_z) pre_z[tn][i] = zeros[at];
+        }
       }
     }
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+      for (int i = 0; i < kStreamMaxGroups / 4; ++i) {
+        const int g = q + 4 * i;
+        const float zf = to_float(pre_z[tn][i]);
+        integral = integral && zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
+        if (g < kStreamMaxGroups) {
+          *(T*)(sz + ((tn * 16 + r16) * kStreamMaxGroups + g) * 2) = pre_s[tn][i];
+          *(T*)(sz + Cfg::SZ_WAVE / 2 + ((tn * 16 + r16) * kStreamMaxGroups + g) * 2) = pre_z[tn][i];
+        }
+      }
+  }
   // small integer zero points fold exactly into the unpack bias (a quarter of the conversion arithmetic less); decided
   // once per wavefront
   const bool fold = __builtin_amdgcn_ballot_w64(integral) == ~0ull;
@@ -190,8 +235,8 @@ __global__ __launch_bounds__(512, 2) void w4a16_stream_kernel(const T* __restric
     T sv[2], zv[2];
 #pragma unroll
     for (int tn = 0; tn < 2; ++tn) {
-      sv[tn] = *(const T*)(sz + ((tn * kStreamMaxGroups + gl) * 16 + r16) * 2);
-      zv[tn] = *(const T*)(sz + Cfg::SZ_WAVE / 2 + ((tn * kStreamMaxGroups + gl) * 16 + r16) * 2);
+      sv[tn] = *(const T*)(sz + ((tn * 16 + r16) * kStreamMaxGroups + gl) * 2);
+      zv[tn] = *(const T*)(sz + Cfg::SZ_WAVE / 2 + ((tn * 16 + r16) * kStreamMaxGroups + gl) * 2);
     }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm)
