@@ -1,6 +1,6 @@
 """Kernels that read weights repacked by interleave_weight for the float16 target (tilelang/quantize/utils.py:73-101; the
 layout the reference's fast decoders consume, tilelang/quantize/lop3.py:17-24): the dequantisation pass, the streaming
-W4A16 kernel and the two passes.  The repacking only moves 4-bit fields inside each 32-bit word, so every result must be
+W4A16 kernel, the decode kernel and the two passes.  The repacking only moves 4-bit fields inside each 32-bit word, so every result must be
 bit-identical to the plain layout on the same logical weights, and the dequantised matrix must equal the oracle's."""
 import numpy as np
 import pytest
@@ -119,14 +119,33 @@ def test_operator_with_interleaved_weights_packed_on_the_gpu():
     check_float_output(inter, w4a16_reference(A, Wp, s, z, group), "operator interleaved vs oracle")
 
 
-def test_interleaved_layout_rejects_decode_sized_problems_and_other_kernels():
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K,group,zeros_kind", [(1, 64, 256, 64, "int"), (16, 1000, 4096, 128, "frac"), (32, 520, 8192, 64, "int"), (7, 2048, 1024, 32, None)])
+def test_decode_kernel_on_interleaved_words(in_dtype, M, N, K, group, zeros_kind):
     from tilelang_ascend_amd import _abi
 
-    A = torch.zeros(16, 128, dtype=torch.float16)
+    dt = DT[in_dtype]
+    A = torch.randn(M, K, generator=gen(77)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=78)
+    rc, plain = run_layout(A, Wp, s, z, group, _abi.W_PLAIN, _abi.ALGO_DECODE)
+    assert rc == 0, _abi.last_error()
+    for algo in (_abi.ALGO_DECODE, _abi.ALGO_AUTO):
+        rc, inter = run_layout(A, interleaved(Wp), s, z, group, _abi.W_INTERLEAVED_F16, algo)
+        assert rc == 0, _abi.last_error()
+        assert_bit_equal(inter, plain, f"decode interleaved vs plain {in_dtype} {M}x{N}x{K} algo {algo}")
+    check_float_output(inter, w4a16_reference(A, Wp, s, z, group), "decode interleaved vs oracle")
+
+
+def test_interleaved_layout_rejects_what_no_kernel_reads():
+    from tilelang_ascend_amd import _abi
+
+    A = torch.zeros(16, 128, dtype=torch.float16)  # K = 128: not a shape of the decode kernel
     Wp = torch.zeros(256, 64, dtype=torch.uint8)
     rc, _ = run_layout(A, Wp, None, None, 128, _abi.W_INTERLEAVED_F16, _abi.ALGO_AUTO)
     assert rc != 0 and "plain layout" in _abi.last_error()
+    rc, _ = run_layout(A, Wp, None, None, 128, _abi.W_INTERLEAVED_F16, _abi.ALGO_DECODE)
+    assert rc != 0 and "decode kernel" in _abi.last_error()
     rc, _ = run_layout(A, Wp, None, None, 128, _abi.W_INTERLEAVED_F16, _abi.ALGO_GEMV)
-    assert rc != 0 and "streaming kernel and the two passes" in _abi.last_error()
+    assert rc != 0 and "decode kernel, the streaming kernel and the two passes" in _abi.last_error()
     rc, _ = run_layout(A, Wp, None, None, 128, 7, _abi.ALGO_AUTO)
     assert rc != 0 and "bad weight layout" in _abi.last_error()

@@ -259,8 +259,8 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
     return tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, algo, workspace,
                              workspace_bytes, stream);
   TLQ_CHECK_DIMS("tlq_gemm_w4a16_layout_ws");
-  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS,
-              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the streaming kernel and the two passes (algo %d)", algo);
+  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS || algo == TLQ_ALGO_DECODE,
+              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the decode kernel, the streaming kernel and the two passes (algo %d)", algo);
   TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_w4a16_layout_ws: in_dtype must be float16 or bfloat16 (got %d)", in_dtype);
   TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_w4a16_layout_ws: bad out_dtype %d", out_dtype);
   if (M == 0 || N == 0) return 0;
@@ -272,6 +272,18 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
   TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16_layout_ws: scales / zeros misaligned");
   TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K / 2), "tlq_gemm_w4a16_layout_ws: a matrix spans 4 GiB or more");
   const bool ws_aligned = workspace && aligned16(workspace);
+  if (M <= 32 && (algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_DECODE)) {
+    const DecodePlan dp = w4a16_decode_plan(M, N, K, group, cu_count_or_default());
+    const bool dec_ok = dp.ok && (((uintptr_t)scales | (uintptr_t)zeros) & 3) == 0 &&
+                        (dp.chunks == 1 || ((M * N) % 4 == 0 && ws_aligned && workspace_bytes >= (int64_t)dp.chunks * M * N * 4));
+    if (dec_ok)
+      return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, dp,
+                               (float*)workspace, (hipStream_t)stream);
+    TLQ_REQUIRE(algo != TLQ_ALGO_DECODE, "tlq_gemm_w4a16_layout_ws: the decode kernel does not take M=%lld N=%lld K=%lld group=%lld with a "
+                "workspace of %lld bytes (K %% 256 == 0, a power-of-two group, dword-aligned scale / zero tensors)", (long long)M, (long long)N,
+                (long long)K, (long long)group, (long long)workspace_bytes);
+  }
+  TLQ_REQUIRE(algo != TLQ_ALGO_DECODE, "tlq_gemm_w4a16_layout_ws: the decode kernel handles M <= 32 (got %lld)", (long long)M);
   if (algo != TLQ_ALGO_TWO_PASS) {
     const StreamPlan sp = w4a16_stream_plan(M, N, K, group, cu_count_or_default());
     const bool ws_ok = sp.ok && (M * N) % 4 == 0 && (sp.split == 1 || (ws_aligned && workspace_bytes >= (int64_t)sp.split * M * N * 4));
@@ -281,7 +293,8 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
     TLQ_REQUIRE(algo != TLQ_ALGO_STREAM, "tlq_gemm_w4a16_layout_ws: the streaming kernel does not take M=%lld N=%lld K=%lld group=%lld "
                 "with a workspace of %lld bytes", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
   }
-  TLQ_REQUIRE(M >= 17, "tlq_gemm_w4a16_layout_ws: decode-sized problems (M=%lld) read the plain layout", (long long)M);
+  TLQ_REQUIRE(M >= 17, "tlq_gemm_w4a16_layout_ws: with M=%lld interleaved weights need the decode kernel's shapes (K %% 256 == 0, power-of-two "
+              "group, dword-aligned scale / zero tensors); other decode-sized problems read the plain layout", (long long)M);
   TLQ_REQUIRE(ws_aligned && workspace_bytes >= N * K * 2 && N % 8 == 0,
               "tlq_gemm_w4a16_layout_ws: M=%lld N=%lld K=%lld needs a 16-byte aligned workspace of %lld bytes (got %lld) and N %% 8 == 0",
               (long long)M, (long long)N, (long long)K, (long long)(N * K * 2), (long long)workspace_bytes);
