@@ -490,6 +490,44 @@ struct EpiRescale {
     return ef;
   }
   static constexpr bool STAGED = true;
+  static constexpr bool HAS_SCALES = true;
+  // The scales a lane needs for its TN x TM accumulators: one per row tile, four per column tile.  Fetched in one go
+  // (indices clamped into the arrays) before the tile is packed: fetched per accumulator, each tile paid a memory round
+  // trip per use (measured on 256 x 256 int8 tiles: 18.7 us of fixed cost per tile against 7 us for the plain epilogue).
+  template <int TM, int TN>
+  struct Scales {
+    float a[TM];
+    float4_t b[TN];
+  };
+  template <int TM, int TN>
+  __device__ __forceinline__ Scales<TM, TN> load_scales(int m_base, int n_base, int lane, int M, int N) const {
+    Scales<TM, TN> s;
+    const int r16 = lane & 15, q = lane >> 4;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      int m = m_base + tm * 16 + r16;
+      m = m < M ? m : M - 1;
+      s.a[tm] = sa ? sa[m] : 1.0f;
+    }
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int n = n_base + tn * 16 + q * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int nn = (n + i < N) ? n + i : N - 1;
+        s.b[tn][i] = p.scale_b ? (p.n_scale_b == 1 ? p.scale_b[0] : p.scale_b[nn]) : 1.0f;
+      }
+    }
+    return s;
+  }
+  // same arithmetic as scaled(): convert, times the row scale, times the column scales (absent scales multiply by an
+  // exact 1.0f, which changes nothing)
+  __device__ __forceinline__ uint4_t pack_scaled(int m, int n, const int4_t& acc, float a, const float4_t& b, int M, int N) const {
+    float4_t f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = ((float)acc[i] * a) * b[i];
+    return as_float().pack(m, n, f, M, N);
+  }
   __device__ __forceinline__ int out_bytes() const { return p.out_dtype == TLQ_F32 ? 4 : 2; }
   __device__ __forceinline__ int64_t pitch() const { return p.ldc; }
   __device__ __forceinline__ uint8_t* addr_of(int m, int n) const { return as_float().addr_of(m, n); }
@@ -512,9 +550,30 @@ struct EpiRescale {
 // and pass, and read back row-wise, 16 bytes per lane, eight lanes per row -- every store instruction then writes eight
 // whole 128-byte lines.  Needs 16-byte aligned rows of C (pitch and N multiples of 16 bytes); otherwise, and for
 // tilings whose wavefront rows are shorter than 128 bytes, the direct path is used.
-template <class Epi, int TM, int TN, class Acc>
-__device__ __forceinline__ void write_tile(const Epi& epi, Acc (&acc)[TN][TM], uint8_t* region, int lane, int m_base, int n_base,
-                                           int M, int N) {
+// epilogues with per-row / per-column scales fetch them once per wavefront tile (HAS_SCALES); the others pack directly
+template <class Epi, typename = void>
+struct EpiHasScales : std::false_type {};
+template <class Epi>
+struct EpiHasScales<Epi, std::enable_if_t<Epi::HAS_SCALES>> : std::true_type {};
+struct NoScales {};
+template <class Epi, int TM, int TN>
+__device__ __forceinline__ auto fetch_scales(const Epi& epi, int m_base, int n_base, int lane, int M, int N) {
+  if constexpr (EpiHasScales<Epi>::value)
+    return epi.template load_scales<TM, TN>(m_base, n_base, lane, M, N);
+  else
+    return NoScales{};
+}
+template <class Epi, class S, class A>
+__device__ __forceinline__ uint4_t pack_with(const Epi& epi, const S& sc, int m, int n, const A& acc, int tm, int tn, int M, int N) {
+  if constexpr (EpiHasScales<Epi>::value)
+    return epi.pack_scaled(m, n, acc, sc.a[tm], sc.b[tn], M, N);
+  else
+    return epi.pack(m, n, acc, M, N);
+}
+
+template <class Epi, int TM, int TN, class Acc, class S>
+__device__ __forceinline__ void write_tile_with(const Epi& epi, const S& scales, Acc (&acc)[TN][TM], uint8_t* region, int lane, int m_base,
+                                                int n_base, int M, int N) {
   const int r16 = lane & 15, q = lane >> 4;
   const int osz = epi.out_bytes();
   bool staged = false;
@@ -537,7 +596,7 @@ __device__ __forceinline__ void write_tile(const Epi& epi, Acc (&acc)[TN][TM], u
 #pragma unroll
           for (int tm = 0; tm < TM; ++tm) {
             const int row = tm * 16 + r16;
-            const uint4_t v = epi.pack(m_base + row, n_base + (p0 + t) * 16 + q * 4, acc[p0 + t][tm], M, N);
+            const uint4_t v = pack_with<Epi>(epi, scales, m_base + row, n_base + (p0 + t) * 16 + q * 4, acc[p0 + t][tm], tm, p0 + t, M, N);
             const int byte = (t * 16 + q * 4) * OSZ;  // offset inside the 128-byte row of this pass
             uint8_t* dst = region + lds_off(row, byte >> 4) + (byte & 15);
             if (OSZ == 2)
@@ -563,6 +622,14 @@ __device__ __forceinline__ void write_tile(const Epi& epi, Acc (&acc)[TN][TM], u
     run(std::integral_constant<int, 2>{});
   else
     run(std::integral_constant<int, 4>{});
+}
+
+// the same with the scales fetched here (callers with registers to spare fetch them before their main loop instead)
+template <class Epi, int TM, int TN, class Acc>
+__device__ __forceinline__ void write_tile(const Epi& epi, Acc (&acc)[TN][TM], uint8_t* region, int lane, int m_base, int n_base,
+                                           int M, int N) {
+  const auto scales = fetch_scales<Epi, TM, TN>(epi, m_base, n_base, lane, M, N);
+  write_tile_with<Epi, TM, TN>(epi, scales, acc, region, lane, m_base, n_base, M, N);
 }
 
 // Work-group -> tile.  Consecutive hardware ids are dealt round-robin to the 8 XCDs; give

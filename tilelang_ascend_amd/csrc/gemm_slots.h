@@ -42,6 +42,10 @@ __global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDi
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = typename Mma::acc_t{0, 0, 0, 0};
 
+  // per-row / per-column output scales travel while the main loop runs (24 registers; this kernel has 256 per lane)
+  const Epi epi(pe, tc.batch);
+  const auto out_scales = fetch_scales<Epi, TM, TN>(epi, tc.m0 + wave_m0, tc.n0 + wave_n0, lane, M, N);
+
   auto slot_of = [&](int t) { return smem + addr::slot_of_tile(t) * TILE; };
   struct Ops {
     decltype(slot_of)& slot;
@@ -81,9 +85,8 @@ __global__ __launch_bounds__(512, 2) void gemm_slots_kernel(typename RowLoaderDi
   } ops{slot_of, al, wl, regs, regs_w, fragA, fragW, acc};
   addr::slots_schedule(KT, ops);
 
-  Epi epi(pe, tc.batch);
   if constexpr (Epi::STAGED) __syncthreads();  // every wavefront is past its last operand read: LDS becomes the output staging area
-  write_tile<Epi, TM, TN>(epi, acc, smem + wave * (TM * 16 * kStageBytes), lane, tc.m0 + wave_m0, tc.n0 + wave_n0, M, N);
+  write_tile_with<Epi, TM, TN>(epi, out_scales, acc, smem + wave * (TM * 16 * kStageBytes), lane, tc.m0 + wave_m0, tc.n0 + wave_n0, M, N);
 }
 
 // tlq_tune_gemm_slots: 0 = the two-stage kernel (default), 1 = this one where it applies
