@@ -1,0 +1,35 @@
+"""Compiler resource report of the hand-scheduled small-M kernels: none of them may spill registers to scratch memory
+(a spill in their inner loops costs more than the kernels gain: the two-activation-tile decode kernel ran 25 us instead of
+17 us when 11 registers spilled).  Compiles the two sources with hipcc's resource remarks; no GPU needed."""
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from tilelang_ascend_amd import build
+
+pytestmark = pytest.mark.skipif(shutil.which("hipcc") is None and not __import__("os").path.exists("/opt/rocm/bin/hipcc"),
+                                reason="hipcc not available")
+
+
+@pytest.mark.parametrize("source,kernels", [
+    ("gemm_w4a16_decode.hip", ["w4a16_decode_kernel"]),
+    ("gemm_w4a16_stream.hip", ["w4a16_stream_kernel"]),
+])
+def test_no_register_spills(tmp_path, source, kernels):
+    cmd = [build.hipcc_path(), *build.HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c",
+           f"{build.CSRC_DIR}/{source}", "-o", str(tmp_path / "out.o")]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout[-2000:]
+    blocks = re.split(r"remark: Function Name: ", res.stdout)[1:]
+    seen = 0
+    for b in blocks:
+        name = b.split()[0]
+        if not any(k in name for k in kernels):
+            continue
+        seen += 1
+        scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1))
+        spills = int(re.search(r"VGPRs Spill: (\d+)", b).group(1))
+        assert scratch == 0 and spills == 0, f"{name}: scratch {scratch} bytes per lane, {spills} registers spilled"
+    assert seen >= 4, f"expected the instances of {kernels} in the report, found {seen}"

@@ -175,57 +175,83 @@ __global__ __launch_bounds__(1024) void w4a16_decode_kernel(const T* __restrict_
     if (active) {
       if (ts > 0 && ts + 2 < my_tiles) issue_tile(ts + 2);  // into the slot that tile ts - 1 was read from (tile 2: issued above)
       const uint8_t* const slotp = mine + (ts % TS) * SLOT;
-      // one wait and one round of LDS reads per tile: both k-blocks, their scales and zero points
-      wait_vm(addr::dec_wait_count(ts, 1, my_tiles));
-      uint4_t wf[2];
-      uint32_t sdw[2], zdw[2];
+      wait_vm(addr::dec_wait_count(ts, 1, my_tiles));  // one wait per tile: both k-blocks, their scales and zero points
+      if constexpr (MT == 1) {
+        // one round of LDS reads per tile, and the two k-blocks accumulate separately (two independent MFMA chains)
+        uint4_t wf[2];
+        uint32_t sdw[2], zdw[2];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        wf[kb] = *(const uint4_t*)(slotp + kb * 1024 + fo_w);
-        sdw[kb] = *(const uint32_t*)(slotp + 2048 + rd_cell[kb]);
-        zdw[kb] = *(const uint32_t*)(slotp + 2304 + rd_cell[kb]);
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      T sv[2], zv[2];
-      bool ok = true;
+        for (int kb = 0; kb < 2; ++kb) {
+          wf[kb] = *(const uint4_t*)(slotp + kb * 1024 + fo_w);
+          sdw[kb] = *(const uint32_t*)(slotp + 2048 + rd_cell[kb]);
+          zdw[kb] = *(const uint32_t*)(slotp + 2304 + rd_cell[kb]);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        T sv[2], zv[2];
+        bool ok = true;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        sv[kb] = has_s ? bitcast<T>((uint16_t)(sdw[kb] >> rd_half[kb])) : one;
-        zv[kb] = has_z ? bitcast<T>((uint16_t)(zdw[kb] >> rd_half[kb])) : zs;
-        const float zf = to_float(zv[kb]);
-        ok = ok && zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
-      }
-      // the two k-blocks accumulate separately (two independent MFMA chains), added when the tile is handed over
-      typename Mma::acc_t acc2[2][MT];
+        for (int kb = 0; kb < 2; ++kb) {
+          sv[kb] = has_s ? bitcast<T>((uint16_t)(sdw[kb] >> rd_half[kb])) : one;
+          zv[kb] = has_z ? bitcast<T>((uint16_t)(zdw[kb] >> rd_half[kb])) : zs;
+          const float zf = to_float(zv[kb]);
+          ok = ok && zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
+        }
+        typename Mma::acc_t acc2[2] = {typename Mma::acc_t{0, 0, 0, 0}, typename Mma::acc_t{0, 0, 0, 0}};
+        if (__builtin_amdgcn_ballot_w64(ok) == ~0ull) {  // integer zero points fold into the unpack bias (exact)
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+          for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc2[kb][mt] = typename Mma::acc_t{0, 0, 0, 0};
-      if (__builtin_amdgcn_ballot_w64(ok) == ~0ull) {  // integer zero points fold into the unpack bias (exact)
+            for (int kb = 0; kb < 2; ++kb) {
+              const Expand8<T, true, 1> ex(sv[kb], zv[kb], mg);
+              const uint32_t w[4] = {wf[kb].x, wf[kb].y, wf[kb].z, wf[kb].w};
+              acc2[kb] = Mma::mma(ex(w[j]), af[kb][j][0], acc2[kb]);
+            }
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+          for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb) {
-            const Expand8<T, true, 1> ex(sv[kb], zv[kb], mg);
-            const uint32_t w[4] = {wf[kb].x, wf[kb].y, wf[kb].z, wf[kb].w};
-            const uint4_t b = ex(w[j]);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc2[kb][mt] = Mma::mma(b, af[kb][j][mt], acc2[kb][mt]);
-          }
+            for (int kb = 0; kb < 2; ++kb) {
+              const Expand8<T, false, 1> ex(sv[kb], zv[kb], mg);
+              const uint32_t w[4] = {wf[kb].x, wf[kb].y, wf[kb].z, wf[kb].w};
+              acc2[kb] = Mma::mma(ex(w[j]), af[kb][j][0], acc2[kb]);
+            }
+        }
+        acc[0] = acc2[0] + acc2[1];
       } else {
+        // two activation tiles: the operands fill the register file (128 per lane with 16 wavefronts per CU), so the
+        // k-blocks go one after the other into one chain per activation tile
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int mt = 0; mt < MT; ++mt) acc[mt] = typename Mma::acc_t{0, 0, 0, 0};
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb) {
-            const Expand8<T, false, 1> ex(sv[kb], zv[kb], mg);
-            const uint32_t w[4] = {wf[kb].x, wf[kb].y, wf[kb].z, wf[kb].w};
-            const uint4_t b = ex(w[j]);
+        for (int kb = 0; kb < 2; ++kb) {
+          const uint4_t wf = *(const uint4_t*)(slotp + kb * 1024 + fo_w);
+          const uint32_t sdw = *(const uint32_t*)(slotp + 2048 + rd_cell[kb]);
+          const uint32_t zdw = *(const uint32_t*)(slotp + 2304 + rd_cell[kb]);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          const T sv = has_s ? bitcast<T>((uint16_t)(sdw >> rd_half[kb])) : one;
+          const T zv = has_z ? bitcast<T>((uint16_t)(zdw >> rd_half[kb])) : zs;
+          const float zf = to_float(zv);
+          const bool ok = zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
+          const uint32_t w[4] = {wf.x, wf.y, wf.z, wf.w};
+          if (__builtin_amdgcn_ballot_w64(ok) == ~0ull) {
+            const Expand8<T, true, 1> ex(sv, zv, mg);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc2[kb][mt] = Mma::mma(b, af[kb][j][mt], acc2[kb][mt]);
+            for (int j = 0; j < 4; ++j) {
+              const uint4_t b = ex(w[j]);
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) acc[mt] = Mma::mma(b, af[kb][j][mt], acc[mt]);
+            }
+          } else {
+            const Expand8<T, false, 1> ex(sv, zv, mg);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const uint4_t b = ex(w[j]);
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) acc[mt] = Mma::mma(b, af[kb][j][mt], acc[mt]);
+            }
           }
+        }
       }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[mt] = acc2[0][mt] + acc2[1][mt];
     }
     if (RB == 1 && ts > 0) __syncthreads();  // the single buffer: the wavefronts that added up tile ts - 1 have read it
     if (active) {
