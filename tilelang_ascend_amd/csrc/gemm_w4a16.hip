@@ -48,7 +48,8 @@ struct W4Loader {
   };
   struct Regs {
     uint4_t v[PASSES];
-    T s[PASSES], z[PASSES];
+    uint32_t sz[PASSES];  // scale in the low half, zero point in the high half: 16-bit members of a struct that crosses
+                          // a stage boundary are passed through scratch memory by the compiler (a round trip per stage)
   };
   const uint8_t* base;  // uniform: first packed row of the tile
   const T* sbase;       // uniform: scales / zeros row of the tile's first row
@@ -94,15 +95,14 @@ struct W4Loader {
       r.v[ps] = *(const uint4_t*)(sb + voff[ps]);
       const T sv = sbase[has_s ? goff[ps] + gk : 0u];
       const T zv = zbase[has_z ? goff[ps] + gk : 0u];
-      r.s[ps] = has_s ? sv : one;
-      r.z[ps] = has_z ? zv : zs;
+      r.sz[ps] = (uint32_t)bitcast<uint16_t>(has_s ? sv : one) | ((uint32_t)bitcast<uint16_t>(has_z ? zv : zs) << 16);
     }
   }
   __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
       if (PARTIAL && ps == PASSES - 1 && !active) continue;
-      const Expand8<T, FOLD> ex(r.s[ps], r.z[ps], mg);
+      const Expand8<T, FOLD> ex(bitcast<T>((uint16_t)(r.sz[ps] & 0xffffu)), bitcast<T>((uint16_t)(r.sz[ps] >> 16)), mg);
       const uint32_t w[4] = {r.v[ps].x, r.v[ps].y, r.v[ps].z, r.v[ps].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(MT >= 4 ? 512 : 1024) void w4a16_skinny_kernel(cons
 
   struct Block {
     uint4_t w[RT];
-    T s[RT], z[RT];
+    uint32_t sz[RT];  // scale | zero point << 16 (16-bit struct members would travel through scratch memory)
     uint4_t a[MT][4];
   };
   auto load = [&](Block& b, int kb) {
@@ -276,8 +276,7 @@ __global__ __launch_bounds__(MT >= 4 ? 512 : 1024) void w4a16_skinny_kernel(cons
       b.w[rt] = *(const uint4_t*)(Wp + woff[rt] + (uint32_t)kb * 64u);
       const T sv = sp[has_s ? goff[rt] + gi : 0u];
       const T zv = zp[has_z ? goff[rt] + gi : 0u];
-      b.s[rt] = has_s ? sv : one;
-      b.z[rt] = has_z ? zv : zs;
+      b.sz[rt] = (uint32_t)bitcast<uint16_t>(has_s ? sv : one) | ((uint32_t)bitcast<uint16_t>(has_z ? zv : zs) << 16);
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -293,7 +292,7 @@ __global__ __launch_bounds__(MT >= 4 ? 512 : 1024) void w4a16_skinny_kernel(cons
   auto compute = [&](const Block& b) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      const Expand8<T, FOLD> ex(b.s[rt], b.z[rt], mg);
+      const Expand8<T, FOLD> ex(bitcast<T>((uint16_t)(b.sz[rt] & 0xffffu)), bitcast<T>((uint16_t)(b.sz[rt] >> 16)), mg);
       const uint32_t w[4] = {b.w[rt].x, b.w[rt].y, b.w[rt].z, b.w[rt].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
