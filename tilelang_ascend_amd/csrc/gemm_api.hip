@@ -79,6 +79,11 @@ int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cu
   return p.ok ? 1 : 0;
 }
 
+// Activation rows from which the decode kernel is ahead of the GEMV kernels, whose time grows with every row: from three
+// rows on, and with two rows once the weights are large enough for the second pass over them to show (measured: level at
+// 4096 x 4096, 10.4 against 12.8 us (fp16) and 11.1 against 15.3 us (bf16, skinny kernel) at 11008 x 4096).
+static bool decode_preferred(int64_t M, int64_t N, int64_t K) { return M > 2 || (M == 2 && N * K >= ((int64_t)1 << 24)); }
+
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                    void* stream) {
@@ -111,7 +116,7 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
     // M.  Measured crossovers: fp16 GEMV wins at M = 1, and at M = 2 while K <= 4096; the bf16 GEMV dequantises
     // element by element and wins only at M = 1 in its register-resident form, for rows of up to 8192 values.
     const bool skinny_ok = M <= 64 && K % 128 == 0 && fits32(M, K * 2) && fits32(N, K / 2);
-    if (M > 2 && decode_ok && g_w4a16_decode)
+    if (decode_preferred(M, N, K) && decode_ok && g_w4a16_decode)
       return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, dp, nullptr, st);
     if (M > 4)
       algo = skinny_ok ? TLQ_ALGO_SKINNY : TLQ_ALGO_MFMA;
@@ -172,7 +177,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                       void* workspace, int64_t workspace_bytes, void* stream) {
   TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_DECODE, "tlq_gemm_w4a16_ws: bad algo %d", algo);
   // decode batches: rows longer than 4096 values run as chunks of K whose fp32 partial sums live in the workspace
-  if (((algo == TLQ_ALGO_AUTO && g_w4a16_decode && M > 2) || algo == TLQ_ALGO_DECODE) && M <= 32 && M >= 1 && N >= 1 && K > 0 && group > 0 &&
+  if (((algo == TLQ_ALGO_AUTO && g_w4a16_decode && decode_preferred(M, N, K)) || algo == TLQ_ALGO_DECODE) && M <= 32 && M >= 1 && N >= 1 && K > 0 && group > 0 &&
       N < kMaxDim && K < kMaxDim) {
     const DecodePlan dp = w4a16_decode_plan(M, N, K, group, cu_count_or_default());
     const bool args_ok = A && w_packed && C && aligned16(A) && aligned16(w_packed) && aligned16(C) &&
