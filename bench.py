@@ -184,7 +184,7 @@ def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
         "config": {"workload": f"W4A16 decode GEMV M=1 N=11008 K=4096 group=128 fp16 scales+zeros, {units} weight set(s) per launch, "
                                f"{sets} sets rotating ({sets * unit_bytes >> 20} MiB); " + WALL_NOTE,
                    "M": M, "N": N, "K": K, "group": g, "units_per_launch": units},
-        "roofline": dict({"kernel": "gemv_w4a16_f16_rows_kernel", "bound": "hbm"}, **tm.roofline(step_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
+        "roofline": dict({"kernel": ("gemv_w4a16_ring_kernel<f16,2,1>" if units == 1 else "gemv_w4a16_f16_rows_kernel<2,2,1024>"), "bound": "hbm"}, **tm.roofline(step_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
                          traffic=(traffic_from_profile("gemv_w4a16_f16_M1_N11008_K4096_g128.txt") if units == 1 else None),
                          bytes_per_launch=step_bytes),
         "cpu_baseline": cpu,

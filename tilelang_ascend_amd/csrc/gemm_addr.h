@@ -186,5 +186,49 @@ __host__ __device__ inline int dec_wait_count(int ts, int kb, int my_tiles) {
   return 4 * younger + (kb == 0 ? 1 : 0);
 }
 
+// ---- GEMV ring kernel (one activation row): a work-group owns `rows_per_block` consecutive weight rows, wavefront w
+// takes rows w, w + waves, ... of them.  A packed row travels global -> LDS directly (no registers on the way), in
+// `iters` instructions of 1 KB (lane l moves chunk 64 it + l, 16 bytes), into one of the wavefront's `depth` private
+// slots; the activations and the work-group's scales / zero points are staged the same way, 16 bytes per lane.
+// LDS map (bytes): [ring: waves x depth x iters KB][activations, K x 2][scales][zero points], each area a whole number of KB
+// so that a wave-wide instruction whose last lanes repeat the final piece still lands inside its area.
+struct RingLayout {
+  uint32_t ring, act, s, z, total;
+};
+__host__ __device__ inline uint32_t ring_kb(uint32_t bytes) { return (bytes + 1023u) & ~1023u; }
+__host__ __device__ inline RingLayout ring_layout(int waves, int depth, int iters, int K, int rows_per_block, int groups) {
+  RingLayout l;
+  l.ring = 0;
+  l.act = (uint32_t)(waves * depth * iters) * 1024u;
+  l.s = l.act + ring_kb((uint32_t)K * 2u);
+  l.z = l.s + ring_kb((uint32_t)(rows_per_block * groups) * 2u);
+  l.total = l.z + ring_kb((uint32_t)(rows_per_block * groups) * 2u);
+  return l;
+}
+// weight instruction `it` of a row: byte offset of the lane's 16 bytes inside the row (chunks past the row repeat the
+// last one: their lanes multiply by a zero scale), and the LDS offset of the instruction's 1 KB
+__host__ __device__ inline uint32_t ring_w_voff(int lane, int it, int chunks) {
+  int c = it * 64 + lane;
+  c = c < chunks ? c : chunks - 1;
+  return (uint32_t)c * 16u;
+}
+__host__ __device__ inline uint32_t ring_w_lds(int wave, int slot, int it, int depth, int iters) {
+  return (uint32_t)((wave * depth + slot) * iters + it) * 1024u;
+}
+// staging: a tensor of `pieces` 16-byte pieces; the instruction that starts at piece p0 (a multiple of 64) moves piece
+// min(p0 + lane, pieces - 1) to bytes 16 (p0 + lane) of the area
+__host__ __device__ inline uint32_t ring_stage_voff(int p0, int lane, int pieces) {
+  int p = p0 + lane;
+  p = p < pieces ? p : pieces - 1;
+  return (uint32_t)p * 16u;
+}
+// rows of wavefront `wave`, and the loads it may leave in flight when it reads its i-th row (row i + depth is issued
+// after row i has been read; loads retire in issue order)
+__host__ __device__ inline int ring_my_rows(int rows, int wave, int waves) { return wave < rows ? (rows - wave + waves - 1) / waves : 0; }
+__host__ __device__ inline int ring_younger_rows(int i, int my_rows, int depth) {
+  const int y = my_rows - 1 - i;
+  return y < depth - 1 ? y : depth - 1;
+}
+
 }  // namespace addr
 }  // namespace tlq

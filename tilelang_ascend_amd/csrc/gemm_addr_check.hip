@@ -431,6 +431,95 @@ int check_decode_ring(int my_tiles) {
 
 using namespace tlq;
 
+// GEMV ring kernel: every direct load of every work-group stays inside its tensor and inside its LDS area, the staging
+// instructions cover every piece, every row is read by exactly one wavefront from the slot its loads went to, and no
+// row is read while one of its loads may be in flight or overwritten before it was read.
+int check_gemv_ring(int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth) {
+  CHECK_OR_FAIL(N >= 1 && K >= 32 && K % 32 == 0 && group >= 32 && K % group == 0 && rows_per_block >= 1 && waves >= 1 && waves <= 16 &&
+                    depth >= 1 && depth <= 3,
+                "gemv ring: bad arguments");
+  const int chunks = (int)(K / 32), groups = (int)(K / group), iters = (chunks + 63) / 64;
+  CHECK_OR_FAIL(iters * depth <= 6, "gemv ring: %d loads per wavefront in flight have no s_waitcnt case", iters * depth);
+  CHECK_OR_FAIL(groups % 8 == 0, "gemv ring: %d groups per row are not a whole number of 16-byte pieces", groups);
+  const int64_t row_bytes = K / 2;
+  const addr::RingLayout L = addr::ring_layout(waves, depth, iters, (int)K, rows_per_block, groups);
+  CHECK_OR_FAIL(L.total <= 160 * 1024, "gemv ring: %u bytes of LDS", L.total);
+  const int64_t blocks = (N + rows_per_block - 1) / rows_per_block;
+  const int64_t probe[6] = {0, 1, blocks / 2, blocks - 2, blocks - 1, blocks / 3};
+  for (int pi = 0; pi < 6; ++pi) {
+    const int64_t b = probe[pi];
+    if (b < 0 || b >= blocks) continue;
+    const int64_t r0 = b * rows_per_block, r1 = r0 + rows_per_block < N ? r0 + rows_per_block : N;
+    // staging: activations, then scales / zero points of rows r0 .. r1 - 1
+    const int a_pieces = chunks * 4, sz_pieces = (int)((r1 - r0) * groups / 8);
+    for (int which = 0; which < 2; ++which) {
+      const int pieces = which == 0 ? a_pieces : sz_pieces;
+      const uint32_t area = which == 0 ? L.act : L.s, area_end = which == 0 ? L.s : L.z;
+      const int64_t src_bytes = which == 0 ? K * 2 : (N - r0) * groups * 2;  // from the base pointer of the instruction
+      std::vector<char> seen(pieces, 0);
+      for (int w = 0; w < waves; ++w)
+        for (int p0 = w * 64; p0 < pieces; p0 += waves * 64)
+          for (int lane = 0; lane < 64; ++lane) {
+            const uint32_t voff = addr::ring_stage_voff(p0, lane, pieces);
+            CHECK_OR_FAIL((int64_t)voff + 16 <= src_bytes, "gemv ring: staging read at byte %u of %lld", voff, (long long)src_bytes);
+            const uint32_t dst = area + (uint32_t)p0 * 16u + (uint32_t)lane * 16u;
+            CHECK_OR_FAIL(dst + 16 <= area_end, "gemv ring: staging write at LDS byte %u, area ends at %u", dst, area_end);
+            if (p0 + lane < pieces) {
+              CHECK_OR_FAIL(voff == (uint32_t)(p0 + lane) * 16u, "gemv ring: piece %d read from byte %u", p0 + lane, voff);
+              seen[p0 + lane] = 1;
+            }
+          }
+      for (int p = 0; p < pieces; ++p) CHECK_OR_FAIL(seen[p], "gemv ring: staging piece %d of %d never loaded", p, pieces);
+    }
+    CHECK_OR_FAIL(L.z + (uint32_t)sz_pieces * 16u <= L.total && L.total - L.z == L.z - L.s, "gemv ring: zero-point area");
+    // weights
+    std::vector<int> reader((size_t)(r1 - r0), -1);
+    for (int w = 0; w < waves; ++w) {
+      const int my_rows = addr::ring_my_rows((int)(r1 - r0), w, waves);
+      std::vector<int> slot(depth, -1);
+      std::vector<char> read(my_rows > 0 ? my_rows : 1, 0);
+      std::vector<int> queue;  // row index of each outstanding load, oldest first
+      auto issue = [&](int i, int sl) -> int {
+        const int64_t row = r0 + w + (int64_t)i * waves;
+        CHECK_OR_FAIL(row < r1, "gemv ring: wavefront %d asks for row %lld past its work-group", w, (long long)row);
+        CHECK_OR_FAIL(slot[sl] < 0 || read[slot[sl]], "gemv ring: row %d overwrites row %d before it was read", i, slot[sl]);
+        for (int it = 0; it < iters; ++it) {
+          for (int lane = 0; lane < 64; ++lane) {
+            const int64_t src = row * row_bytes + addr::ring_w_voff(lane, it, chunks);
+            CHECK_OR_FAIL(src + 16 <= N * row_bytes && addr::ring_w_voff(lane, it, chunks) + 16 <= row_bytes, "gemv ring: weight read past the row");
+            const uint32_t dst = L.ring + addr::ring_w_lds(w, sl, it, depth, iters) + (uint32_t)lane * 16u;
+            CHECK_OR_FAIL(dst + 16 <= L.act, "gemv ring: weight write at LDS byte %u, ring ends at %u", dst, L.act);
+            CHECK_OR_FAIL(dst / (1024u * iters) == (uint32_t)(w * depth + sl), "gemv ring: weight write outside the slot");
+          }
+          queue.push_back(i);
+        }
+        slot[sl] = i;
+        return 0;
+      };
+      for (int d = 0; d < depth; ++d)
+        if (d < my_rows)
+          if (int rc = issue(d, d)) return rc;
+      int sl = 0;
+      for (int i = 0; i < my_rows; ++i) {
+        const int allowed = iters * addr::ring_younger_rows(i, my_rows, depth);
+        while ((int)queue.size() > allowed) queue.erase(queue.begin());
+        for (int q : queue) CHECK_OR_FAIL(q != i, "gemv ring: row %d read while one of its loads may be in flight", i);
+        CHECK_OR_FAIL(slot[sl] == i, "gemv ring: slot %d holds row %d when row %d is read", sl, slot[sl], i);
+        read[i] = 1;
+        const int lrow = w + i * waves;
+        CHECK_OR_FAIL(lrow < r1 - r0 && reader[lrow] < 0, "gemv ring: row %d read twice", lrow);
+        CHECK_OR_FAIL((int64_t)(lrow * groups + groups) * 2 <= (int64_t)(L.z - L.s), "gemv ring: scale row outside its area");
+        reader[lrow] = w;
+        if (i + depth < my_rows)
+          if (int rc = issue(i + depth, sl)) return rc;
+        sl = sl + 1 == depth ? 0 : sl + 1;
+      }
+    }
+    for (size_t r = 0; r < reader.size(); ++r) CHECK_OR_FAIL(reader[r] >= 0, "gemv ring: row %zu of work-group %lld never read", r, (long long)b);
+  }
+  return 0;
+}
+
 extern "C" {
 
 int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads) {
@@ -474,6 +563,10 @@ int tlq_debug_check_slots_schedule(int stages, int loads_per_tile) {
     return 1;
   }
   return 0;
+}
+
+int tlq_debug_check_gemv_ring_addressing(int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth) {
+  return check_gemv_ring(N, K, group, rows_per_block, waves, depth);
 }
 
 }  // extern "C"

@@ -17,6 +17,7 @@
 // (bf16 keeps only 8 mantissa bits, so skipping those roundings would be visible).
 #include "tlq_common.h"
 #include "expand8.h"
+#include "gemm_addr.h"
 
 namespace tlq {
 
@@ -582,6 +583,146 @@ __global__ __launch_bounds__(MAXT) void gemv_w4a16_bf16_rows_kernel(const bf16_t
   gemv_rows_body<bf16_t, ITERS, D>(A, Wp, scales, zeros, C, N, K, group_shift, zero_scalar, out_dtype, rows_per_block, nwaves);
 }
 
+// ---- ring kernel: the rows kernel's arithmetic with every global read a direct global -> LDS load ----
+// Loads that return into registers move about 14 bytes per clock and CU through the address unit, direct loads about 30;
+// a single problem of a few tens of MB is over before the stream settles, so the rate at which a CU can put its
+// requests out is what its time depends on.  Here every wavefront asks for its first `D` rows (all of its rows for the
+// shapes this is used for) before anything else happens, the staging data (activations, scales, zero points of the
+// work-group's rows) travels the same way ahead of them, and a row is read back from the wavefront's private LDS slot
+// by the lane that asked for it.  Same sums in the same order as the rows kernel: the results are the same bits.
+template <typename T, int ITERS, int D>
+__global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
+                                                              const T* __restrict__ scales, const T* __restrict__ zeros,
+                                                              void* __restrict__ C, int N, int K, int group_shift,
+                                                              float zero_scalar, int out_dtype, int rows_per_block) {
+  constexpr bool F16 = __is_same(T, half_t);
+  typedef __attribute__((address_space(3))) uint8_t* lptr_t;
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nwaves = blockDim.x >> 6;
+  const int chunks = K >> 5, row_bytes = K >> 1, groups = K >> group_shift;
+  const int r0 = blockIdx.x * rows_per_block;
+  const int r1 = r0 + rows_per_block < N ? r0 + rows_per_block : N;
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lptr_t)smem);
+  const addr::RingLayout L = addr::ring_layout(nwaves, D, ITERS, K, rows_per_block, groups);
+  const bool has_s = scales != nullptr, has_z = zeros != nullptr;
+  auto dma16 = [&](uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+  };
+  auto wait_vm = [&](int outstanding) {  // a wavefront-uniform count, 0 .. ITERS * D
+    static_assert(ITERS * D <= 6, "cases below");
+    switch (outstanding) {
+      case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+      case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+      case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+      case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+      case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+  };
+
+  // ---- staging data first (loads retire in issue order: once only a wavefront's weight rows are outstanding its
+  // staging loads have landed), then the first D rows ----
+  const int a_pieces = chunks * 4;
+  for (int p0 = wave * 64; p0 < a_pieces; p0 += nwaves * 64)
+    dma16(lds0 + L.act + (uint32_t)p0 * 16u, addr::ring_stage_voff(p0, lane, a_pieces), (const uint8_t*)A);
+  const int sz_pieces = ((r1 - r0) * groups) >> 3;  // groups is a multiple of 8
+  const uint8_t* const s_base = uniform_ptr((const uint8_t*)(scales + (int64_t)r0 * groups));
+  const uint8_t* const z_base = uniform_ptr((const uint8_t*)(zeros + (int64_t)r0 * groups));
+  for (int p0 = wave * 64; p0 < sz_pieces; p0 += nwaves * 64) {
+    const uint32_t voff = addr::ring_stage_voff(p0, lane, sz_pieces);
+    if (has_s) dma16(lds0 + L.s + (uint32_t)p0 * 16u, voff, s_base);
+    if (has_z) dma16(lds0 + L.z + (uint32_t)p0 * 16u, voff, z_base);
+  }
+  uint32_t voff_w[ITERS];
+  int cc[ITERS], gsel[ITERS];
+  bool ok[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = (it << 6) + lane;
+    ok[it] = c < chunks;
+    cc[it] = ok[it] ? c : chunks - 1;
+    gsel[it] = (cc[it] << 5) >> group_shift;
+    voff_w[it] = addr::ring_w_voff(lane, it, chunks);
+  }
+  const int my_rows = addr::ring_my_rows(r1 - r0, wave, nwaves);
+  auto issue = [&](int i, int slot) {  // the wavefront's i-th row into ring slot `slot`
+    const uint8_t* const base = uniform_ptr(Wp + (int64_t)(r0 + wave + i * nwaves) * row_bytes);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) dma16(lds0 + L.ring + addr::ring_w_lds(wave, slot, it, D, ITERS), voff_w[it], base);
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < my_rows) issue(d, d);
+  wait_vm(ITERS * (my_rows < D ? my_rows : D));
+  __syncthreads();
+
+  // every wavefront prepares the activations of its lanes' chunks itself (fp16: pairs in unpack order and the chunk
+  // sums; bf16: the 32 values as they are)
+  ActF16 act[F16 ? ITERS : 1];
+  uint4_t actn[F16 ? 1 : ITERS][4];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    uint4_t raw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) raw[j] = *(const uint4_t*)(smem + L.act + (uint32_t)(cc[it] * 4 + j) * 16u);
+    if constexpr (F16) {
+      permute_act(act[it], raw);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) actn[it][j] = raw[j];
+    }
+  }
+  const T* const lds_s = (const T*)(smem + L.s);
+  const T* const lds_z = (const T*)(smem + L.z);
+  const NibbleMagic mg = make_nibble_magic();
+  const T one = from_float<T>(1.0f), zs = from_float<T>(zero_scalar);
+  int slot = 0;
+  for (int i = 0; i < my_rows; ++i) {
+    wait_vm(ITERS * addr::ring_younger_rows(i, my_rows, D));
+    const int lrow = wave + i * nwaves;
+    uint4_t w[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+      w[it] = *(const uint4_t*)(smem + L.ring + addr::ring_w_lds(wave, slot, it, D, ITERS) + (uint32_t)lane * 16u);
+    T sv[ITERS], zv[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const T s0 = has_s ? lds_s[lrow * groups + gsel[it]] : one;
+      sv[it] = ok[it] ? s0 : from_float<T>(0.0f);  // a chunk past the end contributes 0
+      zv[it] = has_z ? lds_z[lrow * groups + gsel[it]] : zs;
+    }
+    if (i + D < my_rows) {  // the slot takes the row D ahead once this row's words are in registers
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      issue(i + D, slot);
+    }
+    float acc = 0.f;
+    if constexpr (F16) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) acc += chunk_term_biased(w[it], act[it], sv[it], zv[it], mg);
+    } else {
+      bool integral = true;  // small integer zero points fold exactly into one fused multiply-add per weight
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const float zf = to_float(zv[it]);
+        integral = integral && zf == __builtin_rintf(zf) && zf >= -256.0f && zf <= 256.0f;
+      }
+      if (__builtin_amdgcn_ballot_w64(integral) == ~0ull) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) acc += chunk_term_dot2<true>(w[it], actn[it], sv[it], zv[it], mg);
+      } else {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) acc += chunk_term_dot2<false>(w[it], actn[it], sv[it], zv[it], mg);
+      }
+    }
+    const float v = wave_sum_to_lane63(acc);
+    if (lane == 63) store_out(C, r0 + lrow, v, out_dtype);
+    slot = slot + 1 == D ? 0 : slot + 1;
+  }
+}
+
 template <typename T>
 struct ActOf;
 template <>
@@ -760,6 +901,73 @@ static int launch_gemv_rows(const void* A, const void* Wp, const void* scales, c
   return 0;
 }
 
+// Launch geometry of the ring kernel: one work-group of 16 wavefronts per CU, every wavefront's rows in flight from the
+// start where the LDS has room for them (three slots of a row per wavefront at most).  One problem per launch, rows of
+// up to 4096 values, group counts that are multiples of 8 (the staging loads move 16 bytes).
+struct RingPlan {
+  bool ok;
+  int iters, depth, waves, rows_per_block, blocks;
+  uint32_t lds_bytes;
+};
+static RingPlan plan_gemv_ring(int64_t batch, int64_t N, int64_t K, int group_shift, int cus) {
+  RingPlan p{false, 0, 0, 0, 0, 0, 0};
+  if (batch != 1 || N < 1 || N > 0x7fffffff || K < 32 || K % 32 != 0 || K > 4096 || group_shift < 5 || cus < 1) return p;
+  const int groups = (int)(K >> group_shift);
+  if (groups < 8 || groups % 8 != 0 || ((int64_t)groups << group_shift) != K) return p;
+  p.waves = (g_gemv_waves16 >= 1 && g_gemv_waves16 <= 16) ? g_gemv_waves16 : 16;
+  p.iters = K > 2048 ? 2 : 1;
+  int64_t rpb = ceil_div(N, (int64_t)cus);
+  if (rpb < p.waves) rpb = p.waves;
+  if (rpb * groups * 2 > 24 * 1024) return p;  // scales and zero points of the rows: at most 24 KB each
+  p.rows_per_block = (int)rpb;
+  p.blocks = (int)ceil_div(N, rpb);
+  // one row in flight per wavefront: 16 wavefronts on 256 CUs ask for 8 MB at a time, about what the memory system
+  // holds in flight at its full rate; with two or three rows per wavefront the same launch measured 3 - 17 % slower
+  const int per_wave = (int)ceil_div(rpb, (int64_t)p.waves);
+  const int want = (g_gemv_depth >= 1 && g_gemv_depth <= 3) ? g_gemv_depth : 1;
+  p.depth = per_wave < want ? per_wave : want;
+  p.lds_bytes = addr::ring_layout(p.waves, p.depth, p.iters, (int)K, p.rows_per_block, groups).total;
+  p.ok = p.lds_bytes <= 160 * 1024;
+  return p;
+}
+
+template <typename T, int ITERS, int D>
+static int launch_gemv_ring(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int N, int K,
+                            int group_shift, float zero_scalar, int out_dtype, const RingPlan& p, hipStream_t st) {
+  auto kern = gemv_w4a16_ring_kernel<T, ITERS, D>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      set_error("tlq_gemm_w4a16(gemv): cannot reserve the ring kernel's LDS: %s", hipGetErrorString(e));
+      return 1;
+    }
+    attr_set = true;
+  }
+  kern<<<p.blocks, 64 * p.waves, p.lds_bytes, st>>>((const T*)A, (const uint8_t*)Wp, (const T*)scales, (const T*)zeros, C, N, K,
+                                                  group_shift, zero_scalar, out_dtype, p.rows_per_block);
+  return check_launch("tlq_gemm_w4a16(gemv)") ? 0 : 1;
+}
+
+// 1 (default): the ring kernel where it applies; 0: never
+static thread_local int g_gemv_ring = 1;
+
+template <typename T>
+static int dispatch_gemv_ring(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int N, int K,
+                              int group_shift, float zero_scalar, int out_dtype, const RingPlan& p, hipStream_t st) {
+#define TLQ_RING_CASE(IT, DD) \
+  return launch_gemv_ring<T, IT, DD>(A, Wp, scales, zeros, C, N, K, group_shift, zero_scalar, out_dtype, p, st)
+  if (p.iters == 1) {
+    if (p.depth == 1) TLQ_RING_CASE(1, 1);
+    if (p.depth == 2) TLQ_RING_CASE(1, 2);
+    TLQ_RING_CASE(1, 3);
+  }
+  if (p.depth == 1) TLQ_RING_CASE(2, 1);
+  if (p.depth == 2) TLQ_RING_CASE(2, 2);
+  TLQ_RING_CASE(2, 3);
+#undef TLQ_RING_CASE
+}
+
 // wavefronts per work-group and work-groups per CU of the rows kernel for this K
 static void rows_kernel_shape(int64_t K, int& wpb_rows, int& bpc_rows) {
   bpc_rows = g_gemv_unroll ? g_gemv_unroll : 1;
@@ -834,6 +1042,10 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     const int R = g_gemv_rows > 0 ? g_gemv_rows : (streaming ? 2 : 1);
     const int bpc = g_gemv_unroll ? g_gemv_unroll : (streaming ? 64 : 8);  // grid size cap, blocks per CU
     const int depth_req = g_gemv_depth;
+    if (M == 1 && g_gemv_ring && g_gemv_rows >= 0 && (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0) {
+      const RingPlan rp = plan_gemv_ring(batch, N, K, shift, cu_count());
+      if (rp.ok) return dispatch_gemv_ring<half_t>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st);
+    }
     if (M == 1 && K <= 16384 && g_gemv_rows >= 0 && rows_kernel_fits(batch, N, K, shift))
       return dispatch_gemv_rows<half_t>(A, Wp, scales, zeros, C, batch, N, K, shift, zero_scalar, out_dtype, st);
     const bool two_rows = M > 1 && (size_t)2 * (K / 32) * 72 <= 64 * 1024;
@@ -869,6 +1081,10 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
   } else {
     int shift = 0;
     while (((int64_t)1 << shift) < group) ++shift;
+    if (M == 1 && pow2 && g_gemv_ring && g_gemv_rows >= 0 && (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0) {
+      const RingPlan rp = plan_gemv_ring(batch, N, K, shift, cu_count());
+      if (rp.ok) return dispatch_gemv_ring<bf16_t>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st);
+    }
     if (M == 1 && pow2 && K <= 16384 && g_gemv_rows >= 0 && rows_kernel_fits(batch, N, K, shift)) {
       return dispatch_gemv_rows<bf16_t>(A, Wp, scales, zeros, C, batch, N, K, shift, zero_scalar, out_dtype, st);
     }
@@ -910,6 +1126,23 @@ void tlq_tune_gemv(int rows_per_wave, int waves_per_block) {
   tlq::g_gemv_waves = (waves_per_block < 0 || waves_per_block > 4) ? 0 : waves_per_block;
   tlq::g_gemv_waves16 = (waves_per_block < 0 || waves_per_block > 16) ? 0 : waves_per_block;  // register-resident kernel
 }
+void tlq_tune_gemv_ring(int on) { tlq::g_gemv_ring = on != 0; }
+
+int tlq_debug_gemv_ring_plan(int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
+  int shift = 0;
+  while (((int64_t)1 << shift) < group) ++shift;
+  if (group < 1 || ((int64_t)1 << shift) != group) {
+    tlq::set_error("tlq_debug_gemv_ring_plan: the group size must be a power of two");
+    return -1;
+  }
+  const tlq::RingPlan p = tlq::plan_gemv_ring(1, N, K, shift, cus);
+  if (plan_out) {
+    int64_t* o = (int64_t*)plan_out;
+    o[0] = p.iters, o[1] = p.depth, o[2] = p.waves, o[3] = p.rows_per_block, o[4] = p.blocks, o[5] = p.lds_bytes;
+  }
+  return p.ok ? 1 : 0;
+}
+
 void tlq_tune_gemv_unroll(int blocks_per_cu) { tlq::g_gemv_unroll = blocks_per_cu; }
 void tlq_tune_gemv_depth(int steps_in_flight) { tlq::g_gemv_depth = steps_in_flight < 0 ? 0 : steps_in_flight; }
 }
