@@ -286,15 +286,16 @@ int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cu
  * -1 for bad arguments.  No counterpart in the reference. */
 int tlq_debug_gemv_rows_plan(int64_t batch, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
 
-/* The same for the ring kernel, which takes a single decode GEMV (M = 1, fp16, K <= 4096, a multiple of 8 groups per row,
- * 16-byte aligned scale / zero tensors) with every global read a direct global -> LDS load: plan_out receives six int64:
+/* The same for the ring kernel, which takes a single decode GEMV (M = 1, or 2 with fp16 activations; K <= 4096, a
+ * multiple of 8 groups per row, 16-byte aligned scale / zero tensors) with every global read a direct global -> LDS load:
+ * plan_out receives six int64:
  * load instructions per row, ring slots per wavefront, wavefronts per work-group, rows per work-group, work-groups and
  * bytes of dynamic LDS.  Returns 1 when the kernel applies, 0 when not, -1 for bad arguments.
  * tlq_debug_check_gemv_ring_addressing walks, on the host, every load of the first, middle and last work-groups of such a
  * launch (bounds of every global read and LDS write, coverage of the staging data and of the rows, ring order against the
  * kernel's wait counts); 0 = consistent.  No counterpart in the reference. */
-int tlq_debug_gemv_ring_plan(int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
-int tlq_debug_check_gemv_ring_addressing(int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth);
+int tlq_debug_gemv_ring_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
+int tlq_debug_check_gemv_ring_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth);
 
 /* Tuning hooks for benchmark sweeps and the autotuner (each sets a value of the CALLING THREAD, read by that thread's
  * later launches; other threads keep the automatic choice; 0 = automatic choice).
@@ -304,8 +305,9 @@ void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4 (negat
                                                              * M = 1, K <= 4096 kernel), waves 1..4 (that kernel: 1..16) */
 void tlq_tune_gemv_unroll(int blocks_per_cu);               /* resident blocks per CU the GEMV grid is sized for */
 void tlq_tune_gemv_depth(int steps_in_flight);               /* load steps (1 KB per row each) a GEMV wavefront keeps in flight */
-void tlq_tune_gemv_ring(int on);                             /* 1 (default): a single fp16 decode GEMV runs on the ring kernel where it
-                                                              * applies; 0: on the register-resident kernel (same results, bit for bit) */
+void tlq_tune_gemv_ring(int on);                             /* 1 (default): a single decode GEMV (1 or 2 activation rows) runs on the
+                                                              * ring kernel where it applies; 0: on the kernels it replaced (for one
+                                                              * activation row the same results, bit for bit) */
 void tlq_tune_gemm_band(int tile_rows);                       /* tile rows per band of the MFMA kernels' tile order (default 4) */
 void tlq_tune_gemm_slots(int on);                            /* 1 (default): 256 x 256 tiles of the plain 16-bit GEMM with [N, K] weights and of the
                                                               * int8 GEMMs run on the kernel that cuts LDS into five operand-tile slots

@@ -48,9 +48,9 @@ def test_bad_arguments():
     assert plan(0, 16, 4096, 128)[0] == -1
 
 
-def ring_plan(N, K, group, cus=256):
+def ring_plan(N, K, group, cus=256, M=1):
     out = (ctypes.c_int64 * 6)()
-    rc = _abi.load().tlq_debug_gemv_ring_plan(N, K, group, cus, ctypes.cast(out, ctypes.c_void_p))
+    rc = _abi.load().tlq_debug_gemv_ring_plan(M, N, K, group, cus, ctypes.cast(out, ctypes.c_void_p))
     return rc, list(out)
 
 
@@ -64,26 +64,28 @@ def test_ring_kernel_geometry_and_addressing(N, K, group):
     if K % group:
         pytest.skip("group does not divide K")
     lib = _abi.load()
-    for cus in (256, 64, 8):
-        rc, (iters, depth, waves, rpb, blocks, lds) = ring_plan(N, K, group, cus)
+    for cus, M in ((256, 1), (64, 1), (8, 1), (256, 2), (64, 2)):
+        rc, (iters, depth, waves, rpb, blocks, lds) = ring_plan(N, K, group, cus, M)
         groups = K // group
         if groups % 8 or rc == 0:
             assert rc == 0  # 16-byte staging pieces need a multiple of 8 groups per row; or LDS does not hold the rows' scales
             continue
         assert rc == 1
-        assert iters == (2 if K > 2048 else 1) and waves == 16 and 1 <= depth <= 3
-        assert rpb >= 16 and rpb * blocks >= N and rpb * (blocks - 1) < N and (blocks <= cus or rpb == 16)
+        assert iters == (2 if K > 2048 else 1) and waves == 16 and 1 <= depth <= (3 if M == 1 else 2)
+        assert rpb >= waves and rpb * blocks >= N and rpb * (blocks - 1) < N and (blocks <= cus or rpb == waves)
         assert lds <= 160 * 1024
-        assert lib.tlq_debug_check_gemv_ring_addressing(N, K, group, rpb, waves, depth) == 0, _abi.last_error()
+        assert lib.tlq_debug_check_gemv_ring_addressing(M, N, K, group, rpb, waves, depth) == 0, _abi.last_error()
 
 
 def test_ring_walker_catches_a_wrong_launch():
     lib = _abi.load()
     # rows per work-group whose scales overflow the 160 KB of LDS
-    assert lib.tlq_debug_check_gemv_ring_addressing(11008, 4096, 32, 4096, 16, 3) != 0
+    assert lib.tlq_debug_check_gemv_ring_addressing(1, 11008, 4096, 32, 4096, 16, 3) != 0
     assert "LDS" in _abi.last_error()
     # a group count that is not a multiple of 8
-    assert lib.tlq_debug_check_gemv_ring_addressing(1024, 1024, 256, 16, 16, 1) != 0
+    assert lib.tlq_debug_check_gemv_ring_addressing(1, 1024, 1024, 256, 16, 16, 1) != 0
+    assert lib.tlq_debug_check_gemv_ring_addressing(3, 1024, 1024, 32, 16, 16, 1) != 0  # at most two activation rows
+    assert ring_plan(1024, 1024, 32, M=3)[0] == 0
     assert ring_plan(1024, 1024, 256)[0] == 0
     assert ring_plan(1024, 8192, 128)[0] == 0  # rows longer than 4096 values stay with the register-resident kernel
     assert ring_plan(1024, 1024, 96)[0] == -1

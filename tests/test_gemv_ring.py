@@ -13,7 +13,7 @@ def run_gemv(A, Wp, s, z, group, ring, out_dtype=None):
     from tilelang_ascend_amd import _abi
 
     lib, P = _abi.load(), _abi.ptr
-    K = A.shape[1]
+    M, K = A.shape
     N = Wp.shape[0]
     code = {torch.float16: _abi.F16, torch.float32: _abi.F32, torch.bfloat16: _abi.BF16}
     out_dtype = out_dtype or A.dtype
@@ -22,11 +22,11 @@ def run_gemv(A, Wp, s, z, group, ring, out_dtype=None):
     dA, dW = A.cuda(), Wp.cuda()
     dS = s.cuda() if s is not None else None
     dZ = zt.cuda() if zt is not None else None
-    C = torch.full((1, N), float("nan"), dtype=out_dtype, device="cuda")
-    print(f"gemv ring={ring} N={N} K={K} g={group} {A.dtype} out={out_dtype}", flush=True)
+    C = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+    print(f"gemv ring={ring} M={M} N={N} K={K} g={group} {A.dtype} out={out_dtype}", flush=True)
     lib.tlq_tune_gemv_ring(ring)
     try:
-        _abi.check(lib.tlq_gemm_w4a16(P(dA), P(dW), P(dS), P(dZ), P(C), 1, N, K, group, zs, code[A.dtype], code[out_dtype],
+        _abi.check(lib.tlq_gemm_w4a16(P(dA), P(dW), P(dS), P(dZ), P(C), M, N, K, group, zs, code[A.dtype], code[out_dtype],
                                       _abi.ALGO_GEMV, torch.cuda.current_stream().cuda_stream))
         torch.cuda.synchronize()
     finally:
@@ -44,7 +44,7 @@ def test_ring_kernel_equals_the_register_resident_kernel_and_the_oracle(N, K, gr
     from tilelang_ascend_amd import _abi
 
     plan = (torch.zeros(6, dtype=torch.int64)).numpy()
-    assert _abi.load().tlq_debug_gemv_ring_plan(N, K, group, 256, plan.ctypes.data) == 1, "this shape is meant to take the ring kernel"
+    assert _abi.load().tlq_debug_gemv_ring_plan(1, N, K, group, 256, plan.ctypes.data) == 1, "this shape is meant to take the ring kernel"
     dt = DT[in_dtype]
     A = torch.randn(1, K, generator=gen(80)).to(dt)
     Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=81)
@@ -88,3 +88,22 @@ def test_misaligned_scales_fall_back_to_the_register_resident_kernel():
                                   torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     check_float_output(C.cpu(), w4a16_reference(A, Wp, s, z, group), "misaligned scales")
+
+
+@pytest.mark.parametrize("zeros_kind", [None, "scalar8", "int", "frac"])
+@pytest.mark.parametrize("N,K,group", [(11008, 4096, 128), (77, 1024, 32), (1000, 2048, 64), (5000, 2560, 64), (16, 256, 32), (14336, 4096, 64)])
+def test_ring_kernel_with_two_activation_rows(N, K, group, zeros_kind):
+    """fp16, two activation rows: each weight row is expanded once and multiplied with both.  Against the oracle; and each
+    activation row must come out exactly as it does when it is the only one (the rows do not mix)."""
+    from tilelang_ascend_amd import _abi
+
+    M = 2
+    plan = (torch.zeros(6, dtype=torch.int64)).numpy()
+    assert _abi.load().tlq_debug_gemv_ring_plan(M, N, K, group, 256, plan.ctypes.data) == 1
+    A = torch.randn(M, K, generator=gen(88)).to(torch.float16)
+    Wp, s, z = make_w4(N, K, group, torch.float16, zeros_kind, seed=89)
+    got = run_gemv(A, Wp, s, z, group, 1)
+    check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"ring kernel M={M} vs oracle")
+    for m in (0, M - 1):
+        alone = run_gemv(A[m:m + 1].contiguous(), Wp, s, z, group, 1)
+        assert_bit_equal(got[m:m + 1], alone, f"activation row {m} of {M} vs the same row alone")

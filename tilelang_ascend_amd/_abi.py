@@ -62,8 +62,8 @@ SIGNATURES = {
     "tlq_tune_gemv_unroll": (None, [_int]),
     "tlq_tune_gemv_depth": (None, [_int]),
     "tlq_tune_gemv_ring": (None, [_int]),
-    "tlq_debug_gemv_ring_plan": (_int, [_i64, _i64, _i64, _int, _vp]),
-    "tlq_debug_check_gemv_ring_addressing": (_int, [_i64, _i64, _i64, _int, _int, _int]),
+    "tlq_debug_gemv_ring_plan": (_int, [_i64, _i64, _i64, _i64, _int, _vp]),
+    "tlq_debug_check_gemv_ring_addressing": (_int, [_i64, _i64, _i64, _i64, _int, _int, _int]),
     "tlq_tune_gemm_band": (None, [_int]),
     "tlq_tune_gemm_slots": (None, [_int]),
     "tlq_tune_w4a16_stream": (None, [_int]),

@@ -186,21 +186,21 @@ __host__ __device__ inline int dec_wait_count(int ts, int kb, int my_tiles) {
   return 4 * younger + (kb == 0 ? 1 : 0);
 }
 
-// ---- GEMV ring kernel (one activation row): a work-group owns `rows_per_block` consecutive weight rows, wavefront w
+// ---- GEMV ring kernel (one or two activation rows): a work-group owns `rows_per_block` consecutive weight rows, wavefront w
 // takes rows w, w + waves, ... of them.  A packed row travels global -> LDS directly (no registers on the way), in
 // `iters` instructions of 1 KB (lane l moves chunk 64 it + l, 16 bytes), into one of the wavefront's `depth` private
 // slots; the activations and the work-group's scales / zero points are staged the same way, 16 bytes per lane.
-// LDS map (bytes): [ring: waves x depth x iters KB][activations, K x 2][scales][zero points], each area a whole number of KB
+// LDS map (bytes): [ring: waves x depth x iters KB][activations, mt x K x 2][scales][zero points], each area a whole number of KB
 // so that a wave-wide instruction whose last lanes repeat the final piece still lands inside its area.
 struct RingLayout {
   uint32_t ring, act, s, z, total;
 };
 __host__ __device__ inline uint32_t ring_kb(uint32_t bytes) { return (bytes + 1023u) & ~1023u; }
-__host__ __device__ inline RingLayout ring_layout(int waves, int depth, int iters, int K, int rows_per_block, int groups) {
+__host__ __device__ inline RingLayout ring_layout(int waves, int depth, int iters, int K, int rows_per_block, int groups, int mt) {
   RingLayout l;
   l.ring = 0;
   l.act = (uint32_t)(waves * depth * iters) * 1024u;
-  l.s = l.act + ring_kb((uint32_t)K * 2u);
+  l.s = l.act + ring_kb((uint32_t)(K * mt) * 2u);
   l.z = l.s + ring_kb((uint32_t)(rows_per_block * groups) * 2u);
   l.total = l.z + ring_kb((uint32_t)(rows_per_block * groups) * 2u);
   return l;

@@ -434,15 +434,15 @@ using namespace tlq;
 // GEMV ring kernel: every direct load of every work-group stays inside its tensor and inside its LDS area, the staging
 // instructions cover every piece, every row is read by exactly one wavefront from the slot its loads went to, and no
 // row is read while one of its loads may be in flight or overwritten before it was read.
-int check_gemv_ring(int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth) {
-  CHECK_OR_FAIL(N >= 1 && K >= 32 && K % 32 == 0 && group >= 32 && K % group == 0 && rows_per_block >= 1 && waves >= 1 && waves <= 16 &&
-                    depth >= 1 && depth <= 3,
+int check_gemv_ring(int64_t M, int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth) {
+  CHECK_OR_FAIL(M >= 1 && M <= 2 && N >= 1 && K >= 32 && K % 32 == 0 && group >= 32 && K % group == 0 && rows_per_block >= 1 && waves >= 1 &&
+                    waves <= 16 && depth >= 1 && depth <= 3,
                 "gemv ring: bad arguments");
   const int chunks = (int)(K / 32), groups = (int)(K / group), iters = (chunks + 63) / 64;
   CHECK_OR_FAIL(iters * depth <= 6, "gemv ring: %d loads per wavefront in flight have no s_waitcnt case", iters * depth);
   CHECK_OR_FAIL(groups % 8 == 0, "gemv ring: %d groups per row are not a whole number of 16-byte pieces", groups);
   const int64_t row_bytes = K / 2;
-  const addr::RingLayout L = addr::ring_layout(waves, depth, iters, (int)K, rows_per_block, groups);
+  const addr::RingLayout L = addr::ring_layout(waves, depth, iters, (int)K, rows_per_block, groups, (int)M);
   CHECK_OR_FAIL(L.total <= 160 * 1024, "gemv ring: %u bytes of LDS", L.total);
   const int64_t blocks = (N + rows_per_block - 1) / rows_per_block;
   const int64_t probe[6] = {0, 1, blocks / 2, blocks - 2, blocks - 1, blocks / 3};
@@ -451,11 +451,11 @@ int check_gemv_ring(int64_t N, int64_t K, int64_t group, int rows_per_block, int
     if (b < 0 || b >= blocks) continue;
     const int64_t r0 = b * rows_per_block, r1 = r0 + rows_per_block < N ? r0 + rows_per_block : N;
     // staging: activations, then scales / zero points of rows r0 .. r1 - 1
-    const int a_pieces = chunks * 4, sz_pieces = (int)((r1 - r0) * groups / 8);
+    const int a_pieces = chunks * 4 * (int)M, sz_pieces = (int)((r1 - r0) * groups / 8);
     for (int which = 0; which < 2; ++which) {
       const int pieces = which == 0 ? a_pieces : sz_pieces;
       const uint32_t area = which == 0 ? L.act : L.s, area_end = which == 0 ? L.s : L.z;
-      const int64_t src_bytes = which == 0 ? K * 2 : (N - r0) * groups * 2;  // from the base pointer of the instruction
+      const int64_t src_bytes = which == 0 ? M * K * 2 : (N - r0) * groups * 2;  // from the base pointer of the instruction
       std::vector<char> seen(pieces, 0);
       for (int w = 0; w < waves; ++w)
         for (int p0 = w * 64; p0 < pieces; p0 += waves * 64)
@@ -565,8 +565,8 @@ int tlq_debug_check_slots_schedule(int stages, int loads_per_tile) {
   return 0;
 }
 
-int tlq_debug_check_gemv_ring_addressing(int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth) {
-  return check_gemv_ring(N, K, group, rows_per_block, waves, depth);
+int tlq_debug_check_gemv_ring_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth) {
+  return check_gemv_ring(M, N, K, group, rows_per_block, waves, depth);
 }
 
 }  // extern "C"

@@ -5,6 +5,7 @@
 namespace tlq {
 int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch, int64_t M,
                int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
+bool gemv_ring_applies(int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype, const void* scales, const void* zeros);
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group);
@@ -116,6 +117,10 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
     // M.  Measured crossovers: fp16 GEMV wins at M = 1, and at M = 2 while K <= 4096; the bf16 GEMV dequantises
     // element by element and wins only at M = 1 in its register-resident form, for rows of up to 8192 values.
     const bool skinny_ok = M <= 64 && K % 128 == 0 && fits32(M, K * 2) && fits32(N, K / 2);
+    // two fp16 activation rows on many weight rows: the ring GEMV (8.9 against 10.3 us for the decode kernel at
+    // 11008 x 4096, 5.2 against 6.2 us at 8192 x 2048; with 4096 rows, one per wavefront, the decode kernel is 5 % ahead)
+    if (M == 2 && N >= 8192 && gemv_ring_applies(M, N, K, group, in_dtype, scales, zeros))
+      return gemv_w4a16(A, w_packed, scales, zeros, C, 1, M, N, K, group, zero_scalar, in_dtype, out_dtype, st);
     if (decode_preferred(M, N, K) && decode_ok && g_w4a16_decode)
       return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, dp, nullptr, st);
     if (M > 4)

@@ -590,12 +590,17 @@ __global__ __launch_bounds__(MAXT) void gemv_w4a16_bf16_rows_kernel(const bf16_t
 // shapes this is used for) before anything else happens, the staging data (activations, scales, zero points of the
 // work-group's rows) travels the same way ahead of them, and a row is read back from the wavefront's private LDS slot
 // by the lane that asked for it.  Same sums in the same order as the rows kernel: the results are the same bits.
-template <typename T, int ITERS, int D>
+// MT = 2 activation rows (fp16): a row's nibbles are expanded once and multiplied with both activation rows, whose
+// prepared chunks the wavefront keeps in registers (36 per activation row and 2048 values of K).  Every further
+// activation row costs about 2 us on the cfg-2 shape: from three rows on the decode kernel (matrix cores) is ahead.
+template <typename T, int ITERS, int D, int MT>
 __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
-                                                              const T* __restrict__ scales, const T* __restrict__ zeros,
-                                                              void* __restrict__ C, int N, int K, int group_shift,
-                                                              float zero_scalar, int out_dtype, int rows_per_block) {
+                                                                             const T* __restrict__ scales,
+                                                                             const T* __restrict__ zeros, void* __restrict__ C,
+                                                                             int N, int K, int group_shift, float zero_scalar,
+                                                                             int out_dtype, int rows_per_block) {
   constexpr bool F16 = __is_same(T, half_t);
+  static_assert(MT == 1 || (F16 && MT == 2), "two activation rows: fp16 only");
   typedef __attribute__((address_space(3))) uint8_t* lptr_t;
   extern __shared__ __align__(16) uint8_t smem[];
   const int lane = threadIdx.x & 63;
@@ -605,7 +610,7 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
   const int r0 = blockIdx.x * rows_per_block;
   const int r1 = r0 + rows_per_block < N ? r0 + rows_per_block : N;
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lptr_t)smem);
-  const addr::RingLayout L = addr::ring_layout(nwaves, D, ITERS, K, rows_per_block, groups);
+  const addr::RingLayout L = addr::ring_layout(nwaves, D, ITERS, K, rows_per_block, groups, MT);
   const bool has_s = scales != nullptr, has_z = zeros != nullptr;
   auto dma16 = [&](uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
@@ -625,7 +630,7 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
 
   // ---- staging data first (loads retire in issue order: once only a wavefront's weight rows are outstanding its
   // staging loads have landed), then the first D rows ----
-  const int a_pieces = chunks * 4;
+  const int a_pieces = chunks * 4 * MT;  // the activation rows are contiguous
   for (int p0 = wave * 64; p0 < a_pieces; p0 += nwaves * 64)
     dma16(lds0 + L.act + (uint32_t)p0 * 16u, addr::ring_stage_voff(p0, lane, a_pieces), (const uint8_t*)A);
   const int sz_pieces = ((r1 - r0) * groups) >> 3;  // groups is a multiple of 8
@@ -661,20 +666,22 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
 
   // every wavefront prepares the activations of its lanes' chunks itself (fp16: pairs in unpack order and the chunk
   // sums; bf16: the 32 values as they are)
-  ActF16 act[F16 ? ITERS : 1];
+  ActF16 act[MT][F16 ? ITERS : 1];
   uint4_t actn[F16 ? 1 : ITERS][4];
 #pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    uint4_t raw[4];
+  for (int m = 0; m < MT; ++m)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) raw[j] = *(const uint4_t*)(smem + L.act + (uint32_t)(cc[it] * 4 + j) * 16u);
-    if constexpr (F16) {
-      permute_act(act[it], raw);
-    } else {
+    for (int it = 0; it < ITERS; ++it) {
+      uint4_t raw[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) actn[it][j] = raw[j];
+      for (int j = 0; j < 4; ++j) raw[j] = *(const uint4_t*)(smem + L.act + (uint32_t)((m * chunks + cc[it]) * 4 + j) * 16u);
+      if constexpr (F16) {
+        permute_act(act[m][it], raw);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) actn[it][j] = raw[j];
+      }
     }
-  }
   const T* const lds_s = (const T*)(smem + L.s);
   const T* const lds_z = (const T*)(smem + L.z);
   const NibbleMagic mg = make_nibble_magic();
@@ -699,9 +706,40 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
       issue(i + D, slot);
     }
     float acc = 0.f;
-    if constexpr (F16) {
+    if constexpr (F16 && MT > 1) {
+      float accm[MT];
 #pragma unroll
-      for (int it = 0; it < ITERS; ++it) acc += chunk_term_biased(w[it], act[it], sv[it], zv[it], mg);
+      for (int m = 0; m < MT; ++m) accm[m] = 0.f;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        half2_t e[16];  // the chunk's 32 nibbles with the unpack bias left in, once for all activation rows
+        const uint32_t x[4] = {w[it].x, w[it].y, w[it].z, w[it].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t v = x[j], v8 = v >> 8;
+          e[4 * j + 0] = bitcast<half2_t>(bfi(mg.m_lo, v, mg.b_lo));
+          e[4 * j + 1] = bitcast<half2_t>(bfi(mg.m_hi, v, mg.b_hi));
+          e[4 * j + 2] = bitcast<half2_t>(bfi(mg.m_lo, v8, mg.b_lo));
+          e[4 * j + 3] = bitcast<half2_t>(bfi(mg.m_hi, v8, mg.b_hi));
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          float d = 0.f;
+#pragma unroll
+          for (int p = 0; p < 16; ++p) d = __builtin_amdgcn_fdot2(e[p], act[m][it].a[p], d, false);
+          accm[m] += (float)sv[it] * (d - __builtin_fmaf((float)zv[it], act[m][it].sum, act[m][it].bsum));
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const float v = wave_sum_to_lane63(accm[m]);
+        if (lane == 63) store_out(C, (int64_t)m * N + r0 + lrow, v, out_dtype);
+      }
+      slot = slot + 1 == D ? 0 : slot + 1;
+      continue;
+    } else if constexpr (F16) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) acc += chunk_term_biased(w[it], act[0][it], sv[it], zv[it], mg);
     } else {
       bool integral = true;  // small integer zero points fold exactly into one fused multiply-add per weight
 #pragma unroll
@@ -909,9 +947,9 @@ struct RingPlan {
   int iters, depth, waves, rows_per_block, blocks;
   uint32_t lds_bytes;
 };
-static RingPlan plan_gemv_ring(int64_t batch, int64_t N, int64_t K, int group_shift, int cus) {
+static RingPlan plan_gemv_ring(int64_t batch, int64_t M, int64_t N, int64_t K, int group_shift, int cus) {
   RingPlan p{false, 0, 0, 0, 0, 0, 0};
-  if (batch != 1 || N < 1 || N > 0x7fffffff || K < 32 || K % 32 != 0 || K > 4096 || group_shift < 5 || cus < 1) return p;
+  if (batch != 1 || M < 1 || M > 2 || N < 1 || N > 0x7fffffff || K < 32 || K % 32 != 0 || K > 4096 || group_shift < 5 || cus < 1) return p;
   const int groups = (int)(K >> group_shift);
   if (groups < 8 || groups % 8 != 0 || ((int64_t)groups << group_shift) != K) return p;
   p.waves = (g_gemv_waves16 >= 1 && g_gemv_waves16 <= 16) ? g_gemv_waves16 : 16;
@@ -926,15 +964,16 @@ static RingPlan plan_gemv_ring(int64_t batch, int64_t N, int64_t K, int group_sh
   const int per_wave = (int)ceil_div(rpb, (int64_t)p.waves);
   const int want = (g_gemv_depth >= 1 && g_gemv_depth <= 3) ? g_gemv_depth : 1;
   p.depth = per_wave < want ? per_wave : want;
-  p.lds_bytes = addr::ring_layout(p.waves, p.depth, p.iters, (int)K, p.rows_per_block, groups).total;
+  if (M > 1 && p.depth > 2) p.depth = 2;
+  p.lds_bytes = addr::ring_layout(p.waves, p.depth, p.iters, (int)K, p.rows_per_block, groups, (int)M).total;
   p.ok = p.lds_bytes <= 160 * 1024;
   return p;
 }
 
-template <typename T, int ITERS, int D>
+template <typename T, int ITERS, int D, int MT>
 static int launch_gemv_ring(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int N, int K,
                             int group_shift, float zero_scalar, int out_dtype, const RingPlan& p, hipStream_t st) {
-  auto kern = gemv_w4a16_ring_kernel<T, ITERS, D>;
+  auto kern = gemv_w4a16_ring_kernel<T, ITERS, D, MT>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -952,20 +991,31 @@ static int launch_gemv_ring(const void* A, const void* Wp, const void* scales, c
 // 1 (default): the ring kernel where it applies; 0: never
 static thread_local int g_gemv_ring = 1;
 
-template <typename T>
+template <typename T, int MT>
 static int dispatch_gemv_ring(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int N, int K,
                               int group_shift, float zero_scalar, int out_dtype, const RingPlan& p, hipStream_t st) {
 #define TLQ_RING_CASE(IT, DD) \
-  return launch_gemv_ring<T, IT, DD>(A, Wp, scales, zeros, C, N, K, group_shift, zero_scalar, out_dtype, p, st)
+  return launch_gemv_ring<T, IT, DD, MT>(A, Wp, scales, zeros, C, N, K, group_shift, zero_scalar, out_dtype, p, st)
   if (p.iters == 1) {
     if (p.depth == 1) TLQ_RING_CASE(1, 1);
-    if (p.depth == 2) TLQ_RING_CASE(1, 2);
-    TLQ_RING_CASE(1, 3);
+    if (p.depth == 2 || MT > 1) TLQ_RING_CASE(1, 2);
+    if constexpr (MT == 1) TLQ_RING_CASE(1, 3);
   }
   if (p.depth == 1) TLQ_RING_CASE(2, 1);
-  if (p.depth == 2) TLQ_RING_CASE(2, 2);
-  TLQ_RING_CASE(2, 3);
+  if (p.depth == 2 || MT > 1) TLQ_RING_CASE(2, 2);
+  if constexpr (MT == 1) TLQ_RING_CASE(2, 3);
 #undef TLQ_RING_CASE
+  return 1;
+}
+
+// whether the ring kernel takes this problem (the automatic kernel choice of tlq_gemm_w4a16 asks)
+bool gemv_ring_applies(int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype, const void* scales, const void* zeros) {
+  if (!g_gemv_ring || g_gemv_rows < 0 || group < 32 || (group & (group - 1)) != 0) return false;
+  if ((((uintptr_t)scales | (uintptr_t)zeros) & 15) != 0) return false;
+  if (in_dtype != TLQ_F16 && !(in_dtype == TLQ_BF16 && M == 1)) return false;
+  int shift = 0;
+  while (((int64_t)1 << shift) < group) ++shift;
+  return plan_gemv_ring(1, M, N, K, shift, cu_count()).ok;
 }
 
 // wavefronts per work-group and work-groups per CU of the rows kernel for this K
@@ -1042,9 +1092,16 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     const int R = g_gemv_rows > 0 ? g_gemv_rows : (streaming ? 2 : 1);
     const int bpc = g_gemv_unroll ? g_gemv_unroll : (streaming ? 64 : 8);  // grid size cap, blocks per CU
     const int depth_req = g_gemv_depth;
-    if (M == 1 && g_gemv_ring && g_gemv_rows >= 0 && (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0) {
-      const RingPlan rp = plan_gemv_ring(batch, N, K, shift, cu_count());
-      if (rp.ok) return dispatch_gemv_ring<half_t>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st);
+    if (M <= 2 && g_gemv_ring && g_gemv_rows >= 0 && (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0) {
+      const RingPlan rp = plan_gemv_ring(batch, M, N, K, shift, cu_count());
+#define TLQ_RING_M(MM) \
+  case MM:             \
+    return dispatch_gemv_ring<half_t, MM>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st)
+      if (rp.ok) switch ((int)M) {
+          TLQ_RING_M(1);
+          TLQ_RING_M(2);
+        }
+#undef TLQ_RING_M
     }
     if (M == 1 && K <= 16384 && g_gemv_rows >= 0 && rows_kernel_fits(batch, N, K, shift))
       return dispatch_gemv_rows<half_t>(A, Wp, scales, zeros, C, batch, N, K, shift, zero_scalar, out_dtype, st);
@@ -1082,8 +1139,8 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
     int shift = 0;
     while (((int64_t)1 << shift) < group) ++shift;
     if (M == 1 && pow2 && g_gemv_ring && g_gemv_rows >= 0 && (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0) {
-      const RingPlan rp = plan_gemv_ring(batch, N, K, shift, cu_count());
-      if (rp.ok) return dispatch_gemv_ring<bf16_t>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st);
+      const RingPlan rp = plan_gemv_ring(batch, 1, N, K, shift, cu_count());
+      if (rp.ok) return dispatch_gemv_ring<bf16_t, 1>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st);
     }
     if (M == 1 && pow2 && K <= 16384 && g_gemv_rows >= 0 && rows_kernel_fits(batch, N, K, shift)) {
       return dispatch_gemv_rows<bf16_t>(A, Wp, scales, zeros, C, batch, N, K, shift, zero_scalar, out_dtype, st);
@@ -1128,14 +1185,14 @@ void tlq_tune_gemv(int rows_per_wave, int waves_per_block) {
 }
 void tlq_tune_gemv_ring(int on) { tlq::g_gemv_ring = on != 0; }
 
-int tlq_debug_gemv_ring_plan(int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
+int tlq_debug_gemv_ring_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
   int shift = 0;
   while (((int64_t)1 << shift) < group) ++shift;
   if (group < 1 || ((int64_t)1 << shift) != group) {
     tlq::set_error("tlq_debug_gemv_ring_plan: the group size must be a power of two");
     return -1;
   }
-  const tlq::RingPlan p = tlq::plan_gemv_ring(1, N, K, shift, cus);
+  const tlq::RingPlan p = tlq::plan_gemv_ring(1, M, N, K, shift, cus);
   if (plan_out) {
     int64_t* o = (int64_t*)plan_out;
     o[0] = p.iters, o[1] = p.depth, o[2] = p.waves, o[3] = p.rows_per_block, o[4] = p.blocks, o[5] = p.lds_bytes;
