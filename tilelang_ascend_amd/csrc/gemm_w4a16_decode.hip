@@ -131,8 +131,10 @@ __global__ __launch_bounds__(1024) void w4a16_decode_kernel(const T* __restrict_
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const uint32_t voff = (uint32_t)(addr::dec_a_off(lane, mt, kb, i, M, K, k0) - (k0 + kb * 128) * 2);
-        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(mine_lds + STG + (uint32_t)(i * 1024)), "v"(voff), "s"(asb)
-                     : "memory");
+        // rows past M are not fetched: what the staging area holds for them only reaches output rows that are never stored
+        if (mt * 16 + 4 * i + (lane >> 4) < M)
+          asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(mine_lds + STG + (uint32_t)(i * 1024)), "v"(voff), "s"(asb)
+                       : "memory");
       }
     };
     issue_block(0, 0);
