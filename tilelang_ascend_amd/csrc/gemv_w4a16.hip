@@ -962,7 +962,8 @@ static RingPlan plan_gemv_ring(int64_t batch, int64_t M, int64_t N, int64_t K, i
   // one row in flight per wavefront: 16 wavefronts on 256 CUs ask for 8 MB at a time, about what the memory system
   // holds in flight at its full rate; with two or three rows per wavefront the same launch measured 3 - 17 % slower
   const int per_wave = (int)ceil_div(rpb, (int64_t)p.waves);
-  const int want = (g_gemv_depth >= 1 && g_gemv_depth <= 3) ? g_gemv_depth : 1;
+  // (from about 64 MB of weights on the launch is long enough for two rows in flight to be level or 2 - 4 % ahead)
+  const int want = (g_gemv_depth >= 1 && g_gemv_depth <= 3) ? g_gemv_depth : (N * (K / 2) > ((int64_t)64 << 20) ? 2 : 1);
   p.depth = per_wave < want ? per_wave : want;
   if (M > 1 && p.depth > 2) p.depth = 2;
   p.lds_bytes = addr::ring_layout(p.waves, p.depth, p.iters, (int)K, p.rows_per_block, groups, (int)M).total;
