@@ -203,6 +203,22 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
       return 1;
     }
   }
+  if (algo == TLQ_ALGO_AUTO && M >= 1 && N >= 1 && K > 0 && N < kMaxDim && K < kMaxDim) {
+    // Small problems are launch-bound: a second launch (for the partial sums of K slices, or for the dequantisation
+    // pass) costs more than it saves.  Measured: 256^3 6.5 against 9.5 us, M = 128 on 1024 x 512 9.7 against 12.4 us,
+    // M = 64 on 1024^2 6.7 against 11.4 us and on 2048^2 11.0 against 13.0 us; the streaming kernel with its K slices is
+    // ahead from M = 256 on 1024^2 (15.5 against 20.8 us) and for M = 40 on 1024 rows of 4096 values (13.0 against 16.5 us).
+    const int64_t nk = N * K;
+    if ((M <= 64 && (nk <= ((int64_t)1 << 21) || (nk <= ((int64_t)1 << 22) && K <= 2048))) || nk <= ((int64_t)1 << 19))
+      return tlq_gemm_w4a16(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, stream);
+    // 17 .. 32 activation rows whose K is one chunk of the decode kernel: that kernel, which needs no workspace
+    // (M = 32, N = 14336, K = 4096: 16.8 against 20 us for the streaming kernel)
+    if (M > 16 && M <= 32 && g_w4a16_decode && group > 0) {
+      const DecodePlan dp = w4a16_decode_plan(M, N, K, group, cu_count_or_default());
+      if (dp.ok && dp.chunks == 1 && (((uintptr_t)scales | (uintptr_t)zeros) & 3) == 0)
+        return tlq_gemm_w4a16(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, stream);
+    }
+  }
   const int64_t need = (N > 0 && K > 0) ? N * K * 2 : 0;
   const bool have = workspace != nullptr && workspace_bytes >= need && aligned16(workspace);
   if (algo == TLQ_ALGO_TWO_PASS)
