@@ -1,0 +1,58 @@
+"""The automatic kernel choice of tlq_gemm_w4a16_ws (what ops.w4a16_gemm and the benchmark call): small, launch-bound
+problems and 17 .. 32 activation rows take the single-launch kernels although a workspace is there, two fp16 activation
+rows on many weight rows take the ring GEMV.  Observed through the outputs: the automatic choice must return the bits of
+the kernel it is meant to pick (the kernels differ in summation order), and every result is checked against the oracle."""
+import pytest
+import torch
+
+from helpers import assert_bit_equal, check_float_output, gen, make_w4, w4a16_reference
+
+pytestmark = pytest.mark.gpu
+
+
+def run_ws(A, Wp, s, z, group, algo, workspace=True):
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    M, K = A.shape
+    N = Wp.shape[0]
+    dA, dW, dS, dZ = A.cuda(), Wp.cuda(), s.cuda(), z.cuda()
+    need = max(lib.tlq_w4a16_workspace_bytes(M, N, K), N * K * 2, 16) if workspace else 0
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    print(f"kernel choice M={M} N={N} K={K} g={group} algo={algo} workspace={need}", flush=True)
+    _abi.check(lib.tlq_gemm_w4a16_ws(P(dA), P(dW), P(dS), P(dZ), P(C), M, N, K, group, 0.0, _abi.F16, _abi.F16, algo,
+                                     P(ws) if workspace else None, need, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return C.cpu()
+
+
+def cases():
+    from tilelang_ascend_amd import _abi
+
+    return [
+        # M, N, K, group, the kernel the automatic choice is meant to take
+        (256, 256, 256, 128, _abi.ALGO_MFMA),      # the reference's own CPU-runnable case: one launch of the tile kernel
+        (128, 1024, 512, 128, _abi.ALGO_MFMA),
+        (64, 1024, 1024, 128, _abi.ALGO_SKINNY),
+        (48, 4096, 1024, 64, _abi.ALGO_SKINNY),
+        (24, 4096, 4096, 128, _abi.ALGO_DECODE),
+        (32, 1024, 2048, 32, _abi.ALGO_DECODE),
+        (2, 8192, 2048, 64, _abi.ALGO_GEMV),       # ring kernel, two activation rows
+        (2, 4096, 4096, 128, _abi.ALGO_DECODE),    # 4096 rows: one per wavefront, the decode kernel is ahead
+        (64, 4096, 4096, 128, _abi.ALGO_STREAM),   # large enough for K slices and a second launch
+        (256, 1024, 1024, 128, _abi.ALGO_STREAM),
+    ]
+
+
+@pytest.mark.parametrize("case", range(10))
+def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
+    from tilelang_ascend_amd import _abi
+
+    M, N, K, group, algo = cases()[case]
+    A = torch.randn(M, K, generator=gen(90 + case)).to(torch.float16)
+    Wp, s, z = make_w4(N, K, group, torch.float16, "int", seed=110 + case)
+    auto = run_ws(A, Wp, s, z, group, _abi.ALGO_AUTO)
+    want = run_ws(A, Wp, s, z, group, algo)
+    assert_bit_equal(auto, want, f"automatic choice vs algo {algo} for M={M} N={N} K={K}")
+    check_float_output(auto, w4a16_reference(A, Wp, s, z, group), "automatic choice vs oracle")
