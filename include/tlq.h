@@ -294,6 +294,10 @@ int tlq_debug_gemv_rows_plan(int64_t batch, int64_t N, int64_t K, int64_t group,
  * tlq_debug_check_gemv_ring_addressing walks, on the host, every load of the first, middle and last work-groups of such a
  * launch (bounds of every global read and LDS write, coverage of the staging data and of the rows, ring order against the
  * kernel's wait counts); 0 = consistent.  No counterpart in the reference. */
+/* Output tile (128 or 256, square) the MFMA GEMMs take for `batch` problems of M x N outputs on the current device (256 CUs
+ * when there is none): by machine fill, see tlq_tune_gemm_tile.  fused = 1: the fused W4A16 tile kernel's rule.  Host only;
+ * no counterpart in the reference (its block_M / block_N are arguments, example_dequant_gemm_fine_grained.py:437). */
+int tlq_debug_gemm_tile(int64_t batch, int64_t M, int64_t N, int fused);
 int tlq_debug_gemv_ring_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
 int tlq_debug_check_gemv_ring_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth);
 
@@ -309,6 +313,8 @@ void tlq_tune_gemv_ring(int on);                             /* 1 (default): a s
                                                               * ring kernel where it applies; 0: on the kernels it replaced (for one
                                                               * activation row the same results, bit for bit) */
 void tlq_tune_gemm_band(int tile_rows);                       /* tile rows per band of the MFMA kernels' tile order (default 4) */
+void tlq_tune_gemm_tile(int tile);                            /* square tile of the plain 16-bit GEMM (and of the second of the two W4A16 passes):
+                                                              * 128 | 256, 0 = by the number of output tiles */
 void tlq_tune_gemm_slots(int on);                            /* 1 (default): 256 x 256 tiles of the plain 16-bit GEMM with [N, K] weights and of the
                                                               * int8 GEMMs run on the kernel that cuts LDS into five operand-tile slots
                                                               * (whole 128-byte stages of K only); 0: always the two-stage kernel */

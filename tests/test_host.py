@@ -182,3 +182,24 @@ def test_build_lock_is_exclusive_and_stale_libraries_are_detected(tmp_path, monk
     assert build.is_stale()
     (tmp_path / "libtlq.fingerprint").write_text(build.source_fingerprint() + "\n")
     assert not build.is_stale() and build.is_current()
+
+
+def test_tile_choice_by_machine_fill():
+    """128 x 128 or 256 x 256 output tiles: the choice follows how full each makes the machine (256 CUs without a GPU),
+    the small tiles' fill weighted by their pace.  The table is what was measured faster on an MI355X."""
+    from tilelang_ascend_amd import _abi
+
+    tile = _abi.load().tlq_debug_gemm_tile
+    if _abi.load().tlq_device_cu_count() not in (0, -1, 256):
+        import pytest
+
+        pytest.skip("table holds for 256 CUs")
+    plain = {(1, 2048, 4096): 128, (1, 1536, 4096): 128, (1, 3072, 4096): 256, (1, 4096, 4096): 256, (1, 2048, 11008): 256,
+             (1, 1024, 14336): 256, (1, 1024, 4096): 128, (1, 2560, 5120): 256, (1, 512, 14336): 128, (1, 768, 8192): 128,
+             (8, 2048, 4096): 256, (3, 2048, 4096): 256, (2, 1024, 4096): 128, (1, 8192, 14336): 256, (1, 100, 4096): 128}
+    for (b, m, n), want in plain.items():
+        assert tile(b, m, n, 0) == want, (b, m, n)
+    fused = {(1, 2048, 4096): 128, (1, 1536, 4096): 128, (1, 3072, 4096): 256, (1, 2048, 11008): 256, (1, 512, 14336): 128,
+             (1, 1024, 14336): 256, (1, 4096, 4096): 256}
+    for (b, m, n), want in fused.items():
+        assert tile(b, m, n, 1) == want, (b, m, n)

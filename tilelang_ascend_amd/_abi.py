@@ -66,6 +66,8 @@ SIGNATURES = {
     "tlq_debug_check_gemv_ring_addressing": (_int, [_i64, _i64, _i64, _i64, _int, _int, _int]),
     "tlq_tune_gemm_band": (None, [_int]),
     "tlq_tune_gemm_slots": (None, [_int]),
+    "tlq_tune_gemm_tile": (None, [_int]),
+    "tlq_debug_gemm_tile": (_int, [_i64, _i64, _i64, _int]),
     "tlq_tune_w4a16_stream": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),
     "tlq_tune_w4a16_split": (None, [_int]),

@@ -1,6 +1,7 @@
 // extern "C" entry points of the GEMM family: argument validation, then dispatch.
 // Every shape assumption a kernel makes is checked here, before anything is launched.
 #include "tlq_common.h"
+#include "gemm_core.h"
 
 namespace tlq {
 int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch, int64_t M,
@@ -45,6 +46,7 @@ int gemm_w4a16_decode(const void* A, const void* Wp, const void* scales, const v
 
 thread_local int g_gemm_band_rows = 0;
 thread_local int g_gemm_slots = 1;
+extern thread_local int g_gemm_f16_tile;
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // compute units of the current device (256 when it cannot be asked, e.g. without a GPU)
 static int cu_count_or_default() {
@@ -68,6 +70,10 @@ extern "C" {
 
 void tlq_tune_gemm_band(int tile_rows) { tlq::g_gemm_band_rows = tile_rows < 0 ? 0 : tile_rows; }
 void tlq_tune_gemm_slots(int on) { tlq::g_gemm_slots = on != 0; }
+int tlq_debug_gemm_tile(int64_t batch, int64_t M, int64_t N, int fused) {
+  return tlq::prefer_small_tiles(batch, M, N, fused ? 0.65 : 0.72) ? 128 : 256;
+}
+void tlq_tune_gemm_tile(int tile) { tlq::g_gemm_f16_tile = (tile == 128 || tile == 256) ? tile : 0; }
 void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
 void tlq_tune_w4a16_decode(int on) { tlq::g_w4a16_decode = on != 0; }
 

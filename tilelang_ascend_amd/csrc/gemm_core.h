@@ -807,6 +807,24 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
 // were 2 for the int8 kernels, 4 for the plain 16-bit GEMM and 8 for the fused W4A16 kernel; 1 = plain row-major)
 extern thread_local int g_gemm_band_rows;
 
+// 128 x 128 or 256 x 256 output tiles?  The large tiles need half the operand traffic per product and run 1.25 - 1.3 PFLOP/s
+// (bf16) where the small ones reach 1.0 - 1.07, both with every CU busy; but one large tile per CU is a whole round, and
+// a launch with 128 of them leaves half the machine idle.  Fill = tiles / (rounds x CUs); the small tiles are taken
+// when their fill, weighted by 0.72, beats the large tiles' (measured on fifteen shapes: every choice this rule makes
+// was the faster one, e.g. M = 2048, N = 4096: 248 against 322 us; M = 3072, N = 4096: 99 (large) against 111 us).
+// (`weight`: pace of the small tiles relative to the large ones at equal fill; 0.65 for the fused W4A16 tile kernel,
+// whose small tiles also dequantise every weight twice as often.)
+inline bool prefer_small_tiles(int64_t batch, int64_t M, int64_t N, double weight = 0.72) {
+  if (M <= 128) return true;
+  int cus = tlq_device_cu_count();
+  if (cus <= 0) cus = 256;
+  const int64_t t256 = batch * ceil_div(M, (int64_t)256) * ceil_div(N, (int64_t)256);
+  const int64_t t128 = batch * ceil_div(M, (int64_t)128) * ceil_div(N, (int64_t)128);
+  const double fill256 = (double)t256 / (double)(ceil_div(t256, (int64_t)cus) * cus);
+  const double fill128 = (double)t128 / (double)(ceil_div(t128, (int64_t)cus) * cus);
+  return fill128 * weight > fill256;
+}
+
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,
                 int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what, int band_rows = 4) {

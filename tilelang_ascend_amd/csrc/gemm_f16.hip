@@ -124,7 +124,7 @@ static int run_f16_splitk(const void* A, const void* B, float* C, int64_t M, int
 
 int gemm_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
                     int in_dtype, int b_layout, hipStream_t st) {
-  const bool small = M <= 128 || ceil_div(M, 256) * ceil_div(N, 256) * split_k < 128;
+  const bool small = prefer_small_tiles(split_k, M, N);
   if (in_dtype == TLQ_F16)
     return small ? run_f16_splitk<MmaF16, 128, 128, 2, 2>(A, B, C, M, N, K, split_k, b_layout, st)
                  : run_f16_splitk<MmaF16, 256, 256, 2, 4>(A, B, C, M, N, K, split_k, b_layout, st);
@@ -132,10 +132,14 @@ int gemm_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N
                : run_f16_splitk<MmaBF16, 256, 256, 2, 4>(A, B, C, M, N, K, split_k, b_layout, st);
 }
 
+// tlq_tune_gemm_tile: 0 = automatic, 128 / 256 = that square tile
+thread_local int g_gemm_f16_tile = 0;
+
 template <class Mma>
 static int dispatch_f16(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int out_dtype,
                         int b_layout, hipStream_t st) {
-  if (M <= 128 || batch * ceil_div(M, 256) * ceil_div(N, 256) < 128)
+  const bool small = g_gemm_f16_tile ? g_gemm_f16_tile == 128 : prefer_small_tiles(batch, M, N);
+  if (small)
     return run_f16<Mma, 128, 128, 2, 2>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);
   if (g_gemm_slots && b_layout == TLQ_B_NK && K % 64 == 0) {  // whole 128-byte stages
     typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K * 2, M * K * 2, K * 2},

@@ -199,7 +199,7 @@ static int dispatch_w4a16(const W4Args& a) {
       tile = 32;
     else if (M <= 64)
       tile = 64;
-    else if (M <= 128 || (a.split <= 1 && ceil_div(M, 256) * ceil_div(N, 256) < 128))
+    else if (M <= 128 || (a.split <= 1 && prefer_small_tiles(1, M, N, 0.65)))
       tile = 128;  // few large tiles: smaller ones fill more CUs, unless K is being cut for that purpose
     else
       tile = 256;
