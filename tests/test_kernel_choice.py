@@ -42,10 +42,12 @@ def cases():
         (2, 4096, 4096, 128, _abi.ALGO_DECODE),    # 4096 rows: one per wavefront, the decode kernel is ahead
         (64, 4096, 4096, 128, _abi.ALGO_STREAM),   # large enough for K slices and a second launch
         (256, 1024, 1024, 128, _abi.ALGO_STREAM),
+        (16, 5120, 5120, 128, _abi.ALGO_DECODE),   # rows of 5120 values, 320 tiles of 16 weight rows (more than CUs): decode kernel on K chunks
+        (512, 4096, 2048, 128, _abi.ALGO_STREAM),  # 512 rows on 4096 weight rows: the tile kernels would fill half the machine
     ]
 
 
-@pytest.mark.parametrize("case", range(10))
+@pytest.mark.parametrize("case", range(12))
 def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
     from tilelang_ascend_amd import _abi
 

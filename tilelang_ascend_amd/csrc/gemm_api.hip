@@ -197,7 +197,9 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                          (((uintptr_t)scales | (uintptr_t)zeros) & 3) == 0;
     // measured on rows of 14336 values: with up to 16 activation rows the skinny kernel is level or ahead (no second
     // launch for the partial sums), from 17 rows on the decode kernel is 10 - 15 % ahead of the streaming kernel
-    if (dp.ok && dp.chunks > 1 && (algo == TLQ_ALGO_DECODE || M > 16) && args_ok && (M * N) % 4 == 0 && workspace && aligned16(workspace) &&
+    // (and whenever the weight rows make more 16-row tiles than there are CUs, i.e. more than one round of the skinny
+    // kernel's work-groups: N = 5120, K = 13824, M = 16: 15.8 against 23.6 us; N = 28672, K = 8192: 31.6 against 45.6 us)
+    if (dp.ok && dp.chunks > 1 && (algo == TLQ_ALGO_DECODE || M > 16 || ceil_div(N, (int64_t)16) > cu_count_or_default()) && args_ok && (M * N) % 4 == 0 && workspace && aligned16(workspace) &&
         workspace_bytes >= (int64_t)dp.chunks * M * N * 4)
       return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, dp,
                                (float*)workspace, (hipStream_t)stream);
@@ -240,8 +242,13 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                          (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) && (M * N) % 4 == 0 &&
                          ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0 && K > 0 && fits32(M, K * 2) && fits32(N, K / 2);
     const bool ws_ok = sp.ok && (sp.split == 1 || (workspace && aligned16(workspace) && workspace_bytes >= (int64_t)sp.split * M * N * 4));
-    // measured on the MLP shapes: 20 - 35 % ahead of the tile kernel up to 256 rows, level with it at 512
-    if (sp.ok && args_ok && ws_ok && (algo == TLQ_ALGO_STREAM || M <= 256))
+    // measured on the MLP shapes: 20 - 35 % ahead of the tile kernel up to 256 rows, level with it at 512 -- unless the
+    // tile kernels cannot fill the machine there (M = 512 on 4096 weight rows: 128 tiles of 128 x 128; K = 11008: 89
+    // against 137 us for the two passes, K = 4096: 34 against 43 us)
+    // (rows of more than 8192 values that the tile kernel can cut into enough K slices stay with it: N = 5120, K = 13824:
+    // 101 against 127 us)
+    if (sp.ok && args_ok && ws_ok &&
+        (algo == TLQ_ALGO_STREAM || M <= 256 || (tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
     if (algo == TLQ_ALGO_STREAM) {
@@ -319,7 +326,7 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
   if (algo != TLQ_ALGO_TWO_PASS) {
     const StreamPlan sp = w4a16_stream_plan(M, N, K, group, cu_count_or_default());
     const bool ws_ok = sp.ok && (M * N) % 4 == 0 && (sp.split == 1 || (ws_aligned && workspace_bytes >= (int64_t)sp.split * M * N * 4));
-    if (ws_ok && (algo == TLQ_ALGO_STREAM || M <= 256 || !(ws_aligned && workspace_bytes >= N * K * 2)))
+    if (ws_ok && (algo == TLQ_ALGO_STREAM || M <= 256 || tile_fill(1, M, N, 128) < 0.65 || !(ws_aligned && workspace_bytes >= N * K * 2)))  // (no tile kernel reads this layout: the alternative is the two passes)
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, sp,
                                (float*)workspace, (hipStream_t)stream);
     TLQ_REQUIRE(algo != TLQ_ALGO_STREAM, "tlq_gemm_w4a16_layout_ws: the streaming kernel does not take M=%lld N=%lld K=%lld group=%lld "

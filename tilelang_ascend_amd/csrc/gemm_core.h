@@ -812,17 +812,17 @@ extern thread_local int g_gemm_band_rows;
 // a launch with 128 of them leaves half the machine idle.  Fill = tiles / (rounds x CUs); the small tiles are taken
 // when their fill, weighted by 0.72, beats the large tiles' (measured on fifteen shapes: every choice this rule makes
 // was the faster one, e.g. M = 2048, N = 4096: 248 against 322 us; M = 3072, N = 4096: 99 (large) against 111 us).
+inline double tile_fill(int64_t batch, int64_t M, int64_t N, int64_t tile) {
+  int cus = tlq_device_cu_count();
+  if (cus <= 0) cus = 256;
+  const int64_t t = batch * ceil_div(M, tile) * ceil_div(N, tile);
+  return (double)t / (double)(ceil_div(t, (int64_t)cus) * cus);
+}
 // (`weight`: pace of the small tiles relative to the large ones at equal fill; 0.65 for the fused W4A16 tile kernel,
 // whose small tiles also dequantise every weight twice as often.)
 inline bool prefer_small_tiles(int64_t batch, int64_t M, int64_t N, double weight = 0.72) {
   if (M <= 128) return true;
-  int cus = tlq_device_cu_count();
-  if (cus <= 0) cus = 256;
-  const int64_t t256 = batch * ceil_div(M, (int64_t)256) * ceil_div(N, (int64_t)256);
-  const int64_t t128 = batch * ceil_div(M, (int64_t)128) * ceil_div(N, (int64_t)128);
-  const double fill256 = (double)t256 / (double)(ceil_div(t256, (int64_t)cus) * cus);
-  const double fill128 = (double)t128 / (double)(ceil_div(t128, (int64_t)cus) * cus);
-  return fill128 * weight > fill256;
+  return tile_fill(batch, M, N, 128) * weight > tile_fill(batch, M, N, 256);
 }
 
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
