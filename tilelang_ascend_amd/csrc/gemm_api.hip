@@ -121,7 +121,8 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
   if (algo == TLQ_ALGO_AUTO) {
     // The skinny kernel takes the same time for every M up to 16 (the weights bound it); the GEMV kernels grow with
     // M.  Measured crossovers: fp16 GEMV wins at M = 1, and at M = 2 while K <= 4096; the bf16 GEMV dequantises
-    // element by element and wins only at M = 1 in its register-resident form, for rows of up to 8192 values.
+    // element by element and wins only at M = 1 in its register-resident form (rows of up to 16384 values: level with the
+    // skinny kernel on 4096 weight rows, 15 against 25 us on 5120 rows of 13824 values).
     const bool skinny_ok = M <= 64 && K % 128 == 0 && fits32(M, K * 2) && fits32(N, K / 2);
     // two fp16 activation rows on many weight rows: the ring GEMV (8.9 against 10.3 us for the decode kernel at
     // 11008 x 4096, 5.2 against 6.2 us at 8192 x 2048; with 4096 rows, one per wavefront, the decode kernel is 5 % ahead)
@@ -134,9 +135,9 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
     else if (!skinny_ok)
       algo = TLQ_ALGO_GEMV;
     else if (in_dtype == TLQ_BF16)
-      algo = (M == 1 && K <= 8192 && (group & (group - 1)) == 0) ? TLQ_ALGO_GEMV : TLQ_ALGO_SKINNY;
+      algo = (M == 1 && K <= 16384 && (group & (group - 1)) == 0) ? TLQ_ALGO_GEMV : TLQ_ALGO_SKINNY;
     else
-      algo = (M == 1 || (M == 2 && K <= 4096)) ? TLQ_ALGO_GEMV : TLQ_ALGO_SKINNY;
+      algo = ((M == 1 && K <= 16384) || (M == 2 && K <= 4096)) ? TLQ_ALGO_GEMV : TLQ_ALGO_SKINNY;  // (longer rows: no register-resident GEMV)
   }
   if (algo == TLQ_ALGO_SKINNY) {
     TLQ_REQUIRE(M <= 64, "tlq_gemm_w4a16: the skinny kernel handles M <= 64 (got %lld)", (long long)M);
@@ -188,7 +189,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                       void* workspace, int64_t workspace_bytes, void* stream) {
   TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_DECODE, "tlq_gemm_w4a16_ws: bad algo %d", algo);
   // decode batches: rows longer than 4096 values run as chunks of K whose fp32 partial sums live in the workspace
-  if (((algo == TLQ_ALGO_AUTO && g_w4a16_decode && decode_preferred(M, N, K)) || algo == TLQ_ALGO_DECODE) && M <= 32 && M >= 1 && N >= 1 && K > 0 && group > 0 &&
+  if (((algo == TLQ_ALGO_AUTO && g_w4a16_decode && (decode_preferred(M, N, K) || K > 16384)) || algo == TLQ_ALGO_DECODE) && M <= 32 && M >= 1 && N >= 1 && K > 0 && group > 0 &&
       N < kMaxDim && K < kMaxDim) {
     const DecodePlan dp = w4a16_decode_plan(M, N, K, group, cu_count_or_default());
     const bool args_ok = A && w_packed && C && aligned16(A) && aligned16(w_packed) && aligned16(C) &&
@@ -197,9 +198,12 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                          (((uintptr_t)scales | (uintptr_t)zeros) & 3) == 0;
     // measured on rows of 14336 values: with up to 16 activation rows the skinny kernel is level or ahead (no second
     // launch for the partial sums), from 17 rows on the decode kernel is 10 - 15 % ahead of the streaming kernel
-    // (and whenever the weight rows make more 16-row tiles than there are CUs, i.e. more than one round of the skinny
-    // kernel's work-groups: N = 5120, K = 13824, M = 16: 15.8 against 23.6 us; N = 28672, K = 8192: 31.6 against 45.6 us)
-    if (dp.ok && dp.chunks > 1 && (algo == TLQ_ALGO_DECODE || M > 16 || ceil_div(N, (int64_t)16) > cu_count_or_default()) && args_ok && (M * N) % 4 == 0 && workspace && aligned16(workspace) &&
+    // (also for rows of more than 16384 values, which the register-resident GEMV does not take: M = 1, N = 8192,
+    // K = 28672: 32 against 49 us for the generic GEMV;
+    // from 64 MB of weights on -- N = 28672, K = 8192, M = 16: 31.6 against 45.6 us -- and where the skinny kernel's
+    // work-groups, one per 16 weight rows, would leave a fifth of the machine or more idle in their last round:
+    // N = 5120, K = 13824: 15.8 against 23.6 us; with 8192 or 13824 weight rows the skinny kernel is level or ahead)
+    if (dp.ok && dp.chunks > 1 && (algo == TLQ_ALGO_DECODE || M > 16 || K > 16384 || N * (K / 2) >= ((int64_t)64 << 20) || tile_fill(1, 16, N, 16) < 0.8) && args_ok && (M * N) % 4 == 0 && workspace && aligned16(workspace) &&
         workspace_bytes >= (int64_t)dp.chunks * M * N * 4)
       return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, dp,
                                (float*)workspace, (hipStream_t)stream);
