@@ -10,6 +10,7 @@ bool gemv_ring_applies(int64_t M, int64_t N, int64_t K, int64_t group, int in_dt
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group);
+double w4a16_mid_fill(int64_t M, int64_t N, int64_t K, int64_t group);
 int gemm_w4a16_mfma_splitk(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M,
                            int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype,
                            int64_t split, float* partial, hipStream_t st);
@@ -251,8 +252,15 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     // against 137 us for the two passes, K = 4096: 34 against 43 us)
     // (rows of more than 8192 values that the tile kernel can cut into enough K slices stay with it: N = 5120, K = 13824:
     // 101 against 127 us)
+    // Small quantisation groups shorten the K slices (16 groups each): when the partial sums (split x M x N x 4 bytes,
+    // written and read back) outweigh the packed weights, the tile kernel, which cuts K as it likes, is ahead
+    // (groups of 32, M = 256, N = 11008, K = 4096: 56 against 74 us; N = K = 8192: 64 against 90 us).
+    // (Only where the partial sums are tens of MB: on 4096 weight rows, or below, the streaming kernel stays ahead.)
+    // And only where the tile kernel finds a K cut that fills the machine: rows of 11008 = 2 x 43 x 128 values can only be halved.
+    const bool slices_too_short = (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
+                                  w4a16_mid_fill(M, N, K, group) >= 0.66;
     if (sp.ok && args_ok && ws_ok &&
-        (algo == TLQ_ALGO_STREAM || M <= 256 || (tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
+        (algo == TLQ_ALGO_STREAM || (M <= 256 && !slices_too_short) || (!slices_too_short && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
     if (algo == TLQ_ALGO_STREAM) {

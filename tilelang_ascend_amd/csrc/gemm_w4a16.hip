@@ -706,6 +706,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4_t* __re
 // MLP shapes), slices of at least 512 values that are whole stages and whole quantisation groups.  1 = no split.
 static thread_local int g_w4a16_split = 0;  // forced number of K slices for tuning runs (0 = automatic)
 
+// fraction of the work-group places (256, or 512 for the smaller tiles) that the tile kernel fills with the K cut it would take
+double w4a16_mid_fill(int64_t M, int64_t N, int64_t K, int64_t group);
+
 int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group) {
   // Where cutting K pays (measured against the two passes on the MLP shapes): up to M = 512 always, up to
   // M = 2048 while the 256 x 256 output tiles would fill at most a quarter of the chip.
@@ -725,6 +728,13 @@ int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group) {
   for (int64_t s = want < 16 ? want : 16; s >= 2; --s)
     if (K % s == 0 && (K / s) % unit == 0 && K / s >= 512) return (M > 256 && tiles * s * 3 < places * 2) ? 1 : s;
   return 1;
+}
+
+double w4a16_mid_fill(int64_t M, int64_t N, int64_t K, int64_t group) {
+  const int64_t bm = M <= 32 ? 32 : (M <= 64 ? 64 : (M <= 128 ? 128 : 256)), bn = (M <= 32 || (M > 64 && M <= 128)) ? 128 : 256;
+  const int64_t tiles = ceil_div(M, bm) * ceil_div(N, bn), places = bm == 256 ? 256 : 512;
+  const double f = (double)(tiles * w4a16_mid_split(M, N, K, group)) / (double)places;
+  return f > 1.0 ? 1.0 : f;
 }
 
 void launch_splitk_reduce(const float* partial, void* C, int64_t M, int64_t N, int split, int out_dtype, hipStream_t st) {
