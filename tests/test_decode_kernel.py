@@ -41,8 +41,11 @@ def test_decode_plan_rejects_what_the_kernel_cannot_do_and_the_check_catches_a_w
     from tilelang_ascend_amd import _abi
 
     lib = _abi.load()
-    for M, N, K, group in ((33, 64, 256, 64), (0, 64, 256, 64), (4, 64, 384, 64), (4, 64, 256, 96), (4, 64, 256, 16), (4, 3, 256, 256)):
+    for M, N, K, group in ((33, 64, 256, 64), (0, 64, 256, 64), (4, 64, 384, 64), (4, 64, 256, 96), (4, 64, 256, 16), (4, 3, 256, 256),
+                           (24, 100, 256, 64)):  # (two activation tiles on rows of 256 values: one wavefront, nobody adds up the second)
         assert not _plan(M, N, K, group)[0], (M, N, K, group)
+    assert _plan(24, 100, 512, 64)[0] and _plan(16, 100, 256, 64)[0]
+    assert lib.tlq_debug_check_decode_addressing(24, 128, 256, 64, 2, 1, 1, 8) != 0 and "add up" in _abi.last_error()
     # a launch that does not cover K, or leaves tiles out, fails the walk
     assert lib.tlq_debug_check_decode_addressing(16, 512, 4096, 128, 1, 1, 8, 32) != 0 and "slices" in _abi.last_error()
     assert lib.tlq_debug_check_decode_addressing(16, 512, 4096, 128, 1, 1, 16, 64) != 0 and "work-groups" in _abi.last_error()
@@ -103,6 +106,31 @@ def test_decode_one_hot_rows_return_the_dequantised_weights(in_dtype, zeros_kind
     want = W[:, cols].T.contiguous()
     assert_bit_equal(run_decode(A, Wp, s, z, group), want, f"one-hot {in_dtype} zeros={zeros_kind}")
     assert_bit_equal(run_decode(A, Wp, s, z, group, torch.float32), want.float(), f"one-hot f32 out {in_dtype} zeros={zeros_kind}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,group", [(24, 100, 256, 64), (32, 64, 256, 128), (20, 48, 512, 32), (17, 1000, 768, 256)])
+def test_short_rows_with_more_than_sixteen_activation_rows(M, N, K, group):
+    """Rows of 256 values are one wavefront's slice: with two activation tiles the decode kernel does not apply (the
+    automatic choice without a workspace takes another kernel); from 512 values on it does."""
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    A = torch.randn(M, K, generator=gen(64)).to(torch.float16)
+    Wp, s, z = make_w4(N, K, group, torch.float16, "int", seed=65)
+    dA, dW, dS, dZ = A.cuda(), Wp.cuda(), s.cuda(), z.cuda()
+    want = w4a16_reference(A, Wp, s, z, group)
+    for algo in (_abi.ALGO_AUTO, _abi.ALGO_DECODE):
+        C = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        print(f"short rows M={M} N={N} K={K} g={group} algo={algo}", flush=True)
+        rc = lib.tlq_gemm_w4a16(P(dA), P(dW), P(dS), P(dZ), P(C), M, N, K, group, 0.0, _abi.F16, _abi.F16, algo,
+                                torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        if algo == _abi.ALGO_DECODE and K == 256:
+            assert rc != 0 and "decode kernel" in _abi.last_error()
+            continue
+        assert rc == 0, _abi.last_error()
+        check_float_output(C.cpu(), want, f"short rows algo {algo}")
 
 
 @pytest.mark.gpu

@@ -296,6 +296,8 @@ int check_decode(int64_t M, int64_t N, int64_t K, int64_t group, int mt, int chu
   CHECK_OR_FAIL(chunks >= 1 && waves >= 1 && waves <= 16 && (int64_t)chunks * waves >= slices && (int64_t)(chunks - 1) * waves < slices,
                 "decode: %d chunks of %d wavefronts do not cover %lld slices", chunks, waves, (long long)slices);
   CHECK_OR_FAIL(grid_x >= 1 && grid_x <= tiles, "decode: %d work-groups for %lld tiles", grid_x, (long long)tiles);
+  // wavefront (ts mt + a) % waves adds up activation tile a of the ts-th weight tile: two tiles need two wavefronts
+  CHECK_OR_FAIL(waves >= mt, "decode: %d wavefront(s) cannot add up the partial sums of %d activation tiles", waves, mt);
   CHECK_OR_FAIL(((N * groups) & 1) == 0, "decode: scale tensors of an odd number of values");
   CHECK_OR_FAIL((int64_t)waves * addr::dec_wave_bytes(mt) <= 160 * 1024, "decode: LDS");
   int gshift = 0;

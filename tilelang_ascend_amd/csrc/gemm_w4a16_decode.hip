@@ -326,7 +326,9 @@ DecodePlan w4a16_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   gx = gx < 1 ? 1 : gx;
   p.grid_x = (int)(gx < tiles ? gx : tiles);
   p.lds_bytes = (int64_t)p.waves * addr::dec_wave_bytes(p.mt);
-  p.ok = p.lds_bytes <= 160 * 1024 && p.chunks <= 16;
+  // every activation tile's partial sums are added up by a wavefront of its own: a row of 256 values (one wavefront)
+  // cannot serve two activation tiles
+  p.ok = p.lds_bytes <= 160 * 1024 && p.chunks <= 16 && p.waves >= p.mt;
   return p;
 }
 
