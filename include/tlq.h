@@ -260,8 +260,10 @@ int tlq_act_quant_i8(const void* X, void* Y, void* S, int64_t M, int64_t N, int 
  * themselves use (no GPU needed; the reference has no counterpart, its tile addressing is generated by TVM).
  * tlq_debug_check_gemm_addressing walks every tile, thread, load instruction and stage of one operand:
  * source_kind 0 = row-major [rows, row_bytes] operand copied global -> LDS directly in tiles of `tile` rows by
- * `threads` threads; 1 = int8 [K = rows, N = row_bytes] weights in tiles of `tile` (128 | 256) columns.  It checks
- * global extents, LDS extents and coverage, and agreement with the operand-fragment reads.
+ * `threads` threads; 1 = int8 [K = rows, N = row_bytes] weights in tiles of `tile` (128 | 256) columns; 2 = 16-bit
+ * [K = rows, N = row_bytes (the number of columns)] weights in tiles of 128 | 256 columns (N a multiple of 8).  It
+ * checks global extents, LDS extents and coverage, agreement with the (transposing) operand-fragment reads and, for
+ * kind 2, that no half-wavefront read meets a bank twice.
  * tlq_debug_check_slots_schedule simulates the five-slot kernel's issue / wait / barrier order over `stages` stages
  * with `loads_per_tile` load instructions per wavefront and tile (the kernel's waits assume 4).
  * Both return 0 when everything holds, else 1 with tlq_last_error() naming the first violation. */

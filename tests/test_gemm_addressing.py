@@ -46,8 +46,21 @@ def test_the_walker_rejects_what_it_should():
     assert lib.tlq_debug_check_gemm_addressing(0, 256, 256, 64, 1024) != 0      # fewer load instructions than wavefronts
     assert lib.tlq_debug_check_gemm_addressing(0, 1 << 20, 1 << 13, 256, 512) != 0  # 8 GiB operand: 32-bit offsets
     assert lib.tlq_debug_check_gemm_addressing(1, 128, 24, 256, 512) != 0       # N not a multiple of 16
-    assert lib.tlq_debug_check_gemm_addressing(2, 128, 128, 256, 512) != 0
+    assert lib.tlq_debug_check_gemm_addressing(3, 128, 128, 256, 512) != 0
     assert "bad source kind" in _abi.last_error()
+    assert lib.tlq_debug_check_gemm_addressing(2, 128, 100, 256, 512) != 0      # 16-bit [K, N]: N not a multiple of 8
+    assert lib.tlq_debug_check_gemm_addressing(2, 128, 128, 64, 256) != 0       # ... tiles of 128 or 256 columns only
+    assert lib.tlq_debug_check_gemm_addressing(2, 128, 128, 256, 768) != 0      # ... 32 load instructions do not split over 12 wavefronts
+
+
+def test_16_bit_kn_operand_of_the_five_slot_kernel():
+    """[K, N] weights of the plain 16-bit GEMM (the reference's fp16_gemm layout, example_dequant_gemm_fine_grained.py:60-115):
+    direct loads inside the matrix for full, ragged and narrow column tiles, every LDS cell written once, the transposing
+    operand reads on the right rows and columns, and no bank met twice by a half-wavefront."""
+    lib = _abi.load()
+    for K, N in ((64, 8), (64, 256), (128, 264), (256, 1000), (4096, 4096), (1024, 11008), (192, 40), (72, 264), (328, 4104), (1, 8), (40, 72)):
+        _ok(lib.tlq_debug_check_gemm_addressing(2, K, N, 256, 512))   # five-slot and two-stage kernels, 256 x 256 tiles
+        _ok(lib.tlq_debug_check_gemm_addressing(2, K, N, 128, 256))   # two-stage kernel, 128 x 128 tiles
 
 
 def test_five_slot_schedule():

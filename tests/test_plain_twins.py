@@ -153,6 +153,39 @@ def test_fp16_gemm_kn_operand_large_tiles_and_k_tails(M, N, K):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("B,M,N,K", [(1, 2048, 4096, 1024), (1, 1024, 2056, 512), (1, 4096, 4096, 64), (2, 1000, 1288, 192), (3, 300, 264, 128), (1, 257, 8, 64)])
+def test_kn_operand_on_the_five_slot_kernel(dtype, B, M, N, K):
+    """[K, N] weights copied global -> LDS as they are and transposed by the operand read (ds_read_b64_tr_b16): whole 64-value
+    stages of K, N a multiple of 8, forced onto the 256 x 256 tiles so that small, ragged and batched problems take this
+    loader too.  Exact on ternary inputs; random inputs at the float-output bar; and the same bits as the two-stage kernel
+    that reads [K, N] weights through registers (tlq_tune_gemm_slots(0))."""
+    from helpers import check_float_output
+    from tilelang_ascend_amd import _abi
+    from tilelang_ascend_amd.ops import batch_matmul
+
+    lib = _abi.load()
+    kernel = batch_matmul(B, M, N, K, 128, 256, 64, dtype=dtype)
+    lib.tlq_tune_gemm_tile(256)
+    try:
+        a, b = _ternary((B, M, K), 66).to(DT[dtype]), _ternary((B, K, N), 67).to(DT[dtype])
+        got = kernel(a.cuda(), b.cuda()).cpu()
+        assert torch.equal(got, torch.matmul(a.float(), b.float()).to(DT[dtype]))
+        g = torch.Generator().manual_seed(68)
+        a, b = torch.randn(B, M, K, generator=g).to(DT[dtype]), torch.randn(B, K, N, generator=g).to(DT[dtype])
+        got = kernel(a.cuda(), b.cuda()).cpu()
+        want = torch.matmul(a.float(), b.float())
+        for i in range(B):
+            check_float_output(got[i], want[i], f"[K,N] five-slot {dtype} batch {i}")
+        lib.tlq_tune_gemm_slots(0)
+        two_stage = kernel(a.cuda(), b.cuda()).cpu()
+        assert torch.equal(got, two_stage), "five-slot vs two-stage kernel on [K, N] weights"
+    finally:
+        lib.tlq_tune_gemm_slots(1)
+        lib.tlq_tune_gemm_tile(0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
 @pytest.mark.parametrize("B,M,N,K", [(8, 1024, 1024, 1024), (3, 100, 72, 40), (2, 520, 264, 136), (20, 256, 512, 64), (1, 64, 64, 64)])
 def test_batch_matmul_matches_reference(dtype, B, M, N, K):
     from helpers import check_float_output

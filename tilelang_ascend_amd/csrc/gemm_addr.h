@@ -70,6 +70,37 @@ __host__ __device__ inline uint32_t knfrag_off(int lane, int wave_row0, int t) {
   return (uint32_t)(krow * BN + 8 * (r16 & 1)) + (uint32_t)((((wave_row0 >> 4) + t) ^ sw) << 4);
 }
 
+// ---- 16-bit source stored [K, N] (N contiguous): a stage is 64 k rows of BN columns (BN = 256 | 128, rows of 2 BN bytes),
+// copied as it is; the operand read transposes (ds_read_b64_tr_b16: lane i of a group of 16 supplies 8 bytes R[i]; lane j
+// receives the 16-bit values h = 0 .. 3 = R[4 h + j / 4][j % 4] -- established by probing).  With lane i supplying the row
+// of k = i / 4 at columns n_t + 4 (i % 4), lane j receives k = 0 .. 3 of column n_t + j; a second read four rows on
+// completes the eight values of an MFMA operand.  16-byte chunks of a k row are XOR-swizzled by an even number, which
+// keeps the 8-byte halves of a chunk together and spreads the eight rows a half-wavefront touches over all banks.
+__host__ __device__ inline int kn16_swz(int k) { return ((k & 3) << 1) | (((k >> 3) & 1) << 3); }
+// one wavefront instruction covers 512 / BN consecutive k rows
+template <int BN>
+__host__ __device__ inline int kn16_k(int lane, int wave, int j, int waves) {
+  static_assert(BN == 128 || BN == 256, "tile width");
+  return (j * waves + wave) * (512 / BN) + lane / (BN / 8);
+}
+template <int BN>
+__host__ __device__ inline uint32_t kn16_voff(int lane, int wave, int j, int waves, int cols_valid, uint32_t ld_bytes) {
+  const int k = kn16_k<BN>(lane, wave, j, waves);
+  const int pc = lane % (BN / 8);
+  int colb = (pc ^ kn16_swz(k)) * 16;
+  colb = colb < cols_valid * 2 ? colb : cols_valid * 2 - 16;  // whole chunks are clamped; those columns are masked at the store
+  return (uint32_t)k * ld_bytes + (uint32_t)colb;
+}
+// operand read of column block t (16 columns) of a wavefront whose columns start at wave_col0; k-step ks adds 32 rows,
+// the second read 4 rows (neither changes the swizzle)
+template <int BN>
+__host__ __device__ inline uint32_t kn16frag_off(int lane, int wave_col0, int t) {
+  const int i = lane & 15, q = lane >> 4;
+  const int krow = 8 * q + (i >> 2);
+  const int chunk = (wave_col0 >> 3) + 2 * t + ((i & 3) >> 1);
+  return (uint32_t)(krow * 2 * BN) + (uint32_t)((chunk ^ kn16_swz(krow)) << 4) + (uint32_t)(8 * (i & 1));
+}
+
 // ---- five-slot schedule (gemm_slots.h): tile t = 2 * stage (+ 1 for the weights) lives in slot t % 5 ----
 constexpr int kSlots = 5;
 __host__ __device__ inline int slot_of_tile(int t) { return t % kSlots; }

@@ -144,6 +144,79 @@ int check_kn_direct(int64_t K, int64_t N, int threads) {
   return 0;
 }
 
+// 16-bit [K, N] source in tiles of BN columns: every direct load inside the matrix (the partial last stage's register loads
+// too), every LDS cell of the [64 k][2 BN bytes] tile written once, every transposing operand read on the chunk that holds
+// its rows and columns, and no bank met twice by a half-wavefront.
+template <int BN>
+int check_kn16_direct(int64_t K, int64_t N, int threads) {
+  CHECK_OR_FAIL(threads % 64 == 0, "[K,N] 16-bit loader: threads %d", threads);
+  const int waves = threads / 64, kpi = 512 / BN, instr = 64 / kpi, RB = 2 * BN;
+  CHECK_OR_FAIL(instr % waves == 0 && instr >= waves, "[K,N] 16-bit loader: %d load instructions do not split over %d wavefronts", instr, waves);
+  CHECK_OR_FAIL(K >= 1 && N >= 8 && N % 8 == 0, "[K,N] 16-bit loader: bad matrix K=%lld N=%lld", (long long)K, (long long)N);
+  CHECK_OR_FAIL(K * N * 2 < ((int64_t)1 << 32), "[K,N] 16-bit loader: the matrix spans 4 GiB or more");
+  const int per_wave = instr / waves;
+  const int64_t ld = N * 2, extent = K * ld;
+  const int KT = (int)((K + 63) / 64);
+  const bool tail = K % 64 != 0;
+  const int last_full = tail ? KT - 2 : KT - 1;
+  std::vector<int> cell(64 * (BN / 8));
+  for (int64_t col0 = 0; col0 < N; col0 += BN) {
+    const int cols_valid = (int)(N - col0);
+    std::fill(cell.begin(), cell.end(), -1);
+    for (int wave = 0; wave < waves; ++wave)
+      for (int j = 0; j < per_wave; ++j)
+        for (int lane = 0; lane < 64; ++lane) {
+          const uint32_t voff = addr::kn16_voff<BN>(lane, wave, j, waves, cols_valid, (uint32_t)ld);
+          const int k = addr::kn16_k<BN>(lane, wave, j, waves);
+          CHECK_OR_FAIL(k < 64, "[K,N] 16-bit loader: k row %d outside the stage", k);
+          CHECK_OR_FAIL((int64_t)voff - (int64_t)k * ld >= 0 && (int64_t)voff - (int64_t)k * ld + 16 <= ld - col0 * 2,
+                        "[K,N] 16-bit loader: lane %d reads past the end of its k row", lane);
+          for (int kt = 0; kt <= last_full; ++kt) {
+            const int64_t o = col0 * 2 + (int64_t)voff + (int64_t)kt * 64 * ld;
+            CHECK_OR_FAIL(o >= 0 && o + 16 <= extent, "[K,N] 16-bit loader: col %lld wave %d instr %d lane %d stage %d reads [%lld, +16) of %lld",
+                          (long long)col0, wave, j, lane, kt, (long long)o, (long long)extent);
+          }
+          if (tail) {  // k rows past K re-read k row 0 of the matrix (then zeroed)
+            const bool ok = (int64_t)(KT - 1) * 64 + k < K;
+            const int64_t o = col0 * 2 + (ok ? (int64_t)voff + (int64_t)(KT - 1) * 64 * ld : (int64_t)voff - (int64_t)k * ld);
+            CHECK_OR_FAIL(o >= 0 && o + 16 <= extent, "[K,N] 16-bit loader: tail stage reads [%lld, +16) of %lld", (long long)o, (long long)extent);
+          }
+          const uint32_t l = addr::direct_lds_off(lane, wave, j, waves);
+          CHECK_OR_FAIL(l % 16 == 0 && l + 16 <= 64u * RB, "[K,N] 16-bit loader: LDS offset %u outside the tile", l);
+          CHECK_OR_FAIL(cell[l / 16] == -1, "[K,N] 16-bit loader: LDS cell %u written twice", l / 16);
+          const int pc = lane % (BN / 8);
+          CHECK_OR_FAIL(l == (uint32_t)(k * RB + pc * 16), "[K,N] 16-bit loader: lane lands at %u, not on (k %d, chunk %d)", l, k, pc);
+          cell[l / 16] = k * (BN / 8) + (pc ^ addr::kn16_swz(k));  // the logical chunk (8 columns) this cell holds
+        }
+    for (size_t c = 0; c < cell.size(); ++c) CHECK_OR_FAIL(cell[c] >= 0, "[K,N] 16-bit loader: LDS cell %zu never written", c);
+    // operand reads: lane (i, q) of column block t supplies the row of k = 8 q + i / 4 (+ 4 for the second read, + 32 for
+    // k-step 1) at columns wave_col0 + 16 t + 4 (i % 4) .. + 3
+    for (int wave_col0 = 0; wave_col0 + 64 <= BN; wave_col0 += 64)
+      for (int t = 0; t < 4; ++t)
+        for (int ks = 0; ks < 2; ++ks)
+          for (int h = 0; h < 2; ++h) {
+            int bank_use[2][64] = {};
+            for (int lane = 0; lane < 64; ++lane) {
+              const uint32_t off = addr::kn16frag_off<BN>(lane, wave_col0, t) + (uint32_t)(ks * 32 * RB + h * 4 * RB);
+              CHECK_OR_FAIL(off + 8 <= 64u * RB, "[K,N] 16-bit operand read at %u outside the tile", off);
+              const int i = lane & 15, q = lane >> 4;
+              const int k = 8 * q + (i >> 2) + 4 * h + 32 * ks;
+              const int col = wave_col0 + 16 * t + 4 * (i & 3);
+              const int want = k * (BN / 8) + col / 8;
+              CHECK_OR_FAIL(cell[off / 16] == want && (int)(off % 16) == 2 * (col % 8),
+                            "[K,N] 16-bit operand read (lane %d t %d) finds cell %d at byte %u, expects cell %d byte %d", lane, t, cell[off / 16],
+                            off % 16, want, 2 * (col % 8));
+              ++bank_use[lane >> 5][(off / 4) % 64];
+              ++bank_use[lane >> 5][(off / 4 + 1) % 64];
+            }
+            for (int half = 0; half < 2; ++half)
+              for (int b = 0; b < 64; ++b)
+                CHECK_OR_FAIL(bank_use[half][b] <= 1, "[K,N] 16-bit operand read: bank %d used %d times by one half-wavefront", b, bank_use[half][b]);
+          }
+  }
+  return 0;
+}
+
 // One wavefront running addr::slots_schedule; every tile is `loads_per_tile` load instructions of that wavefront.
 struct SlotsSim {
   int loads_per_tile;
@@ -530,6 +603,12 @@ int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_b
     if (tile == 256) return check_kn_direct<256>(rows, row_bytes, threads);
     if (tile == 128) return check_kn_direct<128>(rows, row_bytes, threads);
     set_error("tlq_debug_check_gemm_addressing: [K,N] tiles are 128 or 256 columns wide (got %d)", tile);
+    return 1;
+  }
+  if (source_kind == 2) {
+    if (tile == 256) return check_kn16_direct<256>(rows, row_bytes, threads);
+    if (tile == 128) return check_kn16_direct<128>(rows, row_bytes, threads);
+    set_error("tlq_debug_check_gemm_addressing: 16-bit [K,N] tiles are 128 or 256 columns wide (got %d)", tile);
     return 1;
   }
   set_error("tlq_debug_check_gemm_addressing: bad source kind %d", source_kind);

@@ -84,6 +84,25 @@ struct KNFrag8 {
   }
 };
 
+// [64 k][BN columns] tiles of 16-bit values (a [K, N] source copied as it is): ds_read_b64_tr_b16 hands every lane four
+// consecutive k of its column, two reads make an operand (addressing and the instruction's semantics: gemm_addr.h).
+template <int BN>
+struct KNFrag16 {
+  typedef short v4s_t __attribute__((ext_vector_type(4)));
+  uint32_t off[4];
+  __device__ __forceinline__ KNFrag16(int lane, int wave_col0) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) off[t] = addr::kn16frag_off<BN>(lane, wave_col0, t);
+  }
+  __device__ __forceinline__ uint4_t read(const uint8_t* tile, int ks, int t) const {
+    typedef __attribute__((address_space(3))) v4s_t* lds_ptr;
+    const uint8_t* p = tile + off[t] + ks * 32 * 2 * BN;
+    const uint2_t lo = bitcast<uint2_t>(__builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p)));
+    const uint2_t hi = bitcast<uint2_t>(__builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * 2 * BN)));
+    return uint4_t{lo.x, lo.y, hi.x, hi.y};
+  }
+};
+
 // ---- MFMA wrappers ----------------------------------------------------------------------
 struct MmaF16 {
   typedef float4_t acc_t;
@@ -332,6 +351,82 @@ struct I8KNLoaderDirect {
         const int k = addr::kn_k<BN>(0, wave, j, WAVES) + k_lane;
         const bool ok = kt * kStageBytes + k < k_total;
         uint4_t v = *(const uint4_t*)(ok ? sb + voff[j] : base + (voff[j] - (uint32_t)k * ld_));
+        if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
+        r.v[j] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void lstore_piece(const Regs& r, uint8_t* lds, int pc, int np) const {
+    if (!r.pending) return;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) {
+      if (j * np / UNITS != pc) continue;
+      *(uint4_t*)(lds + wave_off + addr::direct_lds_off(0, 0, j, WAVES) + lane_off) = r.v[j];
+    }
+  }
+  __device__ __forceinline__ void lstore(const Regs& r, uint8_t* lds) const { lstore_piece(r, lds, 0, 1); }
+};
+
+// 16-bit source stored [K, N], N a multiple of 8 (16-byte chunks): the tile is filled by direct global -> LDS loads, one
+// wavefront instruction per 512 / BN consecutive k rows; a partial last stage (rows past K must read as zero) goes
+// through registers.  Other N go through the register loader (H16KNLoader).
+struct H16KNParams {
+  const uint8_t* base;  // B[0, 0] of batch 0
+  int64_t ld;           // bytes per k row (= 2 N)
+  int64_t batch_stride;
+  int64_t k_total;
+};
+template <int BN, int NT>
+struct H16KNLoaderDirect {
+  typedef KNFrag16<BN> Frag;
+  static constexpr bool DIRECT = true;
+  static constexpr bool PREFETCH2 = false;
+  static constexpr int CH = BN / 8;     // 16-byte chunks per k row
+  static constexpr int KPI = 64 / CH;   // k rows per wavefront instruction
+  static constexpr int WAVES = NT / 64;
+  static constexpr int INSTR = 64 / KPI;  // 64 k rows per stage
+  static constexpr int PER_WAVE = INSTR / WAVES;
+  static constexpr int UNITS = PER_WAVE;
+  static_assert(INSTR % WAVES == 0 && PER_WAVE >= 1, "tile does not split into whole wavefront loads");
+  typedef H16KNParams Params;
+  struct Regs {
+    uint4_t v[PER_WAVE];
+    bool pending;
+  };
+  const uint8_t* base;
+  uint32_t voff[PER_WAVE];
+  uint32_t wave_off, lane_off, ld_;
+  int k_lane, wave, k_total;
+  __device__ __forceinline__ H16KNLoaderDirect(const Params& p, int batch, int col0, int cols_total, int tid)
+      : base(p.base + batch * p.batch_stride + (int64_t)col0 * 2), ld_((uint32_t)p.ld), k_total((int)p.k_total) {
+    const int lane = tid & 63;
+    wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    wave_off = addr::direct_lds_off(0, wave, 0, WAVES);
+    lane_off = addr::direct_lds_off(lane, 0, 0, WAVES);
+    k_lane = lane / CH;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) voff[j] = addr::kn16_voff<BN>(lane, wave, j, WAVES, cols_total - col0, ld_);
+  }
+  template <bool TAIL>
+  __device__ __forceinline__ void gload(Regs& r, int kt, uint8_t* lds_next) const {
+    typedef __attribute__((address_space(3))) uint8_t* lptr_t;
+    if (!TAIL) {
+      r.pending = false;
+      const uint8_t* sb = uniform_ptr(base + (int64_t)kt * 64 * ld_);
+      const uint32_t l0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lptr_t)lds_next + wave_off);
+#pragma unroll
+      for (int j = 0; j < PER_WAVE; ++j)
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l0 + addr::direct_lds_off(0, 0, j, WAVES)), "v"(voff[j]),
+                     "s"(sb)
+                     : "memory");
+    } else {
+      r.pending = true;
+      const uint8_t* sb = base + (int64_t)kt * 64 * ld_;
+#pragma unroll
+      for (int j = 0; j < PER_WAVE; ++j) {
+        const int k = addr::kn16_k<BN>(0, wave, j, WAVES) + k_lane;
+        const bool ok = kt * 64 + k < k_total;
+        uint4_t v = *(const uint4_t*)(ok ? sb + voff[j] : base + (voff[j] - (uint32_t)k * ld_));  // (rows past K: row 0, then zeroed)
         if (!ok) v = uint4_t{0u, 0u, 0u, 0u};
         r.v[j] = v;
       }

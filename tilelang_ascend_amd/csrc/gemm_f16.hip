@@ -97,6 +97,11 @@ static int run_f16(const void* A, const void* B, void* C, int64_t batch, int64_t
     typename WL::Params pw{(const uint8_t*)B, K * 2, N * K * 2, K * 2};
     return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16");
   }
+  if (N % 8 == 0) {  // [K, N] rows are whole 16-byte chunks: copied as they are, transposed by the operand read
+    typedef H16KNLoaderDirect<BN, NT> WL;
+    H16KNParams pw{(const uint8_t*)B, N * 2, K * N * 2, K};
+    return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16");
+  }
   typedef H16KNLoader<BN, NT> WL;
   typename WL::Params pw{(const uint8_t*)B, N * 2, K * N * 2, K};
   return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16");
@@ -115,6 +120,11 @@ static int run_f16_splitk(const void* A, const void* B, float* C, int64_t M, int
   if (b_layout == TLQ_B_NK) {
     typedef RowLoaderDirect<BN, NT> WL;
     typename WL::Params pw{(const uint8_t*)B, K * 2, ks * 2, ks * 2};
+    return launch_gemm<Mma, AL, WL, EpiAtomicAdd, BM, BN, WM, WN>(pa, pw, pe, split_k, M, N, ks * 2, st, "tlq_gemm_f16_splitk");
+  }
+  if (N % 8 == 0) {
+    typedef H16KNLoaderDirect<BN, NT> WL;
+    H16KNParams pw{(const uint8_t*)B, N * 2, ks * N * 2, ks};
     return launch_gemm<Mma, AL, WL, EpiAtomicAdd, BM, BN, WM, WN>(pa, pw, pe, split_k, M, N, ks * 2, st, "tlq_gemm_f16_splitk");
   }
   typedef H16KNLoader<BN, NT> WL;
@@ -146,6 +156,12 @@ static int dispatch_f16(const void* A, const void* B, void* C, int64_t batch, in
         pw{(const uint8_t*)B, K * 2, N * K * 2, K * 2};
     EpiFloat::Params pe{C, N, M * N, out_dtype};
     return launch_gemm_slots<Mma, RowLoaderDirect<256, 512>, EpiFloat>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16", 4);
+  }
+  if (g_gemm_slots && b_layout == TLQ_B_KN && K % 64 == 0 && N % 8 == 0) {  // [K, N] weights, transposed in the operand read
+    typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K * 2, M * K * 2, K * 2};
+    H16KNParams pw{(const uint8_t*)B, N * 2, K * N * 2, K};
+    EpiFloat::Params pe{C, N, M * N, out_dtype};
+    return launch_gemm_slots<Mma, H16KNLoaderDirect<256, 512>, EpiFloat>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16", 4);
   }
   return run_f16<Mma, 256, 256, 2, 4>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);
 }
