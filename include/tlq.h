@@ -219,9 +219,15 @@ int tlq_gemm_i8(const void* A, const void* B, void* C, int64_t batch, int64_t M,
 /* int8 activations x packed int4 weights -> int32, replaces w4a8_gemm_cv
  * (example_dequant_gemm_w4a8.py:25-121) and dequant_gemm_int8_wrapper
  * (example_dequant_gemm_fine_grained.py:226-266): C[M,N] = A[M,K] . convert(sign_mode, Wp)[N,K]^T.
- * The reference's caller-supplied int8 [N,K] workspace is not needed (unpack is fused). */
+ * The reference's caller-supplied int8 [N,K] workspace is not needed here (unpack is fused); tlq_gemm_w4a8_ws takes it. */
 int tlq_gemm_w4a8(const void* A, const void* w_packed, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
                   void* stream);
+/* The same with the reference kernel's third positional, the caller's int8 [N, K] workspace
+ * (example_dequant_gemm_w4a8.py:27,69-106 unpacks into it on the vector cores, :108-120 multiplies from it): when it is
+ * given (N * K bytes, 16-byte aligned, K and N multiples of 16) the weights are unpacked into it and the int8 GEMM runs on
+ * it; otherwise this is tlq_gemm_w4a8.  The workspace holds the unpacked weights afterwards, as the reference's does. */
+int tlq_gemm_w4a8_ws(const void* A, const void* w_packed, void* workspace, int64_t workspace_bytes, void* C, int64_t M,
+                     int64_t N, int64_t K, int sign_mode, void* stream);
 
 /* W8A8 matmul with fused rescale epilogue, replaces simple_quant_batch_matmul
  * (examples/quant_batch_matmul/example_quant_batch_matmul.py:8-91), simple_quant_matmul

@@ -39,6 +39,7 @@ SIGNATURES = {
     "tlq_gemm_f16_batched": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
     "tlq_gemm_i8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "tlq_gemm_w4a8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "tlq_gemm_w4a8_ws": (_int, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _int, _vp]),
     "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_w4a16_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "tlq_gemm_w4a16_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp, _i64, _vp]),

@@ -3,9 +3,9 @@
 Surface of examples/dequantize_gemm/example_dequant_gemm_w4a8.py: ``w4a8_gemm_cv(M, N, K)``
 (:25-121) -> ``kernel(A, B_packed, workspace[, C]) -> C`` and ``torch_convert`` (:124-145).
 The reference unpacks on the vector cores into a caller-supplied int8 [N, K] global workspace
-and then runs the cube GEMM; here the two's-complement unpack happens on the way into LDS, so
-the workspace argument is accepted (third positional, as the reference's callers pass it) and
-left untouched.
+and then runs the cube GEMM; so does this one when the workspace (third positional, as the
+reference's callers pass it) is a usable int8 [N, K] buffer: an unpack kernel at the HBM roofline
+and the int8 GEMM, which together beat the kernel that unpacks on the way into LDS.
 """
 from __future__ import annotations
 
@@ -28,8 +28,10 @@ def w4a8_gemm_cv(M, N, K):
     """C[M,N] i32 = A[M,K] i8 . twos_complement_unpack(B_packed)[N,K]^T (exact)."""
 
     def launch(t, sym, stream):
-        A, Bp, _workspace, C = t
-        _abi.check(_abi.load().tlq_gemm_w4a8(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(C), M, N, K, _abi.S4_TWOS, stream))
+        A, Bp, workspace, C = t
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None and workspace.is_contiguous() else 0
+        _abi.check(_abi.load().tlq_gemm_w4a8_ws(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(workspace) if ws_bytes else None, ws_bytes,
+                                                _abi.ptr(C), M, N, K, _abi.S4_TWOS, stream))
 
     return KernelSpec("w4a8_gemm_cv", [Param("A", (M, K), "int8"), Param("B_packed", (N, K // 2), "uint8"),
                                        Param("workspace", (N, K), "int8"), Param("C", (M, N), "int32")], launch)
