@@ -241,6 +241,18 @@ int tlq_gemm_w4a8_ws(const void* A, const void* w_packed, void* workspace, int64
 int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
                   int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, void* stream);
 
+/* The same with an int32 workspace in the place of the reference kernels' workspace_1 [B,M,N]
+ * (example_quant_batch_matmul.py:28,42,66-68; example_quant_matmul.py:27,41; deepseek_v4/int8_gemm.py workspace_idx=[5]):
+ * with one batch and few activation rows (too few output tiles to fill the machine) K is cut into slices that write
+ * their int32 tiles into the workspace, one [M,N] matrix per slice, and a second pass sums and rescales them into C --
+ * the same value bit for bit (integer sums are exact in any order).  tlq_w8a8_workspace_bytes gives the size that
+ * allows the preferred number of slices (0: this shape is not split); a smaller workspace (16-byte aligned) means fewer
+ * slices, none or too small a one means tlq_gemm_w8a8. */
+int64_t tlq_w8a8_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K);
+int tlq_gemm_w8a8_ws(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, void* workspace,
+                     int64_t workspace_bytes, int64_t batch, int64_t M, int64_t N, int64_t K, int64_t n_scale_b,
+                     int b_layout, int out_dtype, void* stream);
+
 /* Offline weight preparation on the GPU.
  * tlq_pack_int4 replaces general_compress (tilelang/quantize/utils.py:53-69, 4-bit source) and, with
  * interleave = 1 (fp16 target) or 2 (int8 target), the interleave_weight that follows it (:73-101):
@@ -333,6 +345,9 @@ void tlq_tune_w4a16_split(int slices);                       /* K slices of the 
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,
                                                                +10 = never stage through LDS, +20 = stage whenever possible */
 void tlq_tune_i8_tile(int block_m);                         /* 32|128|256 */
+void tlq_tune_i8_split(int slices);                         /* K slices of the one-batch int8 kernels: 0 = automatic, 1 = never, n = up to n */
+int tlq_debug_i8_split(int64_t M, int64_t N, int64_t K, int buffers); /* K slices taken for one batch of this shape: with a matrix per
+                                                                      * slice (1, tlq_gemm_w8a8_ws) or atomic adds into C (0, tlq_gemm_i8) */
 
 #ifdef __cplusplus
 }

@@ -41,6 +41,7 @@ SIGNATURES = {
     "tlq_gemm_w4a8": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "tlq_gemm_w4a8_ws": (_int, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _int, _vp]),
     "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "tlq_gemm_w8a8_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_w4a16_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "tlq_gemm_w4a16_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp, _i64, _vp]),
     "tlq_gemm_w4a16_layout_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _int, _vp, _i64, _vp]),
@@ -74,6 +75,9 @@ SIGNATURES = {
     "tlq_tune_w4a16_split": (None, [_int]),
     "tlq_tune_w4a16_skinny": (None, [_int, _int]),
     "tlq_tune_i8_tile": (None, [_int]),
+    "tlq_tune_i8_split": (None, [_int]),
+    "tlq_debug_i8_split": (_int, [_i64, _i64, _i64, _int]),
+    "tlq_w8a8_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
 }
 
 _lock = threading.Lock()

@@ -34,6 +34,12 @@ int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const v
                       int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, hipStream_t st);
 int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
                   hipStream_t st);
+int i8_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K, bool buffers);
+int gemm_i8_i32_splitk(const void* A, const void* B, int32_t* acc, int64_t M, int64_t N, int64_t K, int64_t split,
+                       int b_layout, hipStream_t st);
+int gemm_w8a8_rescale_splitk(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int32_t* partial,
+                             int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int64_t split, int b_layout, int out_dtype,
+                             hipStream_t st);
 
 struct DecodePlan {
   bool ok;
@@ -425,6 +431,9 @@ int tlq_gemm_i8(const void* A, const void* B, void* C, int64_t batch, int64_t M,
   TLQ_REQUIRE(A && B && C, "tlq_gemm_i8: null pointer");
   TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_i8: pointers must be 16-byte aligned");
   TLQ_REQUIRE(fits32(M, K) && fits32(N, K), "tlq_gemm_i8: a matrix spans 4 GiB or more");
+  // few activation rows: K slices add into C itself (int32, exact in any order)
+  if (const int split = i8_split_choice(batch, M, N, K, false); split > 1)
+    return gemm_i8_i32_splitk(A, B, (int32_t*)C, M, N, K, split, b_layout, (hipStream_t)stream);
   return gemm_i8_i32(A, B, C, batch, M, N, K, b_layout, (hipStream_t)stream);
 }
 
@@ -472,6 +481,41 @@ int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void*
   TLQ_REQUIRE(fits32(M, K) && fits32(N, K), "tlq_gemm_w8a8: a matrix spans 4 GiB or more");
   return gemm_w8a8_rescale(A, B, scale_a, scale_b, C, batch, M, N, K, n_scale_b, b_layout, out_dtype,
                            (hipStream_t)stream);
+}
+
+static bool w8a8_dims_split(int64_t batch, int64_t M, int64_t N, int64_t K) {
+  return batch == 1 && M > 0 && N > 0 && K > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim && K % 16 == 0 && N % 16 == 0 &&
+         fits32(M, K) && fits32(N, K);
+}
+
+int64_t tlq_w8a8_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K) {
+  if (!w8a8_dims_split(batch, M, N, K)) return 0;
+  const int split = i8_split_choice(batch, M, N, K, true);
+  return split > 1 ? (int64_t)split * M * N * 4 : 0;
+}
+
+int tlq_gemm_w8a8_ws(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, void* workspace,
+                     int64_t workspace_bytes, int64_t batch, int64_t M, int64_t N, int64_t K, int64_t n_scale_b,
+                     int b_layout, int out_dtype, void* stream) {
+  // One batch, few activation rows: K slices write their int32 tiles into the workspace, a second pass sums and
+  // rescales them into C (the reference's own two steps, example_quant_batch_matmul.py:42,66-68, with a matrix per slice).
+  int split = 1;
+  if (w8a8_dims_split(batch, M, N, K) && workspace != nullptr && aligned16(workspace)) {
+    split = i8_split_choice(batch, M, N, K, true);
+    while (split > 1 && (int64_t)split * M * N * 4 > workspace_bytes) split /= 2;  // as many slices as the workspace holds
+  }
+  if (split <= 1)
+    return tlq_gemm_w8a8(A, B, scale_a, scale_b, C, batch, M, N, K, n_scale_b, b_layout, out_dtype, stream);
+  TLQ_REQUIRE(b_layout == TLQ_B_KN || b_layout == TLQ_B_NK, "tlq_gemm_w8a8_ws: bad b_layout %d", b_layout);
+  TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_w8a8_ws: bad out_dtype %d",
+              out_dtype);
+  TLQ_REQUIRE(scale_b == nullptr || n_scale_b == 1 || n_scale_b == N,
+              "tlq_gemm_w8a8_ws: n_scale_b=%lld must be 1 or N=%lld", (long long)n_scale_b, (long long)N);
+  TLQ_REQUIRE(A && B && C, "tlq_gemm_w8a8_ws: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_w8a8_ws: pointers must be 16-byte aligned");
+  TLQ_REQUIRE(((uintptr_t)scale_a & 3) == 0 && ((uintptr_t)scale_b & 3) == 0, "tlq_gemm_w8a8_ws: scales misaligned");
+  return gemm_w8a8_rescale_splitk(A, B, scale_a, scale_b, C, (int32_t*)workspace, M, N, K, n_scale_b, split, b_layout,
+                                  out_dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -516,6 +516,25 @@ struct EpiAtomicAdd {  // fp32 accumulators added into C (split-K: several work-
   }
 };
 
+struct EpiAtomicAddI32 {  // int32 accumulators added into C (split-K; integer adds commute, so the sum is exact in any order)
+  struct Params {
+    int32_t* C;
+    int64_t ldc;
+  };
+  Params p;
+  __device__ __forceinline__ EpiAtomicAddI32(const Params& pp, int /*split*/) : p(pp) {}
+  static constexpr bool STAGED = false;
+  __device__ __forceinline__ int out_bytes() const { return 4; }
+  __device__ __forceinline__ int64_t pitch() const { return p.ldc; }
+  __device__ __forceinline__ uint8_t* addr_of(int, int) const { return nullptr; }
+  __device__ __forceinline__ uint4_t pack(int, int, const int4_t&, int, int) const { return uint4_t{0u, 0u, 0u, 0u}; }
+  __device__ __forceinline__ void store(int m, int n, const int4_t& acc, int M, int N) const {
+    if (m >= M || n >= N) return;
+    int32_t* c = p.C + (int64_t)m * p.ldc + n;
+    for (int i = 0; i < 4 && n + i < N; ++i) atomicAdd(c + i, acc[i]);
+  }
+};
+
 struct EpiInt32 {  // raw int32 accumulators
   struct Params {
     int32_t* C;
@@ -756,8 +775,8 @@ __device__ __forceinline__ TileCoord tile_of_block(int tiles_m, int tiles_n, int
 // ---- the kernel -----------------------------------------------------------------------------
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma_kernel(
-    typename AL::Params pa, typename WL::Params pw, typename Epi::Params pe, int M, int N, int KT, int k_tail,
-    int tiles_m, int tiles_n, int band_rows) {
+    typename AL::Params pa, typename WL::Params pw, typename Epi::Params pe, int M, int N, int kt_each, int k_tail,
+    int tiles_m, int tiles_n, int band_rows, int kt_total) {
   constexpr int TM = BM / WM / 16;  // 16-row activation tiles per wave
   constexpr int TN = BN / WN / 16;  // 16-row weight tiles per wave
   constexpr int A_TILE = BM * kStageBytes, W_TILE = BN * kStageBytes;
@@ -774,6 +793,8 @@ __global__ __launch_bounds__(WM* WN * 64, (WM * WN >= 8 ? 2 : 1)) void gemm_mfma
   const int wave_n0 = (wave / WM) * (BN / WN);
   const TileCoord tc = tile_of_block<BM, BN>(tiles_m, tiles_n, band_rows);
   const int m0 = tc.m0, n0 = tc.n0, batch = tc.batch;
+  // K slices (the "batches" of a split launch) may be uneven: the last one holds what is left of kt_total stages
+  const int KT = kt_total > 0 && kt_total - batch * kt_each < kt_each ? kt_total - batch * kt_each : kt_each;
 
   AL al(pa, batch, m0, M, tid);
   WL wl(pw, batch, n0, N, tid);
@@ -922,7 +943,9 @@ inline bool prefer_small_tiles(int64_t batch, int64_t M, int64_t N, double weigh
 
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,
-                int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what, int band_rows = 4) {
+                int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what, int band_rows = 4,
+                int kt_total = 0) {
+  // kt_total > 0: the batches are slices of K of k_bytes each (whole stages), the last one shorter: kt_total stages in all
   auto kern = gemm_mfma_kernel<Mma, AL, WL, Epi, BM, BN, WM, WN>;
   constexpr int lds_bytes = 2 * (BM + BN) * kStageBytes;  // two stages
   static bool attr_set = false;  // per instantiation; idempotent, so a race only repeats the call
@@ -943,8 +966,12 @@ int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, co
   }
   const int KT = (int)ceil_div(k_bytes, kStageBytes);
   const int k_tail = (k_bytes % kStageBytes) != 0;
+  if (kt_total > 0 && (k_tail || (batch - 1) * KT >= kt_total || batch * KT < kt_total)) {
+    set_error("%s: %lld slices of %d stages do not cover %d stages", what, (long long)batch, KT, kt_total);
+    return 1;
+  }
   kern<<<(unsigned)blocks, WM * WN * 64, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, KT, k_tail, (int)tiles_m,
-                                                          (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows);
+                                                          (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows, kt_total);
   return check_launch(what) ? 0 : 1;
 }
 

@@ -177,6 +177,135 @@ int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const v
   return dispatch_i8<EpiRescale>(A, B, pe, batch, M, N, K, b_layout, st, "tlq_gemm_w8a8");
 }
 
+// ---- split K (one batch, few activation rows) -------------------------------------------------
+// With few activation rows the output tiles are too few to fill the machine and the kernel is paced by the weight
+// bytes one work-group can pull.  Slice z of K is "batch" z of the loaders (the batch strides step along K) and every
+// slice adds its int32 tile into the one accumulator matrix, cleared beforehand: integer adds commute, so the result
+// is the exact sum whatever the order.
+__global__ __launch_bounds__(256) void i32_clear_kernel(int4_t* __restrict__ p, int64_t n4) {
+  for (int64_t i = blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) p[i] = int4_t{0, 0, 0, 0};
+}
+
+// `split` slices of ceil(stages / split) whole stages each, the last one with what is left (at least one stage).
+template <class Epi, int BM, int BN, int WM, int WN>
+static int run_i8_splitk(const void* A, const void* B, const typename Epi::Params& pe, int64_t M, int64_t N, int64_t K,
+                         int64_t split, int b_layout, hipStream_t st) {
+  constexpr int NT = WM * WN * 64;
+  const int64_t stages = K / kStageBytes;
+  const int64_t ks = ceil_div(stages, split) * kStageBytes;
+  typedef RowLoaderDirect<BM, NT> AL;
+  typename AL::Params pa{(const uint8_t*)A, K, ks, ks};
+  if (b_layout == TLQ_B_NK) {
+    typedef RowLoaderDirect<BN, NT> WL;
+    typename WL::Params pw{(const uint8_t*)B, K, ks, ks};
+    return launch_gemm<MmaI8, AL, WL, Epi, BM, BN, WM, WN>(pa, pw, pe, split, M, N, ks, st, "tlq_gemm_i8 (K slices)", 2, (int)stages);
+  }
+  typedef I8KNLoaderDirect<BN, NT> WL;
+  typename WL::Params pw{(const uint8_t*)B, N, ks * N, ks};
+  return launch_gemm<MmaI8, AL, WL, Epi, BM, BN, WM, WN>(pa, pw, pe, split, M, N, ks, st, "tlq_gemm_i8 (K slices)", 2, (int)stages);
+}
+
+static thread_local int g_i8_split = 0;  // tlq_tune_i8_split: 0 = automatic, 1 = never, n = that many slices where K allows
+
+// Number of K slices for one batch of [M,K] x [N,K]: 1 = do not split.  Slices are whole 128-byte stages.
+// `buffers`: every slice has an int32 [M,N] matrix of its own (plain stores, summed by the pass that follows);
+// otherwise the slices add into one matrix with atomic adds, which cost about 10 ns per thousand.
+// The estimate behind the choice, in microseconds: an under-filled launch is paced by what one work-group
+// streams, (BM + BN) * K bytes at about 40 GB/s; s slices divide that and add the cost of their sums.
+int i8_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K, bool buffers) {
+  if (batch != 1 || g_i8_split == 1 || (g_i8_tile && g_i8_split == 0)) return 1;  // a forced tile means: that kernel
+  const int tile = M <= 32 ? 32 : 128;
+  const int64_t tiles = ceil_div(M, tile) * ceil_div(N, (int64_t)128);
+  int cus = tlq_device_cu_count();
+  if (cus <= 0) cus = 256;
+  const int64_t places = (int64_t)cus * (tile == 32 ? 4 : 2);  // work-groups the machine holds at once (LDS per work-group)
+  if (K % kStageBytes != 0) return 1;
+  const int64_t stages = K / kStageBytes;
+  // the number of slices that s asks for once every slice but the last has ceil(stages / s) stages
+  auto slices = [&](int64_t sl) { return ceil_div(stages, ceil_div(stages, sl)); };
+  if (g_i8_split > 1) return (int)slices(g_i8_split < stages ? g_i8_split : stages);
+  if (tiles * 2 > places) return 1;
+  const double one = (double)(tile + 128) * (double)K / 40e3;
+  const double mn = (double)M * (double)N;
+  double best = one;
+  int64_t best_s = 1;
+  for (int64_t want = 2; want * tiles <= places && want * 2 <= stages; ++want) {
+    const int64_t sl = slices(want);
+    if (sl != want) continue;  // the same cut as a smaller request
+    const double sums = buffers ? 3.0 + (double)sl * mn * 8 / 4e6 : 5.0 + (double)sl * mn / 100e3;
+    const double t = one * (double)ceil_div(stages, sl) / (double)stages + sums;
+    if (t < best * (best_s == 1 ? 0.85 : 0.97)) best = t, best_s = sl;
+  }
+  return (int)best_s;
+}
+
+// any requested count -> the count of non-empty slices of ceil(stages / count) stages
+static int64_t whole_slices(int64_t K, int64_t split) {
+  const int64_t stages = K / kStageBytes;
+  if (split > stages) split = stages;
+  return ceil_div(stages, ceil_div(stages, split));
+}
+
+int gemm_i8_i32_splitk(const void* A, const void* B, int32_t* acc, int64_t M, int64_t N, int64_t K, int64_t split,
+                       int b_layout, hipStream_t st) {
+  split = whole_slices(K, split);
+  const int64_t n4 = M * N / 4;  // N % 16 == 0
+  const int64_t want = ceil_div(n4, (int64_t)256);
+  i32_clear_kernel<<<(int)(want > 4096 ? 4096 : want), 256, 0, st>>>((int4_t*)acc, n4);
+  if (!check_launch("tlq_gemm_i8 (clear)")) return 1;
+  if (M <= 32) return run_i8_splitk<EpiAtomicAddI32, 32, 128, 1, 4>(A, B, {acc, N}, M, N, K, split, b_layout, st);
+  return run_i8_splitk<EpiAtomicAddI32, 128, 128, 2, 2>(A, B, {acc, N}, M, N, K, split, b_layout, st);
+}
+
+// C = rn_out(rn_f32(rn_f32(f32(acc) * scale_a[m]) * scale_b[n])) with acc the sum of the slices' int32 matrices:
+// the arithmetic of EpiRescale on the finished sums (four outputs per thread; N % 16 == 0).
+__global__ __launch_bounds__(256) void i32_sum_rescale_kernel(const int4_t* __restrict__ partial, int split, void* __restrict__ C,
+                                                              const float* __restrict__ scale_a, const float* __restrict__ scale_b,
+                                                              int64_t n_scale_b, int64_t n4_total, int n4_row, int out_dtype) {
+  for (int64_t i = blockIdx.x * 256 + threadIdx.x; i < n4_total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / n4_row;
+    const int n = (int)(i - m * n4_row) * 4;
+    int4_t a = partial[i];
+    for (int z = 1; z < split; ++z) a += partial[(int64_t)z * n4_total + i];
+    float4_t f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f[j] = (float)a[j];
+    if (scale_a) {
+      const float sa = scale_a[m];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f[j] = f[j] * sa;
+    }
+    if (scale_b) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f[j] = f[j] * (n_scale_b == 1 ? scale_b[0] : scale_b[n + j]);
+    }
+    if (out_dtype == TLQ_F32) {
+      ((float4_t*)C)[i] = f;
+    } else if (out_dtype == TLQ_F16) {
+      half_t h[4] = {(half_t)f[0], (half_t)f[1], (half_t)f[2], (half_t)f[3]};
+      ((uint2_t*)C)[i] = bitcast<uint2_t>(h);
+    } else {
+      ((uint2_t*)C)[i] = uint2_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3])};
+    }
+  }
+}
+
+// partial: int32 [split][M][N]
+int gemm_w8a8_rescale_splitk(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int32_t* partial,
+                             int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int64_t split, int b_layout, int out_dtype,
+                             hipStream_t st) {
+  split = whole_slices(K, split);
+  EpiInt32::Params pe{partial, N, M * N};
+  const int rc = M <= 32 ? run_i8_splitk<EpiInt32, 32, 128, 1, 4>(A, B, pe, M, N, K, split, b_layout, st)
+                         : run_i8_splitk<EpiInt32, 128, 128, 2, 2>(A, B, pe, M, N, K, split, b_layout, st);
+  if (rc) return rc;
+  const int64_t n4 = M * N / 4;
+  const int64_t want = ceil_div(n4, (int64_t)256);
+  i32_sum_rescale_kernel<<<(int)(want > 8192 ? 8192 : want), 256, 0, st>>>((const int4_t*)partial, (int)split, C, (const float*)scale_a,
+                                                                            (const float*)scale_b, n_scale_b, n4, (int)(N / 4), out_dtype);
+  return check_launch("tlq_gemm_w8a8 (sum and rescale)") ? 0 : 1;
+}
+
 int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
                   hipStream_t st) {
   EpiInt32::Params pe{(int32_t*)C, N, M * N};
@@ -204,4 +333,10 @@ extern "C" {
 // Tuning hook used by the benchmark sweeps: forces the activation-tile height (32, 128, 256)
 // of the int8 kernels; 0 restores the automatic choice.
 void tlq_tune_i8_tile(int block_m) { tlq::g_i8_tile = block_m; }
+// Forces the number of K slices of the one-batch int8 kernels: 0 = automatic, 1 = never split, n = up to n slices
+// (a power of two, as far as K divides into whole 128-byte stages).
+void tlq_tune_i8_split(int slices) { tlq::g_i8_split = slices; }
+// The number of K slices the automatic choice (or the forced value) takes for one batch of this shape, with a matrix
+// per slice (buffers = 1: tlq_gemm_w8a8_ws) or atomic adds into the one output (0: tlq_gemm_i8).
+int tlq_debug_i8_split(int64_t M, int64_t N, int64_t K, int buffers) { return tlq::i8_split_choice(1, M, N, K, buffers != 0); }
 }

@@ -18,6 +18,7 @@ from typing import Literal
 
 from .. import _abi
 from ..jit import ABI_DTYPE, TORCH_DTYPES, KernelSpec, Param, PassConfigKey, jit
+from .quant_matmul import w8a8_launch
 
 _PASS_CONFIGS = {
     PassConfigKey.TL_ASCEND_AUTO_SYNC: True,
@@ -44,8 +45,7 @@ def int8_gemm_kernel_corrected(N: int, K: int, block_M: int = 32, block_N: int =
     def launch(t, sym, stream):
         A, B, sa, sb, C, _ws = t
         with _abi.tuning(i8_tile=tile):
-            _abi.check(_abi.load().tlq_gemm_w8a8(_abi.ptr(A), _abi.ptr(B), _abi.ptr(sa), _abi.ptr(sb), _abi.ptr(C), 1,
-                                                 sym["M"], N, K, N, _abi.B_NK, tout, stream))
+            w8a8_launch(A, B, sa, sb, C, 1, sym["M"], N, K, N, _abi.B_NK, tout, stream)
 
     return KernelSpec("int8_gemm_kernel_corrected",
                       [Param("A", ("M", K), in_dtype), Param("B", (N, K), in_dtype),
@@ -66,8 +66,7 @@ def quant_batch_matmul_per_token(Batch: int, M: int, N: int, K: int, block_M: in
     def launch(t, sym, stream):
         A, B, sa, sb, C, _ws = t
         with _abi.tuning(i8_tile=tile):
-            _abi.check(_abi.load().tlq_gemm_w8a8(_abi.ptr(A), _abi.ptr(B), _abi.ptr(sa), _abi.ptr(sb), _abi.ptr(C),
-                                                 Batch, M, N, K, N, _abi.B_KN, tout, stream))
+            w8a8_launch(A, B, sa, sb, C, Batch, M, N, K, N, _abi.B_KN, tout, stream)
 
     return KernelSpec("quant_batch_matmul_per_token",
                       [Param("A", (Batch, M, K), "int8"), Param("B", (Batch, K, N), "int8"),

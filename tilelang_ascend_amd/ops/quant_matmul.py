@@ -8,12 +8,16 @@ with ``out_idx=[3]`` and an int32 ``workspace_1`` at ``workspace_idx=[4]``.
     C   = rn_out( f32(acc) * scale[n or 0] )               CAST_RINT = round to nearest even
 
 The reference writes acc to the global workspace and re-reads it on the vector cores
-(:66-68); here the rescale runs on the MFMA accumulators and the workspace is never
-allocated.
+(:66-68); here the rescale runs on the MFMA accumulators.  Only with one batch and few
+activation rows, where the output tiles are too few to fill the machine, K is cut into
+slices that write int32 matrices into a workspace and a second pass sums and rescales
+them (``w8a8_launch``) -- the same values bit for bit.
 """
 from __future__ import annotations
 
 from typing import Literal
+
+import torch
 
 from .. import _abi
 from ..jit import ABI_DTYPE, TORCH_DTYPES, KernelSpec, Param, PassConfigKey, jit
@@ -34,6 +38,18 @@ def _check_types(scale_size, in_dtype, out_dtype, accum_dtype, scale_dtype):
         raise ValueError(f"out_dtype must be float16, bfloat16 or float32, got {out_dtype}")
 
 
+def w8a8_launch(A, B, scale_a, scale_b, C, batch, M, N, K, n_scale_b, b_layout, out_code, stream):
+    """One W8A8 launch with the int32 workspace the library asks for (the reference's workspace_idx buffer,
+    example_quant_batch_matmul.py:28,42): allocated per call on A's device like the reference's, and only where the
+    library cuts K into slices (one batch, few activation rows); otherwise the rescale stays fused and nothing is
+    allocated."""
+    lib = _abi.load()
+    ws_bytes = lib.tlq_w8a8_workspace_bytes(batch, M, N, K)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device) if ws_bytes else None
+    _abi.check(lib.tlq_gemm_w8a8_ws(_abi.ptr(A), _abi.ptr(B), _abi.ptr(scale_a), _abi.ptr(scale_b), _abi.ptr(C), _abi.ptr(ws),
+                                    ws_bytes, batch, M, N, K, n_scale_b, b_layout, out_code, stream))
+
+
 @jit(out_idx=[3], workspace_idx=[4], pass_configs=_PASS_CONFIGS)
 def simple_quant_batch_matmul(Batch: int, M: int, N: int, K: int, scale_size: Literal["1", "N"],
                               block_M: int, block_N: int, block_K: int,
@@ -48,8 +64,7 @@ def simple_quant_batch_matmul(Batch: int, M: int, N: int, K: int, scale_size: Li
 
     def launch(t, sym, stream):
         A, B, scale, C, _ws = t
-        _abi.check(_abi.load().tlq_gemm_w8a8(_abi.ptr(A), _abi.ptr(B), None, _abi.ptr(scale), _abi.ptr(C), Batch, M, N,
-                                             K, N_scale, _abi.B_KN, tout, stream))
+        w8a8_launch(A, B, None, scale, C, Batch, M, N, K, N_scale, _abi.B_KN, tout, stream)
 
     return KernelSpec("simple_quant_batch_matmul",
                       [Param("A", (Batch, M, K), in_dtype), Param("B", (Batch, K, N), in_dtype),
@@ -72,8 +87,7 @@ def simple_quant_matmul(M: int, N: int, K: int, scale_size: Literal["1", "N"],
 
     def launch(t, sym, stream):
         A, B, scale, C, _ws = t
-        _abi.check(_abi.load().tlq_gemm_w8a8(_abi.ptr(A), _abi.ptr(B), None, _abi.ptr(scale), _abi.ptr(C), 1, M, N, K,
-                                             N_scale, _abi.B_KN, tout, stream))
+        w8a8_launch(A, B, None, scale, C, 1, M, N, K, N_scale, _abi.B_KN, tout, stream)
 
     return KernelSpec("simple_quant_matmul",
                       [Param("A", (M, K), in_dtype), Param("B", (K, N), in_dtype),
