@@ -223,9 +223,11 @@ int tlq_gemm_i8(const void* A, const void* B, void* C, int64_t batch, int64_t M,
 int tlq_gemm_w4a8(const void* A, const void* w_packed, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
                   void* stream);
 /* The same with the reference kernel's third positional, the caller's int8 [N, K] workspace
- * (example_dequant_gemm_w4a8.py:27,69-106 unpacks into it on the vector cores, :108-120 multiplies from it): when it is
- * given (N * K bytes, 16-byte aligned, K and N multiples of 16) the weights are unpacked into it and the int8 GEMM runs on
- * it; otherwise this is tlq_gemm_w4a8.  The workspace holds the unpacked weights afterwards, as the reference's does. */
+ * (example_dequant_gemm_w4a8.py:27,69-106 unpacks into it on the vector cores, :108-120 multiplies from it).  With many
+ * activation rows (M > 256) and a usable workspace (N * K bytes, 16-byte aligned, K and N multiples of 16) the weights
+ * are unpacked into it and the int8 GEMM runs on it, as in the reference; the workspace then holds the unpacked
+ * weights.  With few rows the unpack stays fused and K is cut into slices, the workspace holding one int32 [M, N] matrix
+ * per slice (as many slices as fit).  Otherwise this is tlq_gemm_w4a8.  The result is the same in every case. */
 int tlq_gemm_w4a8_ws(const void* A, const void* w_packed, void* workspace, int64_t workspace_bytes, void* C, int64_t M,
                      int64_t N, int64_t K, int sign_mode, void* stream);
 
@@ -345,6 +347,7 @@ void tlq_tune_w4a16_split(int slices);                       /* K slices of the 
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,
                                                                +10 = never stage through LDS, +20 = stage whenever possible */
 void tlq_tune_i8_tile(int block_m);                         /* 32|128|256 */
+void tlq_tune_w4a8_ws(int mode);                            /* tlq_gemm_w4a8_ws: 0 = automatic, 1 = K slices in the workspace, 2 = unpack + int8 GEMM */
 void tlq_tune_i8_split(int slices);                         /* K slices of the one-batch int8 kernels: 0 = automatic, 1 = never, n = up to n */
 int tlq_debug_i8_split(int64_t M, int64_t N, int64_t K, int buffers); /* K slices taken for one batch of this shape: with a matrix per
                                                                       * slice (1, tlq_gemm_w8a8_ws) or atomic adds into C (0, tlq_gemm_i8) */

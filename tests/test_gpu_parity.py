@@ -408,11 +408,13 @@ def test_w4a8(ops, M, N, K):
     assert torch.equal(ref.torch_convert(qB), B_ref)
 
 
-@pytest.mark.parametrize("M,N,K", [(64, 256, 256), (300, 1040, 512), (1024, 4096, 1024), (7, 48, 96)])
+@pytest.mark.parametrize("M,N,K", [(64, 256, 256), (300, 1040, 512), (1024, 4096, 1024), (7, 48, 96), (16, 1024, 2048),
+                                   (200, 512, 128 * 9)])
 def test_w4a8_with_and_without_the_reference_workspace(ops, M, N, K):
-    """tlq_gemm_w4a8_ws: with the reference's int8 [N, K] workspace the weights are unpacked into it (it then holds
-    torch_convert(B_packed), example_dequant_gemm_w4a8.py:69-106) and the int8 GEMM runs on it; without one, or with one
-    that is too small, the fused kernel runs.  Integers: all three results are the oracle's, bit for bit."""
+    """tlq_gemm_w4a8_ws uses the reference's int8 [N, K] workspace in one of two ways: unpack into it (it then holds
+    torch_convert(B_packed), example_dequant_gemm_w4a8.py:69-106) and run the int8 GEMM on it, or -- few activation
+    rows -- keep the unpack fused and cut K into slices whose int32 matrices live in the workspace.  Without a
+    workspace the fused kernel runs (its slices add into C).  Integers: every result is the oracle's, bit for bit."""
     from tilelang_ascend_amd import _abi
 
     lib, P = _abi.load(), _abi.ptr
@@ -422,17 +424,23 @@ def test_w4a8_with_and_without_the_reference_workspace(ops, M, N, K):
     want = ref.int_matmul_exact(A, B_ref.t().contiguous()).to(torch.int32)
     dA, dB = A.cuda(), qB.cuda()
     st = torch.cuda.current_stream().cuda_stream
-    for ws_bytes in (N * K, 0, N * K - 16):
-        ws = torch.full((N * K,), 99, dtype=torch.int8, device="cuda")
-        C = torch.full((M, N), -1, dtype=torch.int32, device="cuda")
-        print(f"w4a8 M={M} N={N} K={K} workspace={ws_bytes}", flush=True)
-        _abi.check(lib.tlq_gemm_w4a8_ws(P(dA), P(dB), P(ws) if ws_bytes else None, ws_bytes, P(C), M, N, K, _abi.S4_TWOS, st))
-        torch.cuda.synchronize()
-        assert_bit_equal(C.cpu(), want, f"w4a8 workspace={ws_bytes}")
-        if ws_bytes == N * K and N % 16 == 0 and K % 16 == 0:
-            assert_bit_equal(ws.cpu().view(N, K), B_ref, "the workspace holds the unpacked weights")
-        else:
-            assert (ws == 99).all(), "a workspace that is not used stays untouched"
+    for mode in (0, 1, 2):  # automatic, K slices in the workspace, unpack + int8 GEMM
+        for ws_bytes in (N * K, 0, N * K - 16, M * N * 8):
+            ws = torch.full((max(N * K, M * N * 8),), 99, dtype=torch.int8, device="cuda")
+            C = torch.full((M, N), -1, dtype=torch.int32, device="cuda")
+            print(f"w4a8 M={M} N={N} K={K} mode={mode} workspace={ws_bytes}", flush=True)
+            lib.tlq_tune_w4a8_ws(mode)
+            try:
+                _abi.check(lib.tlq_gemm_w4a8_ws(P(dA), P(dB), P(ws) if ws_bytes else None, ws_bytes, P(C), M, N, K, _abi.S4_TWOS, st))
+            finally:
+                lib.tlq_tune_w4a8_ws(0)
+            torch.cuda.synchronize()
+            assert_bit_equal(C.cpu(), want, f"w4a8 mode={mode} workspace={ws_bytes}")
+            if mode == 2:
+                if ws_bytes >= N * K and N % 16 == 0 and K % 16 == 0:
+                    assert_bit_equal(ws.cpu()[:N * K].view(N, K), B_ref, "the workspace holds the unpacked weights")
+                else:
+                    assert (ws == 99).all(), "a workspace that is not used stays untouched"
 
 
 @pytest.mark.parametrize("scale_size,out_dtype", [("1", "float16"), ("N", "bfloat16"), ("N", "float16")])

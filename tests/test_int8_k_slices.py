@@ -181,3 +181,38 @@ def test_the_operators_take_the_sliced_path_for_few_rows():
     kernel = ops.int8_gemm_kernel_corrected(N, K, out_dtype="bfloat16")
     got = kernel(A.cuda(), Bnk.cuda(), sa.cuda(), sb.cuda()).cpu()
     assert_bit_equal(got, ref.ref_int8_gemm_sequential(A, Bnk, sa, sb, torch.bfloat16), "int8_gemm_kernel_corrected, few rows")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sign_mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("M,N,K", [(1, 260, 512), (16, 4096, 4096), (33, 400, 128 * 7), (200, 2048, 4096), (32, 1024, 11008)])
+def test_packed_int4_weights_over_k_slices(M, N, K, sign_mode):
+    """tlq_gemm_w4a8 (slices add into C) and tlq_gemm_w4a8_ws (a matrix per slice in the workspace) against the kernel
+    without slices and against the exact integer product of the unpacked weights, for every sign convention."""
+    from oracle import ref
+
+    _abi, lib, P = _lib()
+    g = gen(5 * M + N + K + sign_mode)
+    st = torch.cuda.current_stream().cuda_stream
+    A = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g)
+    Wp = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=g)
+    lo, hi = (Wp & 15).to(torch.int16), (Wp >> 4).to(torch.int16)
+    u = torch.stack([lo, hi], dim=-1).reshape(N, K)
+    vals = {0: u, 1: torch.where(u >= 8, u - 16, u), 2: u - 8, 3: u - 7}[sign_mode].to(torch.int8)
+    want = ref.int_matmul_exact(A, vals.t().contiguous()).to(torch.int32)
+    Ad, Wd = A.cuda(), Wp.cuda()
+    ws = torch.empty(max(N * K, 64 * M * N * 4), dtype=torch.int8, device="cuda")
+    for slices in (1, 0, 2, 3, 5, 64):
+        lib.tlq_tune_i8_split(slices)
+        lib.tlq_tune_w4a8_ws(1)
+        try:
+            C = torch.full((M, N), 7, dtype=torch.int32, device="cuda")
+            _abi.check(lib.tlq_gemm_w4a8(P(Ad), P(Wd), P(C), M, N, K, sign_mode, st))
+            D = torch.full((M, N), 7, dtype=torch.int32, device="cuda")
+            _abi.check(lib.tlq_gemm_w4a8_ws(P(Ad), P(Wd), P(ws), ws.numel(), P(D), M, N, K, sign_mode, st))
+        finally:
+            lib.tlq_tune_i8_split(0)
+            lib.tlq_tune_w4a8_ws(0)
+        torch.cuda.synchronize()
+        assert_bit_equal(C.cpu(), want, f"W4A8 sign mode {sign_mode}, {slices} slices asked, {M}x{N}x{K} (adds into C)")
+        assert_bit_equal(D.cpu(), want, f"W4A8 sign mode {sign_mode}, {slices} slices asked, {M}x{N}x{K} (matrix per slice)")

@@ -76,6 +76,7 @@ SIGNATURES = {
     "tlq_tune_w4a16_skinny": (None, [_int, _int]),
     "tlq_tune_i8_tile": (None, [_int]),
     "tlq_tune_i8_split": (None, [_int]),
+    "tlq_tune_w4a8_ws": (None, [_int]),
     "tlq_debug_i8_split": (_int, [_i64, _i64, _i64, _int]),
     "tlq_w8a8_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
 }

@@ -34,7 +34,9 @@ int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const v
                       int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, hipStream_t st);
 int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
                   hipStream_t st);
-int i8_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K, bool buffers);
+int i8_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K, bool buffers, double pace = 1.0);
+int gemm_w4a8_i32_splitk(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
+                         int64_t split, int32_t* partial, hipStream_t st);
 int gemm_i8_i32_splitk(const void* A, const void* B, int32_t* acc, int64_t M, int64_t N, int64_t K, int64_t split,
                        int b_layout, hipStream_t st);
 int gemm_w8a8_rescale_splitk(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int32_t* partial,
@@ -447,21 +449,42 @@ int tlq_gemm_w4a8(const void* A, const void* w_packed, void* C, int64_t M, int64
   TLQ_REQUIRE(A && w_packed && C, "tlq_gemm_w4a8: null pointer");
   TLQ_REQUIRE(aligned16(A) && aligned16(w_packed) && aligned16(C), "tlq_gemm_w4a8: pointers must be 16-byte aligned");
   TLQ_REQUIRE(fits32(M, K) && fits32(N, K / 2), "tlq_gemm_w4a8: a matrix spans 4 GiB or more");
+  // few activation rows: K slices add into C (int32, exact in any order)
+  if (const int split = i8_split_choice(1, M, N, K, false, 2.5); split > 1)
+    return gemm_w4a8_i32_splitk(A, w_packed, C, M, N, K, sign_mode, split, nullptr, (hipStream_t)stream);
   return gemm_w4a8_i32(A, w_packed, C, M, N, K, sign_mode, (hipStream_t)stream);
 }
 
+static thread_local int g_w4a8_ws_mode = 0;  // tlq_tune_w4a8_ws: 0 = automatic, 1 = K slices in the workspace, 2 = unpack + int8 GEMM
+
 int tlq_gemm_w4a8_ws(const void* A, const void* w_packed, void* workspace, int64_t workspace_bytes, void* C, int64_t M,
                      int64_t N, int64_t K, int sign_mode, void* stream) {
-  // With the reference's int8 [N, K] workspace: its two steps -- unpack into the workspace, int8 GEMM on it -- each at
-  // its own roofline (M = N = K = 4096: 6 + 66 us against 98 us fused; M = 1024: 37 against 65 us).
-  const bool two_steps = workspace != nullptr && aligned16(workspace) && N > 0 && K > 0 && N < kMaxDim && K < kMaxDim &&
-                         workspace_bytes >= N * K && K % 16 == 0 && N % 16 == 0 && M > 0 && fits32(N, K);
+  // The reference's int8 [N, K] workspace is used in one of two ways.  Many activation rows: the reference's own two
+  // steps -- unpack into the workspace, int8 GEMM on it -- each at its own roofline (M = N = K = 4096: 6 + 66 us against
+  // 98 us fused; M = 1024: 37 against 65 us).  Few rows (the unpack pass would cost more than the GEMM): the kernel that
+  // unpacks on the way into LDS over K slices, the workspace holding one int32 [M, N] matrix per slice.
+  const bool usable = workspace != nullptr && aligned16(workspace) && N > 0 && K > 0 && M > 0 && M < kMaxDim && N < kMaxDim &&
+                      K < kMaxDim && fits32(N, K / 2) && fits32(M, K);
+  if (usable && K % 32 == 0 && N % 4 == 0 && g_w4a8_ws_mode != 2 && (M <= 256 || g_w4a8_ws_mode == 1)) {
+    int split = i8_split_choice(1, M, N, K, true, 2.5);
+    while (split > 1 && (int64_t)split * M * N * 4 > workspace_bytes) split /= 2;
+    if (split > 1) {
+      TLQ_REQUIRE(sign_mode >= TLQ_U4 && sign_mode <= TLQ_S4_OFFSET7, "tlq_gemm_w4a8_ws: bad sign_mode %d", sign_mode);
+      TLQ_REQUIRE(A && w_packed && C && aligned16(A) && aligned16(w_packed) && aligned16(C),
+                  "tlq_gemm_w4a8_ws: null or misaligned pointer");
+      return gemm_w4a8_i32_splitk(A, w_packed, C, M, N, K, sign_mode, split, (int32_t*)workspace, (hipStream_t)stream);
+    }
+  }
+  const bool two_steps = usable && workspace_bytes >= N * K && K % 16 == 0 && N % 16 == 0 && fits32(N, K) &&
+                         (M > 64 || g_w4a8_ws_mode == 2);
   if (!two_steps) return tlq_gemm_w4a8(A, w_packed, C, M, N, K, sign_mode, stream);
   TLQ_REQUIRE(sign_mode >= TLQ_U4 && sign_mode <= TLQ_S4_OFFSET7, "tlq_gemm_w4a8_ws: bad sign_mode %d", sign_mode);
   TLQ_REQUIRE(A && w_packed && C && aligned16(w_packed), "tlq_gemm_w4a8_ws: null or misaligned pointer");
   if (int rc = tlq_unpack_int4(w_packed, workspace, N, K, TLQ_I8, sign_mode, stream)) return rc;
   return tlq_gemm_i8(A, workspace, C, 1, M, N, K, TLQ_B_NK, stream);
 }
+
+void tlq_tune_w4a8_ws(int mode) { g_w4a8_ws_mode = mode; }
 
 int tlq_gemm_w8a8(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
                   int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int b_layout, int out_dtype, void* stream) {

@@ -24,6 +24,7 @@ struct W4I8Loader {
     const uint8_t* wp;
     int64_t row_bytes;  // K / 2
     int sign_mode;
+    int64_t batch_stride;  // bytes between the "batches" (K slices: a slice's packed bytes per row)
   };
   struct Regs {
     uint4_t v[PASSES];
@@ -34,8 +35,8 @@ struct W4I8Loader {
   int kb_lane, row_bytes, sign_mode;
   bool active;
 
-  __device__ __forceinline__ W4I8Loader(const Params& p, int /*batch*/, int row0, int rows_total, int tid)
-      : base(p.wp + (int64_t)row0 * p.row_bytes), row_bytes((int)p.row_bytes), sign_mode(p.sign_mode) {
+  __device__ __forceinline__ W4I8Loader(const Params& p, int batch, int row0, int rows_total, int tid)
+      : base(p.wp + batch * p.batch_stride + (int64_t)row0 * p.row_bytes), row_bytes((int)p.row_bytes), sign_mode(p.sign_mode) {
     const int rows_valid = rows_total - row0;
     const int quarter = tid & 3;
     kb_lane = quarter * 16;
@@ -211,8 +212,9 @@ static thread_local int g_i8_split = 0;  // tlq_tune_i8_split: 0 = automatic, 1 
 // `buffers`: every slice has an int32 [M,N] matrix of its own (plain stores, summed by the pass that follows);
 // otherwise the slices add into one matrix with atomic adds, which cost about 10 ns per thousand.
 // The estimate behind the choice, in microseconds: an under-filled launch is paced by what one work-group
-// streams, (BM + BN) * K bytes at about 40 GB/s; s slices divide that and add the cost of their sums.
-int i8_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K, bool buffers) {
+// streams, (BM + BN) * K bytes at about 40 GB/s (times `pace` for a slower loader: the one that unpacks int4 on
+// the way into LDS takes 2.5 times as long); s slices divide that and add the cost of their sums.
+int i8_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K, bool buffers, double pace) {
   if (batch != 1 || g_i8_split == 1 || (g_i8_tile && g_i8_split == 0)) return 1;  // a forced tile means: that kernel
   const int tile = M <= 32 ? 32 : 128;
   const int64_t tiles = ceil_div(M, tile) * ceil_div(N, (int64_t)128);
@@ -225,7 +227,7 @@ int i8_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K, bool buffers
   auto slices = [&](int64_t sl) { return ceil_div(stages, ceil_div(stages, sl)); };
   if (g_i8_split > 1) return (int)slices(g_i8_split < stages ? g_i8_split : stages);
   if (tiles * 2 > places) return 1;
-  const double one = (double)(tile + 128) * (double)K / 40e3;
+  const double one = (double)(tile + 128) * (double)K / 40e3 * pace;
   const double mn = (double)M * (double)N;
   double best = one;
   int64_t best_s = 1;
@@ -266,6 +268,7 @@ __global__ __launch_bounds__(256) void i32_sum_rescale_kernel(const int4_t* __re
     const int64_t m = i / n4_row;
     const int n = (int)(i - m * n4_row) * 4;
     int4_t a = partial[i];
+#pragma unroll 8  // independent loads in flight: with few outputs the pass is paced by their latency
     for (int z = 1; z < split; ++z) a += partial[(int64_t)z * n4_total + i];
     float4_t f;
 #pragma unroll
@@ -313,7 +316,7 @@ int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, 
 #define TLQ_RUN(BM, BN, WM, WN)                                                                  \
   {                                                                                              \
     typedef W4I8Loader<BN, WM * WN * 64> WL;                                                     \
-    typename WL::Params pw{(const uint8_t*)Wp, K / 2, sign_mode};                                \
+    typename WL::Params pw{(const uint8_t*)Wp, K / 2, sign_mode, 0};                             \
     return run_i8<WL, EpiInt32, BM, BN, WM, WN>(A, pw, pe, 1, M, N, K, st, "tlq_gemm_w4a8");     \
   }
   switch (tile) {
@@ -327,6 +330,55 @@ int gemm_w4a8_i32(const void* A, const void* Wp, void* C, int64_t M, int64_t N, 
 #undef TLQ_RUN
 }
 
+// C = the sum of the slices' int32 matrices (N % 4 == 0)
+__global__ __launch_bounds__(256) void i32_sum_kernel(const int4_t* __restrict__ partial, int split, int4_t* __restrict__ C,
+                                                      int64_t n4_total) {
+  for (int64_t i = blockIdx.x * 256 + threadIdx.x; i < n4_total; i += (int64_t)gridDim.x * 256) {
+    int4_t a = partial[i];
+#pragma unroll 8
+    for (int z = 1; z < split; ++z) a += partial[(int64_t)z * n4_total + i];
+    C[i] = a;
+  }
+}
+
+// W4A8 over K slices: the unpacking loader is the slowest of the family per work-group (registers, nibble expansion,
+// LDS stores), so few output tiles hurt it most.  With `partial` (int32 [split][M][N]) every slice stores its own
+// matrix and a second pass sums them; without, the slices add into C (cleared first) with atomic adds.
+int gemm_w4a8_i32_splitk(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
+                         int64_t split, int32_t* partial, hipStream_t st) {
+  split = whole_slices(K, split);
+  const int64_t n4 = M * N / 4;  // N % 4 == 0
+  const int64_t want = ceil_div(n4, (int64_t)256);
+  if (!partial) {
+    i32_clear_kernel<<<(int)(want > 4096 ? 4096 : want), 256, 0, st>>>((int4_t*)C, n4);
+    if (!check_launch("tlq_gemm_w4a8 (clear)")) return 1;
+  }
+  const int64_t stages = K / kStageBytes;
+  const int64_t ks = ceil_div(stages, split) * kStageBytes;
+  int rc;
+#define TLQ_RUN(Epi, pe, BM, BN, WM, WN)                                                                            \
+  {                                                                                                                 \
+    constexpr int NT = WM * WN * 64;                                                                                \
+    typedef RowLoaderDirect<BM, NT> AL;                                                                             \
+    typedef W4I8Loader<BN, NT> WL;                                                                                  \
+    typename AL::Params pa{(const uint8_t*)A, K, ks, ks};                                                           \
+    typename WL::Params pw{(const uint8_t*)Wp, K / 2, sign_mode, ks / 2};                                           \
+    rc = launch_gemm<MmaI8, AL, WL, Epi, BM, BN, WM, WN>(pa, pw, pe, split, M, N, ks, st, "tlq_gemm_w4a8 (K slices)", \
+                                                         2, (int)stages);                                           \
+  }
+  if (partial) {
+    EpiInt32::Params pe{partial, N, M * N};
+    if (M <= 32) TLQ_RUN(EpiInt32, pe, 32, 128, 1, 4) else TLQ_RUN(EpiInt32, pe, 128, 128, 2, 2)
+    if (rc) return rc;
+    i32_sum_kernel<<<(int)(want > 8192 ? 8192 : want), 256, 0, st>>>((const int4_t*)partial, (int)split, (int4_t*)C, n4);
+    return check_launch("tlq_gemm_w4a8 (sum)") ? 0 : 1;
+  }
+  EpiAtomicAddI32::Params pe{(int32_t*)C, N};
+  if (M <= 32) TLQ_RUN(EpiAtomicAddI32, pe, 32, 128, 1, 4) else TLQ_RUN(EpiAtomicAddI32, pe, 128, 128, 2, 2)
+#undef TLQ_RUN
+  return rc;
+}
+
 }  // namespace tlq
 
 extern "C" {
@@ -338,5 +390,5 @@ void tlq_tune_i8_tile(int block_m) { tlq::g_i8_tile = block_m; }
 void tlq_tune_i8_split(int slices) { tlq::g_i8_split = slices; }
 // The number of K slices the automatic choice (or the forced value) takes for one batch of this shape, with a matrix
 // per slice (buffers = 1: tlq_gemm_w8a8_ws) or atomic adds into the one output (0: tlq_gemm_i8).
-int tlq_debug_i8_split(int64_t M, int64_t N, int64_t K, int buffers) { return tlq::i8_split_choice(1, M, N, K, buffers != 0); }
+int tlq_debug_i8_split(int64_t M, int64_t N, int64_t K, int buffers) { return tlq::i8_split_choice(1, M, N, K, buffers != 0, 1.0); }
 }

@@ -3,9 +3,11 @@
 Surface of examples/dequantize_gemm/example_dequant_gemm_w4a8.py: ``w4a8_gemm_cv(M, N, K)``
 (:25-121) -> ``kernel(A, B_packed, workspace[, C]) -> C`` and ``torch_convert`` (:124-145).
 The reference unpacks on the vector cores into a caller-supplied int8 [N, K] global workspace
-and then runs the cube GEMM; so does this one when the workspace (third positional, as the
-reference's callers pass it) is a usable int8 [N, K] buffer: an unpack kernel at the HBM roofline
-and the int8 GEMM, which together beat the kernel that unpacks on the way into LDS.
+and then runs the cube GEMM; so does this one from 257 activation rows on when the workspace
+(third positional, as the reference's callers pass it) is a usable int8 [N, K] buffer: an unpack
+kernel at the HBM roofline and the int8 GEMM, which together beat the kernel that unpacks on the
+way into LDS.  With fewer rows the unpack pass would cost more than the GEMM: the fused kernel
+runs over slices of K and keeps one int32 [M, N] matrix per slice in the workspace.
 """
 from __future__ import annotations
 
