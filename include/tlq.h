@@ -197,6 +197,16 @@ int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, in
 int tlq_gemm_f16_batched(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype,
                          int out_dtype, int b_layout, void* stream);
 
+/* tlq_gemm_f16_batched with a workspace for one batch with few activation rows (too few output tiles to fill the machine):
+ * K is cut into slices of whole 128-byte stages that write fp32 [M,N] matrices into the workspace, and a second pass adds
+ * them in slice order and rounds once (deterministic).  tlq_f16_workspace_bytes gives the size for the preferred number
+ * of slices (0: this shape is not cut); a smaller workspace (16-byte aligned) means fewer slices, none means
+ * tlq_gemm_f16_batched.  No counterpart in the reference: its fp16_gemm (example_dequant_gemm_fine_grained.py:60-115)
+ * has one kernel for every M. */
+int64_t tlq_f16_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K);
+int tlq_gemm_f16_ws(const void* A, const void* B, void* C, void* workspace, int64_t workspace_bytes, int64_t batch, int64_t M,
+                    int64_t N, int64_t K, int in_dtype, int out_dtype, int b_layout, void* stream);
+
 /* Split-K form of the same GEMM, replaces gemm_splitk (examples/gemm_splitk/example_tilelang_gemm_splitk.py:16-48):
  * C (fp32 [M,N], accumulated IN PLACE, the caller zeroes it as the example does) += A[M,K] . B.  K is cut into
  * split_k slices handled by different work-groups that add their partial tiles with atomic adds, so small-M /
@@ -347,6 +357,8 @@ void tlq_tune_w4a16_split(int slices);                       /* K slices of the 
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,
                                                                +10 = never stage through LDS, +20 = stage whenever possible */
 void tlq_tune_i8_tile(int block_m);                         /* 32|128|256 */
+void tlq_tune_f16_split(int slices);                        /* K slices of tlq_gemm_f16_ws: 0 = automatic, 1 = never, n = up to n */
+int tlq_debug_f16_split(int64_t M, int64_t N, int64_t K);  /* K slices tlq_gemm_f16_ws takes for one batch of this shape */
 void tlq_tune_w4a8_ws(int mode);                            /* tlq_gemm_w4a8_ws: 0 = automatic, 1 = K slices in the workspace, 2 = unpack + int8 GEMM */
 void tlq_tune_i8_split(int slices);                         /* K slices of the one-batch int8 kernels: 0 = automatic, 1 = never, n = up to n */
 int tlq_debug_i8_split(int64_t M, int64_t N, int64_t K, int buffers); /* K slices taken for one batch of this shape: with a matrix per

@@ -178,16 +178,23 @@ def test_rejects_bad_arguments_of_the_widened_entry_points():
 
 def test_workspace_size_rules():
     """tlq_w4a16_workspace_bytes: nothing for decode shapes, fp32 partial sums of the K slices for small and middle M,
-    a dequantised copy of the weights (N * K 16-bit values) for large M."""
-    ws = _abi.load().tlq_w4a16_workspace_bytes
+    a dequantised copy of the weights (N * K 16-bit values) for large M -- and, from M = 256 on, where the plain GEMM of
+    the two passes has few output tiles, room for its K slices behind that copy (which of the kernels runs depends on the
+    group size, so the size covers both)."""
+    lib = _abi.load()
+    ws = lib.tlq_w4a16_workspace_bytes
     assert ws(1, 11008, 4096) == 0 and ws(16, 14336, 4096) == 0
     assert ws(4096, 4096, 4096) == 4096 * 4096 * 2
     assert ws(8192, 14336, 4096) == 14336 * 4096 * 2
-    for M, N, K in ((64, 14336, 4096), (256, 4096, 14336), (512, 4096, 4096), (1024, 4096, 14336)):
+    for M, N, K in ((64, 14336, 4096), (200, 4096, 4096), (255, 4096, 14336)):
         b = ws(M, N, K)
         assert b > 0 and b % (M * N * 4) == 0, (M, N, K, b)
         split = b // (M * N * 4)
         assert 2 <= split <= 16, (M, N, K, split)  # room for the most K slices any kernel and group size may cut
+    for M, N, K in ((256, 4096, 14336), (512, 4096, 4096), (1024, 4096, 14336)):
+        b = ws(M, N, K)
+        assert b >= N * K * 2 + lib.tlq_f16_workspace_bytes(1, M, N, K) and b >= 2 * M * N * 4, (M, N, K, b)
+        assert lib.tlq_f16_workspace_bytes(1, M, N, K) > 0
     assert ws(1024, 14336, 4096) == 14336 * 4096 * 2  # many output tiles already: no K slices, two passes
     assert ws(64, 0, 4096) == 0 and ws(64, 128, 0) == 0
 
@@ -201,9 +208,9 @@ def test_tuning_hooks_are_per_thread():
     from tilelang_ascend_amd import _abi
 
     lib = _abi.load()
-    M, N, K = 600, 4096, 4096
+    M, N, K = 200, 4096, 4096
     auto = lib.tlq_w4a16_workspace_bytes(M, N, K)
-    assert auto == 4 * M * N * 4
+    assert auto == 8 * M * N * 4
     lib.tlq_tune_w4a16_split(16)
     try:
         here = lib.tlq_w4a16_workspace_bytes(M, N, K)

@@ -77,6 +77,10 @@ SIGNATURES = {
     "tlq_tune_i8_tile": (None, [_int]),
     "tlq_tune_i8_split": (None, [_int]),
     "tlq_tune_w4a8_ws": (None, [_int]),
+    "tlq_tune_f16_split": (None, [_int]),
+    "tlq_debug_f16_split": (_int, [_i64, _i64, _i64]),
+    "tlq_f16_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
+    "tlq_gemm_f16_ws": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
     "tlq_debug_i8_split": (_int, [_i64, _i64, _i64, _int]),
     "tlq_w8a8_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
 }

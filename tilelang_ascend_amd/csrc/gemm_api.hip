@@ -28,6 +28,10 @@ int gemm_f16_plain(const void* A, const void* B, void* C, int64_t batch, int64_t
                    int out_dtype, int b_layout, hipStream_t st);
 int gemm_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
                     int in_dtype, int b_layout, hipStream_t st);
+extern thread_local int g_f16_split;
+int f16_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K);
+int gemm_f16_slices(const void* A, const void* B, void* C, float* partial, int64_t M, int64_t N, int64_t K, int64_t split,
+                    int in_dtype, int out_dtype, int b_layout, hipStream_t st);
 int gemm_i8_i32(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int b_layout,
                 hipStream_t st);
 int gemm_w8a8_rescale(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int64_t batch,
@@ -179,6 +183,15 @@ static int64_t stream_max_split(int64_t M, int64_t N, int64_t K) {
   return most;
 }
 
+// Second of the two passes: the plain GEMM on the dequantised matrix at the head of the workspace.  What the workspace
+// holds beyond that matrix is room for fp32 matrices of K slices (few output tiles: tlq_gemm_f16_ws).
+static int plain_gemm_on_workspace(const void* A, void* workspace, int64_t workspace_bytes, void* C, int64_t M, int64_t N,
+                                   int64_t K, int in_dtype, int out_dtype, void* stream) {
+  const int64_t head = (N * K * 2 + 15) / 16 * 16;
+  return tlq_gemm_f16_ws(A, workspace, C, (uint8_t*)workspace + head, workspace_bytes - head, 1, M, N, K, in_dtype, out_dtype,
+                         TLQ_B_NK, stream);
+}
+
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
   // small and middle M: fp32 partial sums of the K slices (sized for the smallest group, which allows the most slices)
@@ -189,8 +202,14 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const DecodePlan dp = w4a16_decode_plan(M, N, K, 32, 256);
     if (dp.ok && dp.chunks > split) split = dp.chunks;
   }
-  if (split > 1) return split * M * N * 4;
-  return M >= kTwoPassMinM ? N * K * 2 : 0;
+  int64_t need = split > 1 ? split * M * N * 4 : 0;
+  // two passes (which of the two is taken depends on the group size, so the size covers both): the dequantised matrix,
+  // then room for the K slices of the plain GEMM where it has few output tiles
+  if (M >= kTwoPassMinM) {
+    const int64_t two = (N * K * 2 + 15) / 16 * 16 + tlq_f16_workspace_bytes(1, M, N, K);
+    if (two > need) need = two;
+  }
+  return need;
 }
 
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
@@ -307,7 +326,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
               "tlq_gemm_w4a16_ws: group=%lld must divide K=%lld and be a multiple of 32", (long long)group, (long long)K);
   TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16_ws: scales / zeros misaligned");
   if (int rc = tlq_dequant_w4(w_packed, scales, zeros, workspace, N, K, group, zero_scalar, in_dtype, stream)) return rc;
-  return tlq_gemm_f16(A, workspace, C, M, N, K, in_dtype, out_dtype, TLQ_B_NK, stream);
+  return plain_gemm_on_workspace(A, workspace, workspace_bytes, C, M, N, K, in_dtype, out_dtype, stream);
 }
 
 int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
@@ -358,7 +377,7 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
               "tlq_gemm_w4a16_layout_ws: M=%lld N=%lld K=%lld needs a 16-byte aligned workspace of %lld bytes (got %lld) and N %% 8 == 0",
               (long long)M, (long long)N, (long long)K, (long long)(N * K * 2), (long long)workspace_bytes);
   if (int rc = tlq_dequant_w4_layout(w_packed, scales, zeros, workspace, N, K, group, zero_scalar, in_dtype, w_layout, stream)) return rc;
-  return tlq_gemm_f16(A, workspace, C, M, N, K, in_dtype, out_dtype, TLQ_B_NK, stream);
+  return plain_gemm_on_workspace(A, workspace, workspace_bytes, C, M, N, K, in_dtype, out_dtype, stream);
 }
 
 int tlq_gemv_w4a16_batched(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C,
@@ -404,6 +423,36 @@ int tlq_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, in
                  int b_layout, void* stream) {
   return tlq_gemm_f16_batched(A, B, C, 1, M, N, K, in_dtype, out_dtype, b_layout, stream);
 }
+
+int64_t tlq_f16_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K) {
+  if (batch != 1 || M <= 0 || N <= 0 || K <= 0 || M >= kMaxDim || N >= kMaxDim || K >= kMaxDim || N % 8 != 0) return 0;
+  const int split = f16_split_choice(batch, M, N, K);
+  return split > 1 ? (int64_t)split * M * N * 4 : 0;
+}
+
+int tlq_gemm_f16_ws(const void* A, const void* B, void* C, void* workspace, int64_t workspace_bytes, int64_t batch, int64_t M,
+                    int64_t N, int64_t K, int in_dtype, int out_dtype, int b_layout, void* stream) {
+  // One batch, few activation rows: K slices write fp32 matrices into the workspace, a second pass adds them in slice
+  // order and rounds once.  As many slices as the workspace holds; none, or a shape that is not cut: tlq_gemm_f16_batched.
+  int split = 1;
+  if (tlq_f16_workspace_bytes(batch, M, N, K) > 0 && workspace != nullptr && aligned16(workspace)) {
+    split = f16_split_choice(batch, M, N, K);
+    while (split > 1 && (int64_t)split * M * N * 4 > workspace_bytes) split /= 2;
+  }
+  if (split <= 1) return tlq_gemm_f16_batched(A, B, C, batch, M, N, K, in_dtype, out_dtype, b_layout, stream);
+  TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_f16_ws: in_dtype must be float16 or bfloat16 (got %d)",
+              in_dtype);
+  TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_f16_ws: bad out_dtype %d",
+              out_dtype);
+  TLQ_REQUIRE(b_layout == TLQ_B_KN || b_layout == TLQ_B_NK, "tlq_gemm_f16_ws: bad b_layout %d", b_layout);
+  TLQ_REQUIRE(A && B && C, "tlq_gemm_f16_ws: null pointer");
+  TLQ_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), "tlq_gemm_f16_ws: pointers must be 16-byte aligned");
+  TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K * 2), "tlq_gemm_f16_ws: a matrix spans 4 GiB or more");
+  return gemm_f16_slices(A, B, C, (float*)workspace, M, N, K, split, in_dtype, out_dtype, b_layout, (hipStream_t)stream);
+}
+
+void tlq_tune_f16_split(int slices) { g_f16_split = slices; }
+int tlq_debug_f16_split(int64_t M, int64_t N, int64_t K) { return f16_split_choice(1, M, N, K); }
 
 int tlq_gemm_f16_splitk(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t split_k,
                         int in_dtype, int b_layout, void* stream) {

@@ -85,6 +85,9 @@ struct H16KNLoader {
   }
 };
 
+// tlq_tune_gemm_tile: 0 = automatic, 128 / 256 = that square tile
+thread_local int g_gemm_f16_tile = 0;
+
 template <class Mma, int BM, int BN, int WM, int WN>
 static int run_f16(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int out_dtype,
                    int b_layout, hipStream_t st) {
@@ -142,8 +145,78 @@ int gemm_f16_splitk(const void* A, const void* B, float* C, int64_t M, int64_t N
                : run_f16_splitk<MmaBF16, 256, 256, 2, 4>(A, B, C, M, N, K, split_k, b_layout, st);
 }
 
-// tlq_tune_gemm_tile: 0 = automatic, 128 / 256 = that square tile
-thread_local int g_gemm_f16_tile = 0;
+
+// ---- K slices with a matrix per slice (one batch, few activation rows) ---------------------------
+// With few activation rows the output tiles are too few to fill the machine and a work-group's run of stages is
+// latency bound.  Slice z of K is "batch" z of the loaders; slices are whole 128-byte stages, the last one holds what is
+// left; every slice stores its fp32 tile into its own [M, N] matrix and a second pass adds them in slice order and
+// rounds once (deterministic, unlike the atomic adds of gemm_f16_splitk).
+void launch_splitk_reduce(const float* partial, void* C, int64_t M, int64_t N, int split, int out_dtype, hipStream_t st);
+
+thread_local int g_f16_split = 0;  // tlq_tune_f16_split: 0 = automatic, 1 = never, n = up to n slices
+
+// The estimate is the one of the int8 kernels (i8_split_choice): (BM + BN) rows of K * 2 bytes at about 40 GB/s
+// per work-group, divided by the slices, plus a pass over their matrices.
+int f16_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K) {
+  if (batch != 1 || g_f16_split == 1 || (g_gemm_f16_tile && g_f16_split == 0) || (K * 2) % kStageBytes != 0) return 1;
+  const int tile = M <= 32 ? 32 : 128;
+  const int64_t tiles = ceil_div(M, tile) * ceil_div(N, (int64_t)128);
+  int cus = tlq_device_cu_count();
+  if (cus <= 0) cus = 256;
+  const int64_t places = (int64_t)cus * (tile == 32 ? 4 : 2);
+  const int64_t stages = K * 2 / kStageBytes;
+  auto slices = [&](int64_t sl) { return ceil_div(stages, ceil_div(stages, sl)); };
+  if (g_f16_split > 1) return (int)slices(g_f16_split < stages ? g_f16_split : stages);
+  if (tiles * 2 > places) return 1;
+  const double one = (double)(tile + 128) * (double)K * 2 / 40e3;
+  const double mn = (double)M * (double)N;
+  double best = one;
+  int64_t best_s = 1;
+  for (int64_t want = 2; want * tiles <= places && want * 2 <= stages; ++want) {
+    const int64_t sl = slices(want);
+    if (sl != want) continue;
+    const double t = one * (double)ceil_div(stages, sl) / (double)stages + 3.0 + (double)sl * mn * 8 / 4e6;
+    if (t < best * (best_s == 1 ? 0.85 : 0.97)) best = t, best_s = sl;
+  }
+  return (int)best_s;
+}
+
+template <class Mma, int BM, int BN, int WM, int WN>
+static int run_f16_slices(const void* A, const void* B, float* partial, int64_t M, int64_t N, int64_t K, int64_t split,
+                          int b_layout, hipStream_t st) {
+  constexpr int NT = WM * WN * 64;
+  const int64_t stages = K * 2 / kStageBytes;
+  const int64_t ksb = ceil_div(stages, split) * kStageBytes;  // bytes of K per slice
+  typedef RowLoaderDirect<BM, NT> AL;
+  typename AL::Params pa{(const uint8_t*)A, K * 2, ksb, ksb};
+  EpiFloat::Params pe{partial, N, M * N, TLQ_F32};
+  if (b_layout == TLQ_B_NK) {
+    typedef RowLoaderDirect<BN, NT> WL;
+    typename WL::Params pw{(const uint8_t*)B, K * 2, ksb, ksb};
+    return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, split, M, N, ksb, st, "tlq_gemm_f16 (K slices)", 4, (int)stages);
+  }
+  typedef H16KNLoaderDirect<BN, NT> WL;  // N % 8 == 0
+  H16KNParams pw{(const uint8_t*)B, N * 2, (ksb / 2) * N * 2, ksb / 2};
+  return launch_gemm<Mma, AL, WL, EpiFloat, BM, BN, WM, WN>(pa, pw, pe, split, M, N, ksb, st, "tlq_gemm_f16 (K slices)", 4, (int)stages);
+}
+
+// partial: fp32 [split][M][N]
+int gemm_f16_slices(const void* A, const void* B, void* C, float* partial, int64_t M, int64_t N, int64_t K, int64_t split,
+                    int in_dtype, int out_dtype, int b_layout, hipStream_t st) {
+  const int64_t stages = K * 2 / kStageBytes;
+  if (split > stages) split = stages;
+  split = ceil_div(stages, ceil_div(stages, split));  // no empty slice
+  int rc;
+  if (in_dtype == TLQ_F16)
+    rc = M <= 32 ? run_f16_slices<MmaF16, 32, 128, 1, 4>(A, B, partial, M, N, K, split, b_layout, st)
+                 : run_f16_slices<MmaF16, 128, 128, 2, 2>(A, B, partial, M, N, K, split, b_layout, st);
+  else
+    rc = M <= 32 ? run_f16_slices<MmaBF16, 32, 128, 1, 4>(A, B, partial, M, N, K, split, b_layout, st)
+                 : run_f16_slices<MmaBF16, 128, 128, 2, 2>(A, B, partial, M, N, K, split, b_layout, st);
+  if (rc) return rc;
+  launch_splitk_reduce(partial, C, M, N, (int)split, out_dtype, st);
+  return check_launch("tlq_gemm_f16 (sum of the slices)") ? 0 : 1;
+}
 
 template <class Mma>
 static int dispatch_f16(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int out_dtype,

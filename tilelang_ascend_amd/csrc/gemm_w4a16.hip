@@ -689,6 +689,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4_t* __re
                                                            int64_t n4, int split, int out_dtype) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
     float4_t v = partial[i];
+#pragma unroll 8  // loads of eight slices in flight (with few outputs the pass is paced by their latency); same order of adds
     for (int z = 1; z < split; ++z) v += partial[(int64_t)z * n4 + i];
     if (out_dtype == TLQ_F16) {
       half_t h[4] = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};

@@ -128,8 +128,13 @@ def fp16_gemm(M: int, N: int, K: int, block_M: int, block_N: int, block_K: int):
 
     def launch(t, sym, stream):
         A, B, C = t
-        _abi.check(_abi.load().tlq_gemm_f16(_abi.ptr(A), _abi.ptr(B), _abi.ptr(C), M, N, K, _abi.F16, _abi.F16,
-                                            _abi.B_KN, stream))
+        lib = _abi.load()
+        # few activation rows: K slices with their fp32 matrices in a workspace (allocated per call, like the
+        # reference's workspace_idx buffers); 0 bytes for every other shape
+        ws_bytes = lib.tlq_f16_workspace_bytes(1, M, N, K)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device) if ws_bytes else None
+        _abi.check(lib.tlq_gemm_f16_ws(_abi.ptr(A), _abi.ptr(B), _abi.ptr(C), _abi.ptr(ws), ws_bytes, 1, M, N, K, _abi.F16,
+                                       _abi.F16, _abi.B_KN, stream))
 
     return KernelSpec("fp16_gemm", [Param("A", (M, K), "float16"), Param("B", (K, N), "float16"),
                                     Param("C", (M, N), "float16")], launch,
