@@ -293,7 +293,7 @@ def bench_prefill(args, steps=None, cpu=True):
     out = {"workload": "W4A16 prefill GEMM M=N=K=4096 bf16 group=128 zero=8, automatic choice with a caller-owned workspace "
                        "(dequantisation pass + plain MFMA GEMM; the whole step is priced against the MFMA peak)", "dtype": "bf16",
            "value": round(flops / tm.wall / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": tm.wall * 1e3,
-           "roofline": dict({"kernel": "dequant_w4_vec8<bf16> + gemm_slots_kernel<MmaBF16,RowLoaderDirect,EpiFloat>", "bound": "mfma"},
+           "roofline": dict({"kernel": "dequant_w4_vec8<bf16> + gemm_mfma_kernel<MmaBF16,RowLoaderDirect,RowLoaderDirect,EpiFloat,256,256,2,4>", "bound": "mfma"},
                             **tm.roofline(flops, MFMA_F16_PEAK_TFLOPS, "TFLOP/s", 1e12),
                             traffic=traffic_from_profile("gemm_w4a16_bf16_M4096_N4096_K4096_g128.txt"), flops_per_launch=flops),
            "fused_kernel": {"path": "tlq_gemm_w4a16(algo=mfma): gemm_mfma_kernel<MmaBF16,RowLoaderDirect,W4Loader>, one launch, no workspace",

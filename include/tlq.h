@@ -347,9 +347,10 @@ void tlq_tune_gemv_ring(int on);                             /* 1 (default): a s
 void tlq_tune_gemm_band(int tile_rows);                       /* tile rows per band of the MFMA kernels' tile order (default 4) */
 void tlq_tune_gemm_tile(int tile);                            /* square tile of the plain 16-bit GEMM (and of the second of the two W4A16 passes):
                                                               * 128 | 256, 0 = by the number of output tiles */
-void tlq_tune_gemm_slots(int on);                            /* 1 (default): 256 x 256 tiles of the plain 16-bit GEMM with [N, K] weights and of the
-                                                              * int8 GEMMs run on the kernel that cuts LDS into five operand-tile slots
-                                                              * (whole 128-byte stages of K only); 0: always the two-stage kernel */
+void tlq_tune_gemm_slots(int mode);                          /* the kernel that cuts LDS into five operand-tile slots (256 x 256 tiles, whole 128-byte
+                                                              * stages of K only): 1 (default) where it measured faster than the two-stage kernel
+                                                              * (int8, several batches of up to 2048 rows), 2 wherever it can run (also the plain
+                                                              * 16-bit GEMMs), 0 never */
 void tlq_tune_w4a16_decode(int on);                          /* 0: the decode kernel is never picked automatically */
 void tlq_tune_w4a16_stream(int on);                          /* 0: tlq_gemm_w4a16_ws never picks the streaming kernel by itself */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */

@@ -1,5 +1,6 @@
-"""The two main loops of the 256 x 256 GEMM tiles against each other: the five-slot kernel (csrc/gemm_slots.h, the
-default for whole 128-byte stages of K) and the two-stage kernel (csrc/gemm_core.h, tlq_tune_gemm_slots(0)).  Every case
+"""The two main loops of the 256 x 256 GEMM tiles against each other: the five-slot kernel (csrc/gemm_slots.h, whole
+128-byte stages of K; tlq_tune_gemm_slots(2) takes it wherever it can run) and the two-stage kernel (csrc/gemm_core.h,
+tlq_tune_gemm_slots(0)).  Every case
 runs the same inputs through both: integer GEMMs and the rescaled outputs must agree bit for bit, and so must the
 16-bit GEMMs (same tiling, same order of accumulation inside a tile; the kernels only differ in when data is fetched).
 The default path is also checked against an exact / fp32 evaluation.
@@ -51,7 +52,7 @@ def test_plain_gemm_same_bits_on_both_main_loops(hook, value, dtype, M, N, K):
         torch.cuda.synchronize()
         return C.cpu()
 
-    want = run()
+    want = _with_hook(hook, 2, run)  # the five-slot kernel wherever it can run
     ref32 = A.float().cpu() @ B.float().cpu().t()
     assert float((want.float() - ref32).norm() / ref32.norm()) < 3e-3
     got = _with_hook(hook, value, run)
@@ -85,7 +86,7 @@ def test_w8a8_same_bits_on_both_main_loops(hook, value, layout, B, M, N, K):
             lib.tlq_tune_i8_tile(0)
         return C.cpu(), Ci.cpu()
 
-    want, want_i = run()
+    want, want_i = _with_hook(hook, 2, run)  # the five-slot kernel wherever it can run
     Wt = W.cpu() if layout == "KN" else W.cpu().transpose(1, 2)
     exact = torch.matmul(A.cpu().double(), Wt.double()).to(torch.int64)
     assert torch.equal(want_i.to(torch.int64), exact)

@@ -166,6 +166,7 @@ def test_kn_operand_on_the_five_slot_kernel(dtype, B, M, N, K):
     lib = _abi.load()
     kernel = batch_matmul(B, M, N, K, 128, 256, 64, dtype=dtype)
     lib.tlq_tune_gemm_tile(256)
+    lib.tlq_tune_gemm_slots(2)  # the five-slot kernel wherever it can run
     try:
         a, b = _ternary((B, M, K), 66).to(DT[dtype]), _ternary((B, K, N), 67).to(DT[dtype])
         got = kernel(a.cuda(), b.cuda()).cpu()

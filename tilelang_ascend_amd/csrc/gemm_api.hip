@@ -58,7 +58,7 @@ int gemm_w4a16_decode(const void* A, const void* Wp, const void* scales, const v
                       hipStream_t st);
 
 thread_local int g_gemm_band_rows = 0;
-thread_local int g_gemm_slots = 1;
+thread_local int g_gemm_slots = 1;  // tlq_tune_gemm_slots: 0 = never the five-slot kernel, 1 = where it measured faster, 2 = wherever it can run
 extern thread_local int g_gemm_f16_tile;
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // compute units of the current device (256 when it cannot be asked, e.g. without a GPU)
@@ -82,11 +82,11 @@ using namespace tlq;
 extern "C" {
 
 void tlq_tune_gemm_band(int tile_rows) { tlq::g_gemm_band_rows = tile_rows < 0 ? 0 : tile_rows; }
-void tlq_tune_gemm_slots(int on) { tlq::g_gemm_slots = on != 0; }
+void tlq_tune_gemm_slots(int mode) { tlq::g_gemm_slots = mode < 0 ? 0 : (mode > 2 ? 2 : mode); }
 int tlq_debug_gemm_tile(int64_t batch, int64_t M, int64_t N, int fused) {
   return tlq::prefer_small_tiles(batch, M, N, fused ? 0.65 : 0.72) ? 128 : 256;
 }
-void tlq_tune_gemm_tile(int tile) { tlq::g_gemm_f16_tile = (tile == 128 || tile == 256) ? tile : 0; }
+void tlq_tune_gemm_tile(int tile) { tlq::g_gemm_f16_tile = (tile == 128 || tile == 256 || tile == 2562) ? tile : 0; }
 void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
 void tlq_tune_w4a16_decode(int on) { tlq::g_w4a16_decode = on != 0; }
 

@@ -221,16 +221,19 @@ int gemm_f16_slices(const void* A, const void* B, void* C, float* partial, int64
 template <class Mma>
 static int dispatch_f16(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int out_dtype,
                         int b_layout, hipStream_t st) {
+  if (g_gemm_f16_tile == 2562) return run_f16<Mma, 256, 256, 2, 2>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);  // experiment: four wavefronts, 128 x 128 each
   const bool small = g_gemm_f16_tile ? g_gemm_f16_tile == 128 : prefer_small_tiles(batch, M, N);
   if (small)
     return run_f16<Mma, 128, 128, 2, 2>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);
-  if (g_gemm_slots && b_layout == TLQ_B_NK && K % 64 == 0) {  // whole 128-byte stages
+  // (the five-slot kernel only on request: alternating runs on one box have the two-stage loop 3 - 14 % ahead on ten of
+  // twelve 16-bit shapes, 2 % behind on the other two)
+  if (g_gemm_slots == 2 && b_layout == TLQ_B_NK && K % 64 == 0) {  // whole 128-byte stages
     typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K * 2, M * K * 2, K * 2},
         pw{(const uint8_t*)B, K * 2, N * K * 2, K * 2};
     EpiFloat::Params pe{C, N, M * N, out_dtype};
     return launch_gemm_slots<Mma, RowLoaderDirect<256, 512>, EpiFloat>(pa, pw, pe, batch, M, N, K * 2, st, "tlq_gemm_f16", 4);
   }
-  if (g_gemm_slots && b_layout == TLQ_B_KN && K % 64 == 0 && N % 8 == 0) {  // [K, N] weights, transposed in the operand read
+  if (g_gemm_slots == 2 && b_layout == TLQ_B_KN && K % 64 == 0 && N % 8 == 0) {  // [K, N] weights, transposed in the operand read
     typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K * 2, M * K * 2, K * 2};
     H16KNParams pw{(const uint8_t*)B, N * 2, K * N * 2, K};
     EpiFloat::Params pe{C, N, M * N, out_dtype};

@@ -121,8 +121,11 @@ template <class Epi>
 static int dispatch_i8(const void* A, const void* B, const typename Epi::Params& pe, int64_t batch, int64_t M,
                        int64_t N, int64_t K, int b_layout, hipStream_t st, const char* what) {
   const int tile = pick_tile(batch, M, N);
+  // The five-slot kernel where it measured ahead of the two-stage loop in alternating runs: several batches of up to
+  // 2048 rows (1 - 3 %); with one batch or longer matrices the two-stage loop is 2 - 14 % ahead.
+  const bool slots = g_gemm_slots == 2 || (g_gemm_slots == 1 && batch > 1 && M <= 2048);
   if (b_layout == TLQ_B_KN) {
-    if (g_gemm_slots && tile == 256 && K % 128 == 0) {  // whole 128-byte stages
+    if (slots && tile == 256 && K % 128 == 0) {  // whole 128-byte stages
       typedef I8KNLoaderDirect<256, 512> WL;
       typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K, M * K, K};
       typename WL::Params pw{(const uint8_t*)B, N, K * N, K};
@@ -144,7 +147,7 @@ static int dispatch_i8(const void* A, const void* B, const typename Epi::Params&
     }
 #undef TLQ_RUN
   } else {
-    if (g_gemm_slots && tile == 256 && K % 128 == 0) {  // whole 128-byte stages
+    if (slots && tile == 256 && K % 128 == 0) {  // whole 128-byte stages
       typename RowLoaderDirect<256, 512>::Params pa{(const uint8_t*)A, K, M * K, K}, pw{(const uint8_t*)B, K, N * K, K};
       return launch_gemm_slots<MmaI8, RowLoaderDirect<256, 512>, Epi>(pa, pw, pe, batch, M, N, K, st, what, 2);
     }
