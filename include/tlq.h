@@ -147,6 +147,9 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
  * the weights again in every row block of the fused kernel.  The workspace holds nothing between calls.
  * algo: as tlq_gemm_w4a16, or TLQ_ALGO_TWO_PASS to force the two passes (workspace required). */
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K);
+/* The least workspace with which tlq_gemm_w4a16_ws still takes a workspace-based kernel for this shape (the partial sums
+ * of the K-slice kernels where they apply, else the dequantised matrix of the two passes); for callers short of memory. */
+int64_t tlq_w4a16_workspace_bytes_min(int64_t M, int64_t N, int64_t K);
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream);
@@ -164,8 +167,9 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose wrapper allocates its
  * workspace anew on every call (tilelang/jit/adapter/cython/cython_wrapper.pyx:128-129).  The workspace is
  * a device array built into the library, TLQ_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends; problems whose
- * tlq_w4a16_workspace_bytes(M, N, K) exceeds it are rejected with an error (use tlq_gemm_w4a16_ws for those).  The call
- * allocates and frees nothing; results are those of tlq_gemm_w4a16_ws with a sufficient workspace, bit for bit.  All
+ * tlq_w4a16_workspace_bytes_min(M, N, K) exceeds it are rejected with an error (use tlq_gemm_w4a16_ws for those).  The
+ * call allocates and frees nothing; results are those of tlq_gemm_w4a16_ws with a workspace of
+ * TLQ_NOALLOC_SCRATCH_BYTES bytes (the preferred kernel where tlq_w4a16_workspace_bytes(M, N, K) fits), bit for bit.  All
  * calls on one GPU share the array: calls that overlap there (other streams, other threads) race.
  * tlq_gemm_w4a16_noalloc_init looks the array's address up for the current device (otherwise the first call on a
  * device does it); it allocates nothing either. */

@@ -57,12 +57,39 @@ def test_noalloc_matches_the_workspace_entry_point_twice_in_a_row():
     assert_bit_equal(got, want, "two-pass problem, third call")
 
 
+def test_noalloc_takes_the_next_best_kernel_when_only_that_fits():
+    """M = 300, N = 4096, K = 11008: the two passes would need 86 MiB + the K slices of their GEMM, more than the built-in
+    array; the partial sums of the K-slice kernels (51.6 MiB) fit.  The call must then equal tlq_gemm_w4a16_ws with a
+    workspace of the array's size, bit for bit, and meet the float bar against the oracle."""
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    M, N, K, g = 300, 4096, 11008, 128
+    assert lib.tlq_w4a16_workspace_bytes(M, N, K) > SCRATCH >= lib.tlq_w4a16_workspace_bytes_min(M, N, K) > 0
+    A = torch.randn(M, K, generator=gen(41)).half()
+    Wp, s, z = make_w4(N, K, g, torch.float16, "int", 42)
+    dA, dW, dS, dZ = A.cuda(), Wp.cuda(), s.cuda(), z.cuda()
+    st = torch.cuda.current_stream().cuda_stream
+    ws = torch.empty(SCRATCH, dtype=torch.uint8, device="cuda")
+    want = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    _abi.check(lib.tlq_gemm_w4a16_ws(P(dA), P(dW), P(dS), P(dZ), P(want), M, N, K, g, 0.0, _abi.F16, _abi.F16, _abi.ALGO_AUTO,
+                                     P(ws), SCRATCH, st))
+    got = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    before = torch.cuda.memory_allocated()
+    _abi.check(lib.tlq_gemm_w4a16_noalloc(P(dA), P(dW), P(dS), P(dZ), P(got), M, N, K, g, 0.0, _abi.F16, _abi.F16,
+                                          _abi.ALGO_AUTO, st))
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert_bit_equal(got.cpu(), want.cpu(), "next-best kernel in the built-in array")
+    check_float_output(got.cpu(), w4a16_reference(A, Wp, s, z, g), "next-best kernel vs the oracle")
+
+
 def test_noalloc_rejects_what_does_not_fit():
     from tilelang_ascend_amd import _abi
 
     lib, P = _abi.load(), _abi.ptr
     M, N, K = 2048, 14336, 4096  # two passes would need 112 MiB
-    assert lib.tlq_w4a16_workspace_bytes(M, N, K) > SCRATCH
+    assert lib.tlq_w4a16_workspace_bytes_min(M, N, K) > SCRATCH
     A = torch.zeros(8, dtype=torch.float16, device="cuda")  # never read: the call is rejected before any launch
     rc = lib.tlq_gemm_w4a16_noalloc(P(A), P(A), None, None, P(A), M, N, K, 128, 8.0, _abi.F16, _abi.F16, _abi.ALGO_AUTO, None)
     assert rc != 0

@@ -43,6 +43,7 @@ SIGNATURES = {
     "tlq_gemm_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_gemm_w8a8_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_w4a16_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "tlq_w4a16_workspace_bytes_min": (_i64, [_i64, _i64, _i64]),
     "tlq_gemm_w4a16_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp, _i64, _vp]),
     "tlq_gemm_w4a16_layout_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _int, _vp, _i64, _vp]),
     "tlq_dequant_w4_layout": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _int, _int, _vp]),

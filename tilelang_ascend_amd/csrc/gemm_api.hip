@@ -192,9 +192,9 @@ static int plain_gemm_on_workspace(const void* A, void* workspace, int64_t works
                          TLQ_B_NK, stream);
 }
 
-int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  if (N <= 0 || K <= 0) return 0;
-  // small and middle M: fp32 partial sums of the K slices (sized for the smallest group, which allows the most slices)
+// fp32 partial sums of the K slices of the kernels for small and middle M (sized for the smallest group, which allows the
+// most slices); 0 when none of them cuts K
+static int64_t w4a16_partial_sum_bytes(int64_t M, int64_t N, int64_t K) {
   int64_t split = w4a16_mid_split(M, N, K, 32);
   const int64_t ssplit = stream_max_split(M, N, K);
   if (ssplit > split) split = ssplit;
@@ -202,7 +202,12 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const DecodePlan dp = w4a16_decode_plan(M, N, K, 32, 256);
     if (dp.ok && dp.chunks > split) split = dp.chunks;
   }
-  int64_t need = split > 1 ? split * M * N * 4 : 0;
+  return split > 1 ? split * M * N * 4 : 0;
+}
+
+int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (N <= 0 || K <= 0) return 0;
+  int64_t need = w4a16_partial_sum_bytes(M, N, K);
   // two passes (which of the two is taken depends on the group size, so the size covers both): the dequantised matrix,
   // then room for the K slices of the plain GEMM where it has few output tiles
   if (M >= kTwoPassMinM) {
@@ -210,6 +215,13 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (two > need) need = two;
   }
   return need;
+}
+
+int64_t tlq_w4a16_workspace_bytes_min(int64_t M, int64_t N, int64_t K) {
+  if (N <= 0 || K <= 0) return 0;
+  const int64_t partial = w4a16_partial_sum_bytes(M, N, K);
+  if (partial > 0) return partial;
+  return M >= kTwoPassMinM ? N * K * 2 : 0;
 }
 
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,

@@ -62,7 +62,10 @@ int tlq_gemm_w4a16_noalloc_init(void) {
 int tlq_gemm_w4a16_noalloc(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                            int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                            void* stream) {
-  const int64_t need = tlq_w4a16_workspace_bytes(M, N, K);
+  // The array must hold what the preferred kernel for this shape needs, or at least what the next best one does (the
+  // call then equals tlq_gemm_w4a16_ws with a workspace of TLQ_NOALLOC_SCRATCH_BYTES bytes, which takes what fits).
+  int64_t need = tlq_w4a16_workspace_bytes(M, N, K);
+  if (need > (int64_t)TLQ_NOALLOC_SCRATCH_BYTES) need = tlq_w4a16_workspace_bytes_min(M, N, K);
   if (need > (int64_t)TLQ_NOALLOC_SCRATCH_BYTES) {
     set_error("tlq_gemm_w4a16_noalloc: M=%lld N=%lld K=%lld needs %lld bytes of scratch, the built-in array holds %lld; "
               "use tlq_gemm_w4a16_ws with a caller-owned workspace",
