@@ -710,11 +710,16 @@ static thread_local int g_w4a16_split = 0;  // forced number of K slices for tun
 // fraction of the work-group places (256, or 512 for the smaller tiles) that the tile kernel fills with the K cut it would take
 double w4a16_mid_fill(int64_t M, int64_t N, int64_t K, int64_t group);
 
+int f16_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K);  // gemm_f16.hip
+
 int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group) {
   // Where cutting K pays (measured against the two passes on the MLP shapes): up to M = 512 always, up to
   // M = 2048 while the 256 x 256 output tiles would fill at most a quarter of the chip.
   const bool region = M > 16 && (M <= 512 || (M < 2048 && ceil_div(M, (int64_t)256) * ceil_div(N, (int64_t)256) <= 64));
   if (!region || (group & (group - 1)) != 0 || N % 4 != 0) return 1;
+  // Above 512 rows the two passes are the alternative, and where their plain GEMM cuts K itself (few output tiles) they
+  // are ahead of this kernel: M = 768, N = K = 5120: 66 against 89 us.
+  if (M > 512 && g_w4a16_split == 0 && f16_split_choice(1, M, N, K) > 1) return 1;
   if (g_w4a16_split > 0) {
     const int64_t s = g_w4a16_split, unit0 = group > 64 ? group : 64;
     return (s <= 16 && K % s == 0 && (K / s) % unit0 == 0) ? s : 1;
