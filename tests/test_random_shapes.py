@@ -141,3 +141,22 @@ def test_dequant_unpack_and_activation_quantiser_on_random_shapes(ops, seed):
     wq, wsc = ref.act_quant_torch(x)
     assert_bit_equal(q.cpu(), wq, "act_quant values")
     assert_bit_equal(sc.cpu().reshape(-1), wsc.reshape(-1), "act_quant scales")
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_plain_16_bit_gemm_on_random_shapes(ops, seed):
+    """fp16_gemm (fine_grained.py:60-115) through the operator, which cuts K into slices for few activation rows and takes
+    the tile kernels otherwise: the float-output bar against an fp32 product, and the same bits on a second call."""
+    rnd = random.Random(9000 + seed)
+    M = rnd.choice([1, 7, 16, 32, 33, 100, 128, 129, 256, 300, 513, 1024, 2048])
+    N = rnd.choice([8, 64, 128, 136, 256, 264, 1024, 2056, 4096])
+    K = rnd.choice([8, 64, 128, 192, 448, 512, 1024, 2048, 4096, 11008])
+    while M * N * K > 1 << 31:
+        M = max(1, M // 2)
+    print(f"fp16_gemm seed={seed} M={M} N={N} K={K}", flush=True)
+    A = torch.randn(M, K, generator=gen(9100 + seed)).half()
+    B = torch.randn(K, N, generator=gen(9200 + seed)).half()
+    kernel = ops.fp16_gemm(M, N, K, 128, 256, 64)
+    got = kernel(A.cuda(), B.cuda()).cpu()
+    check_float_output(got, A.float() @ B.float(), f"fp16_gemm {M}x{N}x{K}")
+    assert torch.equal(got, kernel(A.cuda(), B.cuda()).cpu()), "the result must be reproducible"
