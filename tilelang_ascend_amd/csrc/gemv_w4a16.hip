@@ -275,7 +275,7 @@ __global__ __launch_bounds__(256, 4) void gemv_w4a16_f16_kernel(const half_t* __
     for (int r = 0; r < R; ++r) {
       int row = at.rg * R + r;
       row = row < N ? row : N - 1;  // clamp: loads stay in bounds
-      st.w[r] = *(const uint4_t*)(Wp + (uint32_t)(row * row_bytes + (cc << 4)));
+      st.w[r] = __builtin_nontemporal_load((const uint4_t*)(Wp + (uint32_t)(row * row_bytes + (cc << 4))));  // read once
       const uint32_t go = (uint32_t)(row * groups + gi);
       const half_t sv = sp[has_s ? go : 0u];
       const half_t zv = zp[has_z ? go : 0u];
@@ -416,7 +416,8 @@ __device__ __forceinline__ void gemv_rows_body(const T* __restrict__ A, const ui
   };
   auto issue = [&](Stage& st, int row) {
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) st.w[it] = *(const uint4_t*)(Wp + (uint32_t)(row * row_bytes + (cc[it] << 4)));
+    for (int it = 0; it < ITERS; ++it)  // read once: non-temporal (24 weight sets per launch: 94.5 instead of 101.6 us)
+      st.w[it] = __builtin_nontemporal_load((const uint4_t*)(Wp + (uint32_t)(row * row_bytes + (cc[it] << 4))));
   };
   Stage st[D];
   int irow = r0 + wave;  // next row to request
@@ -615,6 +616,11 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
   auto dma16 = [&](uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
   };
+  // the packed weights are read once: non-temporal, so that they do not displace what the caches hold for later
+  // (single launch of 22.5 MB: 6.46 instead of 7.18 us)
+  auto dma16_once = [&](uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+  };
   auto wait_vm = [&](int outstanding) {  // a wavefront-uniform count, 0 .. ITERS * D
     static_assert(ITERS * D <= 6, "cases below");
     switch (outstanding) {
@@ -656,7 +662,7 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
   auto issue = [&](int i, int slot) {  // the wavefront's i-th row into ring slot `slot`
     const uint8_t* const base = uniform_ptr(Wp + (int64_t)(r0 + wave + i * nwaves) * row_bytes);
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) dma16(lds0 + L.ring + addr::ring_w_lds(wave, slot, it, D, ITERS), voff_w[it], base);
+    for (int it = 0; it < ITERS; ++it) dma16_once(lds0 + L.ring + addr::ring_w_lds(wave, slot, it, D, ITERS), voff_w[it], base);
   };
 #pragma unroll
   for (int d = 0; d < D; ++d)
@@ -819,7 +825,7 @@ __global__ __launch_bounds__(256) void gemv_w4a16_kernel(const T* __restrict__ A
       const int g = (c << 5) / group;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        w[r] = *(const uint4_t*)(Wp + rows[r] * row_bytes + ((int64_t)c << 4));
+        w[r] = __builtin_nontemporal_load((const uint4_t*)(Wp + rows[r] * row_bytes + ((int64_t)c << 4)));  // read once
         s[r] = scales ? scales[(int64_t)rows[r] * groups + g] : one;
         z[r] = zeros ? zeros[(int64_t)rows[r] * groups + g] : zs;
       }
