@@ -80,7 +80,8 @@ __global__ __launch_bounds__(1024) void gemv_plain_kernel(const uint8_t* __restr
         const int c = c0 + u * 64 + lane;
         const int cc = c < chunks ? c : chunks - 1;
 #pragma unroll
-        for (int r = 0; r < R; ++r) a[r][u] = ((const uint4_t*)ap[r])[cc];
+        // the matrix is read once: non-temporal (N = 11008, K = 4096 fp16: 16.5 instead of 18.0 us)
+        for (int r = 0; r < R; ++r) a[r][u] = __builtin_nontemporal_load((const uint4_t*)ap[r] + cc);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
