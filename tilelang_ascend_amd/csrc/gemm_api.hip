@@ -296,10 +296,22 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     // (groups of 32, M = 256, N = 11008, K = 4096: 56 against 74 us; N = K = 8192: 64 against 90 us).
     // (Only where the partial sums are tens of MB: on 4096 weight rows, or below, the streaming kernel stays ahead.)
     // And only where the tile kernel finds a K cut that fills the machine: rows of 11008 = 2 x 43 x 128 values can only be halved.
+    // Up to three blocks of 128 activation rows the streaming kernel is level with or ahead of the tile kernel over K
+    // slices on 18 of 20 (N, K) pairs (N = 10240, K = 8192, M = 384: 93 against 155 us; the other two are 4 % behind);
+    // with four blocks only while its work-groups fit the machine at once (N = 8192, K = 4096, M = 512: 51 against 59 us;
+    // N = 13824, K = 5120, 432 work-groups: 114 against 99 us).
+    // Its weak spot: somewhat more work-groups than CUs (one work-group per CU: the second round runs half empty).  Where
+    // K has no cut for the tile kernel either, the two passes, whose plain GEMM cuts K unevenly, are ahead then:
+    // N = 4096, K = 11008 (86 steps: 288 work-groups at M = 384, 384 at M = 512): 69 against 82 us, 78 against 87 us.
+    const int64_t stream_wgs = (int64_t)sp.m_blocks * sp.n_blocks * sp.split;
+    const int64_t cus_now = cu_count_or_default();
+    const bool thin_second_round = M > 256 && have && N % 8 == 0 && stream_wgs > cus_now && stream_wgs * 2 <= cus_now * 3 &&
+                                   w4a16_mid_split(M, N, K, group) <= 1;
+    const bool stream_first = (M <= 384 && !thin_second_round) || stream_wgs <= cus_now;
     const bool slices_too_short = (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
                                   w4a16_mid_fill(M, N, K, group) >= 0.66;
     if (sp.ok && args_ok && ws_ok &&
-        (algo == TLQ_ALGO_STREAM || (M <= 256 && !slices_too_short) || (!slices_too_short && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
+        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
     if (algo == TLQ_ALGO_STREAM) {
@@ -377,7 +389,7 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
   if (algo != TLQ_ALGO_TWO_PASS) {
     const StreamPlan sp = w4a16_stream_plan(M, N, K, group, cu_count_or_default());
     const bool ws_ok = sp.ok && (M * N) % 4 == 0 && (sp.split == 1 || (ws_aligned && workspace_bytes >= (int64_t)sp.split * M * N * 4));
-    if (ws_ok && (algo == TLQ_ALGO_STREAM || M <= 256 || tile_fill(1, M, N, 128) < 0.65 || !(ws_aligned && workspace_bytes >= N * K * 2)))  // (no tile kernel reads this layout: the alternative is the two passes)
+    if (ws_ok && (algo == TLQ_ALGO_STREAM || M <= 384 || (int64_t)sp.m_blocks * sp.n_blocks * sp.split <= cu_count_or_default() || tile_fill(1, M, N, 128) < 0.65 || !(ws_aligned && workspace_bytes >= N * K * 2)))  // (no tile kernel reads this layout: the alternative is the two passes)
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, sp,
                                (float*)workspace, (hipStream_t)stream);
     TLQ_REQUIRE(algo != TLQ_ALGO_STREAM, "tlq_gemm_w4a16_layout_ws: the streaming kernel does not take M=%lld N=%lld K=%lld group=%lld "
