@@ -86,7 +86,7 @@ void tlq_tune_gemm_slots(int mode) { tlq::g_gemm_slots = mode < 0 ? 0 : (mode > 
 int tlq_debug_gemm_tile(int64_t batch, int64_t M, int64_t N, int fused) {
   return tlq::prefer_small_tiles(batch, M, N, fused ? 0.65 : 0.72) ? 128 : 256;
 }
-void tlq_tune_gemm_tile(int tile) { tlq::g_gemm_f16_tile = (tile == 128 || tile == 256 || tile == 2562) ? tile : 0; }
+void tlq_tune_gemm_tile(int tile) { tlq::g_gemm_f16_tile = (tile == 128 || tile == 256) ? tile : 0; }
 void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
 void tlq_tune_w4a16_decode(int on) { tlq::g_w4a16_decode = on != 0; }
 

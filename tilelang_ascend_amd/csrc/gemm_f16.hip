@@ -221,7 +221,6 @@ int gemm_f16_slices(const void* A, const void* B, void* C, float* partial, int64
 template <class Mma>
 static int dispatch_f16(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K, int out_dtype,
                         int b_layout, hipStream_t st) {
-  if (g_gemm_f16_tile == 2562) return run_f16<Mma, 256, 256, 2, 2>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);  // experiment: four wavefronts, 128 x 128 each
   const bool small = g_gemm_f16_tile ? g_gemm_f16_tile == 128 : prefer_small_tiles(batch, M, N);
   if (small)
     return run_f16<Mma, 128, 128, 2, 2>(A, B, C, batch, M, N, K, out_dtype, b_layout, st);
