@@ -719,7 +719,12 @@ int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group) {
   if (!region || (group & (group - 1)) != 0 || N % 4 != 0) return 1;
   // Above 512 rows the two passes are the alternative, and where their plain GEMM cuts K itself (few output tiles) they
   // are ahead of this kernel: M = 768, N = K = 5120: 66 against 89 us.
-  if (M > 512 && g_w4a16_split == 0 && f16_split_choice(1, M, N, K) > 1) return 1;
+  // (Not where that GEMM would only halve rows of 13312 values or more: this kernel over four slices is 7 - 16 % ahead
+  // there -- N = 4096, K = 14336, M = 1024: 146 against 163 us; N = 5120, K = 13824, M = 768: 136 against 159 us.)
+  if (M > 512 && g_w4a16_split == 0) {
+    const int plain_slices = f16_split_choice(1, M, N, K);
+    if (plain_slices > 2 || (plain_slices == 2 && K < 13312)) return 1;
+  }
   if (g_w4a16_split > 0) {
     const int64_t s = g_w4a16_split, unit0 = group > 64 ? group : 64;
     return (s <= 16 && K % s == 0 && (K / s) % unit0 == 0) ? s : 1;
