@@ -291,7 +291,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     // against 137 us for the two passes, K = 4096: 34 against 43 us)
     // (rows of more than 8192 values that the tile kernel can cut into enough K slices stay with it: N = 5120, K = 13824:
     // 101 against 127 us)
-    // Small quantisation groups shorten the K slices (16 groups each): when the partial sums (split x M x N x 4 bytes,
+    // Small quantisation groups (32, 64) shorten the K slices (16 groups each): when the partial sums (split x M x N x 4 bytes,
     // written and read back) outweigh the packed weights, the tile kernel, which cuts K as it likes, is ahead
     // (groups of 32, M = 256, N = 11008, K = 4096: 56 against 74 us; N = K = 8192: 64 against 90 us).
     // (Only where the partial sums are tens of MB: on 4096 weight rows, or below, the streaming kernel stays ahead.)
@@ -308,7 +308,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const bool thin_second_round = M > 256 && have && N % 8 == 0 && stream_wgs > cus_now && stream_wgs * 2 <= cus_now * 3 &&
                                    w4a16_mid_split(M, N, K, group) <= 1;
     const bool stream_first = (M <= 384 && !thin_second_round) || stream_wgs <= cus_now;
-    const bool slices_too_short = (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
+    const bool slices_too_short = group < 128 && (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
                                   w4a16_mid_fill(M, N, K, group) >= 0.66;
     if (sp.ok && args_ok && ws_ok &&
         (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))

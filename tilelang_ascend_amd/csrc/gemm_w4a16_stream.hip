@@ -301,16 +301,34 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   const int unit = group > 128 ? (int)(group / 128) : 1;  // a slice is a whole number of groups
   const int cap = (int)(kStreamMaxGroups * group / 128);   // ... and holds at most 16 of them
   if (cap < unit) return p;
-  // K slices: as many as fill the chip once without a second round of work-groups
-  int64_t slices = (int64_t)cus / ((int64_t)p.n_blocks * p.m_blocks);
-  if (slices < 1) slices = 1;
-  int64_t ss = ceil_div((int64_t)steps_total, slices);
-  ss = ceil_div(ss, (int64_t)unit) * unit;
-  if (ss < 4 && steps_total >= 4) ss = ceil_div((int64_t)4, (int64_t)unit) * unit;  // at least four steps per work-group
-  if (ss > cap) ss = cap - cap % unit;
-  if (ss > steps_total) ss = steps_total;
-  p.slice_steps = (int)ss;
-  p.split = (int)ceil_div(steps_total, ss);
+  // K slices: the cut with the lowest estimate of rounds of work-groups (one work-group per CU) x steps per slice, plus the
+  // cost of writing and adding the slices' partial tiles.  (Filling the chip once is usually that cut; but 43 x 3 blocks on
+  // 256 CUs, say -- N = 11008, M = 384 -- are 258 work-groups with two slices and run a second round for two of them,
+  // where three slices take two rounds of two thirds the length.)
+  const double t_step = p.tm == 8 ? 2.6 : (p.tm == 4 ? 1.65 : 1.0);  // us per step of 128 values of K
+  const double t_slice = (double)M * (double)N * 4.0 / 3e6;           // us per slice for its partial tile, written and read back
+  const int64_t blocks = (int64_t)p.n_blocks * p.m_blocks;
+  double best = 0;
+  int64_t best_ss = 0;
+  for (int64_t want = 1; want <= 16; ++want) {
+    int64_t ss = ceil_div((int64_t)steps_total, want);
+    ss = ceil_div(ss, (int64_t)unit) * unit;
+    if (ss > cap) continue;
+    if (ss < 4 && steps_total >= 4) continue;  // at least four steps per work-group
+    if (ss > steps_total) ss = steps_total;
+    const int64_t sl = ceil_div((int64_t)steps_total, ss);
+    if (sl > 16) continue;
+    const int64_t rounds = ceil_div(blocks * sl, (int64_t)(cus > 0 ? cus : 256));
+    const double t = (double)rounds * (double)(ss + 2) * t_step + (sl > 1 ? (double)sl * t_slice : 0.0);
+    if (best_ss == 0 || t < best * 0.97) best = t, best_ss = ss;
+  }
+  if (best_ss == 0) {  // no cut within the limits: the longest slices the scale area holds
+    int64_t ss = cap - cap % unit;
+    if (ss > steps_total) ss = steps_total;
+    best_ss = ss;
+  }
+  p.slice_steps = (int)best_ss;
+  p.split = (int)ceil_div((int64_t)steps_total, best_ss);
   if (p.split > 16) return p;  // too many partial tiles to add up: the tile kernel with longer slices takes it
   p.ok = true;
   return p;
