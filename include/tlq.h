@@ -139,12 +139,14 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
                    void* stream);
 
 /* The same operator with a caller-owned workspace of tlq_w4a16_workspace_bytes(M, N, K) bytes (0 when a
- * workspace would not be used).  With it, 16 < M <= 512 runs the streaming kernel (TLQ_ALGO_STREAM; K % 128 == 0,
- * power-of-two group, N % 4 == 0) or, where that does not apply and up to M = 2048 while there are few output tiles, the
- * tile kernel, both over slices of K whose fp32 partial sums live in the workspace and are added in slice order, and larger
- * problems take two passes -- tlq_dequant_w4 into the workspace, then tlq_gemm_f16 on it -- which is the structure of the reference's own wrapper
- * (example_dequant_gemm_fine_grained.py:176-223 unpacks, then calls fp16_gemm) and is faster than converting
- * the weights again in every row block of the fused kernel.  The workspace holds nothing between calls.
+ * workspace would not be used).  With it, 16 < M <= 384 runs the streaming kernel (TLQ_ALGO_STREAM; K % 128 == 0,
+ * power-of-two group, N % 4 == 0; up to M = 512 while its work-groups fit the machine at once) or, where that does not
+ * apply and up to M = 2048 while there are few output tiles, the tile kernel, both over slices of K whose fp32 partial sums
+ * live in the workspace and are added in slice order, and larger problems take two passes -- tlq_dequant_w4 into the
+ * workspace, then the plain GEMM on it (itself over K slices, kept behind the dequantised matrix, where it has few output
+ * tiles) -- which is the structure of the reference's own wrapper (example_dequant_gemm_fine_grained.py:176-223 unpacks,
+ * then calls fp16_gemm) and is faster than converting the weights again in every row block of the fused kernel.  The
+ * workspace holds nothing between calls.
  * algo: as tlq_gemm_w4a16, or TLQ_ALGO_TWO_PASS to force the two passes (workspace required). */
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 /* The least workspace with which tlq_gemm_w4a16_ws still takes a workspace-based kernel for this shape (the partial sums
