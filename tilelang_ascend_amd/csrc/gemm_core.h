@@ -941,6 +941,43 @@ inline bool prefer_small_tiles(int64_t batch, int64_t M, int64_t N, double weigh
   return tile_fill(batch, M, N, 128) * weight > tile_fill(batch, M, N, 256);
 }
 
+// ---- K slices of a one-batch GEMM with few activation rows ---------------------------------------------
+// The count of non-empty slices when every slice but the last has ceil(stages / count) stages.
+inline int64_t whole_slices(int64_t stages, int64_t count) {
+  if (count > stages) count = stages;
+  if (count < 1) count = 1;
+  return ceil_div(stages, ceil_div(stages, count));
+}
+
+// Number of K slices (whole 128-byte stages) for one batch of M rows against N weight rows of k_bytes bytes: 1 = do not
+// cut.  Tiles are 32 x 128 (M <= 32) or 128 x 128.  The estimate behind the choice, in microseconds: an under-filled
+// launch is paced by what one work-group streams, (BM + BN) * k_bytes at about 40 GB/s (times `pace` for a slower
+// loader); s slices divide that and add the cost of their sums -- a pass over one [M, N] 32-bit matrix per slice
+// (`buffers`), or atomic adds into one matrix at about 10 ns per thousand.  `forced` > 1 is a requested count.
+inline int slice_choice(int64_t M, int64_t N, int64_t k_bytes, bool buffers, double pace, int forced) {
+  if (k_bytes % kStageBytes != 0) return 1;
+  const int64_t stages = k_bytes / kStageBytes;
+  if (forced > 1) return (int)whole_slices(stages, forced);
+  const int tile = M <= 32 ? 32 : 128;
+  const int64_t tiles = ceil_div(M, (int64_t)tile) * ceil_div(N, (int64_t)128);
+  int cus = tlq_device_cu_count();
+  if (cus <= 0) cus = 256;
+  const int64_t places = (int64_t)cus * (tile == 32 ? 4 : 2);  // work-groups the machine holds at once (LDS per work-group)
+  if (tiles * 2 > places) return 1;
+  const double one = (double)(tile + 128) * (double)k_bytes / 40e3 * pace;
+  const double mn = (double)M * (double)N;
+  double best = one;
+  int64_t best_s = 1;
+  for (int64_t want = 2; want * tiles <= places && want * 2 <= stages; ++want) {
+    const int64_t sl = whole_slices(stages, want);
+    if (sl != want) continue;  // the same cut as a smaller request
+    const double sums = buffers ? 3.0 + (double)sl * mn * 8 / 4e6 : 5.0 + (double)sl * mn / 100e3;
+    const double t = one * (double)ceil_div(stages, sl) / (double)stages + sums;
+    if (t < best * (best_s == 1 ? 0.85 : 0.97)) best = t, best_s = sl;
+  }
+  return (int)best_s;
+}
+
 template <class Mma, class AL, class WL, class Epi, int BM, int BN, int WM, int WN>
 int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, const typename Epi::Params& pe,
                 int64_t batch, int64_t M, int64_t N, int64_t k_bytes, hipStream_t st, const char* what, int band_rows = 4,

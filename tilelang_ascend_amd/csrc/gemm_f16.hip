@@ -155,30 +155,10 @@ void launch_splitk_reduce(const float* partial, void* C, int64_t M, int64_t N, i
 
 thread_local int g_f16_split = 0;  // tlq_tune_f16_split: 0 = automatic, 1 = never, n = up to n slices
 
-// The estimate is the one of the int8 kernels (i8_split_choice): (BM + BN) rows of K * 2 bytes at about 40 GB/s
-// per work-group, divided by the slices, plus a pass over their matrices.
+// The estimate is slice_choice's (gemm_core.h): a row is K * 2 bytes, every slice has a matrix of its own.
 int f16_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K) {
-  if (batch != 1 || g_f16_split == 1 || (g_gemm_f16_tile && g_f16_split == 0) || (K * 2) % kStageBytes != 0) return 1;
-  const int tile = M <= 32 ? 32 : 128;
-  const int64_t tiles = ceil_div(M, tile) * ceil_div(N, (int64_t)128);
-  int cus = tlq_device_cu_count();
-  if (cus <= 0) cus = 256;
-  const int64_t places = (int64_t)cus * (tile == 32 ? 4 : 2);
-  const int64_t stages = K * 2 / kStageBytes;
-  auto slices = [&](int64_t sl) { return ceil_div(stages, ceil_div(stages, sl)); };
-  if (g_f16_split > 1) return (int)slices(g_f16_split < stages ? g_f16_split : stages);
-  if (tiles * 2 > places) return 1;
-  const double one = (double)(tile + 128) * (double)K * 2 / 40e3;
-  const double mn = (double)M * (double)N;
-  double best = one;
-  int64_t best_s = 1;
-  for (int64_t want = 2; want * tiles <= places && want * 2 <= stages; ++want) {
-    const int64_t sl = slices(want);
-    if (sl != want) continue;
-    const double t = one * (double)ceil_div(stages, sl) / (double)stages + 3.0 + (double)sl * mn * 8 / 4e6;
-    if (t < best * (best_s == 1 ? 0.85 : 0.97)) best = t, best_s = sl;
-  }
-  return (int)best_s;
+  if (batch != 1 || g_f16_split == 1 || (g_gemm_f16_tile && g_f16_split == 0)) return 1;
+  return slice_choice(M, N, K * 2, true, 1.0, g_f16_split);
 }
 
 template <class Mma, int BM, int BN, int WM, int WN>
@@ -203,9 +183,7 @@ static int run_f16_slices(const void* A, const void* B, float* partial, int64_t 
 // partial: fp32 [split][M][N]
 int gemm_f16_slices(const void* A, const void* B, void* C, float* partial, int64_t M, int64_t N, int64_t K, int64_t split,
                     int in_dtype, int out_dtype, int b_layout, hipStream_t st) {
-  const int64_t stages = K * 2 / kStageBytes;
-  if (split > stages) split = stages;
-  split = ceil_div(stages, ceil_div(stages, split));  // no empty slice
+  split = whole_slices(K * 2 / kStageBytes, split);  // no empty slice
   int rc;
   if (in_dtype == TLQ_F16)
     rc = M <= 32 ? run_f16_slices<MmaF16, 32, 128, 1, 4>(A, B, partial, M, N, K, split, b_layout, st)

@@ -211,49 +211,17 @@ static int run_i8_splitk(const void* A, const void* B, const typename Epi::Param
 
 static thread_local int g_i8_split = 0;  // tlq_tune_i8_split: 0 = automatic, 1 = never, n = that many slices where K allows
 
-// Number of K slices for one batch of [M,K] x [N,K]: 1 = do not split.  Slices are whole 128-byte stages.
-// `buffers`: every slice has an int32 [M,N] matrix of its own (plain stores, summed by the pass that follows);
-// otherwise the slices add into one matrix with atomic adds, which cost about 10 ns per thousand.
-// The estimate behind the choice, in microseconds: an under-filled launch is paced by what one work-group
-// streams, (BM + BN) * K bytes at about 40 GB/s (times `pace` for a slower loader: the one that unpacks int4 on
-// the way into LDS takes 2.5 times as long); s slices divide that and add the cost of their sums.
+// Number of K slices for one batch of [M,K] x [N,K] (slice_choice in gemm_core.h): `buffers`: every slice has an int32
+// [M,N] matrix of its own, otherwise the slices add into one matrix with atomic adds; `pace`: 2.5 for the loader that
+// unpacks int4 on the way into LDS.
 int i8_split_choice(int64_t batch, int64_t M, int64_t N, int64_t K, bool buffers, double pace) {
   if (batch != 1 || g_i8_split == 1 || (g_i8_tile && g_i8_split == 0)) return 1;  // a forced tile means: that kernel
-  const int tile = M <= 32 ? 32 : 128;
-  const int64_t tiles = ceil_div(M, tile) * ceil_div(N, (int64_t)128);
-  int cus = tlq_device_cu_count();
-  if (cus <= 0) cus = 256;
-  const int64_t places = (int64_t)cus * (tile == 32 ? 4 : 2);  // work-groups the machine holds at once (LDS per work-group)
-  if (K % kStageBytes != 0) return 1;
-  const int64_t stages = K / kStageBytes;
-  // the number of slices that s asks for once every slice but the last has ceil(stages / s) stages
-  auto slices = [&](int64_t sl) { return ceil_div(stages, ceil_div(stages, sl)); };
-  if (g_i8_split > 1) return (int)slices(g_i8_split < stages ? g_i8_split : stages);
-  if (tiles * 2 > places) return 1;
-  const double one = (double)(tile + 128) * (double)K / 40e3 * pace;
-  const double mn = (double)M * (double)N;
-  double best = one;
-  int64_t best_s = 1;
-  for (int64_t want = 2; want * tiles <= places && want * 2 <= stages; ++want) {
-    const int64_t sl = slices(want);
-    if (sl != want) continue;  // the same cut as a smaller request
-    const double sums = buffers ? 3.0 + (double)sl * mn * 8 / 4e6 : 5.0 + (double)sl * mn / 100e3;
-    const double t = one * (double)ceil_div(stages, sl) / (double)stages + sums;
-    if (t < best * (best_s == 1 ? 0.85 : 0.97)) best = t, best_s = sl;
-  }
-  return (int)best_s;
-}
-
-// any requested count -> the count of non-empty slices of ceil(stages / count) stages
-static int64_t whole_slices(int64_t K, int64_t split) {
-  const int64_t stages = K / kStageBytes;
-  if (split > stages) split = stages;
-  return ceil_div(stages, ceil_div(stages, split));
+  return slice_choice(M, N, K, buffers, pace, g_i8_split);
 }
 
 int gemm_i8_i32_splitk(const void* A, const void* B, int32_t* acc, int64_t M, int64_t N, int64_t K, int64_t split,
                        int b_layout, hipStream_t st) {
-  split = whole_slices(K, split);
+  split = whole_slices(K / kStageBytes, split);
   const int64_t n4 = M * N / 4;  // N % 16 == 0
   const int64_t want = ceil_div(n4, (int64_t)256);
   i32_clear_kernel<<<(int)(want > 4096 ? 4096 : want), 256, 0, st>>>((int4_t*)acc, n4);
@@ -300,7 +268,7 @@ __global__ __launch_bounds__(256) void i32_sum_rescale_kernel(const int4_t* __re
 int gemm_w8a8_rescale_splitk(const void* A, const void* B, const void* scale_a, const void* scale_b, void* C, int32_t* partial,
                              int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int64_t split, int b_layout, int out_dtype,
                              hipStream_t st) {
-  split = whole_slices(K, split);
+  split = whole_slices(K / kStageBytes, split);
   EpiInt32::Params pe{partial, N, M * N};
   const int rc = M <= 32 ? run_i8_splitk<EpiInt32, 32, 128, 1, 4>(A, B, pe, M, N, K, split, b_layout, st)
                          : run_i8_splitk<EpiInt32, 128, 128, 2, 2>(A, B, pe, M, N, K, split, b_layout, st);
@@ -349,7 +317,7 @@ __global__ __launch_bounds__(256) void i32_sum_kernel(const int4_t* __restrict__
 // matrix and a second pass sums them; without, the slices add into C (cleared first) with atomic adds.
 int gemm_w4a8_i32_splitk(const void* A, const void* Wp, void* C, int64_t M, int64_t N, int64_t K, int sign_mode,
                          int64_t split, int32_t* partial, hipStream_t st) {
-  split = whole_slices(K, split);
+  split = whole_slices(K / kStageBytes, split);
   const int64_t n4 = M * N / 4;  // N % 4 == 0
   const int64_t want = ceil_div(n4, (int64_t)256);
   if (!partial) {
