@@ -960,7 +960,10 @@ static RingPlan plan_gemv_ring(int64_t batch, int64_t M, int64_t N, int64_t K, i
   if (groups < 8 || groups % 8 != 0 || ((int64_t)groups << group_shift) != K) return p;
   p.waves = (g_gemv_waves16 >= 1 && g_gemv_waves16 <= 16) ? g_gemv_waves16 : 16;
   p.iters = K > 2048 ? 2 : 1;
-  int64_t rpb = ceil_div(N, (int64_t)cus);
+  // work-groups per CU (tlq_tune_gemv_unroll): two of 16 wavefronts fit a CU's registers and LDS, and are slower, as every
+  // other way of putting more requests in flight was: N = 11008, K = 4096: 6.8 us with one, 7.5 with two, 8.8 with three
+  const int per_cu = (g_gemv_unroll >= 1 && g_gemv_unroll <= 4) ? g_gemv_unroll : 1;
+  int64_t rpb = ceil_div(N, (int64_t)cus * per_cu);
   if (rpb < p.waves) rpb = p.waves;
   if (rpb * groups * 2 > 24 * 1024) return p;  // scales and zero points of the rows: at most 24 KB each
   p.rows_per_block = (int)rpb;
