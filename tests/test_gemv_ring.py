@@ -107,3 +107,23 @@ def test_ring_kernel_with_two_activation_rows(N, K, group, zeros_kind):
     for m in (0, M - 1):
         alone = run_gemv(A[m:m + 1].contiguous(), Wp, s, z, group, 1)
         assert_bit_equal(got[m:m + 1], alone, f"activation row {m} of {M} vs the same row alone")
+
+
+@pytest.mark.parametrize("per_cu", [2, 3])
+@pytest.mark.parametrize("N,K,group", [(11008, 4096, 128), (5000, 2560, 64), (14336, 4096, 64), (600, 1024, 32)])
+def test_ring_kernel_with_several_work_groups_per_cu(N, K, group, per_cu):
+    """tlq_tune_gemv_unroll sizes the grid for that many work-groups per CU (fewer rows per work-group): the same rows,
+    each summed in the same order, so the same bits as the default grid."""
+    from tilelang_ascend_amd import _abi
+
+    lib = _abi.load()
+    A = torch.randn(1, K, generator=gen(70)).half()
+    Wp, s, z = make_w4(N, K, group, torch.float16, "int", seed=71)
+    want = run_gemv(A, Wp, s, z, group, 1)
+    lib.tlq_tune_gemv_unroll(per_cu)
+    try:
+        got = run_gemv(A, Wp, s, z, group, 1)
+    finally:
+        lib.tlq_tune_gemv_unroll(0)
+    assert_bit_equal(got, want, f"{per_cu} work-groups per CU, N={N} K={K} g={group}")
+    check_float_output(got, w4a16_reference(A, Wp, s, z, group), "against the oracle")
