@@ -44,10 +44,14 @@ def cases():
         (256, 1024, 1024, 128, _abi.ALGO_STREAM),
         (16, 5120, 5120, 128, _abi.ALGO_DECODE),   # rows of 5120 values, 320 tiles of 16 weight rows (more than CUs): decode kernel on K chunks
         (512, 4096, 2048, 128, _abi.ALGO_STREAM),  # 512 rows on 4096 weight rows: the tile kernels would fill half the machine
+        (384, 10240, 2048, 128, _abi.ALGO_STREAM),  # three blocks of 128 activation rows: streaming kernel whatever the tile kernels' fill
+        (512, 8192, 1024, 128, _abi.ALGO_STREAM),   # four blocks, 32 x 4 x 1 = 128 streaming work-groups: they fit the machine at once
+        (768, 5120, 5120, 128, _abi.ALGO_TWO_PASS),  # above 512 rows, few output tiles: the two passes, whose plain GEMM cuts K itself
+        (224, 28672, 8192, 128, _abi.ALGO_MFMA),    # largest matrices from 192 rows on: tile kernel over two long K slices
     ]
 
 
-@pytest.mark.parametrize("case", range(12))
+@pytest.mark.parametrize("case", range(16))
 def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
     from tilelang_ascend_amd import _abi
 

@@ -307,11 +307,17 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const int64_t cus_now = cu_count_or_default();
     const bool thin_second_round = M > 256 && have && N % 8 == 0 && stream_wgs > cus_now && stream_wgs * 2 <= cus_now * 3 &&
                                    w4a16_mid_split(M, N, K, group) <= 1;
-    const bool stream_first = (M <= 384 && !thin_second_round) || stream_wgs <= cus_now;
+    // On the largest matrices the tile kernel finds a K cut that fills the machine with long slices (3072 values or more
+    // per work-group) and is ahead from 192 rows on: N = 28672, K = 8192, M = 256: 164 against 189 us; N = 8192,
+    // K = 28672: 168 against 185 us (at 128 rows the streaming kernel leads by 20 %, on smaller matrices at every M).
+    const int64_t tile_split = M >= 192 && M <= 256 ? w4a16_mid_split(M, N, K, group) : 1;
+    const bool long_tile_slices = tile_split > 1 && K / tile_split >= 3072 && w4a16_mid_fill(M, N, K, group) >= 0.85 &&
+                                  workspace != nullptr && workspace_bytes >= tile_split * M * N * 4;
+    const bool stream_first = ((M <= 384 && !thin_second_round) || stream_wgs <= cus_now) && !long_tile_slices;
     const bool slices_too_short = group < 128 && (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
                                   w4a16_mid_fill(M, N, K, group) >= 0.66;
     if (sp.ok && args_ok && ws_ok &&
-        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
+        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && !long_tile_slices && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
     if (algo == TLQ_ALGO_STREAM) {
