@@ -359,6 +359,7 @@ void tlq_tune_gemm_slots(int mode);                          /* the kernel that 
                                                               * 16-bit GEMMs), 0 never */
 void tlq_tune_w4a16_decode(int on);                          /* 0: the decode kernel is never picked automatically */
 void tlq_tune_w4a16_stream(int on);                          /* 0: tlq_gemm_w4a16_ws never picks the streaming kernel by itself */
+void tlq_tune_w4a16_stream_slice(int steps);                 /* K slice of the streaming kernel in steps of 128 values (0 = by its estimate) */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
 void tlq_tune_w4a16_split(int slices);                       /* K slices of the tile kernel, 16 < M < 256 with a workspace */
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,

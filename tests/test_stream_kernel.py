@@ -64,6 +64,35 @@ def test_stream_one_hot_rows_return_the_dequantised_weights(in_dtype, zeros_kind
     assert_bit_equal(run_stream(A, Wp, s, z, group, torch.float32), want.float(), f"one-hot f32 out {in_dtype} zeros={zeros_kind}")
 
 
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K,group,slice_steps,zeros_kind", [
+    # a slice longer than the 16 groups whose scales a wavefront holds runs in windows (4 / 8 / 16 steps of 128 values for
+    # groups of 32 / 64 / 128): whole and ragged last windows, one and several slices, every activation tile count
+    (20, 300, 128 * 11, 32, 11, "int"), (50, 516, 128 * 11, 32, 6, "frac"), (130, 260, 128 * 9, 32, 9, "scalar8"),
+    (40, 264, 128 * 19, 64, 19, "int"), (200, 512, 128 * 19, 64, 10, None), (300, 256, 128 * 16, 64, 16, "mixed"),
+    (64, 256, 128 * 35, 128, 35, "int"), (48, 1028, 128 * 35, 128, 18, "mixed"), (24, 256, 128 * 12, 32, 12, "mixed"),
+    (256, 2048, 4096, 64, 0, "int"), (256, 14336, 4096, 64, 0, "int"),
+])
+def test_stream_windows_of_a_long_slice(in_dtype, M, N, K, group, slice_steps, zeros_kind):
+    from tilelang_ascend_amd import _abi
+
+    dt = DT[in_dtype]
+    A = torch.randn(M, K, generator=gen(56)).to(dt)
+    mixed = zeros_kind == "mixed"  # integral zero points in the first windows, fractional ones later: the dequantiser changes on the way
+    Wp, s, z = make_w4(N, K, group, dt, "int" if mixed else zeros_kind, seed=57)
+    if mixed:
+        _, _, zf = make_w4(N, K, group, dt, "frac", seed=58)
+        z = z.clone()
+        z[:, 20:] = zf[:, 20:]
+    lib = _abi.load()
+    lib.tlq_tune_w4a16_stream_slice(slice_steps)
+    try:
+        got = run_stream(A, Wp, s, z, group)
+    finally:
+        lib.tlq_tune_w4a16_stream_slice(0)
+    check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"windows {in_dtype} {M}x{N}x{K} g{group} slice {slice_steps} {zeros_kind}")
+
+
 def test_stream_rejects_what_it_cannot_do():
     from tilelang_ascend_amd import _abi
 

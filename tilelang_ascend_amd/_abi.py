@@ -72,6 +72,7 @@ SIGNATURES = {
     "tlq_tune_gemm_tile": (None, [_int]),
     "tlq_debug_gemm_tile": (_int, [_i64, _i64, _i64, _int]),
     "tlq_tune_w4a16_stream": (None, [_int]),
+    "tlq_tune_w4a16_stream_slice": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),
     "tlq_tune_w4a16_split": (None, [_int]),
     "tlq_tune_w4a16_skinny": (None, [_int, _int]),

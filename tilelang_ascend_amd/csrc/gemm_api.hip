@@ -66,6 +66,7 @@ static int cu_count_or_default() {
   const int n = tlq_device_cu_count();
   return n > 0 ? n : 256;
 }
+extern thread_local int g_stream_slice_steps;
 thread_local int g_w4a16_stream = 1;  // 0: never pick the streaming kernel automatically (tuning runs)
 thread_local int g_w4a16_decode = 1;  // 0: never pick the decode kernel automatically
 // the tile loaders address one matrix with 32-bit byte offsets
@@ -88,6 +89,7 @@ int tlq_debug_gemm_tile(int64_t batch, int64_t M, int64_t N, int fused) {
 }
 void tlq_tune_gemm_tile(int tile) { tlq::g_gemm_f16_tile = (tile == 128 || tile == 256) ? tile : 0; }
 void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
+void tlq_tune_w4a16_stream_slice(int steps) { tlq::g_stream_slice_steps = steps; }
 void tlq_tune_w4a16_decode(int on) { tlq::g_w4a16_decode = on != 0; }
 
 int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
@@ -291,9 +293,9 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     // against 137 us for the two passes, K = 4096: 34 against 43 us)
     // (rows of more than 8192 values that the tile kernel can cut into enough K slices stay with it: N = 5120, K = 13824:
     // 101 against 127 us)
-    // Small quantisation groups (32, 64) shorten the K slices (16 groups each): when the partial sums (split x M x N x 4 bytes,
-    // written and read back) outweigh the packed weights, the tile kernel, which cuts K as it likes, is ahead
-    // (groups of 32, M = 256, N = 11008, K = 4096: 56 against 74 us; N = K = 8192: 64 against 90 us).
+    // When the partial sums of many short K slices (split x M x N x 4 bytes, written and read back) outweigh the packed
+    // weights, the tile kernel, which cuts K as it likes, is ahead.  (Since a slice of the streaming kernel may run over
+    // several windows of 16 groups its plan seldom cuts that short.)
     // (Only where the partial sums are tens of MB: on 4096 weight rows, or below, the streaming kernel stays ahead.)
     // And only where the tile kernel finds a K cut that fills the machine: rows of 11008 = 2 x 43 x 128 values can only be halved.
     // Up to three blocks of 128 activation rows the streaming kernel is level with or ahead of the tile kernel over K
@@ -313,11 +315,17 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const int64_t tile_split = M >= 192 && M <= 256 ? w4a16_mid_split(M, N, K, group) : 1;
     const bool long_tile_slices = tile_split > 1 && K / tile_split >= 3072 && w4a16_mid_fill(M, N, K, group) >= 0.85 &&
                                   workspace != nullptr && workspace_bytes >= tile_split * M * N * 4;
-    const bool stream_first = ((M <= 384 && !thin_second_round) || stream_wgs <= cus_now) && !long_tile_slices;
+    // Groups of 32 values give the streaming kernel windows of four steps, each with a round trip to memory of its own:
+    // from 320 rows on, the tile kernel over K slices is 2 - 11 % ahead wherever its cut fills the machine (N = 4096,
+    // K = 14336, M = 384: 77 against 84 us; N = 5120, K = 13824: 89 against 97 us); where it cannot cut K (rows of 11008
+    // values) the streaming kernel is far ahead (64 against 160 us) and stays.
+    const bool short_windows = group < 64 && M > 256 && sp.ok && (int64_t)sp.slice_steps * 128 > 2 * 16 * group &&
+                               w4a16_mid_split(M, N, K, group) > 1 && w4a16_mid_fill(M, N, K, group) >= 0.8;
+    const bool stream_first = ((M <= 384 && !thin_second_round) || stream_wgs <= cus_now) && !long_tile_slices && !short_windows;
     const bool slices_too_short = group < 128 && (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
                                   w4a16_mid_fill(M, N, K, group) >= 0.66;
     if (sp.ok && args_ok && ws_ok &&
-        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && !long_tile_slices && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
+        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && !long_tile_slices && !short_windows && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
     if (algo == TLQ_ALGO_STREAM) {
