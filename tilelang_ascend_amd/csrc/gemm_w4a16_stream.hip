@@ -344,6 +344,7 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   // where three slices take two rounds of two thirds the length.)
   const double t_step = p.tm == 8 ? 2.6 : (p.tm == 4 ? 1.65 : 1.0);  // us per step of 128 values of K
   const double t_window = 2.0;                                        // us per further window of a slice: one round trip to memory
+  const double t_gather = 2.5;                                        // us per window whose scales are gathered (measured 2.5 - 3)
   const double t_slice = (double)M * (double)N * 4.0 / 3e6;           // us per slice for its partial tile, written and read back
   const int64_t blocks = (int64_t)p.n_blocks * p.m_blocks;
   double best = 0;
@@ -361,7 +362,10 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
     if (sl > 16) continue;
     const int64_t rounds = ceil_div(blocks * sl, (int64_t)(cus > 0 ? cus : 256));
     const int64_t windows = ceil_div(ss, (int64_t)window);
-    const double t = (double)rounds * ((double)(ss + 2) * t_step + (double)(windows - 1) * t_window) + (sl > 1 ? (double)sl * t_slice : 0.0);
+    // slices that do not start at a multiple of eight groups gather their scales two bytes at a time
+    const bool gathers = sl > 1 && (ss * 128 / group) % 8 != 0;
+    const double t = (double)rounds * ((double)(ss + 2) * t_step + (double)(windows - 1) * t_window + (gathers ? t_gather : 0.0)) +
+                     (sl > 1 ? (double)sl * t_slice : 0.0);
     if (best_ss == 0 || t < best * 0.97) best = t, best_ss = ss;
   }
   if (best_ss == 0) return p;
