@@ -72,6 +72,8 @@ def test_stream_one_hot_rows_return_the_dequantised_weights(in_dtype, zeros_kind
     (40, 264, 128 * 19, 64, 19, "int"), (200, 512, 128 * 19, 64, 10, None), (300, 256, 128 * 16, 64, 16, "mixed"),
     (64, 256, 128 * 35, 128, 35, "int"), (48, 1028, 128 * 35, 128, 18, "mixed"), (24, 256, 128 * 12, 32, 12, "mixed"),
     (256, 2048, 4096, 64, 0, "int"), (256, 14336, 4096, 64, 0, "int"),
+    # large groups: windows of 32 and 64 steps
+    (64, 256, 128 * 80, 256, 80, "int"), (40, 260, 128 * 72, 512, 72, "frac"),
 ])
 def test_stream_windows_of_a_long_slice(in_dtype, M, N, K, group, slice_steps, zeros_kind):
     from tilelang_ascend_amd import _abi
