@@ -77,7 +77,7 @@ def test_five_slot_schedule():
 
 
 
-@pytest.mark.parametrize("tm,depth", [(2, 5), (4, 4), (8, 3)])
+@pytest.mark.parametrize("tm,depth", [(2, 5), (4, 4), (6, 3), (8, 3)])
 def test_streaming_kernel_addressing(tm, depth):
     """Streaming W4A16 kernel: every direct load stays inside the packed weights / the activations (rows past the
     matrices are clamped), lands on the LDS cell its operand read expects, and the ring never multiplies a step before

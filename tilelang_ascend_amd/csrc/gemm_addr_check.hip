@@ -272,7 +272,7 @@ struct SlotsSim {
 // Streaming W4A16 kernel: packed weights [N, K / 2], activations [M, K] of 2-byte values, 16 * tm activation rows and
 // 256 weight rows per work-group, steps of 128 values of K.
 int check_stream(int64_t M, int64_t N, int64_t K, int tm) {
-  CHECK_OR_FAIL(tm == 2 || tm == 4 || tm == 8, "stream: %d activation tiles", tm);
+  CHECK_OR_FAIL(tm == 2 || tm == 4 || tm == 6 || tm == 8, "stream: %d activation tiles", tm);
   CHECK_OR_FAIL(M > 0 && N > 0 && K >= 128 && K % 128 == 0, "stream: bad shape");
   CHECK_OR_FAIL(N * (K / 2) < ((int64_t)1 << 32) && M * K * 2 < ((int64_t)1 << 32), "stream: a matrix spans 4 GiB or more");
   const int64_t w_extent = N * (K / 2), a_extent = M * K * 2;

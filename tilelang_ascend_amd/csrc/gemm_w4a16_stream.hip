@@ -6,13 +6,13 @@
 // activation rows can share it, keeps two 128-byte stages, and with few activation rows its work-groups run a handful of
 // stages each, at the pace of one memory round trip per stage (M = 64, N = 14336, K = 4096: 36 us for 29 MB of
 // weights).  Here
-//   * a work-group of 8 wavefronts owns 256 weight rows, 16 TM activation rows (TM = 2, 4, 8) and a slice of K;
+//   * a work-group of 8 wavefronts owns 256 weight rows, 16 TM activation rows (TM = 2, 4, 6, 8) and a slice of K;
 //     wavefront w owns weight rows 32 w .. 32 w + 31 (two MFMA tiles) against all activation rows, so no wavefront
 //     needs another one's weights: packed weights stay private to the wavefront, are read from LDS as packed words
 //     and dequantised in registers right into MFMA operands (no dequantised tile in LDS, nothing dequantised twice);
 //   * a step is 128 values of K: per wavefront two 1 KB loads of packed weights (16 rows x 64 B each) and TM / 2
 //     loads of the shared activation tile (16 TM rows x 256 B); steps live in a ring of D slots (D = 5, 4, 3 for
-//     TM = 2, 4, 8), D - 1 steps are in flight while one is multiplied;
+//     TM = 2, 4, 6 | 8), D - 1 steps are in flight while one is multiplied;
 //   * the scales and zero points of a wavefront's rows are fetched 16 groups at a time into a private 2 KB of LDS:
 //     a slice longer than 16 groups runs in windows, each of which fetches its scales and restarts the ring;
 //   * one barrier per step publishes the shared activation tile and frees the slot that the next loads overwrite.
@@ -45,10 +45,10 @@ struct StreamMma<bf16_t> {
 
 template <int TM>
 struct StreamCfg {
-  static_assert(TM == 2 || TM == 4 || TM == 8, "16-row activation tiles per work-group");
+  static_assert(TM == 2 || TM == 4 || TM == 6 || TM == 8, "16-row activation tiles per work-group");
   // ring depth, one work-group per CU (two per CU on rings of two slots were measured no faster, and need twice
   // the K slices, i.e. twice the partial sums)
-  static constexpr int D = TM == 2 ? 5 : (TM == 4 ? 4 : 3);
+  static constexpr int D = TM == 2 ? 5 : (TM == 4 ? 4 : 3);  // (TM = 6: four slots would need 176 KB)
   static constexpr int PER_CU = 1;
   static constexpr int A_TILE = TM * 16 * 256;                // bytes of activations per step
   static constexpr int W_TILE = 8 * 2 * 1024;                 // packed weights per step: 8 wavefronts x 2 tiles x 1 KB
@@ -332,7 +332,10 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   StreamPlan p{false, 0, 0, 0, 0, 0};
   if (M < 17 || M > 512 || N < 1 || K < 128 || K % 128 != 0 || group < 32 || (group & (group - 1)) != 0 || K % group != 0) return p;
   if (N % 4 != 0) return p;
+  // activation rows per work-group: 32, 64, 96 or 128 -- from 65 rows on whichever pads M with fewer rows (M = 96, 160, 192,
+  // 288: blocks of 96; ties go to the larger block, which streams the weights fewer times)
   p.tm = M > 64 ? 8 : (M > 32 ? 4 : 2);
+  if (M > 64 && ceil_div(M, (int64_t)96) * 96 < ceil_div(M, (int64_t)128) * 128) p.tm = 6;
   p.m_blocks = (int)ceil_div(M, (int64_t)16 * p.tm);
   p.n_blocks = (int)ceil_div(N, (int64_t)256);
   const int steps_total = (int)(K / 128);
@@ -342,7 +345,7 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   // cost of writing and adding the slices' partial tiles.  (Filling the chip once is usually that cut; but 43 x 3 blocks on
   // 256 CUs, say -- N = 11008, M = 384 -- are 258 work-groups with two slices and run a second round for two of them,
   // where three slices take two rounds of two thirds the length.)
-  const double t_step = p.tm == 8 ? 2.6 : (p.tm == 4 ? 1.65 : 1.0);  // us per step of 128 values of K
+  const double t_step = p.tm == 8 ? 2.6 : (p.tm == 6 ? 2.1 : (p.tm == 4 ? 1.65 : 1.0));  // us per step of 128 values of K
   const double t_window = 2.0;                                        // us per further window of a slice: one round trip to memory
   const double t_gather = 2.5;                                        // us per window whose scales are gathered (measured 2.5 - 3)
   const double t_slice = (double)M * (double)N * 4.0 / 3e6;           // us per slice for its partial tile, written and read back
@@ -409,9 +412,9 @@ int gemm_w4a16_stream(const void* A, const void* Wp, const void* scales, const v
 #define TLQ_STREAM3(T, TM, LAY) (many ? TLQ_STREAM4(T, TM, LAY, true) : TLQ_STREAM4(T, TM, LAY, false))
 #define TLQ_STREAM(T, TM) (w_layout == TLQ_W_INTERLEAVED_F16 ? TLQ_STREAM3(T, TM, 1) : TLQ_STREAM3(T, TM, 0))
   if (in_dtype == TLQ_F16)
-    rc = p.tm == 2 ? TLQ_STREAM(half_t, 2) : (p.tm == 4 ? TLQ_STREAM(half_t, 4) : TLQ_STREAM(half_t, 8));
+    rc = p.tm == 2 ? TLQ_STREAM(half_t, 2) : (p.tm == 4 ? TLQ_STREAM(half_t, 4) : (p.tm == 6 ? TLQ_STREAM(half_t, 6) : TLQ_STREAM(half_t, 8)));
   else
-    rc = p.tm == 2 ? TLQ_STREAM(bf16_t, 2) : (p.tm == 4 ? TLQ_STREAM(bf16_t, 4) : TLQ_STREAM(bf16_t, 8));
+    rc = p.tm == 2 ? TLQ_STREAM(bf16_t, 2) : (p.tm == 4 ? TLQ_STREAM(bf16_t, 4) : (p.tm == 6 ? TLQ_STREAM(bf16_t, 6) : TLQ_STREAM(bf16_t, 8)));
 #undef TLQ_STREAM3
 #undef TLQ_STREAM4
 #undef TLQ_STREAM
