@@ -332,10 +332,10 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   StreamPlan p{false, 0, 0, 0, 0, 0};
   if (M < 17 || M > 512 || N < 1 || K < 128 || K % 128 != 0 || group < 32 || (group & (group - 1)) != 0 || K % group != 0) return p;
   if (N % 4 != 0) return p;
-  // activation rows per work-group: 32, 64, 96 or 128 -- from 65 rows on whichever pads M with fewer rows (M = 96, 160, 192,
-  // 288: blocks of 96; ties go to the larger block, which streams the weights fewer times)
+  // activation rows per work-group: 32, 64, 96 or 128 -- from 65 rows on whichever needs less time for a step of all its
+  // blocks (2.1 us per block of 96 rows, 2.6 us per block of 128: M = 96, 160, 192, 288 take blocks of 96)
   p.tm = M > 64 ? 8 : (M > 32 ? 4 : 2);
-  if (M > 64 && ceil_div(M, (int64_t)96) * 96 < ceil_div(M, (int64_t)128) * 128) p.tm = 6;
+  if (M > 64 && (double)ceil_div(M, (int64_t)96) * 2.1 < (double)ceil_div(M, (int64_t)128) * 2.6) p.tm = 6;
   p.m_blocks = (int)ceil_div(M, (int64_t)16 * p.tm);
   p.n_blocks = (int)ceil_div(N, (int64_t)256);
   const int steps_total = (int)(K / 128);
