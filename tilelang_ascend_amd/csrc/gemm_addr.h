@@ -129,22 +129,28 @@ __host__ __device__ inline void slots_schedule(int KT, Ops& ops) {
 // One step is 128 values of K.  A work-group of 8 wavefronts owns 256 weight rows (wavefront w: rows 32 w .. 32 w + 31,
 // two 16-row MFMA tiles) and 16 * TM activation rows.
 // Packed weights: [16 rows][64 B] per MFMA tile, private to the wavefront.  One direct load covers a tile (lane l lands
-// on row l / 4, 16-byte piece l % 4 and fetches logical piece (l % 4) ^ ((row >> 2) & 3)); the operand read of lane
+// on row l / 4, 16-byte piece l % 4 and fetches logical piece (l % 4) ^ sw_swz(row)); the operand read of lane
 // (row r16, k-group q) takes logical piece q: the four 32-bit words 4 q .. 4 q + 3 = values 32 q .. 32 q + 31 of the step.
+// The swizzles of both tiles were chosen by measuring the 16-byte reads of eight wavefronts over whole families of
+// layouts (every 4 x 4 bit matrix for the activations, 24 row orders x 256 piece swizzles for the weights): with
+// pieces swizzled by row / 4 and chunks by the row number itself a read took 61 clocks instead of 37 in bank conflicts.
+__host__ __device__ inline int sw_swz(int row) { return (row >> 1) & 3; }
 __host__ __device__ inline int sw_row(int lane) { return lane >> 2; }
-__host__ __device__ inline int sw_piece(int lane) { return (lane & 3) ^ ((sw_row(lane) >> 2) & 3); }
+__host__ __device__ inline int sw_piece(int lane) { return (lane & 3) ^ sw_swz(sw_row(lane)); }
 __host__ __device__ inline uint32_t sw_frag_off(int lane) {  // inside the 1 KB tile
   const int r16 = lane & 15, q = lane >> 4;
-  return (uint32_t)(r16 * 64 + ((q ^ ((r16 >> 2) & 3)) << 4));
+  return (uint32_t)(r16 * 64 + ((q ^ sw_swz(r16)) << 4));
 }
 // Activations: [16 TM rows][256 B], shared by the work-group.  Direct load I (of 4 TM) covers rows 4 I .. 4 I + 3 (lane
-// l: row 4 I + l / 16, physical chunk l % 16, logical chunk (l % 16) ^ (row & 15)); lane (m = r16, k-group q) reads
+// l: row 4 I + l / 16, physical chunk l % 16, logical chunk (l % 16) ^ sa_swz(row)); lane (m = r16, k-group q) reads
 // logical chunk 4 q + ks for MFMA k-step ks, i.e. the eight values that word 4 q + ks of the weights holds.
+// sa_swz: the row number's low four bits rotated left by one.
+__host__ __device__ inline int sa_swz(int row) { return ((row << 1) & 15) | ((row >> 3) & 1); }
 __host__ __device__ inline int sa_row(int lane, int I) { return 4 * I + (lane >> 4); }
-__host__ __device__ inline int sa_chunk(int lane, int I) { return (lane & 15) ^ (sa_row(lane, I) & 15); }
+__host__ __device__ inline int sa_chunk(int lane, int I) { return (lane & 15) ^ sa_swz(sa_row(lane, I)); }
 __host__ __device__ inline uint32_t sa_frag_off(int lane, int tm, int ks) {
   const int r16 = lane & 15, q = lane >> 4;
-  return (uint32_t)((tm * 16 + r16) * 256 + (((4 * q + ks) ^ r16) << 4));
+  return (uint32_t)((tm * 16 + r16) * 256 + (((4 * q + ks) ^ sa_swz(r16)) << 4));
 }
 // Ring of D steps: step s lives in slot s % D.  Every wavefront issues `per_step` load instructions per step, in
 // step order, and loads retire in issue order: this wavefront's loads of step s have landed once at most the
