@@ -313,10 +313,12 @@ __global__ __launch_bounds__(512, 2) void w4a16_stream_kernel(const T* __restric
   const bool split = gridDim.y > 1;
   EpiFloat::Params pe{split ? (void*)partial : C, N, (int64_t)M * N, split ? TLQ_F32 : out_dtype};
   const EpiFloat epi(pe, split ? (int)blockIdx.y : 0);
-#pragma unroll
-  for (int tn = 0; tn < 2; ++tn)
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm) epi.store(m0 + tm * 16 + r16, n0 + wave * 32 + tn * 16 + q * 4, acc[tn][tm], M, N);
+  // A wavefront's 32 fp32 outputs of a row are one 128-byte line: staged through LDS (the ring is no longer needed once
+  // everyone is past the last step) they leave as whole lines; stored from the accumulators' own layout, 16 bytes per
+  // lane and two instructions per line, the partial tiles of 128 rows cost 1.47 times their bytes in write traffic.
+  static_assert(8 * TM * 16 * kStageBytes <= D * Cfg::SLOT, "the staging areas of the wavefronts fit the ring");
+  __syncthreads();
+  write_tile<EpiFloat, TM, 2>(epi, acc, smem + wave * (TM * 16 * kStageBytes), lane, m0, n0 + wave * 32, M, N);
 }
 
 }  // namespace
