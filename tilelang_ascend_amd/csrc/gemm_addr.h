@@ -259,6 +259,20 @@ __host__ __device__ inline uint32_t ring_stage_voff(int p0, int lane, int pieces
   p = p < pieces ? p : pieces - 1;
   return (uint32_t)p * 16u;
 }
+// The activations (chunk c = 32 values = four 16-byte pieces) are read back by lane c, piece j of all lanes in one
+// instruction: with the pieces in order, lanes four apart sit on the same banks and such a read takes 3.4 times its
+// cycles (measured: 128 against 37 clocks).  Piece j of chunk c is therefore kept at position (j + c / 4) % 4 of the
+// chunk's 64 bytes; the direct load fetches the piece that belongs at the position it lands on.
+__host__ __device__ inline int ring_act_logical(int P) {  // the piece (4 c + j) that physical piece P of the area holds
+  const int c = P >> 2;
+  return (c << 2) | (((P & 3) - (c >> 2)) & 3);
+}
+__host__ __device__ inline uint32_t ring_act_lds(int c, int j) { return (uint32_t)(((c << 2) | ((j + (c >> 2)) & 3)) * 16); }
+__host__ __device__ inline uint32_t ring_act_voff(int p0, int lane, int pieces) {  // pieces: a multiple of 4
+  int P = p0 + lane;
+  P = P < pieces ? P : pieces - 1;
+  return (uint32_t)ring_act_logical(P) * 16u;
+}
 // rows of wavefront `wave`, and the loads it may leave in flight when it reads its i-th row (row i + depth is issued
 // after row i has been read; loads retire in issue order)
 __host__ __device__ inline int ring_my_rows(int rows, int wave, int waves) { return wave < rows ? (rows - wave + waves - 1) / waves : 0; }

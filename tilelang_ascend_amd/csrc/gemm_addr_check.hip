@@ -535,16 +535,26 @@ int check_gemv_ring(int64_t M, int64_t N, int64_t K, int64_t group, int rows_per
       for (int w = 0; w < waves; ++w)
         for (int p0 = w * 64; p0 < pieces; p0 += waves * 64)
           for (int lane = 0; lane < 64; ++lane) {
-            const uint32_t voff = addr::ring_stage_voff(p0, lane, pieces);
+            const uint32_t voff = which == 0 ? addr::ring_act_voff(p0, lane, pieces) : addr::ring_stage_voff(p0, lane, pieces);
             CHECK_OR_FAIL((int64_t)voff + 16 <= src_bytes, "gemv ring: staging read at byte %u of %lld", voff, (long long)src_bytes);
             const uint32_t dst = area + (uint32_t)p0 * 16u + (uint32_t)lane * 16u;
             CHECK_OR_FAIL(dst + 16 <= area_end, "gemv ring: staging write at LDS byte %u, area ends at %u", dst, area_end);
             if (p0 + lane < pieces) {
-              CHECK_OR_FAIL(voff == (uint32_t)(p0 + lane) * 16u, "gemv ring: piece %d read from byte %u", p0 + lane, voff);
-              seen[p0 + lane] = 1;
+              // the activation pieces of a chunk are rotated (ring_act_logical); scales and zero points lie in order
+              const int piece = which == 0 ? addr::ring_act_logical(p0 + lane) : p0 + lane;
+              CHECK_OR_FAIL(piece >= 0 && piece < pieces && !seen[piece], "gemv ring: staging piece %d loaded twice or out of range", piece);
+              CHECK_OR_FAIL(voff == (uint32_t)piece * 16u, "gemv ring: piece %d read from byte %u", piece, voff);
+              seen[piece] = 1;
             }
           }
       for (int p = 0; p < pieces; ++p) CHECK_OR_FAIL(seen[p], "gemv ring: staging piece %d of %d never loaded", p, pieces);
+      if (which == 0)  // the read of piece j of chunk c finds the position that holds it
+        for (int c = 0; c < pieces / 4; ++c)
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t off = addr::ring_act_lds(c, j);
+            CHECK_OR_FAIL(off % 16 == 0 && (int)(off / 16) < pieces && addr::ring_act_logical((int)(off / 16)) == 4 * c + j,
+                          "gemv ring: activation read (chunk %d, piece %d) at byte %u finds another piece", c, j, off);
+          }
     }
     CHECK_OR_FAIL(L.z + (uint32_t)sz_pieces * 16u <= L.total && L.total - L.z == L.z - L.s, "gemv ring: zero-point area");
     // weights

@@ -638,7 +638,7 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
   // staging loads have landed), then the first D rows ----
   const int a_pieces = chunks * 4 * MT;  // the activation rows are contiguous
   for (int p0 = wave * 64; p0 < a_pieces; p0 += nwaves * 64)
-    dma16(lds0 + L.act + (uint32_t)p0 * 16u, addr::ring_stage_voff(p0, lane, a_pieces), (const uint8_t*)A);
+    dma16(lds0 + L.act + (uint32_t)p0 * 16u, addr::ring_act_voff(p0, lane, a_pieces), (const uint8_t*)A);
   const int sz_pieces = ((r1 - r0) * groups) >> 3;  // groups is a multiple of 8
   const uint8_t* const s_base = uniform_ptr((const uint8_t*)(scales + (int64_t)r0 * groups));
   const uint8_t* const z_base = uniform_ptr((const uint8_t*)(zeros + (int64_t)r0 * groups));
@@ -680,7 +680,7 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
     for (int it = 0; it < ITERS; ++it) {
       uint4_t raw[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) raw[j] = *(const uint4_t*)(smem + L.act + (uint32_t)((m * chunks + cc[it]) * 4 + j) * 16u);
+      for (int j = 0; j < 4; ++j) raw[j] = *(const uint4_t*)(smem + L.act + addr::ring_act_lds(m * chunks + cc[it], j));
       if constexpr (F16) {
         permute_act(act[m][it], raw);
       } else {
