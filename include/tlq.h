@@ -74,8 +74,14 @@ enum {
   TLQ_ALGO_TWO_PASS = 4, /* tlq_gemm_w4a16_ws only: dequantise into the workspace, then the plain GEMM */
   TLQ_ALGO_STREAM = 5, /* tlq_gemm_w4a16_ws only: 17 <= M <= 512, weights streamed once per 128 activation rows through a deep
                        * ring of direct loads, dequantised in registers; K slices add up through the workspace */
-  TLQ_ALGO_DECODE = 6 /* 1 <= M <= 32, K % 256 == 0, power-of-two group: persistent work-groups, activations resident in registers, every
+  TLQ_ALGO_DECODE = 6, /* 1 <= M <= 32, K % 256 == 0, power-of-two group: persistent work-groups, activations resident in registers, every
                        * weight read once through deep wavefront-private rings (rows longer than 4096 values need the workspace) */
+  TLQ_ALGO_PANEL = 7 /* tlq_gemm_w4a16_ws / tlq_gemm_w4a16_layout_ws only: large M in one launch, 128 activation rows x 512 weight rows
+                      * per work-group, packed weights copied global -> LDS as they are and dequantised on the MFMA operand read;
+                      * K % 128 == 0, M % 4 == 0, N % 16 == 0, power-of-two group >= 32, (K / group) % 8 == 0, 16-byte aligned scale /
+                      * zero tensors.  Workspace: the fp32 partial tiles where K is cut into slices, plus 16 bytes with a zero-point
+                      * tensor (a flag word: a second launch redoes the product with the unfolded dequantiser when a zero point
+                      * turns out not to be a small integer) */
 };
 
 int tlq_abi_version(void);
@@ -308,6 +314,12 @@ int tlq_debug_check_slots_schedule(int stages, int loads_per_tile);
 /* The same walk for the streaming W4A16 kernel (TLQ_ALGO_STREAM): packed weights [N, K / 2] and 2-byte activations [M, K]
  * with 16 * activation_tiles rows per work-group (2 | 4 | 8), and its ring of `ring_depth` steps for 1 .. 40 steps. */
 int tlq_debug_check_stream_addressing(int64_t M, int64_t N, int64_t K, int activation_tiles, int ring_depth);
+/* The same walk for the panel kernel (TLQ_ALGO_PANEL) with K slices of `slice_steps` steps of 128 values: every direct load of
+ * activations, packed weights and scale windows of every work-group, the LDS map and the operand reads; and the plan the
+ * library would choose on a device with `cus` compute units: plan_out is a HOST array of four int64 that receives the tiles
+ * along M and N, the K slices and the steps per slice; returns 1 when the kernel applies. */
+int tlq_debug_check_panel_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int slice_steps);
+int tlq_debug_panel_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
 
 /* The same walk for the decode kernel (TLQ_ALGO_DECODE) launched as grid_x x chunks work-groups of `waves` wavefronts
  * with 16 * activation_tiles activation rows, and its ring for 2 .. 24 items; tlq_debug_decode_plan gives the geometry
@@ -360,6 +372,8 @@ void tlq_tune_gemm_slots(int mode);                          /* the kernel that 
 void tlq_tune_w4a16_decode(int on);                          /* 0: the decode kernel is never picked automatically */
 void tlq_tune_w4a16_stream(int on);                          /* 0: tlq_gemm_w4a16_ws never picks the streaming kernel by itself */
 void tlq_tune_w4a16_stream_slice(int steps);                 /* K slice of the streaming kernel in steps of 128 values (0 = by its estimate) */
+void tlq_tune_w4a16_panel(int mode);                         /* tlq_gemm_w4a16_ws, large M: 0 = automatic, 1 = never the panel kernel (TLQ_ALGO_PANEL) */
+void tlq_tune_w4a16_panel_slice(int steps);                  /* K slice of the panel kernel in steps of 128 values (0 = its own plan) */
 void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
 void tlq_tune_w4a16_split(int slices);                       /* K slices of the tile kernel, 16 < M < 256 with a workspace */
 void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,

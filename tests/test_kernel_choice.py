@@ -46,12 +46,13 @@ def cases():
         (512, 4096, 2048, 128, _abi.ALGO_STREAM),  # 512 rows on 4096 weight rows: the tile kernels would fill half the machine
         (384, 10240, 2048, 128, _abi.ALGO_STREAM),  # three blocks of 128 activation rows: streaming kernel whatever the tile kernels' fill
         (512, 8192, 1024, 128, _abi.ALGO_STREAM),   # four blocks, 32 x 4 x 1 = 128 streaming work-groups: they fit the machine at once
-        (768, 5120, 5120, 128, _abi.ALGO_TWO_PASS),  # above 512 rows, few output tiles: the two passes, whose plain GEMM cuts K itself
+        (768, 5120, 5120, 128, _abi.ALGO_PANEL),    # above 512 rows where the panel kernel's work-groups fill the machine: 6 x 10 tiles x 3 K slices
+        (2048, 4096, 2048, 128, _abi.ALGO_TWO_PASS),  # 128 panel tiles and too few steps to cut: half the CUs idle, the two passes keep it
         (224, 28672, 8192, 128, _abi.ALGO_MFMA),    # largest matrices from 192 rows on: tile kernel over two long K slices
     ]
 
 
-@pytest.mark.parametrize("case", range(16))
+@pytest.mark.parametrize("case", range(17))
 def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
     from tilelang_ascend_amd import _abi
 

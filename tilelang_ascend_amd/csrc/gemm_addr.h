@@ -161,6 +161,46 @@ __host__ __device__ inline int stream_younger_steps(int s, int steps, int D) {
   return last_issued - s > 0 ? last_issued - s : 0;
 }
 
+// ---- panel kernel for large M (gemm_w4a16_panel.hip): 128 activation rows x 512 weight rows per work-group ----------
+// Steps of 128 values of K in two ring slots.  A slot is the activation tile [128 rows][256 B] (the streaming kernel's
+// layout with eight 16-row tiles: direct load I = 8 j + wave, j = 0 .. 3, rows 4 I .. 4 I + 3) followed by the eight
+// wavefronts' packed weights, four [16 rows][64 B] tiles each (wavefront w: weight rows 64 w + 16 tn + row).  Behind
+// the ring every wavefront has two scale windows of 2 KB: [64 rows][8 groups] scales, then the same for zero points;
+// lane l of the window's direct load fetches the eight groups (16 bytes) of row l.
+constexpr int kPanelTM = 8, kPanelTN = 4;
+constexpr uint32_t kPanelATile = 16 * kPanelTM * 256;
+constexpr uint32_t kPanelSlot = kPanelATile + 8 * kPanelTN * 1024;
+constexpr uint32_t kPanelScBuf = 2048;
+__host__ __device__ inline uint32_t panel_a_lds(int wave, int j) { return (uint32_t)(j * 8 + wave) * 1024u; }
+__host__ __device__ inline uint32_t panel_w_lds(int wave, int tn) { return kPanelATile + (uint32_t)(wave * kPanelTN + tn) * 1024u; }
+__host__ __device__ inline uint32_t panel_sc_lds(int wave, int buf) { return 2 * kPanelSlot + (uint32_t)(wave * 2 + buf) * kPanelScBuf; }
+__host__ __device__ inline uint32_t panel_sc_off(int row, int g) { return (uint32_t)(row * 16 + g * 2); }
+// Source of a direct load = (first byte of the step in row 0) + block offset of the instruction (uniform) + lane offset.
+// An instruction covers 16 weight rows (64 bytes per step and row) or 4 activation rows (256 bytes per step and row);
+// with N % 16 == 0 and M % 4 == 0 it lies wholly inside the matrix or wholly outside, and an outside one repeats the
+// last block of the matrix.
+__host__ __device__ inline uint32_t panel_w_lane(int lane, int K) { return (uint32_t)sw_row(lane) * (uint32_t)(K >> 1) + (uint32_t)(sw_piece(lane) * 16); }
+__host__ __device__ inline int64_t panel_w_block(int wave, int tn, int n0, int N, int K) {
+  int n = n0 + wave * (16 * kPanelTN) + tn * 16;
+  n = n + 16 <= N ? n : N - 16;
+  return (int64_t)n * (K >> 1);
+}
+// lane l of activation load I = 8 j + wave: row 4 I + l / 16, logical chunk (l % 16) ^ sa_swz(that row); sa_swz depends on
+// the row's low four bits = 4 (I % 4) + l / 16 only, and I % 4 = wave % 4 for every j
+__host__ __device__ inline uint32_t panel_a_lane(int lane, int K) { return (uint32_t)(lane >> 4) * (uint32_t)K * 2u; }
+__host__ __device__ inline uint32_t panel_a_chunk(int lane, int wave) { return (uint32_t)(((lane & 15) ^ sa_swz(4 * (wave & 3) + (lane >> 4))) * 16); }
+__host__ __device__ inline int64_t panel_a_block(int wave, int j, int m0, int M, int K) {
+  int m = m0 + 4 * (j * 8 + wave);
+  m = m + 4 <= M ? m : M - 4;
+  return (int64_t)m * K * 2;
+}
+// byte offset from element [0][first group of the window] of the scale / zero-point tensor [N][groups]
+__host__ __device__ inline uint32_t panel_sc_voff(int lane, int wave, int n0, int N, int groups) {
+  int n = n0 + wave * (16 * kPanelTN) + lane;
+  n = n < N ? n : N - 1;
+  return ((uint32_t)n * (uint32_t)groups) * 2u;
+}
+
 // ---- decode kernel (1 .. 32 activation rows): wavefront w of a work-group owns values 256 s .. 256 s + 255 of K
 // (s = chunk * waves + w) for every weight row.  A work item is one 16-row weight tile: two [16 rows][64 B] packed
 // pieces (k-blocks kb = 0, 1 of the slice, 128 values each) plus the scales / zero points of the 16 rows for the

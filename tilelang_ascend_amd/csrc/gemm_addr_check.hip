@@ -334,6 +334,103 @@ int check_stream(int64_t M, int64_t N, int64_t K, int tm) {
   return 0;
 }
 
+// Panel kernel (large M): 128 activation rows x 512 weight rows per work-group, steps of 128 values of K in two ring
+// slots, scale windows of eight groups behind the ring.  Walks every work-group tile of an M x N problem: global
+// extents of all three kinds of loads over every step / window of a slice plan, LDS extents and coverage of a slot,
+// agreement of the landing cells with the operand reads, and that the LDS map stays within 160 KB.
+int check_panel(int64_t M, int64_t N, int64_t K, int64_t group, int slice_steps) {
+  CHECK_OR_FAIL(M >= 4 && N >= 16 && M % 4 == 0 && N % 16 == 0 && K >= 128 && K % 128 == 0, "panel: bad shape");
+  CHECK_OR_FAIL(group >= 32 && (group & (group - 1)) == 0 && K % group == 0 && (K / group) % 8 == 0, "panel: group %lld on K %lld",
+                (long long)group, (long long)K);
+  const int64_t groups = K / group;
+  CHECK_OR_FAIL(N * (K / 2) < ((int64_t)1 << 32) && M * K * 2 < ((int64_t)1 << 32) && N * groups * 2 < ((int64_t)1 << 32),
+                "panel: a matrix spans 4 GiB or more");
+  const int steps_total = (int)(K / 128);
+  const int window = (int)(group >= 128 ? 8 * (group / 128) : 8 / (128 / group));
+  CHECK_OR_FAIL(slice_steps >= 1 && (slice_steps % window == 0 || slice_steps >= steps_total), "panel: slices of %d steps are not whole windows of %d",
+                slice_steps, window);
+  const int TM = addr::kPanelTM, TN = addr::kPanelTN;
+  const int64_t w_extent = N * (K / 2), a_extent = M * K * 2, s_extent = N * groups * 2;
+  const uint32_t lds_total = addr::panel_sc_lds(7, 1) + addr::kPanelScBuf;
+  CHECK_OR_FAIL(lds_total <= 160 * 1024, "panel: %u bytes of LDS", lds_total);
+  const int slices = (steps_total + slice_steps - 1) / slice_steps;
+  std::vector<int> cell(addr::kPanelSlot / 16);
+  for (int64_t m0 = 0; m0 < M; m0 += 16 * TM)
+    for (int64_t n0 = 0; n0 < N; n0 += 8 * 16 * TN) {
+      std::fill(cell.begin(), cell.end(), -1);
+      for (int wave = 0; wave < 8; ++wave) {
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t l0 = addr::panel_a_lds(wave, j);
+          const int I = j * 8 + wave;
+          for (int lane = 0; lane < 64; ++lane) {
+            const int64_t blk = addr::panel_a_block(wave, j, (int)m0, (int)M, (int)K);
+            const int64_t voff = blk + addr::panel_a_lane(lane, (int)K) + addr::panel_a_chunk(lane, wave);
+            CHECK_OR_FAIL(voff >= 0 && voff + (int64_t)(steps_total - 1) * 256 + 16 <= a_extent, "panel: activation load at %lld of %lld",
+                          (long long)voff, (long long)a_extent);
+            // inside the matrix the lane fetches the row and chunk its landing cell stands for
+            if (m0 + 4 * I + 4 <= M)
+              CHECK_OR_FAIL(voff == ((int64_t)(m0 + addr::sa_row(lane, I)) * K) * 2 + addr::sa_chunk(lane, I) * 16, "panel: activation lane %d of load %d fetches the wrong bytes", lane, I);
+            const uint32_t at = l0 / 16 + lane;
+            CHECK_OR_FAIL(at < addr::kPanelATile / 16 && cell[at] == -1, "panel: activation cell %u written twice or outside the tile", at);
+            const int row = addr::sa_row(lane, I), chunk = addr::sa_chunk(lane, I);
+            CHECK_OR_FAIL((int)at == row * 16 + (lane & 15), "panel: activation lane lands on cell %u, not on its row", at);
+            cell[at] = row * 16 + chunk;
+          }
+        }
+        for (int tn = 0; tn < TN; ++tn) {
+          const uint32_t l0 = addr::panel_w_lds(wave, tn);
+          for (int lane = 0; lane < 64; ++lane) {
+            const int64_t voff = addr::panel_w_block(wave, tn, (int)n0, (int)N, (int)K) + addr::panel_w_lane(lane, (int)K);
+            CHECK_OR_FAIL(voff >= 0 && voff + (int64_t)(steps_total - 1) * 64 + 16 <= w_extent, "panel: weight load at %lld of %lld",
+                          (long long)voff, (long long)w_extent);
+            if (n0 + wave * 64 + tn * 16 + 16 <= N)
+              CHECK_OR_FAIL(voff == (int64_t)(n0 + wave * 64 + tn * 16 + addr::sw_row(lane)) * (K / 2) + addr::sw_piece(lane) * 16, "panel: weight lane %d fetches the wrong bytes", lane);
+            const uint32_t at = l0 / 16 + lane;
+            CHECK_OR_FAIL(at >= addr::kPanelATile / 16 && at < addr::kPanelSlot / 16 && cell[at] == -1, "panel: weight cell %u written twice or outside the slot", at);
+            cell[at] = addr::sw_row(lane) * 4 + addr::sw_piece(lane);
+          }
+          for (int lane = 0; lane < 64; ++lane) {
+            const uint32_t off = l0 + addr::sw_frag_off(lane);
+            CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= addr::kPanelSlot, "panel: weight operand read at %u", off);
+            CHECK_OR_FAIL(cell[off / 16] == (lane & 15) * 4 + (lane >> 4), "panel: weight operand read of lane %d finds cell %d", lane, cell[off / 16]);
+          }
+        }
+        // scale windows: lane l fetches 16 bytes of row n0 + 64 wave + l for every window of every slice
+        for (int lane = 0; lane < 64; ++lane) {
+          const int64_t voff = addr::panel_sc_voff(lane, wave, (int)n0, (int)N, (int)groups);
+          for (int sl = 0; sl < slices; ++sl) {
+            const int step0 = sl * slice_steps;
+            const int steps = steps_total - step0 < slice_steps ? steps_total - step0 : slice_steps;
+            const int64_t g0 = ((int64_t)step0 * 128) / group;
+            const int nwin = (steps + window - 1) / window;
+            for (int w = 0; w < nwin; ++w) {
+              const int64_t o = voff + (g0 + 8 * w) * 2;
+              CHECK_OR_FAIL(o >= 0 && o + 16 <= s_extent && o % 16 == 0, "panel: scale load at [%lld, +16) of %lld", (long long)o, (long long)s_extent);
+              CHECK_OR_FAIL((g0 + 8 * w) % groups + 8 <= groups, "panel: a scale window crosses the end of a row of the scale tensor");
+            }
+          }
+          for (int buf = 0; buf < 2; ++buf) {
+            const uint32_t at = addr::panel_sc_lds(wave, buf) + 1024u + (uint32_t)lane * 16u;
+            CHECK_OR_FAIL(at + 16 <= lds_total, "panel: scale window at %u", at);
+          }
+        }
+        for (int row = 0; row < 16 * TN; ++row)
+          for (int g = 0; g < 8; ++g)
+            CHECK_OR_FAIL(addr::panel_sc_off(row, g) + 2 <= 1024 && addr::panel_sc_off(row, g) == (uint32_t)(row * 16 + g * 2), "panel: scale read");
+      }
+      for (uint32_t c = 0; c < addr::kPanelSlot / 16; ++c) CHECK_OR_FAIL(cell[c] >= 0, "panel: cell %u of the slot never written", c);
+      for (int t = 0; t < TM; ++t)
+        for (int ks = 0; ks < 4; ++ks)
+          for (int lane = 0; lane < 64; ++lane) {
+            const uint32_t off = addr::sa_frag_off(lane, t, ks);
+            CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= addr::kPanelATile, "panel: activation operand read at %u", off);
+            const int want = (t * 16 + (lane & 15)) * 16 + 4 * (lane >> 4) + ks;
+            CHECK_OR_FAIL(cell[off / 16] == want, "panel: activation operand read (lane %d, k-step %d) finds cell %d, expects %d", lane, ks, cell[off / 16], want);
+          }
+    }
+  return 0;
+}
+
 // The ring: step s occupies slot s % D; at the top of step s the wavefront waits until only `younger` steps' loads are
 // outstanding, passes the barrier, and then issues step s + D - 1 into the slot of step s - 1.
 int check_stream_ring(int steps, int D) {
@@ -630,6 +727,10 @@ int tlq_debug_check_stream_addressing(int64_t M, int64_t N, int64_t K, int activ
   for (int steps = 1; steps <= 40; ++steps)
     if (int rc = check_stream_ring(steps, ring_depth)) return rc;
   return 0;
+}
+
+int tlq_debug_check_panel_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int slice_steps) {
+  return check_panel(M, N, K, group, slice_steps);
 }
 
 int tlq_debug_check_decode_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int activation_tiles, int chunks, int waves,

@@ -47,6 +47,17 @@ int gemm_w8a8_rescale_splitk(const void* A, const void* B, const void* scale_a, 
                              int64_t M, int64_t N, int64_t K, int64_t n_scale_b, int64_t split, int b_layout, int out_dtype,
                              hipStream_t st);
 
+struct PanelPlan {
+  bool ok;
+  int tiles_m, tiles_n, split, slice_steps;
+};
+PanelPlan w4a16_panel_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus);
+int gemm_w4a16_panel(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N, int64_t K,
+                     int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const PanelPlan& p, float* partial,
+                     uint32_t* flag, hipStream_t st);
+extern thread_local int g_panel_slice_steps;
+thread_local int g_w4a16_panel = 0;  // tlq_tune_w4a16_panel: 1 = the panel kernel is never picked automatically
+
 struct DecodePlan {
   bool ok;
   int mt, chunks, waves, grid_x;
@@ -91,6 +102,18 @@ void tlq_tune_gemm_tile(int tile) { tlq::g_gemm_f16_tile = (tile == 128 || tile 
 void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
 void tlq_tune_w4a16_stream_slice(int steps) { tlq::g_stream_slice_steps = steps; }
 void tlq_tune_w4a16_decode(int on) { tlq::g_w4a16_decode = on != 0; }
+void tlq_tune_w4a16_panel(int mode) { tlq::g_w4a16_panel = mode == 1 ? 1 : 0; }
+void tlq_tune_w4a16_panel_slice(int steps) { tlq::g_panel_slice_steps = steps < 0 ? 0 : steps; }
+
+int tlq_debug_panel_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
+  if (!(M >= 1 && N >= 1 && K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return 0;
+  const PanelPlan p = w4a16_panel_plan(M, N, K, group, cus);
+  if (plan_out) {
+    int64_t* o = (int64_t*)plan_out;
+    o[0] = p.tiles_m, o[1] = p.tiles_n, o[2] = p.split, o[3] = p.slice_steps;
+  }
+  return p.ok ? 1 : 0;
+}
 
 int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
   const DecodePlan p = w4a16_decode_plan(M, N, K, group, cus);
@@ -207,9 +230,27 @@ static int64_t w4a16_partial_sum_bytes(int64_t M, int64_t N, int64_t K) {
   return split > 1 ? split * M * N * 4 : 0;
 }
 
+// what the panel kernel may ask of the workspace for any group size: the partial tiles of its K slices and the flag word
+static int64_t panel_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (!(M >= 1 && N >= 1 && K > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return 0;
+  int64_t need = 0;
+  for (int64_t group = 32; group <= 1024; group *= 2) {
+    if (K % group != 0) continue;
+    const PanelPlan pp = w4a16_panel_plan(M, N, K, group, cu_count_or_default());
+    if (!pp.ok) continue;
+    const int64_t b = (pp.split > 1 ? (int64_t)pp.split * M * N * 4 : 0) + 16;
+    if (b > need) need = b;
+  }
+  return need;
+}
+
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
   int64_t need = w4a16_partial_sum_bytes(M, N, K);
+  if (M > 512) {
+    const int64_t pn = panel_workspace_bytes(M, N, K);
+    if (pn > need) need = pn;
+  }
   // two passes (which of the two is taken depends on the group size, so the size covers both): the dequantised matrix,
   // then room for the K slices of the plain GEMM where it has few output tiles
   if (M >= kTwoPassMinM) {
@@ -226,10 +267,39 @@ int64_t tlq_w4a16_workspace_bytes_min(int64_t M, int64_t N, int64_t K) {
   return M >= kTwoPassMinM ? N * K * 2 : 0;
 }
 
+// The panel kernel (large M, one launch, weights dequantised on the operand read).  Returns -1 when it does not take the
+// problem (nothing launched, no error set), else the launch's return code.
+static int try_panel(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, void* workspace,
+                     int64_t workspace_bytes, void* stream) {
+  if (!(M >= 1 && N >= 1 && K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return -1;
+  const PanelPlan pp = w4a16_panel_plan(M, N, K, group, cu_count_or_default());
+  if (!pp.ok) return -1;
+  const bool args_ok = A && w_packed && C && aligned16(A) && aligned16(w_packed) && aligned16(C) && aligned16(scales) &&
+                       aligned16(zeros) && (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) &&
+                       (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) && (M * N) % 4 == 0 &&
+                       fits32(M, K * 2) && fits32(N, K / 2) && fits32(N, (K / group) * 2);
+  if (!args_ok) return -1;
+  // workspace: the partial tiles of the K slices, then (with a zero-point tensor) one word for the kernel's flag
+  const int64_t part_bytes = pp.split > 1 ? (int64_t)pp.split * M * N * 4 : 0;
+  const int64_t need = part_bytes + (zeros ? 16 : 0);
+  if (need > 0 && !(workspace && aligned16(workspace) && workspace_bytes >= need)) return -1;
+  return gemm_w4a16_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, pp,
+                          (float*)workspace, zeros ? (uint32_t*)((uint8_t*)workspace + part_bytes) : nullptr, (hipStream_t)stream);
+}
+
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
-  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_DECODE, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_PANEL, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  if (algo == TLQ_ALGO_PANEL) {
+    const int rc = try_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
+                             workspace_bytes, stream);
+    TLQ_REQUIRE(rc >= 0, "tlq_gemm_w4a16_ws: the panel kernel needs K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group >= 32 "
+                "with (K / group) %% 8 == 0, 16-byte aligned operands, scale and zero tensors, and a workspace for its K slices and (with a "
+                "zero-point tensor) 16 bytes more (M=%lld N=%lld K=%lld group=%lld, workspace %lld)", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
+    return rc;
+  }
   // decode batches: rows longer than 4096 values run as chunks of K whose fp32 partial sums live in the workspace
   if (((algo == TLQ_ALGO_AUTO && g_w4a16_decode && (decode_preferred(M, N, K) || K > 16384)) || algo == TLQ_ALGO_DECODE) && M <= 32 && M >= 1 && N >= 1 && K > 0 && group > 0 &&
       N < kMaxDim && K < kMaxDim) {
@@ -336,6 +406,27 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
       return 1;
     }
   }
+  // Above 512 rows: the panel kernel (one launch, no dequantised matrix) where its work-groups fill the machine.  Measured
+  // against the choice without it (two passes, tile kernel over K slices) on ten (N, K) pairs x nine values of M, fp16 with
+  // a zero-point tensor and bf16 with a scalar one, groups of 128: from 576 to 2048 rows ahead wherever its last round of
+  // work-groups fills 0.55 of the CUs or more -- by 10 - 45 % on the wide or long matrices (N = 28672, K = 4096, M = 768:
+  // 1.35 - 1.47 x; N = 4096, K = 14336, M = 1280: 1.35 - 1.40 x; 8192 x 8192, M = 640: 1.36 - 1.41 x), within 5 % either
+  // way on 5120 x 5120 -- and 6 - 22 % behind below that fill (M = 2048, N = K = 4096: 128 work-groups).  From 3072 rows on
+  // every weight is dequantised 24 times or more and the two are within 5 % of each other (0.91 - 1.09): the two passes
+  // keep those, except where the panel kernel's work-groups fit the machine in one round and no zero-point tensor asks for
+  // its second launch (4096 x 4096 x 4096 with a scalar zero point: level, and no workspace traffic).
+  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && M > 512 && M <= 4096 && K > 0 && group > 0 && N >= 1 && N < kMaxDim && K < kMaxDim) {
+    const PanelPlan pp = w4a16_panel_plan(M, N, K, group, cu_count_or_default());
+    if (pp.ok) {
+      const int64_t wgs = (int64_t)pp.tiles_m * pp.tiles_n * pp.split, cus_now = cu_count_or_default();
+      const double fill = (double)wgs / (double)(ceil_div(wgs, cus_now) * cus_now);
+      if ((M <= 2048 && fill >= 0.55) || (wgs <= cus_now && fill >= 0.9 && zeros == nullptr)) {
+        const int rc = try_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
+                                 workspace_bytes, stream);
+        if (rc >= 0) return rc;
+      }
+    }
+  }
   const bool split_region = w4a16_mid_split(M, N, K, group > 0 ? group : 32) > 1;
   const bool two_pass = algo == TLQ_ALGO_TWO_PASS ||
                         (algo == TLQ_ALGO_AUTO && have && M >= kTwoPassMinM && N % 8 == 0 && !split_region);
@@ -375,8 +466,8 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
     return tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, algo, workspace,
                              workspace_bytes, stream);
   TLQ_CHECK_DIMS("tlq_gemm_w4a16_layout_ws");
-  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS || algo == TLQ_ALGO_DECODE,
-              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the decode kernel, the streaming kernel and the two passes (algo %d)", algo);
+  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS || algo == TLQ_ALGO_DECODE || algo == TLQ_ALGO_PANEL,
+              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the decode kernel, the streaming kernel, the panel kernel and the two passes (algo %d)", algo);
   TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_w4a16_layout_ws: in_dtype must be float16 or bfloat16 (got %d)", in_dtype);
   TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_w4a16_layout_ws: bad out_dtype %d", out_dtype);
   if (M == 0 || N == 0) return 0;
@@ -400,6 +491,20 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
                 (long long)K, (long long)group, (long long)workspace_bytes);
   }
   TLQ_REQUIRE(algo != TLQ_ALGO_DECODE, "tlq_gemm_w4a16_layout_ws: the decode kernel handles M <= 32 (got %lld)", (long long)M);
+  if (algo == TLQ_ALGO_PANEL || (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && M > 512 && M <= 4096)) {
+    // (the same rule as for plain words: where the panel kernel's tiles fill the machine)
+    const PanelPlan pp = w4a16_panel_plan(M, N, K, group, cu_count_or_default());
+    const int64_t wgs = (int64_t)pp.tiles_m * pp.tiles_n * pp.split, cus_now = cu_count_or_default();
+    const double fill = pp.ok ? (double)wgs / (double)(ceil_div(wgs, cus_now) * cus_now) : 0.0;
+    if (pp.ok && (algo == TLQ_ALGO_PANEL || (M <= 2048 && fill >= 0.55) || (wgs <= cus_now && fill >= 0.9 && zeros == nullptr))) {
+      const int rc = try_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, workspace,
+                               workspace_bytes, stream);
+      if (rc >= 0) return rc;
+    }
+    TLQ_REQUIRE(algo != TLQ_ALGO_PANEL, "tlq_gemm_w4a16_layout_ws: the panel kernel does not take M=%lld N=%lld K=%lld group=%lld with a "
+                "workspace of %lld bytes (K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group with (K / group) %% 8 == 0, 16-byte "
+                "aligned scale / zero tensors)", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
+  }
   if (algo != TLQ_ALGO_TWO_PASS) {
     const StreamPlan sp = w4a16_stream_plan(M, N, K, group, cu_count_or_default());
     const bool ws_ok = sp.ok && (M * N) % 4 == 0 && (sp.split == 1 || (ws_aligned && workspace_bytes >= (int64_t)sp.split * M * N * 4));
