@@ -11,14 +11,20 @@ independent weight sets (default 1).  The weight sets rotate through a pool larg
 HBM before the timed region starts.
 
 Prints ONE JSON line.
-  * `value` is algorithmic bytes / WALL-CLOCK time per step of the K timed steps: it includes the host side of every
+  * A timed REGION is exactly K steps (--steps) between two synchronisations, with a HIP event on the launch stream on
+    either side.  The region is repeated (`regions`: up to 25 times, within about a second per workload) and the MEDIAN
+    region is reported, so that one slow region -- a clock ramp, a noisy neighbour -- does not decide the line; the
+    spread is in `roofline.region_us_min` / `region_us_max`.
+  * `value` is algorithmic bytes / WALL-CLOCK time per step of the median region: it includes the host side of every
     launch (the ctypes call into the C ABI, about 2 us, which a microsecond kernel does not hide).
-  * `roofline.achieved` is algorithmic bytes (or operations) / the average step time between two HIP events recorded on the
-    launch stream around the same K steps.  After the timed region the same step runs again with one event pair per
-    step; `roofline.median_us` and `roofline.min_us` come from those pairs (each pair adds the event markers' own cost,
-    about a microsecond, so they bound the kernel from above and are not comparable with the back-to-back average).
-  * `roofline.traffic` is read from the counter summary under profiles/ for that kernel and workload (a line
-    "traffic_bytes_per_launch: N"), null when the file does not carry one.
+  * `roofline.achieved` is algorithmic bytes (or operations) / the step time between the two HIP events of the median
+    region.  After the timed regions the same step runs again with one event pair per step; `roofline.median_us` and
+    `roofline.min_us` come from those pairs (each pair adds the event markers' own cost, about a microsecond, so they
+    bound the kernel from above and are not comparable with the back-to-back average).
+  * `roofline.kernel` is the library's own launch log of one step (tlq_debug_launch_log: entry point [kernel, variant]
+    of every launch the call made), not a constant of this script.
+  * `roofline.traffic` is NOT measured by this run: it is read from the counter summary under profiles/ for that kernel
+    and workload (a line "traffic_bytes_per_launch: N"; `roofline.traffic_source` names the file), null without one.
   * `cpu_baseline` is the CPU oracle (the reference's torch ref_program arithmetic) timed on the host cores on a bounded
     sample; every entry of `other_workloads` (the other configurations) carries its own.
 """
@@ -45,14 +51,17 @@ WALL_NOTE = "value = algorithmic bytes / wall-clock per step incl. the host-side
 
 
 def traffic_from_profile(name):
-    """HBM bytes per launch as measured with hardware counters: the line 'traffic_bytes_per_launch: N' of
-    profiles/<name> (FETCH_SIZE + WRITE_SIZE, each scaled by a copy kernel of known size); None without one."""
+    """HBM bytes per launch as measured with hardware counters in an earlier profiling run: the line
+    'traffic_bytes_per_launch: N' of profiles/<name> (FETCH_SIZE + WRITE_SIZE, each scaled by a copy kernel of known
+    size).  Returns the two roofline fields {traffic, traffic_source}; traffic is None without such a line."""
+    val = None
     try:
         with open(os.path.join(ROOT, "profiles", name)) as f:
             m = re.search(r"^traffic_bytes_per_launch\s*:\s*(\d+)", f.read(), re.M)
-        return int(m.group(1)) if m else None
+        val = int(m.group(1)) if m else None
     except OSError:
-        return None
+        pass
+    return {"traffic": val, "traffic_source": ("profiles/" + name + " (counters of an earlier run, not of this one)") if val is not None else None}
 
 
 def w4a16_bytes(M, N, K, group, zeros_tensor=True, elem=2):
@@ -65,51 +74,83 @@ def w8a8_bytes(B, M, N, K):
 
 
 class Timing:
-    """wall / ev: seconds per step of the timed region (host clock / HIP events around the whole loop);
-    median / best: seconds per step from one event pair per step, taken after the timed region."""
+    """wall / ev: seconds per step of the median timed region (host clock / HIP events around the region's loop);
+    ev_all: the same for every region; median / best: seconds per step from one event pair per step, taken after the
+    timed regions; kernel: the library's launch log of one step."""
 
-    def __init__(self, wall, ev, per_step):
-        self.wall, self.ev = wall, ev
+    def __init__(self, walls, evs, per_step, kernel):
+        order = sorted(range(len(evs)), key=lambda i: evs[i])
+        mid = order[len(order) // 2]
+        self.wall, self.ev = walls[mid], evs[mid]
+        self.ev_all = evs
         self.median = statistics.median(per_step) if per_step else None
         self.best = min(per_step) if per_step else None
         self.pairs = len(per_step)
+        self.kernel = kernel
 
     def roofline(self, work, peak, unit, scale):
         """work per step (bytes or operations), peak in `unit`, scale = 1e9 for GB/s, 1e12 for T.../s."""
         ach = work / self.ev / scale
-        out = {"achieved": round(ach, 1), "peak": peak, "unit": unit, "frac": round(ach / peak, 4),
-               "avg_launch_us": round(self.ev * 1e6, 3)}
+        out = {"kernel": self.kernel, "achieved": round(ach, 1), "peak": peak, "unit": unit, "frac": round(ach / peak, 4),
+               "avg_launch_us": round(self.ev * 1e6, 3), "regions": len(self.ev_all),
+               "region_us_min": round(min(self.ev_all) * 1e6, 3), "region_us_max": round(max(self.ev_all) * 1e6, 3)}
         if self.pairs:
             out.update({"median_us": round(self.median * 1e6, 3), "min_us": round(self.best * 1e6, 3),
                         "per_step_event_pairs": self.pairs})
         return out
 
 
-def timed(fn, steps, warmup, pairs=None):
-    """warmup untimed steps, then exactly `steps` timed ones between two synchronisations; then `pairs` more
-    (default min(steps, 200)) with one event pair each."""
+def launch_log_of(fn):
+    """What one step launches, by the library's own record."""
+    from tilelang_ascend_amd import _abi
+
+    lib = _abi.load()
+    lib.tlq_debug_launch_log(1)
+    try:
+        fn(0)
+        text = lib.tlq_debug_launch_log_text()
+    finally:
+        lib.tlq_debug_launch_log(0)
+    return text.decode() if isinstance(text, bytes) else str(text)
+
+
+def timed(fn, steps, warmup, pairs=None, regions=None):
+    """warmup untimed steps, then regions of exactly `steps` timed ones between two synchronisations each (up to 25
+    regions, fewer when a region is long: about a second in all); then `pairs` more steps (default min(steps, 200)) with
+    one event pair each."""
     import torch
 
+    kernel = launch_log_of(fn)
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        fn(i)
-    e1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    walls, evs = [], []
+    budget_s, t_begin = 1.0, time.perf_counter()
+    want = 25 if regions is None else regions
+    base = 0
+    while len(evs) < want:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            fn(base + i)
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        walls.append((t1 - t0) / steps)
+        evs.append(e0.elapsed_time(e1) * 1e-3 / steps)
+        base += steps
+        if len(evs) >= 5 and time.perf_counter() - t_begin > budget_s:
+            break
     n = min(steps, 200) if pairs is None else pairs
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
-    for i, (a, b) in enumerate(evs):
+    pair_evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for i, (a, b) in enumerate(pair_evs):
         a.record()
-        fn(steps + i)
+        fn(base + i)
         b.record()
     torch.cuda.synchronize()
-    per_step = [a.elapsed_time(b) * 1e-3 for a, b in evs]
-    return Timing((t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps, per_step)
+    per_step = [a.elapsed_time(b) * 1e-3 for a, b in pair_evs]
+    return Timing(walls, evs, per_step, kernel)
 
 
 def cpu_time(fn, budget_s, max_reps=200):
@@ -184,8 +225,8 @@ def bench_gemv(args, units=None, steps=None, warmup=None, cpu=True):
         "config": {"workload": f"W4A16 decode GEMV M=1 N=11008 K=4096 group=128 fp16 scales+zeros, {units} weight set(s) per launch, "
                                f"{sets} sets rotating ({sets * unit_bytes >> 20} MiB); " + WALL_NOTE,
                    "M": M, "N": N, "K": K, "group": g, "units_per_launch": units},
-        "roofline": dict({"kernel": ("gemv_w4a16_ring_kernel<f16,2,1>" if units == 1 else "gemv_w4a16_f16_rows_kernel<2,2,1024>"), "bound": "hbm"}, **tm.roofline(step_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
-                         traffic=(traffic_from_profile("gemv_w4a16_f16_M1_N11008_K4096_g128.txt") if units == 1 else None),
+        "roofline": dict({"bound": "hbm"}, **tm.roofline(step_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
+                         **(traffic_from_profile("gemv_w4a16_f16_M1_N11008_K4096_g128.txt") if units == 1 else {"traffic": None}),
                          bytes_per_launch=step_bytes),
         "cpu_baseline": cpu,
         "parity_rel_l2": rel,
@@ -234,8 +275,7 @@ def bench_small(args, steps=None, cpu=True):
     flops, nbytes = 2.0 * M * N * K, w4a16_bytes(M, N, K, g, zeros_tensor=False)
     out = {"workload": "W4A16 dequant-GEMM M=N=K=256 fp16 group=128 zero=8 (launch bound: 0.03 GFLOP, 0.3 MB)", "dtype": "f16",
            "value": round(flops / tm.wall / 1e12, 3), "unit": "TFLOP/s", "ms_per_step": tm.wall * 1e3,
-           "roofline": dict({"kernel": "automatic choice of tlq_gemm_w4a16_ws", "bound": "hbm"},
-                            **tm.roofline(nbytes, HBM_PEAK_GBS, "GB/s", 1e9), traffic=None, bytes_per_launch=nbytes)}
+           "roofline": dict({"bound": "hbm"}, **tm.roofline(nbytes, HBM_PEAK_GBS, "GB/s", 1e9), traffic=None, bytes_per_launch=nbytes)}
     if cpu:
         from oracle import ref
 
@@ -276,28 +316,36 @@ def bench_prefill(args, steps=None, cpu=True):
     ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
 
-    def step(i):  # what the library chooses with a workspace: dequantise into it, then the plain MFMA GEMM (two launches)
+    def step(i):  # what the library chooses with a workspace (the launch log of a step is in roofline.kernel)
         rc = lib.tlq_gemm_w4a16_ws(P(A), P(Wp), P(S), None, P(C), M, N, K, g, 8.0, _abi.BF16, _abi.BF16, _abi.ALGO_AUTO,
                                    P(ws), ws_bytes, stream)
         if rc:
             raise RuntimeError(_abi.last_error())
 
-    def step_fused(i):  # the single fused kernel, for comparison
+    def step_two(i):  # the reference's own structure, for comparison: dequantise into the workspace, then the plain GEMM
+        rc = lib.tlq_gemm_w4a16_ws(P(A), P(Wp), P(S), None, P(C), M, N, K, g, 8.0, _abi.BF16, _abi.BF16, _abi.ALGO_TWO_PASS,
+                                   P(ws), ws_bytes, stream)
+        if rc:
+            raise RuntimeError(_abi.last_error())
+
+    def step_fused(i):  # the tile kernel that dequantises into LDS through registers, for comparison
         rc = lib.tlq_gemm_w4a16(P(A), P(Wp), P(S), None, P(C), M, N, K, g, 8.0, _abi.BF16, _abi.BF16, _abi.ALGO_MFMA, stream)
         if rc:
             raise RuntimeError(_abi.last_error())
 
     tm = timed(step, steps or args.steps, args.warmup)
-    fused = timed(step_fused, steps or args.steps, min(args.warmup, 4), pairs=0)
+    two = timed(step_two, steps or args.steps, min(args.warmup, 4), pairs=0, regions=9)
+    fused = timed(step_fused, steps or args.steps, min(args.warmup, 4), pairs=0, regions=9)
     flops = 2.0 * M * N * K
     out = {"workload": "W4A16 prefill GEMM M=N=K=4096 bf16 group=128 zero=8, automatic choice with a caller-owned workspace "
-                       "(dequantisation pass + plain MFMA GEMM; the whole step is priced against the MFMA peak)", "dtype": "bf16",
+                       "(the whole step is priced against the MFMA peak)", "dtype": "bf16",
            "value": round(flops / tm.wall / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": tm.wall * 1e3,
-           "roofline": dict({"kernel": "dequant_w4_vec8<bf16> + gemm_mfma_kernel<MmaBF16,RowLoaderDirect,RowLoaderDirect,EpiFloat,256,256,2,4>", "bound": "mfma"},
-                            **tm.roofline(flops, MFMA_F16_PEAK_TFLOPS, "TFLOP/s", 1e12),
-                            traffic=traffic_from_profile("gemm_w4a16_bf16_M4096_N4096_K4096_g128.txt"), flops_per_launch=flops),
-           "fused_kernel": {"path": "tlq_gemm_w4a16(algo=mfma): gemm_mfma_kernel<MmaBF16,RowLoaderDirect,W4Loader>, one launch, no workspace",
-                            "value": round(flops / fused.wall / 1e12, 1), "unit": "TFLOP/s", "us_per_step": round(fused.ev * 1e6, 2),
+           "roofline": dict({"bound": "mfma"}, **tm.roofline(flops, MFMA_F16_PEAK_TFLOPS, "TFLOP/s", 1e12),
+                            **traffic_from_profile("panel_w4a16_bf16_M4096_N4096_K4096_g128.txt"), flops_per_launch=flops),
+           "two_passes": {"path": two.kernel, "value": round(flops / two.wall / 1e12, 1), "unit": "TFLOP/s",
+                          "us_per_step": round(two.ev * 1e6, 2), "frac_of_mfma_peak": round(flops / two.ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)},
+           "fused_kernel": {"path": fused.kernel, "value": round(flops / fused.wall / 1e12, 1), "unit": "TFLOP/s",
+                            "us_per_step": round(fused.ev * 1e6, 2),
                             "frac_of_mfma_peak": round(flops / fused.ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}}
     if cpu:
         from oracle import ref
@@ -337,8 +385,8 @@ def bench_skinny(args, steps=None, cpu=True):
     tm = timed(step, steps or args.steps, args.warmup)
     out = {"workload": f"W4A16 decode batch M=16 N=14336 K=4096 group=128 fp16 scales+zeros, {sets} weight sets rotating",
            "dtype": "f16", "value": round(unit_bytes / tm.wall / 1e9, 1), "unit": "GB/s", "ms_per_step": tm.wall * 1e3,
-           "roofline": dict({"kernel": "w4a16_decode_kernel<f16,1>", "bound": "hbm"}, **tm.roofline(unit_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
-                            traffic=traffic_from_profile("decode_w4a16_f16_M16_N14336_K4096_g128.txt"), bytes_per_launch=unit_bytes)}
+           "roofline": dict({"bound": "hbm"}, **tm.roofline(unit_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
+                            **traffic_from_profile("decode_w4a16_f16_M16_N14336_K4096_g128.txt"), bytes_per_launch=unit_bytes)}
     if cpu:
         from oracle import ref
 
@@ -376,8 +424,8 @@ def bench_act_quant(args, steps=None):
     tm = timed(step, steps or args.steps, args.warmup)
     return {"workload": f"per-token int8 activation quantiser M=16384 N=4096 bf16 in, {sets} inputs rotating",
             "dtype": "f32", "value": round(unit_bytes / tm.wall / 1e9, 1), "unit": "GB/s", "ms_per_step": tm.wall * 1e3,
-            "roofline": dict({"kernel": "act_quant_rows_kernel<bf16,8,1>", "bound": "hbm"}, **tm.roofline(unit_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
-                             traffic=traffic_from_profile("act_quant_bf16_M16384_N4096.txt"), bytes_per_launch=unit_bytes)}
+            "roofline": dict({"bound": "hbm"}, **tm.roofline(unit_bytes, HBM_PEAK_GBS, "GB/s", 1e9),
+                             **traffic_from_profile("act_quant_bf16_M16384_N4096.txt"), bytes_per_launch=unit_bytes)}
 
 
 def bench_mlp_sweep(args, steps=None):
@@ -412,10 +460,10 @@ def bench_mlp_sweep(args, steps=None):
                         raise RuntimeError(_abi.last_error())
 
                 n = steps or (12 if M < 8192 else 4)
-                tm = timed(step, n, 3, pairs=n)
+                tm = timed(step, n, 3, pairs=n, regions=7)
                 ev = tm.ev
                 flops, nbytes = 2.0 * M * N * K, w4a16_bytes(M, N, K, g)
-                rows.append({"M": M, "N": N, "K": K, "group": g, "us": round(ev * 1e6, 1), "median_us": round(tm.median * 1e6, 1),
+                rows.append({"M": M, "N": N, "K": K, "group": g, "kernel": tm.kernel, "us": round(ev * 1e6, 1), "median_us": round(tm.median * 1e6, 1),
                              "min_us": round(tm.best * 1e6, 1),
                              "TFLOP/s": round(flops / ev / 1e12, 1), "frac_mfma": round(flops / ev / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                              "GB/s": round(nbytes / ev / 1e9), "frac_hbm": round(nbytes / ev / 1e9 / HBM_PEAK_GBS, 4)})
@@ -455,9 +503,8 @@ def bench_w8a8(args, steps=None, cpu=True):
     ops = 2.0 * B * M * N * K
     out = {"workload": "W8A8 quant batch matmul B=8 M=2048 N=K=4096, per-token x per-channel rescale, fp16 out",
            "dtype": "i8", "value": round(ops / tm.wall / 1e12, 1), "unit": "TOP/s", "ms_per_step": tm.wall * 1e3,
-           "roofline": dict({"kernel": "gemm_slots_kernel<MmaI8,I8KNLoaderDirect,EpiRescale>", "bound": "mfma"},
-                            **tm.roofline(ops, MFMA_I8_PEAK_TOPS, "TOP/s", 1e12),
-                            traffic=traffic_from_profile("gemm_w8a8_B8_M2048_N4096_K4096.txt"), ops_per_launch=ops)}
+           "roofline": dict({"bound": "mfma"}, **tm.roofline(ops, MFMA_I8_PEAK_TOPS, "TOP/s", 1e12),
+                            **traffic_from_profile("gemm_w8a8_B8_M2048_N4096_K4096.txt"), ops_per_launch=ops)}
     if cpu:
         from oracle import ref
 
@@ -546,7 +593,7 @@ def main():
         line = {"metric": METRIC, "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
                 "config": {"workload": res["workload"] + ("; every figure from HIP events" if args.workload == "mlp-sweep" else "; " + WALL_NOTE)}, "roofline": res["roofline"],
                 "cpu_baseline": res.get("cpu_baseline")}
-        for extra in ("shapes", "fused_kernel"):
+        for extra in ("shapes", "fused_kernel", "two_passes"):
             if extra in res:
                 line[extra] = res[extra]
     if args.calibrate_copy:

@@ -174,10 +174,11 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
 /* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose wrapper allocates its
  * workspace anew on every call (tilelang/jit/adapter/cython/cython_wrapper.pyx:128-129).  The workspace is
- * a device array built into the library, TLQ_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends; problems whose
- * tlq_w4a16_workspace_bytes_min(M, N, K) exceeds it are rejected with an error (use tlq_gemm_w4a16_ws for those).  The
+ * a device array built into the library, TLQ_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends.  The
  * call allocates and frees nothing; results are those of tlq_gemm_w4a16_ws with a workspace of
- * TLQ_NOALLOC_SCRATCH_BYTES bytes (the preferred kernel where tlq_w4a16_workspace_bytes(M, N, K) fits), bit for bit.  All
+ * TLQ_NOALLOC_SCRATCH_BYTES bytes (the preferred kernel where tlq_w4a16_workspace_bytes(M, N, K) fits), bit for bit;
+ * problems whose tlq_w4a16_workspace_bytes_min(M, N, K) exceeds the array run as tlq_gemm_w4a16_ws runs them without a
+ * workspace (the kernels that need no scratch), never with an error for lack of room.  All
  * calls on one GPU share the array: calls that overlap there (other streams, other threads) race.
  * tlq_gemm_w4a16_noalloc_init looks the array's address up for the current device (otherwise the first call on a
  * device does it); it allocates nothing either. */
@@ -298,93 +299,9 @@ int tlq_quantize_sym4(const void* W, void* q_minus8, void* scales, int64_t N, in
  * Its outputs are the A / scale_a operands of tlq_gemm_w8a8. */
 int tlq_act_quant_i8(const void* X, void* Y, void* S, int64_t M, int64_t N, int in_dtype, int round_scale, void* stream);
 
-/* Self-checks of the MFMA GEMM kernels' address arithmetic, evaluated on the HOST with the functions the kernels
- * themselves use (no GPU needed; the reference has no counterpart, its tile addressing is generated by TVM).
- * tlq_debug_check_gemm_addressing walks every tile, thread, load instruction and stage of one operand:
- * source_kind 0 = row-major [rows, row_bytes] operand copied global -> LDS directly in tiles of `tile` rows by
- * `threads` threads; 1 = int8 [K = rows, N = row_bytes] weights in tiles of `tile` (128 | 256) columns; 2 = 16-bit
- * [K = rows, N = row_bytes (the number of columns)] weights in tiles of 128 | 256 columns (N a multiple of 8).  It
- * checks global extents, LDS extents and coverage, agreement with the (transposing) operand-fragment reads and, for
- * kind 2, that no half-wavefront read meets a bank twice.
- * tlq_debug_check_slots_schedule simulates the five-slot kernel's issue / wait / barrier order over `stages` stages
- * with `loads_per_tile` load instructions per wavefront and tile (the kernel's waits assume 4).
- * Both return 0 when everything holds, else 1 with tlq_last_error() naming the first violation. */
-int tlq_debug_check_gemm_addressing(int source_kind, int64_t rows, int64_t row_bytes, int tile, int threads);
-int tlq_debug_check_slots_schedule(int stages, int loads_per_tile);
-/* The same walk for the streaming W4A16 kernel (TLQ_ALGO_STREAM): packed weights [N, K / 2] and 2-byte activations [M, K]
- * with 16 * activation_tiles rows per work-group (2 | 4 | 8), and its ring of `ring_depth` steps for 1 .. 40 steps. */
-int tlq_debug_check_stream_addressing(int64_t M, int64_t N, int64_t K, int activation_tiles, int ring_depth);
-/* The same walk for the panel kernel (TLQ_ALGO_PANEL) with K slices of `slice_steps` steps of 128 values: every direct load of
- * activations, packed weights and scale windows of every work-group, the LDS map and the operand reads; and the plan the
- * library would choose on a device with `cus` compute units: plan_out is a HOST array of four int64 that receives the tiles
- * along M and N, the K slices and the steps per slice; returns 1 when the kernel applies. */
-int tlq_debug_check_panel_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int slice_steps);
-int tlq_debug_panel_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
-
-/* The same walk for the decode kernel (TLQ_ALGO_DECODE) launched as grid_x x chunks work-groups of `waves` wavefronts
- * with 16 * activation_tiles activation rows, and its ring for 2 .. 24 items; tlq_debug_decode_plan gives the geometry
- * the library would choose on a device with `cus` compute units: plan_out is a HOST array of five int64 that receives
- * activation tiles, chunks, wavefronts per work-group, grid_x and bytes of dynamic LDS; returns 1 when the kernel applies. */
-int tlq_debug_check_decode_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int activation_tiles, int chunks, int waves,
-                                      int grid_x);
-int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
-
-/* Launch geometry the register-resident decode GEMV (M = 1, K <= 16384, power-of-two group) would use on a device with
- * `cus` compute units, computed on the host: plan_out is a HOST array of four int64 that receives rows per work-group,
- * work-groups, bytes of dynamic LDS and wavefronts per work-group.  Returns 1 when the kernel applies (its LDS stays
- * within the 64 KB a kernel may use without further set-up), 0 when the launcher falls back to the streaming GEMV,
- * -1 for bad arguments.  No counterpart in the reference. */
-int tlq_debug_gemv_rows_plan(int64_t batch, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
-
-/* The same for the ring kernel, which takes a single decode GEMV (M = 1, or 2 with fp16 activations; K <= 4096, a
- * multiple of 8 groups per row, 16-byte aligned scale / zero tensors) with every global read a direct global -> LDS load:
- * plan_out receives six int64:
- * load instructions per row, ring slots per wavefront, wavefronts per work-group, rows per work-group, work-groups and
- * bytes of dynamic LDS.  Returns 1 when the kernel applies, 0 when not, -1 for bad arguments.
- * tlq_debug_check_gemv_ring_addressing walks, on the host, every load of the first, middle and last work-groups of such a
- * launch (bounds of every global read and LDS write, coverage of the staging data and of the rows, ring order against the
- * kernel's wait counts); 0 = consistent.  No counterpart in the reference. */
-/* Output tile (128 or 256, square) the MFMA GEMMs take for `batch` problems of M x N outputs on the current device (256 CUs
- * when there is none): by machine fill, see tlq_tune_gemm_tile.  fused = 1: the fused W4A16 tile kernel's rule.  Host only;
- * no counterpart in the reference (its block_M / block_N are arguments, example_dequant_gemm_fine_grained.py:437). */
-int tlq_debug_gemm_tile(int64_t batch, int64_t M, int64_t N, int fused);
-int tlq_debug_gemv_ring_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out);
-int tlq_debug_check_gemv_ring_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int rows_per_block, int waves, int depth);
-
-/* Tuning hooks for benchmark sweeps and the autotuner (each sets a value of the CALLING THREAD, read by that thread's
- * later launches; other threads keep the automatic choice; 0 = automatic choice).
- * They play the role of the reference's block_M / block_N / block_K factory arguments
- * (example_dequant_gemm_fine_grained.py:437,462), which here select among pre-built tilings. */
-void tlq_tune_gemv(int rows_per_wave, int waves_per_block); /* rows 1|2|4 (negative: never the register-resident
-                                                             * M = 1, K <= 4096 kernel), waves 1..4 (that kernel: 1..16) */
-void tlq_tune_gemv_unroll(int blocks_per_cu);               /* resident blocks per CU the GEMV grid is sized for */
-void tlq_tune_gemv_depth(int steps_in_flight);               /* load steps (1 KB per row each) a GEMV wavefront keeps in flight */
-void tlq_tune_gemv_ring(int on);                             /* 1 (default): a single decode GEMV (1 or 2 activation rows) runs on the
-                                                              * ring kernel where it applies; 0: on the kernels it replaced (for one
-                                                              * activation row the same results, bit for bit) */
-void tlq_tune_gemm_band(int tile_rows);                       /* tile rows per band of the MFMA kernels' tile order (default 4) */
-void tlq_tune_gemm_tile(int tile);                            /* square tile of the plain 16-bit GEMM (and of the second of the two W4A16 passes):
-                                                              * 128 | 256, 0 = by the number of output tiles */
-void tlq_tune_gemm_slots(int mode);                          /* the kernel that cuts LDS into five operand-tile slots (256 x 256 tiles, whole 128-byte
-                                                              * stages of K only): 1 (default) where it measured faster than the two-stage kernel
-                                                              * (int8, several batches of up to 2048 rows), 2 wherever it can run (also the plain
-                                                              * 16-bit GEMMs), 0 never */
-void tlq_tune_w4a16_decode(int on);                          /* 0: the decode kernel is never picked automatically */
-void tlq_tune_w4a16_stream(int on);                          /* 0: tlq_gemm_w4a16_ws never picks the streaming kernel by itself */
-void tlq_tune_w4a16_stream_slice(int steps);                 /* K slice of the streaming kernel in steps of 128 values (0 = by its estimate) */
-void tlq_tune_w4a16_panel(int mode);                         /* tlq_gemm_w4a16_ws, large M: 0 = automatic, 1 = never the panel kernel (TLQ_ALGO_PANEL) */
-void tlq_tune_w4a16_panel_slice(int steps);                  /* K slice of the panel kernel in steps of 128 values (0 = its own plan) */
-void tlq_tune_w4a16_tile(int block_m);                      /* 16|32|64|128|256 */
-void tlq_tune_w4a16_split(int slices);                       /* K slices of the tile kernel, 16 < M < 256 with a workspace */
-void tlq_tune_w4a16_skinny(int waves, int row_tiles);       /* wavefronts per group 1..16; 16-row tiles per wavefront 1|2,
-                                                               +10 = never stage through LDS, +20 = stage whenever possible */
-void tlq_tune_i8_tile(int block_m);                         /* 32|128|256 */
-void tlq_tune_f16_split(int slices);                        /* K slices of tlq_gemm_f16_ws: 0 = automatic, 1 = never, n = up to n */
-int tlq_debug_f16_split(int64_t M, int64_t N, int64_t K);  /* K slices tlq_gemm_f16_ws takes for one batch of this shape */
-void tlq_tune_w4a8_ws(int mode);                            /* tlq_gemm_w4a8_ws: 0 = automatic, 1 = K slices in the workspace, 2 = unpack + int8 GEMM */
-void tlq_tune_i8_split(int slices);                         /* K slices of the one-batch int8 kernels: 0 = automatic, 1 = never, n = up to n */
-int tlq_debug_i8_split(int64_t M, int64_t N, int64_t K, int buffers); /* K slices taken for one batch of this shape: with a matrix per
-                                                                      * slice (1, tlq_gemm_w8a8_ws) or atomic adds into C (0, tlq_gemm_i8) */
+/* The host-side self-checks of the kernels' address arithmetic (tlq_debug_*) and the tuning hooks that benchmark sweeps and
+ * the autotuner use (tlq_tune_*) are exported by the same library and declared in tlq_debug.h: they are not part of the
+ * operator boundary above. */
 
 #ifdef __cplusplus
 }

@@ -1,5 +1,6 @@
-"""The C-ABI shared library: it loads without a GPU, exports every symbol include/tlq.h declares
-with the declared argument lists, and rejects bad arguments before touching a device."""
+"""The C-ABI shared library: it loads without a GPU, exports every symbol include/tlq.h (the operator boundary) and
+include/tlq_debug.h (self-checks and tuning hooks) declare, with the declared argument lists, and rejects bad arguments
+before touching a device."""
 import ctypes
 import os
 import re
@@ -10,15 +11,16 @@ from tilelang_ascend_amd import _abi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "tlq.h")
+DEBUG_HEADER = os.path.join(ROOT, "include", "tlq_debug.h")
 
 CTYPE = {"const void*": ctypes.c_void_p, "void*": ctypes.c_void_p, "int64_t": ctypes.c_int64, "int": ctypes.c_int,
          "float": ctypes.c_float}
 RESTYPE = {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "void": None, "const char*": ctypes.c_char_p}
 
 
-def declared():
-    """name -> (return type, [argument types]) parsed from the header text."""
-    text = open(HEADER).read()
+def declared(headers=(HEADER, DEBUG_HEADER)):
+    """name -> (return type, [argument types]) parsed from the header texts."""
+    text = "\n".join(open(h).read() for h in headers)
     text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
     out = {}
     for m in re.finditer(r"(const char\*|int64_t|int|void)\s+(tlq_\w+)\s*\(([^)]*)\)\s*;", text):
@@ -38,6 +40,13 @@ def test_header_declares_only_plain_c_types():
     d = declared()
     assert len(d) >= 15
     assert "torch" not in open(HEADER).read().lower().replace("torch_unpack", "").replace("torch_convert", "")
+
+
+def test_the_operator_header_carries_no_test_or_tuning_hooks():
+    ops = declared((HEADER,))
+    assert ops and not [n for n in ops if n.startswith(("tlq_debug_", "tlq_tune_"))]
+    dev = declared((DEBUG_HEADER,))
+    assert dev and all(n.startswith(("tlq_debug_", "tlq_tune_")) for n in dev)
 
 
 def test_library_exports_every_declared_symbol():

@@ -145,3 +145,31 @@ def test_gen_quant4_results_feed_the_w4a16_operands(groupsize):
         gpu.pack_gen_quant4(q8, s, saturate=False)
     with pytest.raises(ValueError):
         gpu.pack_gen_quant4(q8 + 5, s)
+
+
+def test_packed_weights_round_trip_through_a_file(tmp_path):
+    """save_packed / load_packed: plain tensors and numbers only, read back with a loader that executes nothing."""
+    from tilelang_ascend_amd.quantize import load_packed, save_packed
+
+    g = torch.Generator().manual_seed(5)
+    N, K, group = 48, 256, 64
+    Bp = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=g)
+    s = (torch.rand(N, K // group, generator=g) * 0.015 + 0.005).half()
+    z = torch.randint(6, 10, (N, K // group), generator=g).half()
+    for layout, zeros in (("plain", z), ("interleaved", 8), ("plain", None)):
+        path = tmp_path / f"w_{layout}_{type(zeros).__name__}.pt"
+        save_packed(path, Bp, s, zeros, layout=layout, group=group)
+        got = load_packed(path)
+        assert got["layout"] == layout and got["group"] == group and (got["N"], got["K"]) == (N, K)
+        assert torch.equal(got["B_packed"], Bp) and torch.equal(got["scales"], s)
+        if torch.is_tensor(zeros):
+            assert torch.equal(got["zeros"], zeros)
+        else:
+            assert got["zeros"] == zeros
+    with pytest.raises(ValueError):
+        save_packed(tmp_path / "bad.pt", Bp, s[:, :1], None, group=group)
+    with pytest.raises(ValueError):
+        save_packed(tmp_path / "bad.pt", Bp, s, None, layout="tiled", group=group)
+    torch.save({"format": "something else"}, tmp_path / "other.pt")
+    with pytest.raises(ValueError):
+        load_packed(tmp_path / "other.pt")

@@ -59,6 +59,8 @@ SIGNATURES = {
     "tlq_debug_check_stream_addressing": (_int, [_i64, _i64, _i64, _int, _int]),
     "tlq_debug_check_decode_addressing": (_int, [_i64, _i64, _i64, _i64, _int, _int, _int, _int]),
     "tlq_debug_decode_plan": (_int, [_i64, _i64, _i64, _i64, _int, _vp]),
+    "tlq_debug_launch_log": (None, [_int]),
+    "tlq_debug_launch_log_text": (ctypes.c_char_p, []),
     "tlq_debug_check_panel_addressing": (_int, [_i64, _i64, _i64, _i64, _int]),
     "tlq_debug_panel_plan": (_int, [_i64, _i64, _i64, _i64, _int, _vp]),
     "tlq_tune_w4a16_decode": (None, [_int]),
@@ -189,3 +191,18 @@ def tuning(w4a16_tile: int = 0, i8_tile: int = 0, gemv: tuple = None, skinny: tu
                 lib.tlq_tune_gemv_depth(0)
             if skinny:
                 lib.tlq_tune_w4a16_skinny(0, 0)
+
+
+def scratch(nbytes: int, device, stream: int):
+    """A per-call workspace of `nbytes` bytes from torch's caching allocator, safe to hand to a kernel launched on the raw
+    stream `stream`: the allocator orders reuse of a block by the stream that was current when it was allocated, so when
+    the launch stream is another one the block is recorded on it (otherwise the block could be handed out again, on the
+    current stream, while the kernel still writes it).  None for nbytes == 0."""
+    import torch
+
+    if not nbytes:
+        return None
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    if stream and stream != torch.cuda.current_stream(ws.device).cuda_stream:
+        ws.record_stream(torch.cuda.ExternalStream(stream, device=ws.device))
+    return ws

@@ -73,7 +73,7 @@ def source_fingerprint() -> str:
     cache key (tilelang/cache/kernel_cache.py:71-117: hash of source + target + options)."""
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    names = sorted(os.listdir(CSRC_DIR)) + ["../../include/tlq.h"]
+    names = sorted(os.listdir(CSRC_DIR)) + ["../../include/tlq.h", "../../include/tlq_debug.h"]
     for name in names:
         path = os.path.join(CSRC_DIR, name)
         if os.path.isfile(path):

@@ -1,6 +1,7 @@
 // Error channel, version and device queries of libtlq.
 #include <stdarg.h>
 #include <stdio.h>
+#include <string.h>
 
 #include "tlq_common.h"
 
@@ -15,8 +16,28 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
-// Called right after a kernel launch: turns a launch failure into an error string.
-bool check_launch(const char* what) {
+// Launch log of the calling thread (tlq_debug_launch_log): which kernels an entry point really launched, for benchmarks
+// and tests that name the kernel they measured.  Off by default; a repeated entry is written once.
+static thread_local bool g_log_on = false;
+static thread_local char g_log[1024] = "";
+static thread_local char g_log_last[160] = "";
+static void log_launch(const char* what, const char* detail) {
+  char entry[160];
+  if (detail && detail[0])
+    snprintf(entry, sizeof(entry), "%s [%s]", what, detail);
+  else
+    snprintf(entry, sizeof(entry), "%s", what);
+  if (strcmp(entry, g_log_last) == 0) return;
+  snprintf(g_log_last, sizeof(g_log_last), "%s", entry);
+  const size_t used = strlen(g_log);
+  if (used + strlen(entry) + 4 >= sizeof(g_log)) return;
+  snprintf(g_log + used, sizeof(g_log) - used, "%s%s", used ? " + " : "", entry);
+}
+
+// Called right after a kernel launch: turns a launch failure into an error string.  detail: the kernel and its
+// variant, for the launch log.
+bool check_launch(const char* what, const char* detail) {
+  if (g_log_on) log_launch(what, detail);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("%s: launch failed: %s", what, hipGetErrorString(e));
@@ -32,6 +53,13 @@ extern "C" {
 int tlq_abi_version(void) { return TLQ_ABI_VERSION; }
 
 const char* tlq_last_error(void) { return tlq::g_error; }
+
+void tlq_debug_launch_log(int on) {
+  tlq::g_log_on = on != 0;
+  if (on) tlq::g_log[0] = 0, tlq::g_log_last[0] = 0;
+}
+
+const char* tlq_debug_launch_log_text(void) { return tlq::g_log; }
 
 int tlq_device_cu_count(void) {
   int dev = 0;

@@ -186,7 +186,7 @@ static int run_act_quant(const void* Xv, void* Yv, void* Sv, int64_t M, int64_t 
     const int64_t want = ceil_div(M, (int64_t)4);
     act_quant_generic_kernel<T><<<(int)(want > 65536 ? 65536 : want), 256, 0, st>>>(X, Y, S, M, N, round_scale);
   }
-  return check_launch("tlq_act_quant_i8") ? 0 : 1;
+  return check_launch("tlq_act_quant_i8", "act_quant kernel") ? 0 : 1;
 }
 
 }  // namespace tlq

@@ -202,7 +202,7 @@ static int64_t stream_max_split(int64_t M, int64_t N, int64_t K) {
   int64_t most = 0;
   for (int64_t group = 32; group <= K; group *= 2) {
     if (K % group) continue;
-    const StreamPlan p = w4a16_stream_plan(M, N, K, group, 256);
+    const StreamPlan p = w4a16_stream_plan(M, N, K, group, cu_count_or_default());  // (the count the launch plans with)
     if (p.ok && p.split > most) most = p.split;
   }
   return most;
@@ -224,7 +224,7 @@ static int64_t w4a16_partial_sum_bytes(int64_t M, int64_t N, int64_t K) {
   const int64_t ssplit = stream_max_split(M, N, K);
   if (ssplit > split) split = ssplit;
   if (M <= 32) {  // the decode kernel cuts rows longer than 4096 values into chunks
-    const DecodePlan dp = w4a16_decode_plan(M, N, K, 32, 256);
+    const DecodePlan dp = w4a16_decode_plan(M, N, K, 32, cu_count_or_default());
     if (dp.ok && dp.chunks > split) split = dp.chunks;
   }
   return split > 1 ? split * M * N * 4 : 0;

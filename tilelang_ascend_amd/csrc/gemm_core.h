@@ -691,7 +691,9 @@ __device__ __forceinline__ void write_tile_with(const Epi& epi, const S& scales,
   const int r16 = lane & 15, q = lane >> 4;
   const int osz = epi.out_bytes();
   bool staged = false;
-  if constexpr (Epi::STAGED) staged = ((epi.pitch() * osz) & 15) == 0 && ((N * osz) & 15) == 0 && TN * 16 * osz >= 128;
+  // (whole passes of 128 output bytes per row only: a wavefront tile whose width is not a multiple of a pass goes the direct way)
+  if constexpr (Epi::STAGED)
+    staged = ((epi.pitch() * osz) & 15) == 0 && ((N * osz) & 15) == 0 && TN * 16 * osz >= 128 && (TN * 16 * osz) % 128 == 0;
   if (!staged) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
@@ -1009,7 +1011,9 @@ int launch_gemm(const typename AL::Params& pa, const typename WL::Params& pw, co
   }
   kern<<<(unsigned)blocks, WM * WN * 64, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, KT, k_tail, (int)tiles_m,
                                                           (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows, kt_total);
-  return check_launch(what) ? 0 : 1;
+  char detail[96];
+  snprintf(detail, sizeof(detail), "gemm_mfma_kernel %dx%d tiles, two stages%s", BM, BN, WL::DIRECT ? "" : ", weights through registers");
+  return check_launch(what, detail) ? 0 : 1;
 }
 
 }  // namespace tlq

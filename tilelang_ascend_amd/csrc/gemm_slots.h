@@ -117,7 +117,7 @@ int launch_gemm_slots(const typename RowLoaderDirect<256, 512>::Params& pa, cons
   }
   kern<<<(unsigned)blocks, 512, lds_bytes, st>>>(pa, pw, pe, (int)M, (int)N, (int)(k_bytes / kStageBytes), (int)tiles_m,
                                                  (int)tiles_n, g_gemm_band_rows > 0 ? g_gemm_band_rows : band_rows);
-  return check_launch(what) ? 0 : 1;
+  return check_launch(what, "gemm_slots_kernel 256x256 tiles, five slots") ? 0 : 1;
 }
 
 }  // namespace tlq

@@ -597,7 +597,7 @@ static int launch_skinny(const W4Args& a, int waves) {
   const size_t lds = (size_t)waves * RT * MT * 64 * sizeof(float4_t);
   kern<<<blocks, waves * 64, lds, a.st>>>((const T*)a.A, (const uint8_t*)a.Wp, (const T*)a.scales, (const T*)a.zeros, a.C,
                                           (int)a.M, (int)a.N, (int)a.K, (int)a.group, a.zero_scalar, a.out_dtype);
-  return check_launch("tlq_gemm_w4a16(skinny)") ? 0 : 1;
+  return check_launch("tlq_gemm_w4a16(skinny)", "w4a16_skinny_kernel") ? 0 : 1;
 }
 
 template <typename T, bool FOLD, int RT>
@@ -617,7 +617,7 @@ static int launch_skinny_lds(const W4Args& a, int waves, int gshift) {
   kern<<<blocks, waves * 64, (size_t)waves * WAVE_LDS, a.st>>>((const T*)a.A, (const uint8_t*)a.Wp, (const T*)a.scales,
                                                                 (const T*)a.zeros, a.C, (int)a.M, (int)a.N, (int)a.K,
                                                                 gshift, a.zero_scalar, a.out_dtype);
-  return check_launch("tlq_gemm_w4a16(skinny)") ? 0 : 1;
+  return check_launch("tlq_gemm_w4a16(skinny)", "w4a16_skinny_lds_kernel") ? 0 : 1;
 }
 
 static thread_local int g_skinny_lds = -1;  // tuning override: 0 = never, 1 = whenever possible, -1 = automatic

@@ -349,7 +349,7 @@ static int launch_decode(const void* A, const void* Wp, const void* scales, cons
   kern<<<dim3(p.grid_x, p.chunks), p.waves * 64, (size_t)p.lds_bytes, st>>>(
       (const T*)A, (const uint8_t*)Wp, (const T*)scales, (const T*)zeros, C, p.chunks > 1 ? partial : nullptr, (int)M, (int)N, (int)K,
       gshift, zero_scalar, out_dtype, tiles, (int)(K / addr::kDecSlice));
-  return check_launch("tlq_gemm_w4a16(decode)") ? 0 : 1;
+  return check_launch("tlq_gemm_w4a16(decode)", "w4a16_decode_kernel") ? 0 : 1;
 }
 
 // partial: fp32 [chunks][M][N] when the plan has more than one chunk (ignored otherwise)
@@ -373,8 +373,9 @@ int gemm_w4a16_decode(const void* A, const void* Wp, const void* scales, const v
   }
 #undef TLQ_DEC
   if (rc) return rc;
-  if (p.chunks > 1) launch_splitk_reduce(partial, C, M, N, p.chunks, out_dtype, st);
-  return check_launch("tlq_gemm_w4a16(decode, reduce)") ? 0 : 1;
+  if (p.chunks == 1) return 0;
+  launch_splitk_reduce(partial, C, M, N, p.chunks, out_dtype, st);
+  return check_launch("tlq_gemm_w4a16(decode, reduce)", "splitk_reduce_kernel") ? 0 : 1;
 }
 
 }  // namespace tlq

@@ -66,12 +66,10 @@ int tlq_gemm_w4a16_noalloc(const void* A, const void* w_packed, const void* scal
   // call then equals tlq_gemm_w4a16_ws with a workspace of TLQ_NOALLOC_SCRATCH_BYTES bytes, which takes what fits).
   int64_t need = tlq_w4a16_workspace_bytes(M, N, K);
   if (need > (int64_t)TLQ_NOALLOC_SCRATCH_BYTES) need = tlq_w4a16_workspace_bytes_min(M, N, K);
-  if (need > (int64_t)TLQ_NOALLOC_SCRATCH_BYTES) {
-    set_error("tlq_gemm_w4a16_noalloc: M=%lld N=%lld K=%lld needs %lld bytes of scratch, the built-in array holds %lld; "
-              "use tlq_gemm_w4a16_ws with a caller-owned workspace",
-              (long long)M, (long long)N, (long long)K, (long long)need, (long long)TLQ_NOALLOC_SCRATCH_BYTES);
-    return 1;
-  }
+  // Not even that: the kernels that need no scratch at all (the fused tile kernel for large M) take the problem, as
+  // tlq_gemm_w4a16_ws does when it is handed no workspace -- a caller who cannot allocate has nowhere else to go.
+  if (need > (int64_t)TLQ_NOALLOC_SCRATCH_BYTES)
+    return tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, algo, nullptr, 0, stream);
   uint8_t* ws = nullptr;
   if (scratch_of_current_device(&ws)) return 1;
   // from here on only `ws`, the device address, stands for the array

@@ -400,7 +400,7 @@ static int launch_panel(const void* A, const void* Wp, const void* scales, const
   const unsigned blocks = (unsigned)((int64_t)p.tiles_m * p.tiles_n * p.split);
   kern<<<blocks, 512, lds_bytes, st>>>((const T*)A, (const uint8_t*)Wp, (const T*)scales, (const T*)zeros, C, partial, (int)M, (int)N,
                                        (int)K, gshift, zero_scalar, out_dtype, p.slice_steps, p.tiles_m, p.tiles_n, band_rows, flag, epoch);
-  return check_launch("tlq_gemm_w4a16(panel)") ? 0 : 1;
+  return check_launch("tlq_gemm_w4a16(panel)", ZM == 0 ? "w4a16_panel_kernel, zero-point tensor folded" : (ZM == 3 ? "w4a16_panel_kernel, unfolded behind the flag" : "w4a16_panel_kernel")) ? 0 : 1;
 }
 
 // partial: fp32 [split][M][N] workspace, needed when the plan has more than one K slice
@@ -430,7 +430,7 @@ int gemm_w4a16_panel(const void* A, const void* Wp, const void* scales, const vo
   if (rc) return rc;
   if (p.split > 1) {
     launch_splitk_reduce(partial, C, M, N, p.split, out_dtype, st);
-    return check_launch("tlq_gemm_w4a16(panel, reduce)") ? 0 : 1;
+    return check_launch("tlq_gemm_w4a16(panel, reduce)", "splitk_reduce_kernel") ? 0 : 1;
   }
   return 0;
 }

@@ -399,7 +399,9 @@ static int launch_stream(const void* A, const void* Wp, const void* scales, cons
   kern<<<dim3(p.n_blocks, p.split, p.m_blocks), 512, lds_bytes, st>>>((const T*)A, (const uint8_t*)Wp, (const T*)scales,
                                                                      (const T*)zeros, C, partial, (int)M, (int)N, (int)K, gshift,
                                                                      zero_scalar, out_dtype, p.slice_steps);
-  return check_launch("tlq_gemm_w4a16(stream)") ? 0 : 1;
+  char detail[64];
+  snprintf(detail, sizeof(detail), "w4a16_stream_kernel, %d activation rows per work-group", 16 * TM);
+  return check_launch("tlq_gemm_w4a16(stream)", detail) ? 0 : 1;
 }
 
 // partial: fp32 [split][M][N] workspace, needed when the plan has more than one K slice
@@ -421,8 +423,9 @@ int gemm_w4a16_stream(const void* A, const void* Wp, const void* scales, const v
 #undef TLQ_STREAM4
 #undef TLQ_STREAM
   if (rc) return rc;
-  if (p.split > 1) launch_splitk_reduce(partial, C, M, N, p.split, out_dtype, st);
-  return check_launch("tlq_gemm_w4a16(stream, reduce)") ? 0 : 1;
+  if (p.split == 1) return 0;
+  launch_splitk_reduce(partial, C, M, N, p.split, out_dtype, st);
+  return check_launch("tlq_gemm_w4a16(stream, reduce)", "splitk_reduce_kernel") ? 0 : 1;
 }
 
 }  // namespace tlq

@@ -15,6 +15,8 @@
 // at least as accurate as multiplying rounded fp16 weights.
 // bf16 path: weights are dequantised element-wise with bfloat16 rounding after each step
 // (bf16 keeps only 8 mantissa bits, so skipping those roundings would be visible).
+#include <type_traits>
+
 #include "tlq_common.h"
 #include "expand8.h"
 #include "gemm_addr.h"
@@ -995,7 +997,7 @@ static int launch_gemv_ring(const void* A, const void* Wp, const void* scales, c
   }
   kern<<<p.blocks, 64 * p.waves, p.lds_bytes, st>>>((const T*)A, (const uint8_t*)Wp, (const T*)scales, (const T*)zeros, C, N, K,
                                                   group_shift, zero_scalar, out_dtype, p.rows_per_block);
-  return check_launch("tlq_gemm_w4a16(gemv)") ? 0 : 1;
+  return check_launch("tlq_gemm_w4a16(gemv)", "gemv_w4a16_ring_kernel") ? 0 : 1;
 }
 
 // 1 (default): the ring kernel where it applies; 0: never
@@ -1084,7 +1086,7 @@ static int dispatch_gemv_rows(const void* A, const void* Wp, const void* scales,
 #undef TLQ_LONG_CASE
   }
 #undef TLQ_ROWS_CASE
-  return check_launch("tlq_gemm_w4a16(gemv)") ? 0 : 1;
+  return check_launch("tlq_gemm_w4a16(gemv)", std::is_same<T, half_t>::value ? "gemv_w4a16_f16_rows_kernel" : "gemv_w4a16_bf16_rows_kernel") ? 0 : 1;
 }
 
 int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch, int64_t M,

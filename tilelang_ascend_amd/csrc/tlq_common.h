@@ -3,14 +3,16 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 
 #include "tlq.h"
+#include "tlq_debug.h"
 
 namespace tlq {
 
 // ---- error reporting (thread local, read back through tlq_last_error) -------------------
 void set_error(const char* fmt, ...);
-bool check_launch(const char* what);
+bool check_launch(const char* what, const char* detail = nullptr);
 
 #define TLQ_REQUIRE(cond, ...)      \
   do {                              \

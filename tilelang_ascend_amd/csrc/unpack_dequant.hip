@@ -137,7 +137,7 @@ static int launch_dequant(const void* wp, const void* scales, const void* zeros,
     dequant_w4_scalar<T><<<grid_for(N * K), 256, 0, st>>>((const uint8_t*)wp, (const T*)scales, (const T*)zeros, (T*)out,
                                                          N, K, (int)group, zero_scalar);
   }
-  return check_launch("tlq_dequant_w4") ? 0 : 1;
+  return check_launch("tlq_dequant_w4", "dequant_w4_vec8") ? 0 : 1;
 }
 
 }  // namespace tlq

@@ -27,7 +27,7 @@ _PASS_CONFIGS = {
 }
 _SIGN_MODES = {"unsigned": _abi.U4, "twos": _abi.S4_TWOS, "offset8": _abi.S4_OFFSET8, "offset7": _abi.S4_OFFSET7}
 _ALGOS = {"auto": _abi.ALGO_AUTO, "gemv": _abi.ALGO_GEMV, "mfma": _abi.ALGO_MFMA, "skinny": _abi.ALGO_SKINNY,
-          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM, "decode": _abi.ALGO_DECODE}
+          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM, "decode": _abi.ALGO_DECODE, "panel": _abi.ALGO_PANEL}
 # arrangement of the 4-bit fields in each 32-bit word: general_compress order, or interleave_weight(target float16)
 _LAYOUTS = {"plain": _abi.W_PLAIN, "interleaved": _abi.W_INTERLEAVED_F16}
 
@@ -132,7 +132,7 @@ def fp16_gemm(M: int, N: int, K: int, block_M: int, block_N: int, block_K: int):
         # few activation rows: K slices with their fp32 matrices in a workspace (allocated per call, like the
         # reference's workspace_idx buffers); 0 bytes for every other shape
         ws_bytes = lib.tlq_f16_workspace_bytes(1, M, N, K)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device) if ws_bytes else None
+        ws = _abi.scratch(ws_bytes, A.device, stream)
         _abi.check(lib.tlq_gemm_f16_ws(_abi.ptr(A), _abi.ptr(B), _abi.ptr(C), _abi.ptr(ws), ws_bytes, 1, M, N, K, _abi.F16,
                                        _abi.F16, _abi.B_KN, stream))
 
@@ -170,9 +170,12 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
     algo: "auto" | "gemv" (split-K wavefront kernel, M <= 16) | "decode" (M <= 32, K % 256 == 0: persistent work-groups with the
     activations in registers: what "auto" does for 3 <= M <= 16) | "skinny" (M <= 64) | "mfma" (LDS-staged MFMA kernel)
     | "stream" (wavefront-private packed weights dequantised in registers, 17 <= M <= 512: what "auto" does up to
-    M = 256) | "two_pass" (dequantise into a workspace, then the plain GEMM: what "auto" does above).  A workspace
+    M = 384) | "panel" (large M in one launch: packed weights copied to LDS as they are and dequantised on the MFMA operand
+    read; what "auto" does from 513 to 2048 rows where its work-groups fill the machine) | "two_pass" (dequantise into a
+    workspace, then the plain GEMM: what "auto" does otherwise above 512 rows).  A workspace
     (split-K partial sums or the [N, K] dequantised weights) is taken from torch's stream-ordered allocator on every
-    call, as the reference allocates its workspace_idx buffers per call, so launches on different streams do not share one.
+    call, as the reference allocates its workspace_idx buffers per call, so launches on different streams do not share one;
+    when the launch stream (forward(stream=...)) is not torch's current stream the block is recorded on it (_abi.scratch).
     weight_layout: "plain" (general_compress order) or "interleaved" (B_packed went through interleave_weight for the
     float16 target, e.g. quantize.gpu.pack_int4(..., interleave="float16")); interleaved weights are read by the "decode" and
     "stream" kernels and the two passes, with results bit-identical to the plain layout.
@@ -216,12 +219,12 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
         lib = _abi.load()
         ws = None
         ws_bytes = 0
-        if algo in ("auto", "two_pass", "stream", "decode"):
+        if algo in ("auto", "two_pass", "stream", "decode", "panel"):
             ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
             if algo == "two_pass" or (layout_code != _abi.W_PLAIN and algo == "auto" and M > 256):
                 ws_bytes = max(ws_bytes, N * K * 2)
         if ws_bytes:
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
+            ws = _abi.scratch(ws_bytes, A.device, stream)
         with _abi.tuning(w4a16_tile=tile, gemv=gemv_tuning, skinny=skinny_tuning):
             _abi.check(lib.tlq_gemm_w4a16_layout_ws(_abi.ptr(A), _abi.ptr(Bp), _abi.ptr(S), _abi.ptr(Z), _abi.ptr(C), M, N, K,
                                                     group_size, zero_scalar, tin, tout, algo_code, layout_code, _abi.ptr(ws),

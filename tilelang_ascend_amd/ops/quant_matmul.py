@@ -45,7 +45,7 @@ def w8a8_launch(A, B, scale_a, scale_b, C, batch, M, N, K, n_scale_b, b_layout, 
     allocated."""
     lib = _abi.load()
     ws_bytes = lib.tlq_w8a8_workspace_bytes(batch, M, N, K)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device) if ws_bytes else None
+    ws = _abi.scratch(ws_bytes, A.device, stream)
     _abi.check(lib.tlq_gemm_w8a8_ws(_abi.ptr(A), _abi.ptr(B), _abi.ptr(scale_a), _abi.ptr(scale_b), _abi.ptr(C), _abi.ptr(ws),
                                     ws_bytes, batch, M, N, K, n_scale_b, b_layout, out_code, stream))
 

@@ -11,3 +11,4 @@ from .quantization import (  # noqa: F401
     _tir_u8_to_f8_e4m3_to_f16,
 )
 from .utils import gen_quant4, general_compress, interleave_weight  # noqa: F401
+from .pack_io import load_packed, save_packed  # noqa: F401  (no counterpart in the reference: the on-disk form of repacked weights)
