@@ -82,6 +82,12 @@ enum {
                       * zero tensors.  Workspace: the fp32 partial tiles where K is cut into slices, plus 16 bytes with a zero-point
                       * tensor (a flag word: a second launch redoes the product with the unfolded dequantiser when a zero point
                       * turns out not to be a small integer) */
+  ,
+  TLQ_ALGO_PANEL256 = 8 /* the same with 256 activation rows x 256 weight rows per work-group on four wavefronts that each own a
+                         * full register file: per MFMA half the dequantiser arithmetic and half the LDS operand traffic; scales
+                         * and zero points are gathered into registers, so any number of groups per row and 2-byte aligned
+                         * scale / zero tensors will do.  K % 128 == 0, M % 4 == 0, N % 16 == 0, power-of-two group >= 32; workspace
+                         * as for TLQ_ALGO_PANEL */
 };
 
 int tlq_abi_version(void);

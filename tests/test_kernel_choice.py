@@ -46,8 +46,8 @@ def cases():
         (512, 4096, 2048, 128, _abi.ALGO_STREAM),  # 512 rows on 4096 weight rows: the tile kernels would fill half the machine
         (384, 10240, 2048, 128, _abi.ALGO_STREAM),  # three blocks of 128 activation rows: streaming kernel whatever the tile kernels' fill
         (512, 8192, 1024, 128, _abi.ALGO_STREAM),   # four blocks, 32 x 4 x 1 = 128 streaming work-groups: they fit the machine at once
-        (768, 5120, 5120, 128, _abi.ALGO_PANEL),    # above 512 rows where the panel kernel's work-groups fill the machine: 6 x 10 tiles x 3 K slices
-        (2048, 4096, 2048, 128, _abi.ALGO_TWO_PASS),  # 128 panel tiles and too few steps to cut: half the CUs idle, the two passes keep it
+        (768, 8192, 4096, 128, _abi.ALGO_PANEL256),  # above 512 rows where the 256-row panel kernel's work-groups fill the machine: 3 x 32 tiles x 2 K slices on 256 CUs
+        (2048, 4096, 2048, 128, _abi.ALGO_TWO_PASS),  # 8 x 16 panel tiles and too few steps to cut: half the CUs idle, the two passes keep it
         (224, 28672, 8192, 128, _abi.ALGO_MFMA),    # largest matrices from 192 rows on: tile kernel over two long K slices
     ]
 

@@ -72,7 +72,7 @@ struct Expand8<half_t, FOLD, LAYOUT> {
     __device__ __forceinline__ void pin(int i) {
       if (i == 0) asm volatile("" : "+v"(q0), "+v"(q1));
       if (i == 1) asm volatile("" : "+v"(f0), "+v"(f1));
-      if (i == 2) asm volatile("" : "+v"(f2), "+v"(f3));
+      if (i == 2) asm volatile("" : "+v"(f0), "+v"(f1), "+v"(f2), "+v"(f3));  // (all four: piece 3 packs both words)
       if (i == 3) asm volatile("" : "+v"(a), "+v"(b));
     }
   };
@@ -179,7 +179,7 @@ struct Expand8<bf16_t, FOLD, LAYOUT> {
     __device__ __forceinline__ void pin(int i) {
       if (i == 0) asm volatile("" : "+v"(q0), "+v"(q1));
       if (i == 1) asm volatile("" : "+v"(f0), "+v"(f1));
-      if (i == 2) asm volatile("" : "+v"(f2), "+v"(f3));
+      if (i == 2) asm volatile("" : "+v"(f0), "+v"(f1), "+v"(f2), "+v"(f3));  // (all four: piece 3 packs both words)
       if (i == 3) asm volatile("" : "+v"(a), "+v"(b));
     }
   };

@@ -201,6 +201,66 @@ __host__ __device__ inline uint32_t panel_sc_voff(int lane, int wave, int n0, in
   return ((uint32_t)n * (uint32_t)groups) * 2u;
 }
 
+// ---- panel kernel with 256 activation rows (gemm_w4a16_panel256.hip): four wavefronts, 256 x 256 outputs per work-group
+// A ring slot is the activation tile [256 rows][256 B] (sixteen 16-row tiles: direct load I = 4 j + wave, j = 0 .. 15, rows
+// 4 I .. 4 I + 3) followed by the four wavefronts' packed weights, four [16 rows][64 B] tiles each.  Scales and zero
+// points are gathered into registers: lane (row r16, k-group q) reads, for weight tile tn, the 2-byte value of row
+// 64 wave + 16 tn + r16 and of the group its 32 values of the step lie in.
+constexpr int kPanel2TM = 16, kPanel2TN = 4;
+constexpr uint32_t kPanel2ATile = 16 * kPanel2TM * 256;
+constexpr uint32_t kPanel2Slot = kPanel2ATile + 4 * kPanel2TN * 1024;
+__host__ __device__ inline uint32_t panel2_a_lds(int wave, int j) { return (uint32_t)(j * 4 + wave) * 1024u; }
+__host__ __device__ inline uint32_t panel2_w_lds(int wave, int tn) { return kPanel2ATile + (uint32_t)(wave * kPanel2TN + tn) * 1024u; }
+__host__ __device__ inline int64_t panel2_a_block(int wave, int j, int m0, int M, int K) {
+  int m = m0 + 4 * (j * 4 + wave);
+  m = m + 4 <= M ? m : M - 4;
+  return (int64_t)m * K * 2;
+}
+// byte offsets into a scale / zero-point tensor [N][groups] of 2-byte values: row block of the tile (uniform), the group of
+// step `step` of the matrix (uniform), the lane's row and -- for groups of fewer than 128 values -- its k-group's group
+__host__ __device__ inline int64_t panel2_sc_block(int wave, int tn, int n0, int N, int groups) {
+  int n = n0 + wave * (16 * kPanel2TN) + tn * 16;
+  n = n + 16 <= N ? n : N - 16;
+  return (int64_t)n * groups * 2;
+}
+__host__ __device__ inline int64_t panel2_sc_step(int step, int gshift) { return (((int64_t)step << 7) >> gshift) * 2; }
+__host__ __device__ inline uint32_t panel2_sc_lane(int lane, int groups, int gshift) {
+  const int r16 = lane & 15, q = lane >> 4;
+  return (uint32_t)(r16 * groups + ((q << 5) >> gshift)) * 2u;
+}
+
+// The kernel's schedule of a step of 64 slots (a slot = one activation tile against the wavefront's four weight tiles)
+// for its three kinds of loads, and the two waits that follow from it.  Loads retire in issue order, so a wait for "at
+// most n outstanding" stands for "all but the youngest n have landed".
+//   slot  0 .. 15: one load each of the activation tile of step s + 1
+//   slot 16 .. 23: one gather each of the scales / zero points of step s + 2
+//   slot 58 .. 61: one load each of the wavefront's packed weights of step s + 2
+// The wait in front of slot kPanel2WaitWSlot needs the packed weights of step s + 1 (issued one step earlier); the wait in
+// front of slot kPanel2BarrierSlot needs the activation tile and the gathers issued in this step (the gathers are
+// compiler-visible loads whose wait the compiler writes itself, for everything issued before: no load may be
+// younger there), and the barrier behind it separates the last operand read of this step's tile (slot
+// kPanel2BarrierSlot - 1 reads kPanel2Ahead - 1 slots ahead) from the first read of the next.
+enum { kPanel2LoadNone = 0, kPanel2LoadA, kPanel2LoadScale, kPanel2LoadW };
+constexpr int kPanel2Slots = 4 * kPanel2TM, kPanel2Ahead = 8;
+constexpr int kPanel2WaitWSlot = 32, kPanel2BarrierSlot = kPanel2Slots - (kPanel2Ahead - 1);
+// Packed word ks + 2 (of step s + 1 from phase 2 on) of weight tile wt is read in slot kPanel2WordSlot + wt of phase ks;
+// the dequantiser constants of tile tn for step s + 1 are made in slot kPanel2ExpanderSlot + 4 tn, between the last piece of
+// expansion that uses the old ones (slot 32 + 4 tn + 3) and the first that uses the new ones (slot 48 + 4 tn).
+constexpr int kPanel2WordSlot = 8, kPanel2ExpanderSlot = 40, kPanel2WSlot = kPanel2BarrierSlot + 1;
+__host__ __device__ constexpr int panel2_slot_load(int t) {
+  return t < 16 ? kPanel2LoadA : t < 24 ? kPanel2LoadScale : (t >= kPanel2WSlot && t < kPanel2WSlot + kPanel2TN) ? kPanel2LoadW : kPanel2LoadNone;
+}
+__host__ __device__ constexpr int panel2_slot_load_index(int t) { return t < 16 ? t : t < 24 ? t - 16 : t - kPanel2WSlot; }
+__host__ __device__ constexpr int panel2_loads_in(int t0, int t1) {  // loads issued in slots t0 .. t1 - 1 of one step
+  int n = 0;
+  for (int t = t0; t < t1; ++t) n += panel2_slot_load(t) != kPanel2LoadNone;
+  return n;
+}
+constexpr int kPanel2WaitW = panel2_loads_in(kPanel2WSlot + kPanel2TN, kPanel2Slots) + panel2_loads_in(0, kPanel2WaitWSlot);
+constexpr int kPanel2WaitA = panel2_loads_in(24, kPanel2BarrierSlot);
+static_assert(kPanel2WaitW == 24 && kPanel2WaitA == 0 && kPanel2BarrierSlot == 57 && kPanel2WSlot + kPanel2TN <= kPanel2Slots,
+              "the 256-row panel kernel's waits");
+
 // ---- decode kernel (1 .. 32 activation rows): wavefront w of a work-group owns values 256 s .. 256 s + 255 of K
 // (s = chunk * waves + w) for every weight row.  A work item is one 16-row weight tile: two [16 rows][64 B] packed
 // pieces (k-blocks kb = 0, 1 of the slice, 128 values each) plus the scales / zero points of the 16 rows for the

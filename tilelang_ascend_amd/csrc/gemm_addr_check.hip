@@ -431,6 +431,176 @@ int check_panel(int64_t M, int64_t N, int64_t K, int64_t group, int slice_steps)
   return 0;
 }
 
+// Panel kernel with 256 activation rows: 256 x 256 outputs per work-group of four wavefronts, steps of 128 values of K in
+// two ring slots, scales / zero points gathered into registers.  Walks every work-group tile: global extents of the
+// activation, weight and scale loads over every step of every slice (and of the steps past the end, which repeat the
+// last), LDS extents and coverage of a slot, agreement of the landing cells with the operand reads.
+int check_panel256(int64_t M, int64_t N, int64_t K, int64_t group, int slice_steps) {
+  CHECK_OR_FAIL(M >= 4 && N >= 16 && M % 4 == 0 && N % 16 == 0 && K >= 128 && K % 128 == 0, "panel256: bad shape");
+  CHECK_OR_FAIL(group >= 32 && (group & (group - 1)) == 0 && K % group == 0, "panel256: group %lld on K %lld", (long long)group, (long long)K);
+  const int64_t groups = K / group;
+  int gshift = 0;
+  while (((int64_t)1 << gshift) < group) ++gshift;
+  CHECK_OR_FAIL(N * (K / 2) < ((int64_t)1 << 32) && M * K * 2 < ((int64_t)1 << 32) && N * groups * 2 < ((int64_t)1 << 32),
+                "panel256: a matrix spans 4 GiB or more");
+  const int steps_total = (int)(K / 128);
+  CHECK_OR_FAIL(slice_steps >= 1 && (slice_steps * 128 % group == 0 || slice_steps >= steps_total), "panel256: slices of %d steps are not whole groups", slice_steps);
+  const int TM = addr::kPanel2TM, TN = addr::kPanel2TN;
+  const int64_t w_extent = N * (K / 2), a_extent = M * K * 2, s_extent = N * groups * 2;
+  CHECK_OR_FAIL(2 * addr::kPanel2Slot <= 160 * 1024, "panel256: %u bytes of LDS", 2 * addr::kPanel2Slot);
+  std::vector<int> cell(addr::kPanel2Slot / 16);
+  for (int64_t m0 = 0; m0 < M; m0 += 16 * TM)
+    for (int64_t n0 = 0; n0 < N; n0 += 4 * 16 * TN) {
+      std::fill(cell.begin(), cell.end(), -1);
+      for (int wave = 0; wave < 4; ++wave) {
+        for (int j = 0; j < 16; ++j) {
+          const uint32_t l0 = addr::panel2_a_lds(wave, j);
+          const int I = j * 4 + wave;
+          for (int lane = 0; lane < 64; ++lane) {
+            const int64_t voff = addr::panel2_a_block(wave, j, (int)m0, (int)M, (int)K) + addr::panel_a_lane(lane, (int)K) + addr::panel_a_chunk(lane, wave);
+            CHECK_OR_FAIL(voff >= 0 && voff + (int64_t)(steps_total - 1) * 256 + 16 <= a_extent, "panel256: activation load at %lld of %lld",
+                          (long long)voff, (long long)a_extent);
+            const uint32_t at = l0 / 16 + lane;
+            CHECK_OR_FAIL(at < addr::kPanel2ATile / 16 && cell[at] == -1, "panel256: activation cell %u written twice or outside the tile", at);
+            const int row = addr::sa_row(lane, I), chunk = addr::sa_chunk(lane, I);
+            CHECK_OR_FAIL((int)at == row * 16 + (lane & 15), "panel256: activation lane lands on cell %u, not on its row", at);
+            if (m0 + 4 * I + 4 <= M)
+              CHECK_OR_FAIL(voff == ((int64_t)(m0 + row) * K) * 2 + chunk * 16, "panel256: activation lane %d of load %d fetches the wrong bytes", lane, I);
+            cell[at] = row * 16 + chunk;
+          }
+        }
+        for (int tn = 0; tn < TN; ++tn) {
+          const uint32_t l0 = addr::panel2_w_lds(wave, tn);
+          for (int lane = 0; lane < 64; ++lane) {
+            const int64_t voff = addr::panel_w_block(wave, tn, (int)n0, (int)N, (int)K) + addr::panel_w_lane(lane, (int)K);
+            CHECK_OR_FAIL(voff >= 0 && voff + (int64_t)(steps_total - 1) * 64 + 16 <= w_extent, "panel256: weight load at %lld of %lld",
+                          (long long)voff, (long long)w_extent);
+            if (n0 + wave * 64 + tn * 16 + 16 <= N)
+              CHECK_OR_FAIL(voff == (int64_t)(n0 + wave * 64 + tn * 16 + addr::sw_row(lane)) * (K / 2) + addr::sw_piece(lane) * 16, "panel256: weight lane %d fetches the wrong bytes", lane);
+            const uint32_t at = l0 / 16 + lane;
+            CHECK_OR_FAIL(at >= addr::kPanel2ATile / 16 && at < addr::kPanel2Slot / 16 && cell[at] == -1, "panel256: weight cell %u written twice or outside the slot", at);
+            cell[at] = addr::sw_row(lane) * 4 + addr::sw_piece(lane);
+          }
+          for (int lane = 0; lane < 64; ++lane) {
+            const uint32_t off = l0 + addr::sw_frag_off(lane);
+            CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= addr::kPanel2Slot, "panel256: weight operand read at %u", off);
+            CHECK_OR_FAIL(cell[off / 16] == (lane & 15) * 4 + (lane >> 4), "panel256: weight operand read of lane %d finds cell %d", lane, cell[off / 16]);
+          }
+          // the gathers of scales / zero points: the value of (row, group of the lane's 32 values) for every step
+          for (int lane = 0; lane < 64; ++lane)
+            for (int step = 0; step < steps_total; ++step) {
+              const int64_t o = addr::panel2_sc_block(wave, tn, (int)n0, (int)N, (int)groups) + addr::panel2_sc_step(step, gshift) + addr::panel2_sc_lane(lane, (int)groups, gshift);
+              CHECK_OR_FAIL(o >= 0 && o + 2 <= s_extent && o % 2 == 0, "panel256: scale gather at %lld of %lld", (long long)o, (long long)s_extent);
+              if (n0 + wave * 64 + tn * 16 + 16 <= N) {
+                const int64_t row = n0 + wave * 64 + tn * 16 + (lane & 15);
+                const int64_t g = ((int64_t)step * 128 + 32 * (lane >> 4)) / group;
+                CHECK_OR_FAIL(o == (row * groups + g) * 2, "panel256: scale gather of lane %d at step %d reads group %lld of row %lld", lane, step,
+                              (long long)((o / 2) % groups), (long long)((o / 2) / groups));
+              }
+            }
+        }
+      }
+      for (uint32_t c = 0; c < addr::kPanel2Slot / 16; ++c) CHECK_OR_FAIL(cell[c] >= 0, "panel256: cell %u of the slot never written", c);
+      for (int t = 0; t < TM; ++t)
+        for (int ks = 0; ks < 4; ++ks)
+          for (int lane = 0; lane < 64; ++lane) {
+            const uint32_t off = addr::sa_frag_off(lane, t, ks);
+            CHECK_OR_FAIL(off == ((addr::sa_frag_off(lane, 0, 0) ^ (uint32_t)(ks << 4)) + (uint32_t)(t * 16 * 256)), "panel256: the k-step offset is not an exclusive-or");
+            CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= addr::kPanel2ATile, "panel256: activation operand read at %u", off);
+            const int want = (t * 16 + (lane & 15)) * 16 + 4 * (lane >> 4) + ks;
+            CHECK_OR_FAIL(cell[off / 16] == want, "panel256: activation operand read (lane %d, k-step %d) finds cell %d, expects %d", lane, ks, cell[off / 16], want);
+          }
+    }
+  return 0;
+}
+
+// The 256-row panel kernel's schedule, played through for one wavefront over `steps` steps: loads issued per
+// addr::panel2_slot_load retire in issue order, the two waits leave addr::kPanel2WaitW / kPanel2WaitA of them outstanding;
+// every LDS read must find its data landed (for the shared activation tile: landed and behind a barrier), every load
+// into a ring slot must come after the last read of what the slot held (for the shared tile: with a barrier between),
+// and the dequantiser constants of a step must be made from that step's gathers.  (The wait counts are arguments so that
+// a test can show that wrong ones fail.)
+int check_panel256_schedule(int steps, int wait_w, int wait_a) {
+  CHECK_OR_FAIL(steps >= 1 && steps <= 64 && wait_w >= 0 && wait_a >= 0, "panel256 schedule: bad arguments");
+  struct Load { int kind, step; };
+  std::vector<Load> fifo;  // oldest first
+  const int S = steps + 4;
+  std::vector<int> landed_a(S, 0), landed_w(S, 0), landed_sc(S, 0), published_a(S, 0);
+  std::vector<int64_t> last_read_a(S, -1), last_read_w(S, -1), barrier_times;
+  int64_t now = -1;
+  int pinned_sc = -1;
+  auto issue = [&](int kind, int step) { fifo.push_back(Load{kind, step}); };
+  auto wait = [&](size_t n) {
+    while (fifo.size() > n) {
+      const Load l = fifo.front();
+      fifo.erase(fifo.begin());
+      (l.kind == addr::kPanel2LoadA ? landed_a : l.kind == addr::kPanel2LoadW ? landed_w : landed_sc)[l.step]++;
+    }
+  };
+  auto barrier = [&]() {
+    for (int st = 0; st < S; ++st) published_a[st] = landed_a[st] == 16;  // (every wavefront has waited for its own part)
+    barrier_times.push_back(now);
+  };
+  auto barrier_between = [&](int64_t t0, int64_t t1) {  // a barrier at a time in (t0, t1]
+    for (int64_t b : barrier_times)
+      if (b > t0 && b <= t1) return true;
+    return false;
+  };
+  // prologue (as the kernel's)
+  for (int i = 0; i < 8; ++i) issue(addr::kPanel2LoadScale, 0);
+  for (int i = 0; i < 4; ++i) issue(addr::kPanel2LoadW, 0);
+  for (int i = 0; i < 16; ++i) issue(addr::kPanel2LoadA, 0);
+  wait(0);  // (the compiler's own, at the first touch of the gathered values)
+  CHECK_OR_FAIL(landed_sc[0] == 8, "panel256 schedule: the first gathers have not landed behind the prologue's first wait");
+  for (int i = 0; i < 8; ++i) issue(addr::kPanel2LoadScale, 1);
+  for (int i = 0; i < 4; ++i) issue(addr::kPanel2LoadW, 1);
+  wait(0);
+  CHECK_OR_FAIL(landed_sc[1] == 8 && landed_w[0] == 4 && landed_a[0] == 16, "panel256 schedule: the prologue's second wait leaves step 0 incomplete");
+  pinned_sc = 1;
+  barrier();
+  for (int s = 0; s < steps; ++s)
+    for (int t = 0; t < addr::kPanel2Slots; ++t) {
+      now = (int64_t)s * addr::kPanel2Slots + t;
+      const int ks = t / addr::kPanel2TM, tm = t % addr::kPanel2TM;
+      if (t == addr::kPanel2WaitWSlot) {
+        wait((size_t)wait_w);
+        CHECK_OR_FAIL(landed_w[s + 1] == 4, "panel256 schedule: step %d: the next step's packed weights have not landed at their wait", s);
+      }
+      if (t >= addr::kPanel2ExpanderSlot && t < addr::kPanel2ExpanderSlot + 4 * addr::kPanel2TN && (t - addr::kPanel2ExpanderSlot) % 4 == 0)
+        CHECK_OR_FAIL(pinned_sc == s + 1, "panel256 schedule: step %d slot %d: constants made from the gathers of step %d", s, t, pinned_sc);
+      if (t == addr::kPanel2BarrierSlot) {
+        wait((size_t)wait_a);
+        CHECK_OR_FAIL(landed_a[s + 1] == 16 && landed_sc[s + 2] == 8, "panel256 schedule: step %d: activation tile or gathers not landed at the barrier", s);
+        pinned_sc = s + 2;
+        barrier();
+      }
+      // behind MFMA 1: the slot's load, the operand read kPanel2Ahead - 1 slots on, a packed word
+      const int kind = addr::panel2_slot_load(t);
+      if (kind == addr::kPanel2LoadA) {
+        if (s >= 1)
+          CHECK_OR_FAIL(barrier_between(last_read_a[s - 1], now - 1), "panel256 schedule: step %d slot %d: the tile of step %d may still be read", s, t, s - 1);
+        issue(kind, s + 1);
+      } else if (kind == addr::kPanel2LoadW) {
+        CHECK_OR_FAIL(last_read_w[s] >= 0 && last_read_w[s] < now, "panel256 schedule: step %d slot %d: this step's words are not all read", s, t);
+        CHECK_OR_FAIL(ks >= 2, "panel256 schedule: packed weights overwritten before the phase that reads this step's last word has passed");
+        CHECK_OR_FAIL(t > addr::kPanel2BarrierSlot, "panel256 schedule: a direct load in flight where the compiler waits for the gathers");
+        issue(kind, s + 2);
+      } else if (kind == addr::kPanel2LoadScale) {
+        issue(kind, s + 2);
+      }
+      const int at = t + addr::kPanel2Ahead - 1;
+      const int a_step = at < addr::kPanel2Slots ? s : s + 1;
+      CHECK_OR_FAIL(published_a[a_step], "panel256 schedule: step %d slot %d reads an operand of step %d before the barrier that publishes it", s, t, a_step);
+      last_read_a[a_step] = now;
+      if (tm >= addr::kPanel2WordSlot && tm < addr::kPanel2WordSlot + addr::kPanel2TN) {
+        const int w_step = ks < 2 ? s : s + 1;
+        CHECK_OR_FAIL(landed_w[w_step] == 4, "panel256 schedule: step %d slot %d reads a word of step %d that has not landed", s, t, w_step);
+        last_read_w[w_step] = now;
+      }
+    }
+  return 0;
+}
+
 // The ring: step s occupies slot s % D; at the top of step s the wavefront waits until only `younger` steps' loads are
 // outstanding, passes the barrier, and then issues step s + D - 1 into the slot of step s - 1.
 int check_stream_ring(int steps, int D) {
@@ -727,6 +897,17 @@ int tlq_debug_check_stream_addressing(int64_t M, int64_t N, int64_t K, int activ
   for (int steps = 1; steps <= 40; ++steps)
     if (int rc = check_stream_ring(steps, ring_depth)) return rc;
   return 0;
+}
+
+int tlq_debug_check_panel256_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int slice_steps) {
+  if (int rc = check_panel256(M, N, K, group, slice_steps)) return rc;
+  for (int steps : {1, 2, 3, 4, 7})
+    if (int rc = check_panel256_schedule(steps, addr::kPanel2WaitW, addr::kPanel2WaitA)) return rc;
+  return 0;
+}
+
+int tlq_debug_check_panel256_schedule(int steps, int wait_w, int wait_a) {
+  return check_panel256_schedule(steps, wait_w < 0 ? addr::kPanel2WaitW : wait_w, wait_a < 0 ? addr::kPanel2WaitA : wait_a);
 }
 
 int tlq_debug_check_panel_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int slice_steps) {

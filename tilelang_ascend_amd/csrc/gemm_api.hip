@@ -56,7 +56,16 @@ int gemm_w4a16_panel(const void* A, const void* Wp, const void* scales, const vo
                      int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const PanelPlan& p, float* partial,
                      uint32_t* flag, hipStream_t st);
 extern thread_local int g_panel_slice_steps;
-thread_local int g_w4a16_panel = 0;  // tlq_tune_w4a16_panel: 1 = the panel kernel is never picked automatically
+thread_local int g_w4a16_panel = 0;  // tlq_tune_w4a16_panel: non-zero = no panel kernel is picked automatically
+struct Panel2Plan {
+  bool ok;
+  int tiles_m, tiles_n, split, slice_steps;
+};
+Panel2Plan w4a16_panel256_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus);
+int gemm_w4a16_panel256(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N, int64_t K,
+                        int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const Panel2Plan& p, float* partial,
+                        uint32_t* flag, hipStream_t st);
+extern thread_local int g_panel2_slice_steps;
 
 struct DecodePlan {
   bool ok;
@@ -102,12 +111,22 @@ void tlq_tune_gemm_tile(int tile) { tlq::g_gemm_f16_tile = (tile == 128 || tile 
 void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
 void tlq_tune_w4a16_stream_slice(int steps) { tlq::g_stream_slice_steps = steps; }
 void tlq_tune_w4a16_decode(int on) { tlq::g_w4a16_decode = on != 0; }
-void tlq_tune_w4a16_panel(int mode) { tlq::g_w4a16_panel = mode == 1 ? 1 : 0; }
-void tlq_tune_w4a16_panel_slice(int steps) { tlq::g_panel_slice_steps = steps < 0 ? 0 : steps; }
+void tlq_tune_w4a16_panel(int mode) { tlq::g_w4a16_panel = mode != 0 ? 1 : 0; }
+void tlq_tune_w4a16_panel_slice(int steps) { tlq::g_panel_slice_steps = tlq::g_panel2_slice_steps = steps < 0 ? 0 : steps; }
 
 int tlq_debug_panel_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
   if (!(M >= 1 && N >= 1 && K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return 0;
   const PanelPlan p = w4a16_panel_plan(M, N, K, group, cus);
+  if (plan_out) {
+    int64_t* o = (int64_t*)plan_out;
+    o[0] = p.tiles_m, o[1] = p.tiles_n, o[2] = p.split, o[3] = p.slice_steps;
+  }
+  return p.ok ? 1 : 0;
+}
+
+int tlq_debug_panel256_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
+  if (!(M >= 1 && N >= 1 && K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return 0;
+  const Panel2Plan p = w4a16_panel256_plan(M, N, K, group, cus);
   if (plan_out) {
     int64_t* o = (int64_t*)plan_out;
     o[0] = p.tiles_m, o[1] = p.tiles_n, o[2] = p.split, o[3] = p.slice_steps;
@@ -237,9 +256,15 @@ static int64_t panel_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   for (int64_t group = 32; group <= 1024; group *= 2) {
     if (K % group != 0) continue;
     const PanelPlan pp = w4a16_panel_plan(M, N, K, group, cu_count_or_default());
-    if (!pp.ok) continue;
-    const int64_t b = (pp.split > 1 ? (int64_t)pp.split * M * N * 4 : 0) + 16;
-    if (b > need) need = b;
+    if (pp.ok) {
+      const int64_t b = (pp.split > 1 ? (int64_t)pp.split * M * N * 4 : 0) + 16;
+      if (b > need) need = b;
+    }
+    const Panel2Plan p2 = w4a16_panel256_plan(M, N, K, group, cu_count_or_default());
+    if (p2.ok) {
+      const int64_t b = (p2.split > 1 ? (int64_t)p2.split * M * N * 4 : 0) + 16;
+      if (b > need) need = b;
+    }
   }
   return need;
 }
@@ -267,6 +292,15 @@ int64_t tlq_w4a16_workspace_bytes_min(int64_t M, int64_t N, int64_t K) {
   return M >= kTwoPassMinM ? N * K * 2 : 0;
 }
 
+// The automatic choice takes the 256-row panel kernel where the last round of its work-groups fills 0.55 of the CUs or more.
+static bool panel256_fills(int64_t M, int64_t N, int64_t K, int64_t group) {
+  const int64_t cus_now = cu_count_or_default();
+  const Panel2Plan pp = w4a16_panel256_plan(M, N, K, group, (int)cus_now);
+  if (!pp.ok) return false;
+  const int64_t wgs = (int64_t)pp.tiles_m * pp.tiles_n * pp.split;
+  return (double)wgs / (double)(ceil_div(wgs, cus_now) * cus_now) >= 0.55;
+}
+
 // The panel kernel (large M, one launch, weights dequantised on the operand read).  Returns -1 when it does not take the
 // problem (nothing launched, no error set), else the launch's return code.
 static int try_panel(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
@@ -288,10 +322,37 @@ static int try_panel(const void* A, const void* w_packed, const void* scales, co
                           (float*)workspace, zeros ? (uint32_t*)((uint8_t*)workspace + part_bytes) : nullptr, (hipStream_t)stream);
 }
 
+// The 256-row panel kernel: the same contract.
+static int try_panel256(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                        int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, void* workspace,
+                        int64_t workspace_bytes, void* stream) {
+  if (!(M >= 1 && N >= 1 && K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return -1;
+  const Panel2Plan pp = w4a16_panel256_plan(M, N, K, group, cu_count_or_default());
+  if (!pp.ok) return -1;
+  const bool args_ok = A && w_packed && C && aligned16(A) && aligned16(w_packed) && aligned16(C) && ((uintptr_t)scales & 1) == 0 &&
+                       ((uintptr_t)zeros & 1) == 0 && (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) &&
+                       (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) && (M * N) % 4 == 0 &&
+                       fits32(M, K * 2) && fits32(N, K / 2) && fits32(N, (K / group) * 2);
+  if (!args_ok) return -1;
+  const int64_t part_bytes = pp.split > 1 ? (int64_t)pp.split * M * N * 4 : 0;
+  const int64_t need = part_bytes + (zeros ? 16 : 0);
+  if (need > 0 && !(workspace && aligned16(workspace) && workspace_bytes >= need)) return -1;
+  return gemm_w4a16_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, pp,
+                             (float*)workspace, zeros ? (uint32_t*)((uint8_t*)workspace + part_bytes) : nullptr, (hipStream_t)stream);
+}
+
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
-  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_PANEL, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_PANEL256, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  if (algo == TLQ_ALGO_PANEL256) {
+    const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
+                                workspace_bytes, stream);
+    TLQ_REQUIRE(rc >= 0, "tlq_gemm_w4a16_ws: the 256-row panel kernel needs K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group "
+                ">= 32, 16-byte aligned operands and a workspace for its K slices and (with a zero-point tensor) 16 bytes more (M=%lld "
+                "N=%lld K=%lld group=%lld, workspace %lld)", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
+    return rc;
+  }
   if (algo == TLQ_ALGO_PANEL) {
     const int rc = try_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
                              workspace_bytes, stream);
@@ -406,25 +467,19 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
       return 1;
     }
   }
-  // Above 512 rows: the panel kernel (one launch, no dequantised matrix) where its work-groups fill the machine.  Measured
-  // against the choice without it (two passes, tile kernel over K slices) on ten (N, K) pairs x nine values of M, fp16 with
-  // a zero-point tensor and bf16 with a scalar one, groups of 128: from 576 to 2048 rows ahead wherever its last round of
-  // work-groups fills 0.55 of the CUs or more -- by 10 - 45 % on the wide or long matrices (N = 28672, K = 4096, M = 768:
-  // 1.35 - 1.47 x; N = 4096, K = 14336, M = 1280: 1.35 - 1.40 x; 8192 x 8192, M = 640: 1.36 - 1.41 x), within 5 % either
-  // way on 5120 x 5120 -- and 6 - 22 % behind below that fill (M = 2048, N = K = 4096: 128 work-groups).  From 3072 rows on
-  // every weight is dequantised 24 times or more and the two are within 5 % of each other (0.91 - 1.09): the two passes
-  // keep those, except where the panel kernel's work-groups fit the machine in one round and no zero-point tensor asks for
-  // its second launch (4096 x 4096 x 4096 with a scalar zero point: level, and no workspace traffic).
-  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && M > 512 && M <= 4096 && K > 0 && group > 0 && N >= 1 && N < kMaxDim && K < kMaxDim) {
-    const PanelPlan pp = w4a16_panel_plan(M, N, K, group, cu_count_or_default());
-    if (pp.ok) {
-      const int64_t wgs = (int64_t)pp.tiles_m * pp.tiles_n * pp.split, cus_now = cu_count_or_default();
-      const double fill = (double)wgs / (double)(ceil_div(wgs, cus_now) * cus_now);
-      if ((M <= 2048 && fill >= 0.55) || (wgs <= cus_now && fill >= 0.9 && zeros == nullptr)) {
-        const int rc = try_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
-                                 workspace_bytes, stream);
-        if (rc >= 0) return rc;
-      }
+  // Above 512 rows: the 256-row panel kernel (one launch, no dequantised matrix) where its work-groups fill the machine.
+  // Measured against the choice without it (two passes, tile kernel over K slices) and against the 128-row panel kernel
+  // on ten (N, K) pairs x eleven values of M from 576 to 8192, fp16 with a zero-point tensor and bf16 with a scalar one,
+  // groups of 128: wherever its last round of work-groups fills 0.55 of the CUs or more it is level or ahead -- by 3 - 16 %
+  // from 3072 rows on (4096 x 4096 x 4096 bf16: 104 against 113 - 119 us; 8192 x 8192 x 8192: 1.11 x), by 10 - 56 % between
+  // 576 and 2048 rows on wide or long matrices (N = 28672, K = 4096, M = 768: 1.40 - 1.54 x; N = 4096, K = 14336, M = 1280:
+  // 1.50 - 1.56 x), 0.98 - 0.99 on a few of the largest fp16 problems -- and 2 - 21 % behind below that fill (N = K = 4096,
+  // M <= 1024: 96 work-groups).  The 128-row kernel is ahead of it nowhere by more than 4 % and stays an explicit choice.
+  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && M > 512 && K > 0 && group > 0 && N >= 1 && N < kMaxDim && K < kMaxDim && M < kMaxDim) {
+    if (panel256_fills(M, N, K, group)) {
+      const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
+                                  workspace_bytes, stream);
+      if (rc >= 0) return rc;
     }
   }
   const bool split_region = w4a16_mid_split(M, N, K, group > 0 ? group : 32) > 1;
@@ -466,8 +521,8 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
     return tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, algo, workspace,
                              workspace_bytes, stream);
   TLQ_CHECK_DIMS("tlq_gemm_w4a16_layout_ws");
-  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS || algo == TLQ_ALGO_DECODE || algo == TLQ_ALGO_PANEL,
-              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the decode kernel, the streaming kernel, the panel kernel and the two passes (algo %d)", algo);
+  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS || algo == TLQ_ALGO_DECODE || algo == TLQ_ALGO_PANEL || algo == TLQ_ALGO_PANEL256,
+              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the decode kernel, the streaming kernel, the panel kernels and the two passes (algo %d)", algo);
   TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_w4a16_layout_ws: in_dtype must be float16 or bfloat16 (got %d)", in_dtype);
   TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_w4a16_layout_ws: bad out_dtype %d", out_dtype);
   if (M == 0 || N == 0) return 0;
@@ -491,17 +546,25 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
                 (long long)K, (long long)group, (long long)workspace_bytes);
   }
   TLQ_REQUIRE(algo != TLQ_ALGO_DECODE, "tlq_gemm_w4a16_layout_ws: the decode kernel handles M <= 32 (got %lld)", (long long)M);
-  if (algo == TLQ_ALGO_PANEL || (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && M > 512 && M <= 4096)) {
-    // (the same rule as for plain words: where the panel kernel's tiles fill the machine)
+  if (algo == TLQ_ALGO_PANEL256 || (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && M > 512)) {
+    // (the same rule as for plain words: where the 256-row panel kernel's tiles fill the machine)
+    if (algo == TLQ_ALGO_PANEL256 || panel256_fills(M, N, K, group)) {
+      const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, workspace,
+                                  workspace_bytes, stream);
+      if (rc >= 0) return rc;
+    }
+    TLQ_REQUIRE(algo != TLQ_ALGO_PANEL256, "tlq_gemm_w4a16_layout_ws: the 256-row panel kernel does not take M=%lld N=%lld K=%lld group=%lld "
+                "with a workspace of %lld bytes (K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group >= 32)", (long long)M,
+                (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
+  }
+  if (algo == TLQ_ALGO_PANEL) {
     const PanelPlan pp = w4a16_panel_plan(M, N, K, group, cu_count_or_default());
-    const int64_t wgs = (int64_t)pp.tiles_m * pp.tiles_n * pp.split, cus_now = cu_count_or_default();
-    const double fill = pp.ok ? (double)wgs / (double)(ceil_div(wgs, cus_now) * cus_now) : 0.0;
-    if (pp.ok && (algo == TLQ_ALGO_PANEL || (M <= 2048 && fill >= 0.55) || (wgs <= cus_now && fill >= 0.9 && zeros == nullptr))) {
+    if (pp.ok) {
       const int rc = try_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, workspace,
                                workspace_bytes, stream);
       if (rc >= 0) return rc;
     }
-    TLQ_REQUIRE(algo != TLQ_ALGO_PANEL, "tlq_gemm_w4a16_layout_ws: the panel kernel does not take M=%lld N=%lld K=%lld group=%lld with a "
+    TLQ_REQUIRE(false, "tlq_gemm_w4a16_layout_ws: the panel kernel does not take M=%lld N=%lld K=%lld group=%lld with a "
                 "workspace of %lld bytes (K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group with (K / group) %% 8 == 0, 16-byte "
                 "aligned scale / zero tensors)", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
   }

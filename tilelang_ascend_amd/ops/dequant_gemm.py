@@ -27,7 +27,7 @@ _PASS_CONFIGS = {
 }
 _SIGN_MODES = {"unsigned": _abi.U4, "twos": _abi.S4_TWOS, "offset8": _abi.S4_OFFSET8, "offset7": _abi.S4_OFFSET7}
 _ALGOS = {"auto": _abi.ALGO_AUTO, "gemv": _abi.ALGO_GEMV, "mfma": _abi.ALGO_MFMA, "skinny": _abi.ALGO_SKINNY,
-          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM, "decode": _abi.ALGO_DECODE, "panel": _abi.ALGO_PANEL}
+          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM, "decode": _abi.ALGO_DECODE, "panel": _abi.ALGO_PANEL, "panel256": _abi.ALGO_PANEL256}
 # arrangement of the 4-bit fields in each 32-bit word: general_compress order, or interleave_weight(target float16)
 _LAYOUTS = {"plain": _abi.W_PLAIN, "interleaved": _abi.W_INTERLEAVED_F16}
 
@@ -219,7 +219,7 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
         lib = _abi.load()
         ws = None
         ws_bytes = 0
-        if algo in ("auto", "two_pass", "stream", "decode", "panel"):
+        if algo in ("auto", "two_pass", "stream", "decode", "panel", "panel256"):
             ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
             if algo == "two_pass" or (layout_code != _abi.W_PLAIN and algo == "auto" and M > 256):
                 ws_bytes = max(ws_bytes, N * K * 2)
