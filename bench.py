@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|small|prefill|w8a8|skinny|actquant|mlp-sweep] [--units U]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|small|prefill|w8a8|skinny|actquant|mlp-sweep|vendor-gemm] [--units U]
 
 Headline workload (default): the W4A16 decode GEMV -- M=1, N=11008, K=4096, fp16 activations,
 uint4 weights packed low-nibble-first, group 128, fp16 scales U[0.005,0.02] and fp16 zeros U{6..9},
@@ -428,6 +428,80 @@ def bench_act_quant(args, steps=None):
                              **traffic_from_profile("act_quant_bf16_M16384_N4096.txt"), bytes_per_launch=unit_bytes)}
 
 
+def bench_vendor_gemm(args, steps=None):
+    """The vendor library's GEMMs (torch.matmul / torch._int_mm, hipBLASLt underneath) beside this library's kernels on
+    the same dense problems, alternating in one process (boxes and thermal states differ by several percent, so only
+    figures from one process compare): the plain 16-bit GEMM core, the W4A16 path on the same shape (which reads a
+    quarter of the weight bytes and dequantises on the way), and the int8 core.  Random operands.  A kernel trace of
+    this command holds the vendor kernels' names and launch records (work-group size, LDS, registers)."""
+    import torch
+
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device=dev).manual_seed(11)
+    steps = steps or min(args.steps, 10)
+    rows = []
+
+    def med(fns, rounds=5):  # alternating rounds; median us per launch for each callable
+        acc = [[] for _ in fns]
+        for r in range(rounds):
+            for k, fn in enumerate(fns):
+                fn(); fn()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(steps):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                acc[k].append(e0.elapsed_time(e1) * 1e3 / steps)
+        return [statistics.median(a) for a in acc]
+
+    def check(rc):
+        if rc:
+            raise RuntimeError(_abi.last_error())
+
+    g = 128
+    for dt, code, peak in ((torch.bfloat16, _abi.BF16, MFMA_F16_PEAK_TFLOPS), (torch.float16, _abi.F16, MFMA_F16_PEAK_TFLOPS)):
+        for (M, N, K) in ((4096, 4096, 4096), (8192, 8192, 8192), (8192, 14336, 4096)):
+            A = torch.randn(M, K, dtype=dt, device=dev, generator=gen)
+            W = (torch.randn(N, K, dtype=dt, device=dev, generator=gen) * 0.05)
+            C = torch.empty(M, N, dtype=dt, device=dev)
+            Wp = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, device=dev, generator=gen)
+            S = (torch.rand(N, K // g, device=dev, generator=gen) * 0.015 + 0.005).to(dt)
+            ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+            fns = [lambda: torch.matmul(A, W.t(), out=C),
+                   lambda: check(lib.tlq_gemm_f16(P(A), P(W), P(C), M, N, K, code, code, _abi.B_NK, stream)),
+                   lambda: check(lib.tlq_gemm_w4a16_ws(P(A), P(Wp), P(S), None, P(C), M, N, K, g, 8.0, code, code, _abi.ALGO_AUTO, P(ws), ws_bytes, stream))]
+            v, own, w4 = med(fns)
+            flops = 2.0 * M * N * K
+            rows.append({"problem": f"{str(dt)[6:]} M={M} N={N} K={K}, weights [N,K]", "vendor_us": round(v, 1), "gemm_f16_us": round(own, 1),
+                         "w4a16_us": round(w4, 1), "vendor_frac_of_peak": round(flops / v / 1e6 / peak, 4),
+                         "gemm_f16_frac_of_peak": round(flops / own / 1e6 / peak, 4), "w4a16_frac_of_peak": round(flops / w4 / 1e6 / peak, 4)})
+            del A, W, C, Wp, S, ws
+    for (M, N, K) in ((16384, 4096, 4096), (8192, 8192, 8192)):
+        A = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=gen)
+        B = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=gen)
+        C = torch.empty(M, N, dtype=torch.int32, device=dev)
+        fns = [lambda: torch._int_mm(A, B, out=C), lambda: check(lib.tlq_gemm_i8(P(A), P(B), P(C), 1, M, N, K, _abi.B_KN, stream))]
+        v, own = med(fns)
+        ops = 2.0 * M * N * K
+        rows.append({"problem": f"int8 M={M} N={N} K={K}, weights [K,N]", "vendor_us": round(v, 1), "gemm_i8_us": round(own, 1),
+                     "vendor_frac_of_peak": round(ops / v / 1e6 / MFMA_I8_PEAK_TOPS, 4), "gemm_i8_frac_of_peak": round(ops / own / 1e6 / MFMA_I8_PEAK_TOPS, 4)})
+        del A, B, C
+    first = rows[0]
+    flops = 2.0 * 4096 ** 3
+    return {"workload": "vendor library (hipBLASLt through torch.matmul / torch._int_mm) beside this library's GEMMs, alternating in one "
+                        "process, random operands; value: this library's W4A16 path on bf16 4096^3",
+            "dtype": "bf16", "value": round(flops / first["w4a16_us"] / 1e6, 1), "unit": "TFLOP/s", "ms_per_step": first["w4a16_us"] * 1e-3,
+            "roofline": {"bound": "mfma", "achieved": round(flops / first["w4a16_us"] / 1e6, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": first["w4a16_frac_of_peak"], "traffic": None},
+            "shapes": rows}
+
+
 def bench_mlp_sweep(args, steps=None):
     """MLP-shaped sweep: M in {16, 64, 256, 1024, 8192} x (N, K) in {(14336, 4096), (4096, 14336)} x group in {128, 64},
     fp16, per-group scales and zeros, automatic kernel choice with a workspace (tlq_gemm_w4a16_ws).  Inputs are drawn
@@ -522,7 +596,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=48)
-    ap.add_argument("--workload", default="gemv", choices=["gemv", "small", "prefill", "w8a8", "skinny", "actquant", "mlp-sweep"])
+    ap.add_argument("--workload", default="gemv", choices=["gemv", "small", "prefill", "w8a8", "skinny", "actquant", "mlp-sweep", "vendor-gemm"])
     ap.add_argument("--units", type=int, default=1, help="independent weight sets per GEMV launch")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
@@ -589,9 +663,9 @@ def main():
         cpu = not args.no_cpu_baseline
         res = {"prefill": lambda a: bench_prefill(a, cpu=cpu), "w8a8": lambda a: bench_w8a8(a, cpu=cpu),
                "skinny": lambda a: bench_skinny(a, cpu=cpu), "small": lambda a: bench_small(a, cpu=cpu),
-               "actquant": bench_act_quant, "mlp-sweep": bench_mlp_sweep}[args.workload](args)
+               "actquant": bench_act_quant, "mlp-sweep": bench_mlp_sweep, "vendor-gemm": bench_vendor_gemm}[args.workload](args)
         line = {"metric": METRIC, "value": res["value"], "unit": res["unit"], "ms_per_step": res["ms_per_step"], "dtype": res["dtype"],
-                "config": {"workload": res["workload"] + ("; every figure from HIP events" if args.workload == "mlp-sweep" else "; " + WALL_NOTE)}, "roofline": res["roofline"],
+                "config": {"workload": res["workload"] + ("; every figure from HIP events" if args.workload in ("mlp-sweep", "vendor-gemm") else "; " + WALL_NOTE)}, "roofline": res["roofline"],
                 "cpu_baseline": res.get("cpu_baseline")}
         for extra in ("shapes", "fused_kernel", "two_passes"):
             if extra in res:
