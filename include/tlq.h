@@ -88,6 +88,13 @@ enum {
                          * and zero points are gathered into registers, so any number of groups per row and 2-byte aligned
                          * scale / zero tensors will do.  K % 128 == 0, M % 4 == 0, N % 16 == 0, power-of-two group >= 32; workspace
                          * as for TLQ_ALGO_PANEL */
+  ,
+  TLQ_ALGO_PANELM = 9 /* middle M (tens to hundreds of activation rows): the four-wavefront panel structure on 64 or 128
+                       * activation rows x 256 weight rows per work-group, a ring of four / three LDS slots, scales and zero
+                       * points through LDS windows; a zero-point tensor is handled inside the one launch (folded while the
+                       * zero points are small integers, unfolded from the first window that is not).  K % 128 == 0, M % 4 == 0,
+                       * N % 16 == 0, power-of-two group >= 64 with (K / group) % 8 == 0, 16-byte aligned scale / zero tensors;
+                       * plain word layout.  Workspace: the fp32 partial tiles where K is cut into slices */
 };
 
 int tlq_abi_version(void);

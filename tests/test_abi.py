@@ -178,7 +178,7 @@ def test_rejects_bad_arguments_of_the_widened_entry_points():
     _rejected(lib.tlq_gemv(ODD, FAKE, FAKE, 8, 64, _abi.F16, _abi.F16, NULL), "16-byte aligned")
     _rejected(lib.tlq_gemm_w4a16_ws(FAKE, FAKE, NULL, NULL, FAKE, 512, 64, 128, 32, 0.0, _abi.F16, _abi.F16, _abi.ALGO_TWO_PASS,
                                     NULL, 0, NULL), "two-pass path needs", "workspace")
-    _rejected(lib.tlq_gemm_w4a16_ws(FAKE, FAKE, NULL, NULL, FAKE, 512, 64, 128, 32, 0.0, _abi.F16, _abi.F16, 9, NULL, 0, NULL),
+    _rejected(lib.tlq_gemm_w4a16_ws(FAKE, FAKE, NULL, NULL, FAKE, 512, 64, 128, 32, 0.0, _abi.F16, _abi.F16, 10, NULL, 0, NULL),
               "bad algo")
     # empty problems launch nothing
     assert lib.tlq_act_quant_i8(NULL, NULL, NULL, 0, 64, _abi.BF16, 0, NULL) == 0

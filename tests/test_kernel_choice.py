@@ -49,10 +49,11 @@ def cases():
         (768, 8192, 4096, 128, _abi.ALGO_PANEL256),  # above 512 rows where the 256-row panel kernel's work-groups fill the machine: 3 x 32 tiles x 2 K slices on 256 CUs
         (2048, 4096, 2048, 128, _abi.ALGO_TWO_PASS),  # 8 x 16 panel tiles and too few steps to cut: half the CUs idle, the two passes keep it
         (224, 28672, 8192, 128, _abi.ALGO_MFMA),    # largest matrices from 192 rows on: tile kernel over two long K slices
+        (256, 14336, 4096, 128, _abi.ALGO_PANELM),  # 256 .. 512 rows on 2^25 weights or more: the middle-M panel kernel
     ]
 
 
-@pytest.mark.parametrize("case", range(17))
+@pytest.mark.parametrize("case", range(18))
 def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
     from tilelang_ascend_amd import _abi
 

@@ -19,7 +19,7 @@ F16, BF16, F32, I8, I32 = 0, 1, 2, 3, 4
 U4, S4_TWOS, S4_OFFSET8, S4_OFFSET7 = 0, 1, 2, 3
 B_KN, B_NK = 0, 1
 W_PLAIN, W_INTERLEAVED_F16 = 0, 1
-ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY, ALGO_TWO_PASS, ALGO_STREAM, ALGO_DECODE, ALGO_PANEL, ALGO_PANEL256 = 0, 1, 2, 3, 4, 5, 6, 7, 8
+ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY, ALGO_TWO_PASS, ALGO_STREAM, ALGO_DECODE, ALGO_PANEL, ALGO_PANEL256, ALGO_PANELM = 0, 1, 2, 3, 4, 5, 6, 7, 8, 9
 ABI_VERSION = 1
 
 _vp, _i64, _int, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
@@ -66,6 +66,9 @@ SIGNATURES = {
     "tlq_debug_check_panel256_addressing": (_int, [_i64, _i64, _i64, _i64, _int]),
     "tlq_debug_panel256_plan": (_int, [_i64, _i64, _i64, _i64, _int, _vp]),
     "tlq_debug_check_panel256_schedule": (_int, [_int, _int, _int]),
+    "tlq_debug_panelm_plan": (_int, [_i64, _i64, _i64, _i64, _int, _vp]),
+    "tlq_debug_check_panelm_addressing": (_int, [_i64, _i64, _i64, _i64, _int, _int]),
+    "tlq_debug_check_panelm_schedule": (_int, [_int, _int, _int, _int, _int]),
     "tlq_tune_w4a16_decode": (None, [_int]),
     "tlq_debug_gemv_rows_plan": (_int, [_i64, _i64, _i64, _i64, _int, _vp]),
     "tlq_tune_gemv": (None, [_int, _int]),
@@ -82,6 +85,7 @@ SIGNATURES = {
     "tlq_tune_w4a16_stream_slice": (None, [_int]),
     "tlq_tune_w4a16_panel": (None, [_int]),
     "tlq_tune_w4a16_panel_slice": (None, [_int]),
+    "tlq_tune_w4a16_panelm_rows": (None, [_int]),
     "tlq_tune_w4a16_tile": (None, [_int]),
     "tlq_tune_w4a16_split": (None, [_int]),
     "tlq_tune_w4a16_skinny": (None, [_int, _int]),

@@ -71,7 +71,7 @@ struct Expand8<half_t, FOLD, LAYOUT> {
     // that puts pin(i) behind its next MFMA statement keeps piece i ahead of that point and piece i + 1 behind it.
     __device__ __forceinline__ void pin(int i) {
       if (i == 0) asm volatile("" : "+v"(q0), "+v"(q1));
-      if (i == 1) asm volatile("" : "+v"(f0), "+v"(f1));
+      if (i == 1) asm volatile("" : "+v"(q0), "+v"(q1), "+v"(f0), "+v"(f1));  // (also what piece 2 reads: it must not move ahead of this point)
       if (i == 2) asm volatile("" : "+v"(f0), "+v"(f1), "+v"(f2), "+v"(f3));  // (all four: piece 3 packs both words)
       if (i == 3) asm volatile("" : "+v"(a), "+v"(b));
     }
@@ -178,7 +178,7 @@ struct Expand8<bf16_t, FOLD, LAYOUT> {
     // (see the binary16 decoder)
     __device__ __forceinline__ void pin(int i) {
       if (i == 0) asm volatile("" : "+v"(q0), "+v"(q1));
-      if (i == 1) asm volatile("" : "+v"(f0), "+v"(f1));
+      if (i == 1) asm volatile("" : "+v"(q0), "+v"(q1), "+v"(f0), "+v"(f1));  // (also what piece 2 reads: it must not move ahead of this point)
       if (i == 2) asm volatile("" : "+v"(f0), "+v"(f1), "+v"(f2), "+v"(f3));  // (all four: piece 3 packs both words)
       if (i == 3) asm volatile("" : "+v"(a), "+v"(b));
     }

@@ -261,6 +261,44 @@ constexpr int kPanel2WaitA = panel2_loads_in(24, kPanel2BarrierSlot);
 static_assert(kPanel2WaitW == 24 && kPanel2WaitA == 0 && kPanel2BarrierSlot == 57 && kPanel2WSlot + kPanel2TN <= kPanel2Slots,
               "the 256-row panel kernel's waits");
 
+// ---- panel kernel for middle M (gemm_w4a16_panelm.hip): the 256-row kernel's four wavefronts and slot structure on
+// 16 TM activation rows (TM = 4 or 8), 256 weight rows, a ring of D slots and the 128-row kernel's scale windows in LDS.
+// Ring slot: activation tile [16 TM rows][256 B] (direct load I = 4 j + wave, j = 0 .. TM - 1, rows 4 I .. 4 I + 3, as in
+// the 256-row kernel) + the four wavefronts' packed weights, four [16 rows][64 B] tiles each; behind the ring two scale
+// windows per wavefront ([scales | zero points][64 rows][8 groups] of 2 bytes, see the 128-row kernel).
+// A step of 128 values of K is 4 TM slots of four MFMAs (phase ks = slots ks TM .. ks TM + TM - 1).  Step s issues, in this
+// order: the TM loads of the activation tile of step s + D - 1 (slots 0 .. TM - 1), at the first step of a scale window
+// the two loads of the next window (slot TM), and from slot 2 TM + 1 on (the step's last packed word was read in phase 1)
+// the four loads of the wavefront's packed weights of step s + D.  Loads retire in issue order; the two waits of a step are written for the FEWEST
+// loads that can be younger than what they wait for (no window loads), so a step with window loads waits a little more:
+//   slot 2 TM (its packed words are read from there on): the packed weights of step s + 1, issued in step s + 1 - D;
+//        younger: steps s + 2 - D .. s - 1 whole and this step's activation loads
+//   slot B: the activation tile of step s + 1, issued in step s + 2 - D; younger: that step's weights, steps
+//        s + 3 - D .. s - 1 whole and all of this step's loads
+// The barrier at slot B stands behind the last operand read of this step's tile (slot B - 1 reads AR - 1 slots ahead);
+// slots B .. 4 TM - 1 read the first operands of step s + 1.  A window's loads, issued in step x, have landed behind the
+// slot-B wait of step x + D - 2 and are first looked at at the top of the window's last step: a window must span D steps.
+__host__ __device__ constexpr int panelm_depth(int tm) { return tm >= 16 ? 2 : tm >= 8 ? 3 : 4; }
+__host__ __device__ constexpr int panelm_ahead(int tm) { return tm >= 8 ? 8 : 4; }
+__host__ __device__ constexpr int panelm_slots(int tm) { return 4 * tm; }
+__host__ __device__ constexpr int panelm_barrier_slot(int tm) { return 4 * tm - (panelm_ahead(tm) - 1); }
+__host__ __device__ constexpr int panelm_w_slot(int tm) { return 2 * tm + 1; }
+__host__ __device__ constexpr int panelm_step_loads(int tm) { return tm + kPanel2TN; }  // without window loads
+__host__ __device__ constexpr int panelm_wait_w(int tm) { return (panelm_depth(tm) - 2) * panelm_step_loads(tm) + tm; }
+__host__ __device__ constexpr int panelm_wait_a(int tm) { return kPanel2TN + (panelm_depth(tm) - 3) * panelm_step_loads(tm) + panelm_step_loads(tm); }
+static_assert(panelm_depth(4) >= 3 && panelm_depth(8) >= 3, "the waits are written for rings of three slots or more");
+static_assert(panelm_w_slot(4) + kPanel2TN <= panelm_barrier_slot(4) && panelm_w_slot(8) + kPanel2TN <= panelm_barrier_slot(8),
+              "the weight loads are issued between the wait for the next step's weights and the barrier");
+static_assert(panelm_wait_w(8) == 20 && panelm_wait_a(8) == 16 && panelm_wait_w(4) == 20 && panelm_wait_a(4) == 20, "the middle-M panel kernel's waits");
+__host__ __device__ constexpr uint32_t panelm_a_tile(int tm) { return (uint32_t)tm * 4096u; }
+__host__ __device__ constexpr uint32_t panelm_slot_bytes(int tm) { return panelm_a_tile(tm) + 4u * kPanel2TN * 1024u; }
+__host__ __device__ constexpr uint32_t panelm_w_lds(int tm, int wave, int tn) { return panelm_a_tile(tm) + (uint32_t)(wave * kPanel2TN + tn) * 1024u; }
+__host__ __device__ constexpr uint32_t panelm_sc_lds(int tm, int wave, int buf) {
+  return (uint32_t)panelm_depth(tm) * panelm_slot_bytes(tm) + (uint32_t)(wave * 2 + buf) * kPanelScBuf;
+}
+__host__ __device__ constexpr uint32_t panelm_lds_bytes(int tm) { return panelm_sc_lds(tm, 4, 0); }
+static_assert(panelm_lds_bytes(8) <= 160 * 1024 && panelm_lds_bytes(4) <= 160 * 1024, "ring and scale windows fit the CU's LDS");
+
 // ---- decode kernel (1 .. 32 activation rows): wavefront w of a work-group owns values 256 s .. 256 s + 255 of K
 // (s = chunk * waves + w) for every weight row.  A work item is one 16-row weight tile: two [16 rows][64 B] packed
 // pieces (k-blocks kb = 0, 1 of the slice, 128 values each) plus the scales / zero points of the 16 rows for the

@@ -514,6 +514,203 @@ int check_panel256(int64_t M, int64_t N, int64_t K, int64_t group, int slice_ste
   return 0;
 }
 
+// Middle-M panel kernel: 16 tm x 256 outputs per work-group of four wavefronts (tm = 4 or 8), a ring of D slots, scale
+// windows in LDS.  Walks every work-group tile: global extents of the activation, weight and scale-window loads over every
+// step and window of every slice, LDS extents and coverage of a ring slot and of the window buffers, agreement of the
+// landing cells with the operand reads.
+int check_panelm(int64_t M, int64_t N, int64_t K, int64_t group, int tm, int slice_steps) {
+  CHECK_OR_FAIL(tm == 4 || tm == 8, "panelm: %d activation tiles per work-group", tm);
+  CHECK_OR_FAIL(M >= 4 && N >= 16 && M % 4 == 0 && N % 16 == 0 && K >= 128 && K % 128 == 0, "panelm: bad shape");
+  CHECK_OR_FAIL(group >= 32 && (group & (group - 1)) == 0 && K % group == 0 && (K / group) % 8 == 0, "panelm: group %lld on K %lld",
+                (long long)group, (long long)K);
+  const int64_t groups = K / group;
+  CHECK_OR_FAIL(N * (K / 2) < ((int64_t)1 << 32) && M * K * 2 < ((int64_t)1 << 32) && N * groups * 2 < ((int64_t)1 << 32),
+                "panelm: a matrix spans 4 GiB or more");
+  const int steps_total = (int)(K / 128);
+  const int window = (int)(group >= 128 ? 8 * (group / 128) : 8 / (128 / group));
+  CHECK_OR_FAIL(window >= addr::panelm_depth(tm), "panelm: windows of %d steps on a ring of %d slots", window, addr::panelm_depth(tm));
+  CHECK_OR_FAIL(slice_steps >= 1 && (slice_steps % window == 0 || slice_steps >= steps_total), "panelm: slices of %d steps are not whole windows of %d",
+                slice_steps, window);
+  const int TN = addr::kPanel2TN;
+  const int64_t w_extent = N * (K / 2), a_extent = M * K * 2, s_extent = N * groups * 2;
+  const uint32_t slot_bytes = addr::panelm_slot_bytes(tm), a_tile = addr::panelm_a_tile(tm), lds_total = addr::panelm_lds_bytes(tm);
+  CHECK_OR_FAIL(lds_total <= 160 * 1024 && addr::panelm_sc_lds(tm, 0, 0) == (uint32_t)addr::panelm_depth(tm) * slot_bytes, "panelm: %u bytes of LDS", lds_total);
+  const int slices = (steps_total + slice_steps - 1) / slice_steps;
+  std::vector<int> cell(slot_bytes / 16);
+  for (int64_t m0 = 0; m0 < M; m0 += 16 * tm)
+    for (int64_t n0 = 0; n0 < N; n0 += 4 * 16 * TN) {
+      std::fill(cell.begin(), cell.end(), -1);
+      for (int wave = 0; wave < 4; ++wave) {
+        for (int j = 0; j < tm; ++j) {
+          const uint32_t l0 = addr::panel2_a_lds(wave, j);
+          const int I = j * 4 + wave;
+          for (int lane = 0; lane < 64; ++lane) {
+            const int64_t voff = addr::panel2_a_block(wave, j, (int)m0, (int)M, (int)K) + addr::panel_a_lane(lane, (int)K) + addr::panel_a_chunk(lane, wave);
+            CHECK_OR_FAIL(voff >= 0 && voff + (int64_t)(steps_total - 1) * 256 + 16 <= a_extent, "panelm: activation load at %lld of %lld",
+                          (long long)voff, (long long)a_extent);
+            const uint32_t at = l0 / 16 + lane;
+            CHECK_OR_FAIL(at < a_tile / 16 && cell[at] == -1, "panelm: activation cell %u written twice or outside the tile", at);
+            const int row = addr::sa_row(lane, I), chunk = addr::sa_chunk(lane, I);
+            CHECK_OR_FAIL((int)at == row * 16 + (lane & 15), "panelm: activation lane lands on cell %u, not on its row", at);
+            if (m0 + 4 * I + 4 <= M)
+              CHECK_OR_FAIL(voff == ((int64_t)(m0 + row) * K) * 2 + chunk * 16, "panelm: activation lane %d of load %d fetches the wrong bytes", lane, I);
+            cell[at] = row * 16 + chunk;
+          }
+        }
+        for (int tn = 0; tn < TN; ++tn) {
+          const uint32_t l0 = addr::panelm_w_lds(tm, wave, tn);
+          for (int lane = 0; lane < 64; ++lane) {
+            const int64_t voff = addr::panel_w_block(wave, tn, (int)n0, (int)N, (int)K) + addr::panel_w_lane(lane, (int)K);
+            CHECK_OR_FAIL(voff >= 0 && voff + (int64_t)(steps_total - 1) * 64 + 16 <= w_extent, "panelm: weight load at %lld of %lld",
+                          (long long)voff, (long long)w_extent);
+            if (n0 + wave * 64 + tn * 16 + 16 <= N)
+              CHECK_OR_FAIL(voff == (int64_t)(n0 + wave * 64 + tn * 16 + addr::sw_row(lane)) * (K / 2) + addr::sw_piece(lane) * 16, "panelm: weight lane %d fetches the wrong bytes", lane);
+            const uint32_t at = l0 / 16 + lane;
+            CHECK_OR_FAIL(at >= a_tile / 16 && at < slot_bytes / 16 && cell[at] == -1, "panelm: weight cell %u written twice or outside the slot", at);
+            cell[at] = addr::sw_row(lane) * 4 + addr::sw_piece(lane);
+          }
+          for (int lane = 0; lane < 64; ++lane) {
+            const uint32_t off = l0 + addr::sw_frag_off(lane);
+            CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= slot_bytes, "panelm: weight operand read at %u", off);
+            CHECK_OR_FAIL(cell[off / 16] == (lane & 15) * 4 + (lane >> 4), "panelm: weight operand read of lane %d finds cell %d", lane, cell[off / 16]);
+          }
+        }
+        // scale windows: lane l fetches 16 bytes of row n0 + 64 wave + l for every window of every slice
+        for (int lane = 0; lane < 64; ++lane) {
+          const int64_t voff = addr::panel_sc_voff(lane, wave, (int)n0, (int)N, (int)groups);
+          for (int sl = 0; sl < slices; ++sl) {
+            const int step0 = sl * slice_steps;
+            const int steps = steps_total - step0 < slice_steps ? steps_total - step0 : slice_steps;
+            const int64_t g0 = ((int64_t)step0 * 128) / group;
+            const int nwin = (steps + window - 1) / window;
+            for (int w = 0; w < nwin; ++w) {
+              const int64_t o = voff + (g0 + 8 * w) * 2;
+              CHECK_OR_FAIL(o >= 0 && o + 16 <= s_extent && o % 16 == 0, "panelm: scale load at [%lld, +16) of %lld", (long long)o, (long long)s_extent);
+              CHECK_OR_FAIL((g0 + 8 * w) % groups + 8 <= groups, "panelm: a scale window crosses the end of a row of the scale tensor");
+            }
+            // the group a lane reads for step s of the slice lies in the window the kernel reads it from
+            for (int s2 = 0; s2 < steps; ++s2)
+              for (int q = 0; q < 4; ++q) {
+                const int w = s2 / window, pos = s2 - w * window;
+                const int64_t gl = ((int64_t)pos * 128 + q * 32) / group;
+                CHECK_OR_FAIL(gl >= 0 && gl < 8 && g0 + 8 * w + gl == ((int64_t)(step0 + s2) * 128 + q * 32) / group, "panelm: step %d reads group %lld of its window", s2, (long long)gl);
+              }
+          }
+          for (int buf = 0; buf < 2; ++buf) {
+            const uint32_t at = addr::panelm_sc_lds(tm, wave, buf) + 1024u + (uint32_t)lane * 16u;
+            CHECK_OR_FAIL(at + 16 <= lds_total && at >= (uint32_t)addr::panelm_depth(tm) * slot_bytes, "panelm: scale window at %u", at);
+          }
+        }
+      }
+      for (uint32_t c = 0; c < slot_bytes / 16; ++c) CHECK_OR_FAIL(cell[c] >= 0, "panelm: cell %u of the slot never written", c);
+      for (int t = 0; t < tm; ++t)
+        for (int ks = 0; ks < 4; ++ks)
+          for (int lane = 0; lane < 64; ++lane) {
+            const uint32_t off = addr::sa_frag_off(lane, t, ks);
+            CHECK_OR_FAIL(off == ((addr::sa_frag_off(lane, 0, 0) ^ (uint32_t)(ks << 4)) + (uint32_t)(t * 16 * 256)), "panelm: the k-step offset is not an exclusive-or");
+            CHECK_OR_FAIL(off % 16 == 0 && off + 16 <= a_tile, "panelm: activation operand read at %u", off);
+            const int want = (t * 16 + (lane & 15)) * 16 + 4 * (lane >> 4) + ks;
+            CHECK_OR_FAIL(cell[off / 16] == want, "panelm: activation operand read (lane %d, k-step %d) finds cell %d, expects %d", lane, ks, cell[off / 16], want);
+          }
+    }
+  return 0;
+}
+
+// The middle-M kernel's schedule, played through for one wavefront: `steps` steps with windows of `window` steps, loads
+// issued in the kernel's order and retired in issue order, the two waits leaving wait_w / wait_a of them outstanding.
+// Every LDS read must find its data landed (the shared activation tile: landed and behind a barrier), every load into a
+// ring slot or window buffer must come after the last read of what it held (the shared tile: with a barrier between).
+int check_panelm_schedule(int tm, int steps, int window, int wait_w, int wait_a) {
+  CHECK_OR_FAIL((tm == 4 || tm == 8) && steps >= 1 && steps <= 256 && window >= 1 && wait_w >= 0 && wait_a >= 0, "panelm schedule: bad arguments");
+  const int D = addr::panelm_depth(tm), AR = addr::panelm_ahead(tm), S = addr::panelm_slots(tm), B = addr::panelm_barrier_slot(tm);
+  const int WS = addr::panelm_w_slot(tm), TN = addr::kPanel2TN, word_slot = tm >= 8 ? tm / 2 : 0;
+  enum { LA = 1, LW, LSC };
+  struct Load { int kind, idx; };
+  std::vector<Load> fifo;
+  const int X = steps + D + 2, nwin = (steps + window - 1) / window;
+  std::vector<int> landed_a(X, 0), landed_w(X, 0), landed_sc(nwin + 2, 0), published_a(X, 0);
+  std::vector<int64_t> last_read_a(X, -1), last_read_w(X, -1), last_read_sc(nwin + 2, -1), barrier_times;
+  int64_t now = -1;
+  auto issue = [&](int kind, int idx) { fifo.push_back(Load{kind, idx}); };
+  auto wait = [&](size_t n) {
+    while (fifo.size() > n) {
+      const Load l = fifo.front();
+      fifo.erase(fifo.begin());
+      (l.kind == LA ? landed_a : l.kind == LW ? landed_w : landed_sc)[l.idx]++;
+    }
+  };
+  auto barrier = [&]() {
+    for (int st = 0; st < X; ++st) published_a[st] = landed_a[st] >= tm;
+    barrier_times.push_back(now);
+  };
+  auto barrier_between = [&](int64_t t0, int64_t t1) {
+    for (int64_t b : barrier_times)
+      if (b > t0 && b <= t1) return true;
+    return false;
+  };
+  // prologue
+  for (int i = 0; i < 2; ++i) issue(LSC, 0);
+  for (int i = 0; i < TN; ++i) issue(LW, 0);
+  for (int i = 0; i < D - 1; ++i) {
+    for (int j = 0; j < tm; ++j) issue(LA, i);
+    for (int j = 0; j < TN; ++j) issue(LW, i + 1);
+  }
+  wait(0);
+  barrier();
+  for (int s = 0; s < steps; ++s) {
+    const int win = s / window, pos = s - win * window;
+    const int nwin_idx = pos + 1 == window ? win + 1 : win;
+    for (int t = 0; t < S; ++t) {
+      now = (int64_t)s * S + t;
+      const int ks = t / tm, slot_in_phase = t % tm;
+      if (t == 2 * tm) {
+        wait((size_t)wait_w);
+        CHECK_OR_FAIL(landed_w[s + 1] >= TN, "panelm schedule: step %d: the next step's packed weights have not landed at their wait", s);
+      }
+      if (t == B) {
+        wait((size_t)wait_a);
+        CHECK_OR_FAIL(landed_a[s + 1] >= tm, "panelm schedule: step %d: the next activation tile has not landed at the barrier", s);
+        barrier();
+      }
+      // behind MFMA 1 of the slot
+      if (t < tm) {
+        if (t == 0 && s >= 1)
+          CHECK_OR_FAIL(barrier_between(last_read_a[s - 1], now - 1), "panelm schedule: step %d: the tile of step %d may still be read", s, s - 1);
+        issue(LA, s + D - 1);  // into the slot of step s - 1
+      }
+      if (t == tm && pos == 0 && win + 1 < nwin) {
+        if (win >= 1) CHECK_OR_FAIL(last_read_sc[win - 1] < now, "panelm schedule: window %d is overwritten while it is read", win - 1);
+        issue(LSC, win + 1);
+        issue(LSC, win + 1);
+      }
+      if (t >= WS && t < WS + TN) {
+        CHECK_OR_FAIL(ks >= 2 && last_read_w[s] >= 0 && last_read_w[s] < now, "panelm schedule: step %d slot %d: this step's words are not all read", s, t);
+        issue(LW, s + D);  // into the slot of step s
+      }
+      const int at = t + AR - 1, a_step = at < S ? s : s + 1;
+      CHECK_OR_FAIL(published_a[a_step], "panelm schedule: step %d slot %d reads an operand of step %d before the barrier that publishes it", s, t, a_step);
+      last_read_a[a_step] = now;
+      if (slot_in_phase >= word_slot && slot_in_phase < word_slot + TN) {
+        const int w_step = ks < 2 ? s : s + 1;
+        CHECK_OR_FAIL(landed_w[w_step] >= TN, "panelm schedule: step %d slot %d reads a word of step %d that has not landed", s, t, w_step);
+        last_read_w[w_step] = now;
+      }
+      if (t == 2 * tm && s + 1 < steps) {  // the scales of step s + 1
+        CHECK_OR_FAIL(landed_sc[nwin_idx] >= 2, "panelm schedule: step %d reads scales of window %d, which has not landed", s, nwin_idx);
+        last_read_sc[nwin_idx] = now;
+      }
+    }
+    // the zero points of the next window are looked at at the top of the last step of a window: by then (the end of the
+    // step before) they must have landed
+    if (s + 1 < steps) {
+      const int win1 = (s + 1) / window, pos1 = (s + 1) - win1 * window;
+      if (pos1 + 1 == window && win1 + 1 < nwin)
+        CHECK_OR_FAIL(landed_sc[win1 + 1] >= 2, "panelm schedule: the zero points of window %d are looked at before they have landed", win1 + 1);
+    }
+  }
+  return 0;
+}
+
 // The 256-row panel kernel's schedule, played through for one wavefront over `steps` steps: loads issued per
 // addr::panel2_slot_load retire in issue order, the two waits leave addr::kPanel2WaitW / kPanel2WaitA of them outstanding;
 // every LDS read must find its data landed (for the shared activation tile: landed and behind a barrier), every load
@@ -904,6 +1101,26 @@ int tlq_debug_check_panel256_addressing(int64_t M, int64_t N, int64_t K, int64_t
   for (int steps : {1, 2, 3, 4, 7})
     if (int rc = check_panel256_schedule(steps, addr::kPanel2WaitW, addr::kPanel2WaitA)) return rc;
   return 0;
+}
+
+int tlq_debug_check_panelm_addressing(int64_t M, int64_t N, int64_t K, int64_t group, int rows, int slice_steps) {
+  if (rows != 64 && rows != 128) {
+    set_error("tlq_debug_check_panelm_addressing: %d activation rows per work-group", rows);
+    return 1;
+  }
+  const int tm = rows / 16;
+  if (int rc = check_panelm(M, N, K, group, tm, slice_steps)) return rc;
+  const int window = (int)(group >= 128 ? 8 * (group / 128) : 8 / (128 / group));
+  const int steps_total = (int)(K / 128), slice = slice_steps < steps_total ? slice_steps : steps_total;
+  for (int steps : {slice, steps_total % slice ? steps_total % slice : slice})
+    if (int rc = check_panelm_schedule(tm, steps, window, addr::panelm_wait_w(tm), addr::panelm_wait_a(tm))) return rc;
+  return 0;
+}
+
+int tlq_debug_check_panelm_schedule(int rows, int steps, int window, int wait_w, int wait_a) {
+  const int tm = rows / 16;
+  if (tm != 4 && tm != 8) return 1;
+  return check_panelm_schedule(tm, steps, window, wait_w < 0 ? addr::panelm_wait_w(tm) : wait_w, wait_a < 0 ? addr::panelm_wait_a(tm) : wait_a);
 }
 
 int tlq_debug_check_panel256_schedule(int steps, int wait_w, int wait_a) {

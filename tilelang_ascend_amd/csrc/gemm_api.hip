@@ -66,6 +66,15 @@ int gemm_w4a16_panel256(const void* A, const void* Wp, const void* scales, const
                         int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const Panel2Plan& p, float* partial,
                         uint32_t* flag, hipStream_t st);
 extern thread_local int g_panel2_slice_steps;
+struct PanelMPlan {
+  bool ok;
+  int tm, tiles_m, tiles_n, split, slice_steps;
+};
+PanelMPlan w4a16_panelm_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus);
+int gemm_w4a16_panelm(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N, int64_t K,
+                      int64_t group, float zero_scalar, int in_dtype, int out_dtype, const PanelMPlan& p, float* partial, hipStream_t st);
+extern thread_local int g_panelm_slice_steps;
+extern thread_local int g_panelm_rows;
 
 struct DecodePlan {
   bool ok;
@@ -112,7 +121,8 @@ void tlq_tune_w4a16_stream(int on) { tlq::g_w4a16_stream = on != 0; }
 void tlq_tune_w4a16_stream_slice(int steps) { tlq::g_stream_slice_steps = steps; }
 void tlq_tune_w4a16_decode(int on) { tlq::g_w4a16_decode = on != 0; }
 void tlq_tune_w4a16_panel(int mode) { tlq::g_w4a16_panel = mode != 0 ? 1 : 0; }
-void tlq_tune_w4a16_panel_slice(int steps) { tlq::g_panel_slice_steps = tlq::g_panel2_slice_steps = steps < 0 ? 0 : steps; }
+void tlq_tune_w4a16_panel_slice(int steps) { tlq::g_panel_slice_steps = tlq::g_panel2_slice_steps = tlq::g_panelm_slice_steps = steps < 0 ? 0 : steps; }
+void tlq_tune_w4a16_panelm_rows(int rows) { tlq::g_panelm_rows = (rows == 64 || rows == 128) ? rows : 0; }
 
 int tlq_debug_panel_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
   if (!(M >= 1 && N >= 1 && K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return 0;
@@ -130,6 +140,16 @@ int tlq_debug_panel256_plan(int64_t M, int64_t N, int64_t K, int64_t group, int 
   if (plan_out) {
     int64_t* o = (int64_t*)plan_out;
     o[0] = p.tiles_m, o[1] = p.tiles_n, o[2] = p.split, o[3] = p.slice_steps;
+  }
+  return p.ok ? 1 : 0;
+}
+
+int tlq_debug_panelm_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus, void* plan_out) {
+  if (!(M >= 1 && N >= 1 && K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return 0;
+  const PanelMPlan p = w4a16_panelm_plan(M, N, K, group, cus);
+  if (plan_out) {
+    int64_t* o = (int64_t*)plan_out;
+    o[0] = p.tiles_m, o[1] = p.tiles_n, o[2] = p.split, o[3] = p.slice_steps, o[4] = 16 * p.tm;
   }
   return p.ok ? 1 : 0;
 }
@@ -269,9 +289,32 @@ static int64_t panel_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return need;
 }
 
+// the same for the middle-M panel kernel
+static int64_t panelm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (!(M >= 1 && N >= 1 && K > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return 0;
+  int64_t need = 0;
+  for (int64_t group = 32; group <= 1024; group *= 2) {
+    if (K % group != 0) continue;
+    const PanelMPlan pm = w4a16_panelm_plan(M, N, K, group, cu_count_or_default());
+    if (pm.ok && pm.split > 1 && (int64_t)pm.split * M * N * 4 > need) need = (int64_t)pm.split * M * N * 4;
+  }
+  return need;
+}
+
+// The automatic choice takes the middle-M panel kernel from 256 to 512 activation rows on matrices of 2^25 weights or more
+// (measured against the streaming kernel on five (N, K) pairs, groups of 128 and 64, fp16 with a zero-point tensor:
+// 14336 x 4096 and 4096 x 14336: 43.5 - 43.9 against 45.8 - 47.0 us at 256 rows, 56 - 59 against 65 - 71 us at 384, 62 - 76 against
+// 70 - 80 us at 512; 8192 x 8192: 47 / 66 / 77 against 49 / 74 / 82 us; below 256 rows and on 4096 x 4096 or 5120 x 5120 the
+// streaming kernel is level or ahead by up to 15 %).
+static bool panelm_preferred(int64_t M, int64_t N, int64_t K) { return M >= 256 && M <= 512 && N * K >= ((int64_t)1 << 25); }
+
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
   int64_t need = w4a16_partial_sum_bytes(M, N, K);
+  if (panelm_preferred(M, N, K)) {
+    const int64_t pm = panelm_workspace_bytes(M, N, K);
+    if (pm > need) need = pm;
+  }
   if (M > 512) {
     const int64_t pn = panel_workspace_bytes(M, N, K);
     if (pn > need) need = pn;
@@ -341,10 +384,35 @@ static int try_panel256(const void* A, const void* w_packed, const void* scales,
                              (float*)workspace, zeros ? (uint32_t*)((uint8_t*)workspace + part_bytes) : nullptr, (hipStream_t)stream);
 }
 
+// The middle-M panel kernel.  Returns -1 when it does not take the problem (nothing launched, no error set).
+static int try_panelm(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                      int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, void* workspace,
+                      int64_t workspace_bytes, void* stream) {
+  if (!(M >= 1 && N >= 1 && K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)) return -1;
+  const PanelMPlan pp = w4a16_panelm_plan(M, N, K, group, cu_count_or_default());
+  if (!pp.ok) return -1;
+  const bool args_ok = A && w_packed && C && aligned16(A) && aligned16(w_packed) && aligned16(C) && aligned16(scales) &&
+                       aligned16(zeros) && (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) &&
+                       (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) && (M * N) % 4 == 0 &&
+                       fits32(M, K * 2) && fits32(N, K / 2) && fits32(N, (K / group) * 2);
+  if (!args_ok) return -1;
+  const int64_t need = pp.split > 1 ? (int64_t)pp.split * M * N * 4 : 0;
+  if (need > 0 && !(workspace && aligned16(workspace) && workspace_bytes >= need)) return -1;
+  return gemm_w4a16_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, pp, (float*)workspace,
+                           (hipStream_t)stream);
+}
+
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
-  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_PANEL256, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_PANELM, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  if (algo == TLQ_ALGO_PANELM) {
+    const int rc = try_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, workspace, workspace_bytes, stream);
+    TLQ_REQUIRE(rc >= 0, "tlq_gemm_w4a16_ws: the middle-M panel kernel needs K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group "
+                ">= 64 with (K / group) %% 8 == 0, 16-byte aligned operands, scale and zero tensors, and a workspace for its K slices (M=%lld "
+                "N=%lld K=%lld group=%lld, workspace %lld)", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
+    return rc;
+  }
   if (algo == TLQ_ALGO_PANEL256) {
     const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
                                 workspace_bytes, stream);
@@ -409,6 +477,11 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
   if (algo == TLQ_ALGO_TWO_PASS)
     TLQ_REQUIRE(have, "tlq_gemm_w4a16_ws: the two-pass path needs a 16-byte aligned workspace of %lld bytes (got %lld)",
                 (long long)need, (long long)workspace_bytes);
+  // 256 .. 512 activation rows on large matrices: the middle-M panel kernel
+  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && panelm_preferred(M, N, K) && group > 0) {
+    const int rc = try_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, workspace, workspace_bytes, stream);
+    if (rc >= 0) return rc;
+  }
   // 17 .. 512 activation rows: the streaming kernel (weights once per 128 rows, deep ring of direct loads)
   if ((algo == TLQ_ALGO_AUTO && g_w4a16_stream) || algo == TLQ_ALGO_STREAM) {
     const StreamPlan sp = (K > 0 && group > 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim)

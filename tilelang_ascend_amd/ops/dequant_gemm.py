@@ -27,7 +27,7 @@ _PASS_CONFIGS = {
 }
 _SIGN_MODES = {"unsigned": _abi.U4, "twos": _abi.S4_TWOS, "offset8": _abi.S4_OFFSET8, "offset7": _abi.S4_OFFSET7}
 _ALGOS = {"auto": _abi.ALGO_AUTO, "gemv": _abi.ALGO_GEMV, "mfma": _abi.ALGO_MFMA, "skinny": _abi.ALGO_SKINNY,
-          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM, "decode": _abi.ALGO_DECODE, "panel": _abi.ALGO_PANEL, "panel256": _abi.ALGO_PANEL256}
+          "two_pass": _abi.ALGO_TWO_PASS, "stream": _abi.ALGO_STREAM, "decode": _abi.ALGO_DECODE, "panel": _abi.ALGO_PANEL, "panel256": _abi.ALGO_PANEL256, "panelm": _abi.ALGO_PANELM}
 # arrangement of the 4-bit fields in each 32-bit word: general_compress order, or interleave_weight(target float16)
 _LAYOUTS = {"plain": _abi.W_PLAIN, "interleaved": _abi.W_INTERLEAVED_F16}
 
