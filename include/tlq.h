@@ -86,8 +86,9 @@ enum {
   TLQ_ALGO_PANEL256 = 8 /* the same with 256 activation rows x 256 weight rows per work-group on four wavefronts that each own a
                          * full register file: per MFMA half the dequantiser arithmetic and half the LDS operand traffic; scales
                          * and zero points are gathered into registers, so any number of groups per row and 2-byte aligned
-                         * scale / zero tensors will do.  K % 128 == 0, M % 4 == 0, N % 16 == 0, power-of-two group >= 32; workspace
-                         * as for TLQ_ALGO_PANEL */
+                         * scale / zero tensors will do; a zero-point tensor is handled inside the one launch (folded while the
+                         * zero points are small integers, unfolded from the first step whose are not).  K % 128 == 0, M % 4 == 0,
+                         * N % 16 == 0, power-of-two group >= 32.  Workspace: the fp32 partial tiles where K is cut into slices */
   ,
   TLQ_ALGO_PANELM = 9 /* middle M (tens to hundreds of activation rows): the four-wavefront panel structure on 64 or 128
                        * activation rows x 256 weight rows per work-group, a ring of four / three LDS slots, scales and zero

@@ -6,7 +6,7 @@ unpack-then-GEMM wrapper, examples/dequantize_gemm/example_dequant_gemm_fine_gra
 Without a GPU: their plans, the host walk over every direct load, gather, LDS cell and operand read of a launch, and for
 the 256-row kernel its schedule of loads, waits and barriers played through on the host (with wrong wait counts it must
 fail).  On the GPU: against the oracle on ragged shapes, all zero-point kinds (a zero-point tensor with fractional values
-takes the second, unfolded launch), every group size, one and many K slices, both activation types and both word layouts;
+makes the 256-row kernel change dequantiser on the way and the 128-row kernel take a second, unfolded launch), every group size, one and many K slices, both activation types and both word layouts;
 with one-hot activations the outputs must be the dequantised weights bit for bit."""
 import ctypes
 

@@ -64,7 +64,7 @@ struct Panel2Plan {
 Panel2Plan w4a16_panel256_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cus);
 int gemm_w4a16_panel256(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N, int64_t K,
                         int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const Panel2Plan& p, float* partial,
-                        uint32_t* flag, hipStream_t st);
+                        hipStream_t st);
 extern thread_local int g_panel2_slice_steps;
 struct PanelMPlan {
   bool ok;
@@ -377,11 +377,10 @@ static int try_panel256(const void* A, const void* w_packed, const void* scales,
                        (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) && (M * N) % 4 == 0 &&
                        fits32(M, K * 2) && fits32(N, K / 2) && fits32(N, (K / group) * 2);
   if (!args_ok) return -1;
-  const int64_t part_bytes = pp.split > 1 ? (int64_t)pp.split * M * N * 4 : 0;
-  const int64_t need = part_bytes + (zeros ? 16 : 0);
+  const int64_t need = pp.split > 1 ? (int64_t)pp.split * M * N * 4 : 0;
   if (need > 0 && !(workspace && aligned16(workspace) && workspace_bytes >= need)) return -1;
   return gemm_w4a16_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, pp,
-                             (float*)workspace, zeros ? (uint32_t*)((uint8_t*)workspace + part_bytes) : nullptr, (hipStream_t)stream);
+                             (float*)workspace, (hipStream_t)stream);
 }
 
 // The middle-M panel kernel.  Returns -1 when it does not take the problem (nothing launched, no error set).
@@ -417,7 +416,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
                                 workspace_bytes, stream);
     TLQ_REQUIRE(rc >= 0, "tlq_gemm_w4a16_ws: the 256-row panel kernel needs K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group "
-                ">= 32, 16-byte aligned operands and a workspace for its K slices and (with a zero-point tensor) 16 bytes more (M=%lld "
+                ">= 32, 16-byte aligned operands and a workspace for its K slices (M=%lld "
                 "N=%lld K=%lld group=%lld, workspace %lld)", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
     return rc;
   }

@@ -17,9 +17,10 @@
 //     of the step after next in flight, vmcnt(16) in the middle leaves the next activation tile), every step issues the
 //     same number of loads (past the end: the last step again, into a slot nobody reads).
 // The k assignment inside a step, both LDS tile layouts and their swizzles are the streaming kernel's (gemm_addr.h:
-// sw_*, sa_* with sixteen activation tiles).  Zero-point tensors: as in the 128-row kernel, one step loop per kernel
-// and a flag word for the unfolded second launch.
-#include <atomic>
+// sw_*, sa_* with sixteen activation tiles).  Zero-point tensors: the kernel holds both step loops (the accumulators sit in
+// the accumulation registers either way, so two loops do not cost spills) and runs folded while the zero points of the
+// step ahead are small integers; from the first step whose zero points are not, the rest runs unfolded (on integral
+// zero points the two dequantisers give the same bits, so the switch does not show in the result).
 #include <type_traits>
 
 #include "expand8.h"
@@ -70,25 +71,19 @@ struct Panel2Cfg {
   static_assert(SLOT == (int)addr::kPanel2Slot && LA == 16 && TN == 4, "layout shared with the host walker; the waits below count these loads");
 };
 
-// ZM as in the 128-row kernel: 0 = zero-point tensor, folded, *flag = epoch when a zero point is not a small integer;
-// 1 = no tensor, integer zero point (folded); 2 = no tensor (unfolded); 3 = tensor, unfolded, runs only if *flag == epoch.
+// ZM: 0 = zero-point tensor (folded while the zero points allow it, then unfolded); 1 = no tensor, integer zero point
+// (folded); 2 = no tensor (unfolded)
 template <typename T, int LAYOUT, int ZM>
 __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
                                                                const T* __restrict__ scales, const T* __restrict__ zeros,
                                                                void* __restrict__ C, float* __restrict__ partial, int M, int N, int K,
                                                                int gshift, float zero_scalar, int out_dtype, int slice_steps,
-                                                               int tiles_m, int tiles_n, int band_rows, uint32_t* __restrict__ flag,
-                                                               uint32_t epoch) {
+                                                               int tiles_m, int tiles_n, int band_rows) {
   typedef Panel2Cfg Cfg;
   typedef Panel2Mma<T> Mma;
   typedef __attribute__((address_space(3))) uint8_t* lptr_t;
-  if constexpr (ZM == 3) {
-    if (__builtin_nontemporal_load(flag) != epoch) return;  // (uniform: every wavefront of the launch takes the same way)
-  }
   constexpr int TM = Cfg::TM, TN = Cfg::TN, LA = Cfg::LA;
-  constexpr bool HAS_Z = ZM == 0 || ZM == 3;
-  constexpr bool FOLD = ZM == 0 || ZM == 1;
-  typedef Expand8<T, FOLD, LAYOUT> Ex;
+  constexpr bool HAS_Z = ZM == 0;
   extern __shared__ __align__(16) uint8_t smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -141,7 +136,8 @@ __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restr
   auto sc_src = [&](const uint8_t* tensor, bool present, int s) {
     return uniform_ptr(present ? tensor + addr::panel2_sc_step(step0 + clamp_step(s), gshift) : tensor);
   };
-  uint32_t sv_raw[TN], zv_raw[TN];    // the step's whose dequantiser constants are made next
+  uint32_t sv_step[TN], zv_step[TN];  // of the current step (kept for a change of dequantiser)
+  uint32_t sv_raw[TN], zv_raw[TN];    // of the next step: the dequantiser constants made next
   uint32_t sv_load[TN], zv_load[TN];  // in flight
   auto issue_sc1 = [&](int i, const uint8_t* ssrc, const uint8_t* zsrc) {  // gather i (of 8)
     const int tn = i >> 1;
@@ -159,25 +155,23 @@ __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restr
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
       asm volatile("" : "+v"(sv_load[tn]), "+v"(zv_load[tn]));
+      sv_step[tn] = sv_raw[tn], zv_step[tn] = zv_raw[tn];
       sv_raw[tn] = sv_load[tn], zv_raw[tn] = zv_load[tn];
     }
   };
   const uint32_t one_bits = (uint32_t)bitcast<uint16_t>(from_float<T>(1.0f)), zs_bits = (uint32_t)bitcast<uint16_t>(from_float<T>(zero_scalar));
-  uint32_t z_fract_bits = 0;
-  float z_max_abs = 0.0f;
-  Ex exs[TN];
   const NibbleMagic mg = make_nibble_magic();
-  auto make_expander = [&](int tn) {  // from sv_raw / zv_raw, absent tensors replaced by their constants
-    const uint32_t sb = has_s ? sv_raw[tn] : one_bits, zb = HAS_Z ? zv_raw[tn] : zs_bits;
-    const T sv = bitcast<T>((uint16_t)sb), zv = bitcast<T>((uint16_t)zb);
-    if constexpr (ZM == 0) {
-      // three instructions per zero point, the comparisons once behind the loop: the fractional parts' bits or-ed
-      // together (not zero for a fraction or a NaN), and the largest magnitude
-      const float zf = to_float(zv);
-      z_fract_bits |= bitcast<uint32_t>(__builtin_amdgcn_fractf(zf));
-      z_max_abs = __builtin_fmaxf(z_max_abs, __builtin_fabsf(zf));
+  // are these raw zero points (one per weight tile and lane) small integers, for every lane of the wavefront?
+  auto integral = [&](const uint32_t (&zb)[TN]) -> bool {
+    uint32_t fract_bits = 0;  // not zero for a fraction or a NaN
+    float max_abs = 0.0f;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const float zf = to_float(bitcast<T>((uint16_t)zb[tn]));
+      fract_bits |= bitcast<uint32_t>(__builtin_amdgcn_fractf(zf));
+      max_abs = __builtin_fmaxf(max_abs, __builtin_fabsf(zf));
     }
-    exs[tn] = Ex(sv, zv, mg);
+    return __builtin_amdgcn_ballot_w64(fract_bits == 0 && max_abs <= 256.0f) == ~0ull;
   };
 
   typename Mma::acc_t acc[TN][TM];
@@ -195,36 +189,6 @@ __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restr
   // two vector instructions behind every second MFMA), the words of k-step ks + 2 are read.
   uint4_t wop[2][TN];   // expanded weight operands: [k-step parity][tn]
   uint32_t ww[2][TN];   // packed words: [k-step parity][tn]
-  auto read_words = [&](int s, int ks) {  // word ks of step s of every weight tile, into set ks % 2
-    const uint8_t* slot = smem + (s & 1) * Cfg::SLOT;
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn) ww[ks & 1][tn] = *(const uint32_t*)(slot + fo_w + tn * 1024 + ks * 4);
-  };
-  auto expand_piece = [&](int part, int ks, int i, typename Ex::Pieces& st, uint32_t shifted) {
-    const int tn = part >> 1, p = part & 1;
-    uint4_t& o = wop[ks & 1][tn];
-    uint32_t& w = ww[ks & 1][tn];
-    if constexpr (Ex::SPLITS) {
-      if (i == 0) {
-        if (p == 0) {
-          asm volatile("" : "+v"(w));
-          exs[tn].piece(st, w, 0, 0);
-        } else {
-          exs[tn].piece(st, shifted, 0, 0);  // (shifted = w >> 8: the word's second half, read like a first)
-        }
-      } else {
-        st.pin(i - 1);
-        exs[tn].piece(st, w, p, i);
-      }
-      if (i == 3) {
-        st.pin(3);
-        Ex::place(o, uint2_t{st.a, st.b}, p);
-      }
-    } else {
-      if (p == 0 && i == 0) o = exs[tn](w);
-    }
-  };
-
   // Loads of one step, in issue order (addr::panel2_slot_load): 16 of the activation tile of step s + 1 (phase 0, one per
   // slot), 8 gathers of the scales of step s + 2 (phase 1), 4 of the packed weights of step s + 2 (behind the barrier).
   // Loads retire in order, so "at most n outstanding" means "everything but the youngest n has landed":
@@ -251,8 +215,6 @@ __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restr
 #pragma unroll
     for (int j = 0; j < LA; ++j) issue_a1(0, j, asrc);
     pin_scales();  // (the compiler's wait: everything so far)
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn) make_expander(tn);
     const uint8_t *s1 = sc_src(s_tensor, has_s, 1), *z1 = sc_src(z_tensor, HAS_Z, 1);
 #pragma unroll
     for (int i = 0; i < 8; ++i) issue_sc1(i, s1, z1);
@@ -262,19 +224,10 @@ __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restr
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     pin_scales();
   }
-  __syncthreads();
-  read_words(0, 0);
-  read_words(0, 1);
+  __syncthreads();  // (sv_step / zv_step: step 0, sv_raw / zv_raw: step 1)
 #pragma unroll
   for (int j = 0; j < AR - 1; ++j) af[j] = *(const uint4_t*)(smem + fo_a(0) + j * 16 * 256);
   af[AR - 1] = af[0];  // (read in slot 0)
-  {
-    typename Ex::Pieces st;
-#pragma unroll
-    for (int part = 0; part < 2 * TN; ++part)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) expand_piece(part, 0, i, st, ww[0][part >> 1] >> 8);
-  }
   // Where what stands inside a slot of four MFMAs (measured on this part with one wavefront per SIMD: an MFMA takes
   // 16 cycles of the matrix pipeline and 8 of the wavefront's issue; two vector instructions behind it are free, a third
   // costs 4 cycles; an LDS read is free behind an MFMA that another MFMA follows, and costs 4 cycles when a wait for LDS
@@ -296,7 +249,63 @@ __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restr
   for (int ks = 0; ks < 4; ++ks) a_k[ks] = lds0 + fo_a(ks);
   uint32_t w_cur = lds0 + fo_w, w_nxt = lds0 + fo_w + Cfg::SLOT;
   const uint8_t* asrc = a_src(1);
-  for (int s = 0; s < steps; ++s) {
+  // One pass over steps [s_begin, s_end) with one dequantiser.  On entry the ring, the loads in flight and the operand ring
+  // af are as the previous pass (or the prologue) left them; the words, the dequantiser constants and the expanded first
+  // k-step of step s_begin are (re)made here, because the previous pass made them with the other dequantiser.  With
+  // stop_on_fraction the pass ends in front of the first step during which constants would be made from zero points that
+  // are not small integers, and returns that step.
+  auto run_steps = [&](int s_begin, int s_end, auto fold_tag, bool stop_on_fraction) -> int {
+    constexpr bool FOLD = decltype(fold_tag)::value;
+    typedef Expand8<T, FOLD, LAYOUT> Ex;
+    Ex exs[TN];
+    auto make_expander = [&](int tn, const uint32_t (&sraw)[TN], const uint32_t (&zraw)[TN]) {  // absent tensors replaced by their constants
+      const uint32_t sb = has_s ? sraw[tn] : one_bits, zb = HAS_Z ? zraw[tn] : zs_bits;
+      exs[tn] = Ex(bitcast<T>((uint16_t)sb), bitcast<T>((uint16_t)zb), mg);
+    };
+    auto expand_piece = [&](int part, int ks, int i, typename Ex::Pieces& st, uint32_t shifted) {
+      const int tn = part >> 1, p = part & 1;
+      uint4_t& o = wop[ks & 1][tn];
+      uint32_t& w = ww[ks & 1][tn];
+      if constexpr (Ex::SPLITS) {
+        if (i == 0) {
+          if (p == 0) {
+            asm volatile("" : "+v"(w));
+            exs[tn].piece(st, w, 0, 0);
+          } else {
+            exs[tn].piece(st, shifted, 0, 0);  // (shifted = w >> 8: the word's second half, read like a first)
+          }
+        } else {
+          st.pin(i - 1);
+          exs[tn].piece(st, w, p, i);
+        }
+        if (i == 3) {
+          st.pin(3);
+          Ex::place(o, uint2_t{st.a, st.b}, p);
+        }
+      } else {
+        if (p == 0 && i == 0) o = exs[tn](w);
+      }
+    };
+
+    {
+      const uint8_t* slot = smem + (s_begin & 1) * Cfg::SLOT;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        ww[0][tn] = *(const uint32_t*)(slot + fo_w + tn * 1024);
+        ww[1][tn] = *(const uint32_t*)(slot + fo_w + tn * 1024 + 4);
+        make_expander(tn, sv_step, zv_step);
+      }
+      typename Ex::Pieces st;
+#pragma unroll
+      for (int part = 0; part < 2 * TN; ++part)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) expand_piece(part, 0, i, st, ww[0][part >> 1] >> 8);
+    }
+    int s = s_begin;
+    for (; s < s_end; ++s) {
+    if constexpr (ZM == 0) {
+      if (stop_on_fraction && !integral(zv_raw)) break;  // (zv_raw: the zero points of step s + 1)
+    }
     const uint8_t *const ssrc = sc_src(s_tensor, has_s, s + 2), *const zsrc = sc_src(z_tensor, HAS_Z, s + 2);
     const uint8_t* const wsrc = w_src(s + 2);
     uint32_t wsh = 0;
@@ -311,7 +320,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restr
       }
       // the dequantiser constants of step s + 1, from the values taken over a step ago
       if constexpr (t >= addr::kPanel2ExpanderSlot && t < addr::kPanel2ExpanderSlot + 4 * TN && (t - addr::kPanel2ExpanderSlot) % 4 == 0)
-        make_expander((t - addr::kPanel2ExpanderSlot) / 4);
+        make_expander((t - addr::kPanel2ExpanderSlot) / 4, sv_raw, zv_raw);
       if constexpr (t == addr::kPanel2BarrierSlot) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(addr::kPanel2WaitA) : "memory");
         pin_scales();  // those of step s + 2
@@ -362,11 +371,17 @@ __global__ __launch_bounds__(256, 1) void w4a16_panel256_kernel(const T* __restr
       a_nxt = x;
     }
     { const uint32_t x = w_cur; w_cur = w_nxt; w_nxt = x; }
-  }
+    }
+    return s;
+  };
   if constexpr (ZM == 0) {
-    const bool all_integral = z_fract_bits == 0 && z_max_abs <= 256.0f;
-    if (__builtin_amdgcn_ballot_w64(all_integral) != ~0ull && lane == 0)
-      __hip_atomic_store(flag, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    int s = 0;
+    if (integral(zv_step)) s = run_steps(0, steps, std::true_type{}, true);
+    if (s < steps) run_steps(s, steps, std::false_type{}, false);
+  } else if constexpr (ZM == 1) {
+    run_steps(0, steps, std::true_type{}, false);
+  } else {
+    run_steps(0, steps, std::false_type{}, false);
   }
 
   // lane (r16, q) holds C[m = m0 + 16 tm + r16][n = n0 + 64 wave + 16 tn + 4 q + 0..3]
@@ -427,7 +442,7 @@ Panel2Plan w4a16_panel256_plan(int64_t M, int64_t N, int64_t K, int64_t group, i
 template <typename T, int LAYOUT, int ZM>
 static int launch_panel256(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, float* partial, int64_t M,
                            int64_t N, int64_t K, int gshift, float zero_scalar, int out_dtype, const Panel2Plan& p, int band_rows,
-                           uint32_t* flag, uint32_t epoch, hipStream_t st) {
+                           hipStream_t st) {
   auto kern = w4a16_panel256_kernel<T, LAYOUT, ZM>;
   constexpr int lds_bytes = Panel2Cfg::LDS;
   static bool attr_set = false;
@@ -441,34 +456,28 @@ static int launch_panel256(const void* A, const void* Wp, const void* scales, co
   }
   const unsigned blocks = (unsigned)((int64_t)p.tiles_m * p.tiles_n * p.split);
   kern<<<blocks, 256, lds_bytes, st>>>((const T*)A, (const uint8_t*)Wp, (const T*)scales, (const T*)zeros, C, partial, (int)M, (int)N,
-                                       (int)K, gshift, zero_scalar, out_dtype, p.slice_steps, p.tiles_m, p.tiles_n, band_rows, flag, epoch);
-  return check_launch("tlq_gemm_w4a16(panel256)", ZM == 0 ? "w4a16_panel256_kernel, zero-point tensor folded"
-                                                        : (ZM == 3 ? "w4a16_panel256_kernel, unfolded behind the flag" : "w4a16_panel256_kernel"))
+                                       (int)K, gshift, zero_scalar, out_dtype, p.slice_steps, p.tiles_m, p.tiles_n, band_rows);
+  return check_launch("tlq_gemm_w4a16(panel256)", ZM == 0 ? "w4a16_panel256_kernel, zero-point tensor" : "w4a16_panel256_kernel")
              ? 0
              : 1;
 }
 
 // partial: fp32 [split][M][N] workspace, needed when the plan has more than one K slice
-// flag: one 32-bit word of device memory of the caller's (any contents), needed with a zero-point tensor
 int gemm_w4a16_panel256(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N, int64_t K,
                         int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, const Panel2Plan& p, float* partial,
-                        uint32_t* flag, hipStream_t st) {
+                        hipStream_t st) {
   int gshift = 0;
   while (((int64_t)1 << gshift) < group) ++gshift;
   const int band = g_gemm_band_rows > 0 ? g_gemm_band_rows : 4;
   const bool fold_scalar = zero_scalar == (float)(int)zero_scalar && zero_scalar >= -256.0f && zero_scalar <= 256.0f;
-  static std::atomic<uint32_t> epochs{0x5eed8001u};
-  const uint32_t epoch = zeros != nullptr ? epochs.fetch_add(1, std::memory_order_relaxed) : 0u;
   int rc;
-#define TLQ_PANEL3(T, LAY, ZM) launch_panel256<T, LAY, ZM>(A, Wp, scales, zeros, C, partial, M, N, K, gshift, zero_scalar, out_dtype, p, band, flag, epoch, st)
+#define TLQ_PANEL3(T, LAY, ZM) launch_panel256<T, LAY, ZM>(A, Wp, scales, zeros, C, partial, M, N, K, gshift, zero_scalar, out_dtype, p, band, st)
 #define TLQ_PANEL2(T, ZM) (w_layout == TLQ_W_INTERLEAVED_F16 ? TLQ_PANEL3(T, 1, ZM) : TLQ_PANEL3(T, 0, ZM))
 #define TLQ_PANEL(ZM) (in_dtype == TLQ_F16 ? TLQ_PANEL2(half_t, ZM) : TLQ_PANEL2(bf16_t, ZM))
-  if (zeros != nullptr) {
+  if (zeros != nullptr)
     rc = TLQ_PANEL(0);
-    if (!rc) rc = TLQ_PANEL(3);
-  } else {
+  else
     rc = fold_scalar ? TLQ_PANEL(1) : TLQ_PANEL(2);
-  }
 #undef TLQ_PANEL
 #undef TLQ_PANEL2
 #undef TLQ_PANEL3
