@@ -172,6 +172,9 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 /* The least workspace with which tlq_gemm_w4a16_ws still takes a workspace-based kernel for this shape (the partial sums
  * of the K-slice kernels where they apply, else the dequantised matrix of the two passes); for callers short of memory. */
 int64_t tlq_w4a16_workspace_bytes_min(int64_t M, int64_t N, int64_t K);
+/* What the explicitly named family `algo` may ask of the workspace for this shape (any group size); 0 for the families that
+ * use none.  TLQ_ALGO_AUTO: tlq_w4a16_workspace_bytes. */
+int64_t tlq_w4a16_workspace_bytes_for(int64_t M, int64_t N, int64_t K, int algo);
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream);
@@ -184,6 +187,24 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
 int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                              int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                              int w_layout, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Tuned kernel choice.  The reference searches its configurations per call signature and keeps the winner, in memory and
+ * on disk (tilelang/autotuner/tuner.py:102-760 AutoTuner.run, tilelang/cache/tuner_cache.py).  The kernels here are pre-built,
+ * so what a search finds is WHICH family runs: a process-wide table (M, N, K, group, in_dtype) -> TLQ_ALGO_* that
+ * tlq_gemm_w4a16, tlq_gemm_w4a16_ws (and through it tlq_gemm_w4a16_noalloc and tlq_gemm_w4a16_layout_ws with TLQ_W_PLAIN)
+ * consult before their own rules when called with TLQ_ALGO_AUTO.  A chosen family that refuses the call -- its shape rules,
+ * the alignment of an operand, a workspace smaller than tlq_w4a16_workspace_bytes_for asks -- launches nothing and the
+ * call proceeds by the rules, without an error.  tlq_w4a16_workspace_bytes covers the choices present for (M, N, K).
+ * choice_set with TLQ_ALGO_AUTO removes an entry.  choice_save / choice_load: one entry per text line,
+ * "M N K group in_dtype algo" in the codes of this header, '#' comments; load adds to (and overrides) what the table holds
+ * and changes nothing when a line is malformed.  All six are thread safe; a choice made on one GPU model is not meant for
+ * another (keep one file per device).  tilelang_ascend_amd.autotuner.tune_w4a16_choice fills the table by measurement. */
+int tlq_w4a16_choice_set(int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype, int algo);
+int tlq_w4a16_choice_get(int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype);
+void tlq_w4a16_choice_clear(void);
+int64_t tlq_w4a16_choice_count(void);
+int tlq_w4a16_choice_save(const char* path);
+int tlq_w4a16_choice_load(const char* path);
 
 /* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose wrapper allocates its

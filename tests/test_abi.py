@@ -14,7 +14,7 @@ HEADER = os.path.join(ROOT, "include", "tlq.h")
 DEBUG_HEADER = os.path.join(ROOT, "include", "tlq_debug.h")
 
 CTYPE = {"const void*": ctypes.c_void_p, "void*": ctypes.c_void_p, "int64_t": ctypes.c_int64, "int": ctypes.c_int,
-         "float": ctypes.c_float}
+         "float": ctypes.c_float, "const char*": ctypes.c_char_p}
 RESTYPE = {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "void": None, "const char*": ctypes.c_char_p}
 
 
@@ -29,7 +29,7 @@ def declared(headers=(HEADER, DEBUG_HEADER)):
         if args != "void":
             for a in args.split(","):
                 a = a.strip()
-                t = re.match(r"(const void\*|void\*|int64_t|int|float)\s*\w+$", a)
+                t = re.match(r"(const void\*|void\*|const char\*|int64_t|int|float)\s*\w+$", a)
                 assert t, f"{name}: argument '{a}' is not a plain pointer / size / code"
                 types.append(t.group(1))
         out[name] = (ret, types)

@@ -22,7 +22,7 @@ W_PLAIN, W_INTERLEAVED_F16 = 0, 1
 ALGO_AUTO, ALGO_GEMV, ALGO_MFMA, ALGO_SKINNY, ALGO_TWO_PASS, ALGO_STREAM, ALGO_DECODE, ALGO_PANEL, ALGO_PANEL256, ALGO_PANELM = 0, 1, 2, 3, 4, 5, 6, 7, 8, 9
 ABI_VERSION = 1
 
-_vp, _i64, _int, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+_vp, _i64, _int, _f32, _cstr = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_char_p
 
 # name -> (restype, argtypes); kept in step with include/tlq.h (a test compares the two)
 SIGNATURES = {
@@ -44,6 +44,13 @@ SIGNATURES = {
     "tlq_gemm_w8a8_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "tlq_w4a16_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "tlq_w4a16_workspace_bytes_min": (_i64, [_i64, _i64, _i64]),
+    "tlq_w4a16_workspace_bytes_for": (_i64, [_i64, _i64, _i64, _int]),
+    "tlq_w4a16_choice_set": (_int, [_i64, _i64, _i64, _i64, _int, _int]),
+    "tlq_w4a16_choice_get": (_int, [_i64, _i64, _i64, _i64, _int]),
+    "tlq_w4a16_choice_clear": (None, []),
+    "tlq_w4a16_choice_count": (_i64, []),
+    "tlq_w4a16_choice_save": (_int, [_cstr]),
+    "tlq_w4a16_choice_load": (_int, [_cstr]),
     "tlq_gemm_w4a16_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp, _i64, _vp]),
     "tlq_gemm_w4a16_layout_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _int, _vp, _i64, _vp]),
     "tlq_dequant_w4_layout": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _int, _int, _vp]),

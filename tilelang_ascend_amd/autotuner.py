@@ -324,3 +324,161 @@ def autotune(func: Callable = None, *, configs: Union[Sequence[dict], Callable],
         return AutoTuneImpl(factory, **opts)
 
     return decorator
+
+
+# ---- tuned kernel choice for the C entry points ------------------------------------------------------------------
+# The reference's tuner result selects a compiled kernel; here it selects which pre-built W4A16 family
+# ``tlq_gemm_w4a16_ws`` runs for a call signature when asked for TLQ_ALGO_AUTO.  The result lives in the library's own
+# table (tlq_w4a16_choice_set), so callers of the C ABI get it too, and in one text file per device size under
+# ``<cache dir>/autotuner`` (the reference's tuner cache lives there as well, tilelang/cache/tuner_cache.py), which
+# ``cache.clear_cache()`` removes and which ``ops.w4a16_gemm`` installs once per process.
+
+W4A16_FAMILIES = {"gemv": 1, "mfma": 2, "skinny": 3, "two_pass": 4, "stream": 5, "decode": 6, "panel": 7, "panel256": 8,
+                  "panelm": 9}
+_choices_lock = threading.Lock()
+_choices_loaded = False
+
+
+def w4a16_choice_path(cus: Optional[int] = None) -> str:
+    """The file that holds the tuned choices for devices with ``cus`` compute units (default: the current device)."""
+    from . import _abi
+    if cus is None:
+        cus = _abi.load().tlq_device_cu_count()
+    return os.path.join(AutoTuner.cache_dir(), f"w4a16_choices_{int(cus)}cu.txt")
+
+
+def load_w4a16_choices(path: Optional[str] = None) -> int:
+    """Install the entries of ``path`` (default: the current device's file) into the library's table; returns how many
+    entries the table holds afterwards.  A missing file installs nothing."""
+    from . import _abi
+    lib = _abi.load()
+    path = path or w4a16_choice_path()
+    if os.path.exists(path):
+        _abi.check(lib.tlq_w4a16_choice_load(path.encode()))
+    return int(lib.tlq_w4a16_choice_count())
+
+
+def save_w4a16_choices(path: Optional[str] = None) -> str:
+    """Write the library's table to ``path`` (default: the current device's file)."""
+    from . import _abi
+    path = path or w4a16_choice_path()
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    tmp = f"{path}.tmp{os.getpid()}"
+    _abi.check(_abi.load().tlq_w4a16_choice_save(tmp.encode()))
+    os.replace(tmp, path)
+    return path
+
+
+def clear_w4a16_choices() -> None:
+    """Empty the library's table (the file stays; ``cache.clear_cache()`` removes it)."""
+    from . import _abi
+    _abi.load().tlq_w4a16_choice_clear()
+
+
+def ensure_w4a16_choices_loaded() -> None:
+    """Once per process: install the current device's persisted choices, if there are any.  ``TLQ_TUNED_CHOICES=0``
+    turns this off.  Touches the GPU only when a choice file exists."""
+    global _choices_loaded
+    if _choices_loaded:
+        return
+    with _choices_lock:
+        if _choices_loaded:
+            return
+        _choices_loaded = True
+        if os.environ.get("TLQ_TUNED_CHOICES", "1") == "0":
+            return
+        try:
+            d = AutoTuner.cache_dir()
+            if not any(n.startswith("w4a16_choices_") and n.endswith("cu.txt") for n in os.listdir(d)):
+                return
+            load_w4a16_choices()
+        except (OSError, RuntimeError) as e:
+            logger.warning("tuned W4A16 kernel choices not installed: %s", e)
+
+
+def tune_w4a16_choice(M: int, N: int, K: int, group_size: int = 128, dtype: str = "float16", zeros: Optional[str] = "tensor",
+                      candidates: Optional[Sequence[str]] = None, rep: int = 20, rounds: int = 5, min_gain: float = 0.03,
+                      persist: bool = True, seed: int = 0) -> Dict[str, Any]:
+    """Measure the W4A16 kernel families on one call signature and make the fastest the library's choice for it.
+
+    Every family in ``candidates`` (default: all) is run through ``tlq_gemm_w4a16_ws`` by name with the workspace it asks
+    for (``tlq_w4a16_workspace_bytes_for``); families that refuse the shape are recorded under ``"skipped"`` with the
+    library's message, a family whose output is not close to the rule-based choice's is recorded under ``"rejected"``.
+    Timings are medians over ``rounds`` rounds of ``rep`` back-to-back launches, the families taking turns inside a round.
+    The winner is installed (``tlq_w4a16_choice_set``) when it beats the rule-based choice by ``min_gain`` or more;
+    otherwise any earlier entry for the signature is removed.  ``persist`` rewrites the device's choice file.
+
+    Returns ``{"choice": name | "auto", "latency_us": {name: us}, "skipped": {...}, "rejected": {...}, "path": file | None}``.
+    """
+    import statistics
+    from . import _abi
+    lib = _abi.load()
+    tdt = {"float16": torch.float16, "bfloat16": torch.bfloat16}[dtype]
+    code = {"float16": _abi.F16, "bfloat16": _abi.BF16}[dtype]
+    if zeros not in ("tensor", "scalar", None):
+        raise ValueError("zeros must be 'tensor', 'scalar' or None")
+    if K % group_size != 0:
+        raise ValueError("group_size must divide K")
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    Wp = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=g).to(dev)  # two random 4-bit codes per byte
+    A = torch.randn(M, K, generator=g).to(tdt).to(dev)
+    S = (torch.rand(N, K // group_size, generator=g) * 0.02 + 0.005).to(tdt).to(dev)
+    Z = torch.randint(0, 16, (N, K // group_size), generator=g).to(tdt).to(dev) if zeros == "tensor" else None
+    zs = 8.0 if zeros == "scalar" else 0.0
+    stream = torch.cuda.current_stream().cuda_stream
+    names = ["auto"] + [n for n in (candidates or W4A16_FAMILIES) if n != "auto"]
+    for n in names[1:]:
+        if n not in W4A16_FAMILIES:
+            raise ValueError(f"unknown family {n!r}; known: {sorted(W4A16_FAMILIES)}")
+    # the rule-based choice is the baseline: no entry for this signature while measuring
+    _abi.check(lib.tlq_w4a16_choice_set(M, N, K, group_size, code, 0))
+    need = max([lib.tlq_w4a16_workspace_bytes(M, N, K)] + [lib.tlq_w4a16_workspace_bytes_for(M, N, K, W4A16_FAMILIES[n]) for n in names[1:]])
+    ws = torch.empty(max(int(need), 16), dtype=torch.uint8, device=dev)
+    C = torch.empty(M, N, dtype=tdt, device=dev)
+
+    def call(name: str) -> int:
+        algo = 0 if name == "auto" else W4A16_FAMILIES[name]
+        return lib.tlq_gemm_w4a16_ws(_abi.ptr(A), _abi.ptr(Wp), _abi.ptr(S), _abi.ptr(Z), _abi.ptr(C), M, N, K, group_size, zs, code,
+                                     code, algo, _abi.ptr(ws), ws.numel(), stream)
+
+    _abi.check(call("auto"))
+    torch.cuda.synchronize()
+    want = C.float().clone()
+    scale = float(want.abs().max().clamp_min(1e-6))
+    alive, skipped, rejected = ["auto"], {}, {}
+    for n in names[1:]:
+        C.zero_()
+        if call(n) != 0:
+            skipped[n] = _abi.last_error()
+            continue
+        torch.cuda.synchronize()
+        err = float((C.float() - want).abs().max()) / scale
+        if not err <= 2e-2:
+            rejected[n] = f"max |difference| / max |C| = {err:.3g} against the rule-based choice"
+            continue
+        alive.append(n)
+    times: Dict[str, List[float]] = {n: [] for n in alive}
+    for _ in range(max(1, rounds)):
+        for n in alive:
+            for _ in range(3):
+                call(n)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(rep):
+                call(n)
+            e1.record()
+            torch.cuda.synchronize()
+            times[n].append(e0.elapsed_time(e1) * 1000.0 / rep)
+    lat = {n: statistics.median(v) for n, v in times.items()}
+    named = [n for n in lat if n != "auto"]
+    best = min(named, key=lat.get) if named else "auto"
+    choice = best if best != "auto" and lat[best] <= lat["auto"] * (1.0 - min_gain) else "auto"
+    _abi.check(lib.tlq_w4a16_choice_set(M, N, K, group_size, code, 0 if choice == "auto" else W4A16_FAMILIES[choice]))
+    path = None
+    if persist:
+        try:
+            path = save_w4a16_choices()
+        except (OSError, RuntimeError) as e:
+            logger.warning("tuned W4A16 kernel choices not saved: %s", e)
+    return {"choice": choice, "latency_us": lat, "skipped": skipped, "rejected": rejected, "path": path}

@@ -40,6 +40,7 @@ SOURCES = [
     "gemm_w4a16_panel.hip",
     "gemm_w4a16_panel256.hip",
     "gemm_w4a16_panelm.hip",
+    "w4a16_choice.hip",
     "gemm_w4a16_decode.hip",
     "gemm_int8.hip",
     "gemm_f16.hip",

@@ -35,8 +35,13 @@ static void log_launch(const char* what, const char* detail) {
 }
 
 // Called right after a kernel launch: turns a launch failure into an error string.  detail: the kernel and its
-// variant, for the launch log.
+// variant, for the launch log.  launch_count: how often the calling thread has come through here -- an entry point that
+// returned an error without the count moving has refused its arguments and launched nothing.
+static thread_local uint64_t g_launches = 0;
+uint64_t launch_count() { return g_launches; }
+
 bool check_launch(const char* what, const char* detail) {
+  ++g_launches;
   if (g_log_on) log_launch(what, detail);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {

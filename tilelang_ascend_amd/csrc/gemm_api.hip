@@ -101,6 +101,10 @@ thread_local int g_w4a16_decode = 1;  // 0: never pick the decode kernel automat
 // the tile loaders address one matrix with 32-bit byte offsets
 static bool fits32(int64_t rows, int64_t row_bytes) { return rows * row_bytes < ((int64_t)1 << 32); }
 static const int64_t kMaxDim = (int64_t)1 << 30;
+// the table of tuned kernel choices (w4a16_choice.hip)
+int w4a16_choice_lookup(int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype);
+void w4a16_choice_for_shape(int64_t M, int64_t N, int64_t K, void (*fn)(int algo, void* ctx), void* ctx);
+
 }  // namespace tlq
 
 using namespace tlq;
@@ -178,6 +182,17 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
               "tlq_gemm_w4a16: out_dtype must be float16, bfloat16 or float32 (got %d)", out_dtype);
   TLQ_REQUIRE((algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_SKINNY) || algo == TLQ_ALGO_DECODE, "tlq_gemm_w4a16: bad algo %d", algo);
   if (M == 0 || N == 0) return 0;
+  if (algo == TLQ_ALGO_AUTO) {
+    // a tuned choice for this call signature (tlq_w4a16_choice_set) goes first; where that kernel refuses the call (its
+    // shape or alignment rules: nothing launched), the rules below decide as if there were none
+    const int chosen = w4a16_choice_lookup(M, N, K, group, in_dtype);
+    if ((chosen >= TLQ_ALGO_GEMV && chosen <= TLQ_ALGO_SKINNY) || chosen == TLQ_ALGO_DECODE) {
+      const uint64_t before = launch_count();
+      const int rc = tlq_gemm_w4a16(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, chosen, stream);
+      if (rc == 0 || launch_count() != before) return rc;
+      set_error("%s", "");
+    }
+  }
   TLQ_REQUIRE(K > 0 && K % 64 == 0, "tlq_gemm_w4a16: K=%lld must be a positive multiple of 64", (long long)K);
   TLQ_REQUIRE(group > 0 && K % group == 0 && group % 32 == 0,
               "tlq_gemm_w4a16: group=%lld must divide K=%lld and be a multiple of 32", (long long)group, (long long)K);
@@ -308,9 +323,44 @@ static int64_t panelm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 // streaming kernel is level or ahead by up to 15 %).
 static bool panelm_preferred(int64_t M, int64_t N, int64_t K) { return M >= 256 && M <= 512 && N * K >= ((int64_t)1 << 25); }
 
+// What an explicitly named kernel family may ask of the workspace for any group size.
+int64_t tlq_w4a16_workspace_bytes_for(int64_t M, int64_t N, int64_t K, int algo) {
+  if (M <= 0 || N <= 0 || K <= 0 || M >= kMaxDim || N >= kMaxDim || K >= kMaxDim) return 0;
+  switch (algo) {
+    case TLQ_ALGO_AUTO: return tlq_w4a16_workspace_bytes(M, N, K);
+    case TLQ_ALGO_TWO_PASS: return (N * K * 2 + 15) / 16 * 16 + tlq_f16_workspace_bytes(1, M, N, K);
+    case TLQ_ALGO_STREAM: {
+      const int64_t split = stream_max_split(M, N, K);
+      return split > 1 ? split * M * N * 4 : 0;
+    }
+    case TLQ_ALGO_DECODE: {
+      if (M > 32) return 0;
+      const DecodePlan dp = w4a16_decode_plan(M, N, K, 32, cu_count_or_default());
+      return dp.ok && dp.chunks > 1 ? (int64_t)dp.chunks * M * N * 4 : 0;
+    }
+    case TLQ_ALGO_MFMA: {  // with a workspace the tile kernel runs over K slices where it has few output tiles
+      const int64_t split = w4a16_mid_split(M, N, K, 32);
+      return split > 1 ? split * M * N * 4 : 0;
+    }
+    case TLQ_ALGO_PANEL:
+    case TLQ_ALGO_PANEL256: return panel_workspace_bytes(M, N, K);
+    case TLQ_ALGO_PANELM: return panelm_workspace_bytes(M, N, K);
+    default: return 0;  // GEMV, skinny: no workspace
+  }
+}
+
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
   int64_t need = w4a16_partial_sum_bytes(M, N, K);
+  // tuned choices for this shape (any group, any type): room for the chosen family as well
+  int64_t tuned[4] = {0, M, N, K};
+  w4a16_choice_for_shape(M, N, K, [](int algo, void* ctx) {
+    int64_t* const n = (int64_t*)ctx;
+    if (algo == TLQ_ALGO_AUTO) return;
+    const int64_t b = tlq_w4a16_workspace_bytes_for(n[1], n[2], n[3], algo);
+    if (b > n[0]) n[0] = b;
+  }, tuned);
+  if (tuned[0] > need) need = tuned[0];
   if (panelm_preferred(M, N, K)) {
     const int64_t pm = panelm_workspace_bytes(M, N, K);
     if (pm > need) need = pm;
@@ -405,6 +455,18 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
   TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_PANELM, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  if (algo == TLQ_ALGO_AUTO && M >= 1 && N >= 1) {
+    // a tuned choice for this call signature goes first (as in tlq_gemm_w4a16); a kernel that refuses the call -- its shape
+    // rules, the alignment of an operand, a workspace smaller than it needs -- has launched nothing, and the rules decide
+    const int chosen = w4a16_choice_lookup(M, N, K, group, in_dtype);
+    if (chosen != TLQ_ALGO_AUTO) {
+      const uint64_t before = launch_count();
+      const int rc = tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, chosen, workspace,
+                                       workspace_bytes, stream);
+      if (rc == 0 || launch_count() != before) return rc;
+      set_error("%s", "");
+    }
+  }
   if (algo == TLQ_ALGO_PANELM) {
     const int rc = try_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, workspace, workspace_bytes, stream);
     TLQ_REQUIRE(rc >= 0, "tlq_gemm_w4a16_ws: the middle-M panel kernel needs K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group "

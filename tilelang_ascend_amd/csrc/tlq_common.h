@@ -13,6 +13,7 @@ namespace tlq {
 // ---- error reporting (thread local, read back through tlq_last_error) -------------------
 void set_error(const char* fmt, ...);
 bool check_launch(const char* what, const char* detail = nullptr);
+uint64_t launch_count();
 
 #define TLQ_REQUIRE(cond, ...)      \
   do {                              \

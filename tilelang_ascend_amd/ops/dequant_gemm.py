@@ -172,7 +172,9 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
     | "stream" (wavefront-private packed weights dequantised in registers, 17 <= M <= 512: what "auto" does up to
     M = 384) | "panel" (large M in one launch: packed weights copied to LDS as they are and dequantised on the MFMA operand
     read; what "auto" does from 513 to 2048 rows where its work-groups fill the machine) | "two_pass" (dequantise into a
-    workspace, then the plain GEMM: what "auto" does otherwise above 512 rows).  A workspace
+    workspace, then the plain GEMM: what "auto" does otherwise above 512 rows).  "auto" first consults the library's table
+    of tuned choices (autotuner.tune_w4a16_choice; the device's persisted choices are installed on the first launch unless
+    TLQ_TUNED_CHOICES=0).  A workspace
     (split-K partial sums or the [N, K] dequantised weights) is taken from torch's stream-ordered allocator on every
     call, as the reference allocates its workspace_idx buffers per call, so launches on different streams do not share one;
     when the launch stream (forward(stream=...)) is not torch's current stream the block is recorded on it (_abi.scratch).
@@ -218,11 +220,13 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
         C = t[i]
         lib = _abi.load()
         ws = None
-        ws_bytes = 0
-        if algo in ("auto", "two_pass", "stream", "decode", "panel", "panel256"):
-            ws_bytes = lib.tlq_w4a16_workspace_bytes(M, N, K)
-            if algo == "two_pass" or (layout_code != _abi.W_PLAIN and algo == "auto" and M > 256):
-                ws_bytes = max(ws_bytes, N * K * 2)
+        if algo == "auto":
+            from ..autotuner import ensure_w4a16_choices_loaded
+            ensure_w4a16_choices_loaded()  # (once per process: the device's persisted tuned choices, if any)
+        # what the named family asks for ("auto": the rule-based choice and any tuned choice for this shape)
+        ws_bytes = lib.tlq_w4a16_workspace_bytes_for(M, N, K, algo_code)
+        if layout_code != _abi.W_PLAIN and algo == "auto" and M > 256:
+            ws_bytes = max(ws_bytes, N * K * 2)
         if ws_bytes:
             ws = _abi.scratch(ws_bytes, A.device, stream)
         with _abi.tuning(w4a16_tile=tile, gemv=gemv_tuning, skinny=skinny_tuning):
