@@ -608,3 +608,15 @@ def test_auto_picks_a_kernel_for_every_m(ops, in_dtype, N, K, group):
         A = torch.randn(M, K, generator=gen(44)).to(dt)
         got = _run_w4a16(ops, A, Wp, s, z, group, in_dtype, "auto", in_dtype)
         check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"auto {in_dtype} M={M} K={K}")
+
+
+@pytest.mark.parametrize("M,N,K,algo", [(64, 4096, 4096, "auto"), (256, 2048, 4096, "panelm"), (16, 2048, 8192, "decode"),
+                                        (1024, 1024, 1024, "panel256")])
+def test_profiler_assert_consistent_on_kernels_that_add_partial_sums(ops, M, N, K, algo):
+    """The reference's race check (tilelang/profiler/__init__.py:188-205) on the kernels whose K slices or wavefronts add
+    partial sums: every repeat must reproduce the first run bit for bit."""
+    kernel = ops.w4a16_gemm(M, N, K, group_size=128, zeros="tensor", algo=algo)
+    Wp, s, z = make_w4(N, K, 128, torch.float16, "int", seed=M)
+    A = torch.randn(M, K, generator=gen(N)).half()
+    print(f"assert_consistent M={M} N={N} K={K} algo={algo}", flush=True)
+    kernel.get_profiler().assert_consistent(repeat=5, input_tensors=[A.cuda(), Wp.cuda(), s.cuda(), z.cuda()])

@@ -156,6 +156,35 @@ def test_profiler_module_surface():
     assert profiler.TensorSupplyType.Auto.value == 7 and callable(profiler.do_bench)
 
 
+def test_profiler_assert_consistent_compares_repeated_runs(monkeypatch):
+    """The reference's race check (tilelang/profiler/__init__.py:188-205) on a stand-in kernel: equal runs pass, a run
+    that differs in one bit fails, and the inputs of every run are the same tensors."""
+    from tilelang_ascend_amd import profiler
+
+    monkeypatch.setattr(torch.cuda, "synchronize", lambda *a, **k: None)
+
+    class Fake:
+        params, result_idx, workspace_idx = [], [], []
+
+        def __init__(self, flaky_at=None):
+            self.calls, self.flaky_at = 0, flaky_at
+
+        def __call__(self, x):
+            self.calls += 1
+            out = x * 2
+            if self.calls == self.flaky_at:
+                out = out.clone()
+                out.view(torch.int16)[3] ^= 1  # one mantissa bit: allclose would let it pass
+            return out
+
+    x = torch.arange(16, dtype=torch.float16)
+    good = Fake()
+    profiler.Profiler(good).assert_consistent(repeat=4, input_tensors=[x])
+    assert good.calls == 5
+    with pytest.raises(AssertionError, match="not consistent: run 3"):
+        profiler.Profiler(Fake(flaky_at=3)).assert_consistent(repeat=4, input_tensors=[x])
+
+
 def test_build_lock_is_exclusive_and_stale_libraries_are_detected(tmp_path, monkeypatch):
     """Two builders never run at once (advisory file lock), and a library whose build record names other sources
     than those on disk counts as stale; one without a record is taken as it is."""

@@ -145,6 +145,27 @@ class Profiler:
                 raise AssertionError(f"{n_bad} of {got.numel()} elements mismatch (allowed {allowed}); "
                                      f"max abs diff {(got.double() - want.double()).abs().max().item():.4g}")
 
+    def assert_consistent(self, repeat: int = 10, input_tensors: Optional[Sequence[torch.Tensor]] = None) -> None:
+        """The reference's race check (tilelang/profiler/__init__.py:188-205): the kernel is run ``repeat`` more times
+        on the same inputs and every run must reproduce the first.  The reference asks for ``torch.allclose``; the
+        kernels here add their partial sums in a fixed order, so the bits must be equal."""
+        ins = list(self._get_inputs() if input_tensors is None else input_tensors)
+        as_list = lambda o: [o] if isinstance(o, torch.Tensor) else list(o or [])  # noqa: E731
+        # (an output the kernel returns may be a buffer it reuses: keep copies)
+        ref_outs = [o.clone() for o in as_list(self.func(*ins))]
+        torch.cuda.synchronize()
+        for i in range(repeat):
+            lib_outs = as_list(self.func(*ins))
+            torch.cuda.synchronize()
+            assert len(lib_outs) == len(ref_outs)
+            for lhs, rhs in zip(lib_outs, ref_outs):
+                same = lhs.dtype == rhs.dtype and lhs.shape == rhs.shape and torch.equal(
+                    lhs.view(torch.uint8) if lhs.dtype.is_floating_point else lhs,
+                    rhs.view(torch.uint8) if rhs.dtype.is_floating_point else rhs)
+                if not same:
+                    raise AssertionError(f"result is not consistent: run {i + 2} differs from the first run in "
+                                         f"{int((lhs != rhs).sum())} of {lhs.numel()} elements")
+
     def do_bench(self, func: Optional[Callable] = None, warmup: int = 25, rep: int = 100, n_warmup: int = 1,
                  n_repeat: int = 1, input_tensors: Optional[Sequence[torch.Tensor]] = None) -> float:
         """tilelang/profiler/__init__.py:228-285 (its defaults n_warmup = n_repeat = 1 included)."""
