@@ -180,10 +180,13 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                       void* workspace, int64_t workspace_bytes, void* stream);
 
 /* tlq_gemm_w4a16_ws for weights whose words were repacked by interleave_weight (w_layout TLQ_W_INTERLEAVED_F16, e.g. by
- * tlq_pack_int4(interleave = 1)); TLQ_W_PLAIN is tlq_gemm_w4a16_ws itself.  Consumers of the repacked layout: the decode
- * kernel (M <= 32, K % 256 == 0), the streaming kernel (17 <= M <= 512; the fp16 decode saves the four byte permutes per word
- * that only undo the plain layout) and the two passes (M >= 256 with a workspace of N * K 16-bit values).  Other shapes are
- * rejected.  Results are bit-identical to the plain layout on the same logical weights. */
+ * tlq_pack_int4(interleave = 1)); TLQ_W_PLAIN is tlq_gemm_w4a16_ws itself.  Consumers of the repacked layout: the ring GEMV
+ * (one activation row, or two fp16 rows; K <= 4096, (K / group) % 8 == 0; TLQ_ALGO_GEMV or the automatic choice), the
+ * decode kernel (M <= 32, K % 256 == 0), the streaming kernel (17 <= M <= 512; the fp16 decode saves the four byte permutes
+ * per word that only undo the plain layout), the panel kernels and the two passes (M >= 256 with a workspace of N * K
+ * 16-bit values).  Other shapes are rejected.  Results are bit-identical to the plain layout on the same logical weights,
+ * except for the GEMV, whose dot products pair neighbouring elements instead of elements four apart: there the two
+ * layouts agree to the rounding of the fp32 sums (and bit for bit on one-hot activations). */
 int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                              int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                              int w_layout, void* workspace, int64_t workspace_bytes, void* stream);

@@ -139,6 +139,40 @@ def test_decode_kernel_on_interleaved_words(in_dtype, M, N, K, group, zeros_kind
     check_float_output(inter, w4a16_reference(A, Wp, s, z, group), "decode interleaved vs oracle")
 
 
+@pytest.mark.parametrize("in_dtype,M,N,K,group,zeros_kind", [
+    ("float16", 1, 1024, 4096, 128, "int"), ("float16", 1, 520, 1024, 32, "frac"), ("float16", 2, 8192, 2048, 64, "int"),
+    ("float16", 2, 300, 4096, 128, None), ("bfloat16", 1, 1024, 4096, 128, "int"), ("bfloat16", 1, 264, 2048, 64, "frac")])
+def test_ring_gemv_on_interleaved_words(in_dtype, M, N, K, group, zeros_kind):
+    """One or two activation rows: the ring GEMV reads the repacked words too.  Its sums pair other elements than with plain
+    words, so the two layouts agree to rounding, not bit for bit -- except on one-hot activations, where a single product
+    is summed."""
+    from tilelang_ascend_amd import _abi
+
+    lib = _abi.load()
+    dt = DT[in_dtype]
+    A = torch.randn(M, K, generator=gen(81)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=82)
+    want = w4a16_reference(A, Wp, s, z, group)
+    rc, plain = run_layout(A, Wp, s, z, group, _abi.W_PLAIN, _abi.ALGO_GEMV)
+    assert rc == 0, _abi.last_error()
+    for algo in (_abi.ALGO_GEMV,) + ((_abi.ALGO_AUTO,) if (M == 1 or N >= 8192) else ()):
+        lib.tlq_debug_launch_log(1)
+        rc, inter = run_layout(A, interleaved(Wp), s, z, group, _abi.W_INTERLEAVED_F16, algo)
+        log = lib.tlq_debug_launch_log_text().decode()
+        lib.tlq_debug_launch_log(0)
+        assert rc == 0, _abi.last_error()
+        assert "interleaved words" in log, log
+        check_float_output(inter, want, f"ring GEMV on interleaved words, algo {algo}")
+        assert torch.allclose(inter.float(), plain.float(), rtol=2e-3, atol=2e-3)
+    hot = torch.zeros(M, K, dtype=dt)
+    hot[0, 5] = 1.0
+    hot[M - 1, K - 3] = 1.0 if M > 1 else hot[M - 1, K - 3]
+    rc, plain_hot = run_layout(hot, Wp, s, z, group, _abi.W_PLAIN, _abi.ALGO_GEMV)
+    rc2, inter_hot = run_layout(hot, interleaved(Wp), s, z, group, _abi.W_INTERLEAVED_F16, _abi.ALGO_GEMV)
+    assert rc == 0 and rc2 == 0
+    assert_bit_equal(inter_hot, plain_hot, "one-hot activations: the dequantised weights themselves")
+
+
 def test_interleaved_layout_rejects_what_no_kernel_reads():
     from tilelang_ascend_amd import _abi
 
@@ -149,6 +183,8 @@ def test_interleaved_layout_rejects_what_no_kernel_reads():
     rc, _ = run_layout(A, Wp, None, None, 128, _abi.W_INTERLEAVED_F16, _abi.ALGO_DECODE)
     assert rc != 0 and "decode kernel" in _abi.last_error()
     rc, _ = run_layout(A, Wp, None, None, 128, _abi.W_INTERLEAVED_F16, _abi.ALGO_GEMV)
+    assert rc != 0 and "M <= 2" in _abi.last_error()
+    rc, _ = run_layout(A, Wp, None, None, 128, _abi.W_INTERLEAVED_F16, _abi.ALGO_MFMA)
     assert rc != 0 and "interleaved weights are read by" in _abi.last_error()
     rc, _ = run_layout(A, Wp, None, None, 128, 7, _abi.ALGO_AUTO)
     assert rc != 0 and "bad weight layout" in _abi.last_error()

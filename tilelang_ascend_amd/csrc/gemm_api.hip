@@ -7,6 +7,8 @@ namespace tlq {
 int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch, int64_t M,
                int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 bool gemv_ring_applies(int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype, const void* scales, const void* zeros);
+int gemv_w4a16_ring_interleaved(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                                int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int64_t w4a16_mid_split(int64_t M, int64_t N, int64_t K, int64_t group);
@@ -655,8 +657,8 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
     return tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, algo, workspace,
                              workspace_bytes, stream);
   TLQ_CHECK_DIMS("tlq_gemm_w4a16_layout_ws");
-  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS || algo == TLQ_ALGO_DECODE || algo == TLQ_ALGO_PANEL || algo == TLQ_ALGO_PANEL256,
-              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the decode kernel, the streaming kernel, the panel kernels and the two passes (algo %d)", algo);
+  TLQ_REQUIRE(algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_GEMV || algo == TLQ_ALGO_STREAM || algo == TLQ_ALGO_TWO_PASS || algo == TLQ_ALGO_DECODE || algo == TLQ_ALGO_PANEL || algo == TLQ_ALGO_PANEL256,
+              "tlq_gemm_w4a16_layout_ws: interleaved weights are read by the ring GEMV, the decode kernel, the streaming kernel, the panel kernels and the two passes (algo %d)", algo);
   TLQ_REQUIRE(in_dtype == TLQ_F16 || in_dtype == TLQ_BF16, "tlq_gemm_w4a16_layout_ws: in_dtype must be float16 or bfloat16 (got %d)", in_dtype);
   TLQ_REQUIRE(out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32, "tlq_gemm_w4a16_layout_ws: bad out_dtype %d", out_dtype);
   if (M == 0 || N == 0) return 0;
@@ -668,6 +670,17 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
   TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16_layout_ws: scales / zeros misaligned");
   TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K / 2), "tlq_gemm_w4a16_layout_ws: a matrix spans 4 GiB or more");
   const bool ws_aligned = workspace && aligned16(workspace);
+  // one or two activation rows: the ring GEMV where the plain layout takes it too (one row; two fp16 rows on 8192 weight
+  // rows or more), or when asked for by name
+  if (M <= 2 && (algo == TLQ_ALGO_GEMV || (algo == TLQ_ALGO_AUTO && (M == 1 || N >= 8192)))) {
+    const int rc = gemv_w4a16_ring_interleaved(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype,
+                                               (hipStream_t)stream);
+    if (rc >= 0) return rc;
+    TLQ_REQUIRE(algo != TLQ_ALGO_GEMV, "tlq_gemm_w4a16_layout_ws: the GEMV kernel reads interleaved weights for M <= 2 (fp16; bf16 M = 1), "
+                "K <= 4096, a power-of-two group with (K / group) %% 8 == 0 and 16-byte aligned scale / zero tensors (M=%lld N=%lld K=%lld "
+                "group=%lld)", (long long)M, (long long)N, (long long)K, (long long)group);
+  }
+  TLQ_REQUIRE(algo != TLQ_ALGO_GEMV, "tlq_gemm_w4a16_layout_ws: the GEMV kernel reads interleaved weights for M <= 2 only (got %lld)", (long long)M);
   if (M <= 32 && (algo == TLQ_ALGO_AUTO || algo == TLQ_ALGO_DECODE)) {
     const DecodePlan dp = w4a16_decode_plan(M, N, K, group, cu_count_or_default());
     const bool dec_ok = dp.ok && (((uintptr_t)scales | (uintptr_t)zeros) & 3) == 0 &&

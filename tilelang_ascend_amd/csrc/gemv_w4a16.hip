@@ -75,7 +75,11 @@ __device__ __forceinline__ void load_act(ActF16& r, const half_t* __restrict__ A
   r.bsum = 1024.0f * se + 64.0f * (s - se);
 }
 
-// the same from four 16-byte words already loaded
+// the same from four 16-byte words already loaded.  LAYOUT 1: the weight words went through interleave_weight for the fp16
+// target (nibbles hold elements 0, 2, 4, 6, 1, 3, 5, 7): the pair that the low / high nibble mask picks out of a word and of
+// the word shifted by 8 is then (0, 1), (2, 3), (4, 5), (6, 7) -- the activations as they lie in memory; pairs 0 and 2 are
+// still the ones that carry the bias 1024.
+template <int LAYOUT = 0>
 __device__ __forceinline__ void permute_act(ActF16& r, const uint4_t (&p)[4]) {
   float s = 0.f, se = 0.f;
   const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
@@ -84,10 +88,17 @@ __device__ __forceinline__ void permute_act(ActF16& r, const uint4_t (&p)[4]) {
     const uint4_t v = p[j];
     half2_t q0 = bitcast<half2_t>(v.x), q1 = bitcast<half2_t>(v.y);
     half2_t q2 = bitcast<half2_t>(v.z), q3 = bitcast<half2_t>(v.w);
-    r.a[4 * j + 0] = half2_t{q0.x, q2.x};
-    r.a[4 * j + 1] = half2_t{q0.y, q2.y};
-    r.a[4 * j + 2] = half2_t{q1.x, q3.x};
-    r.a[4 * j + 3] = half2_t{q1.y, q3.y};
+    if (LAYOUT == 1) {
+      r.a[4 * j + 0] = q0;
+      r.a[4 * j + 1] = q1;
+      r.a[4 * j + 2] = q2;
+      r.a[4 * j + 3] = q3;
+    } else {
+      r.a[4 * j + 0] = half2_t{q0.x, q2.x};
+      r.a[4 * j + 1] = half2_t{q0.y, q2.y};
+      r.a[4 * j + 2] = half2_t{q1.x, q3.x};
+      r.a[4 * j + 3] = half2_t{q1.y, q3.y};
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) s = __builtin_amdgcn_fdot2(r.a[4 * j + i], ones, s, false);
     se = __builtin_amdgcn_fdot2(r.a[4 * j + 0], ones, se, false);
@@ -187,11 +198,11 @@ __device__ __forceinline__ float chunk_term(const uint4_t& w, const ActBF16& act
 
 // the same value with the weights dequantised eight at a time (Expand8: bf16((u - z) * s), exact) and the packed
 // bf16 dot instruction; `a` holds the chunk's 32 activations in memory order
-template <bool FOLD>
+template <bool FOLD, int LAYOUT = 0>
 __device__ __forceinline__ float chunk_term_dot2(const uint4_t& w, const uint4_t (&a)[4], bf16_t s, bf16_t z,
                                                  const NibbleMagic& mg) {
   typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-  const Expand8<bf16_t, FOLD> ex(s, z, mg);
+  const Expand8<bf16_t, FOLD, LAYOUT> ex(s, z, mg);
   const uint32_t x[4] = {w.x, w.y, w.z, w.w};
   float acc = 0.f;
 #pragma unroll
@@ -596,7 +607,7 @@ __global__ __launch_bounds__(MAXT) void gemv_w4a16_bf16_rows_kernel(const bf16_t
 // MT = 2 activation rows (fp16): a row's nibbles are expanded once and multiplied with both activation rows, whose
 // prepared chunks the wavefront keeps in registers (36 per activation row and 2048 values of K).  Every further
 // activation row costs about 2 us on the cfg-2 shape: from three rows on the decode kernel (matrix cores) is ahead.
-template <typename T, int ITERS, int D, int MT>
+template <typename T, int ITERS, int D, int MT, int LAYOUT = 0>
 __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
                                                                              const T* __restrict__ scales,
                                                                              const T* __restrict__ zeros, void* __restrict__ C,
@@ -684,7 +695,7 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
 #pragma unroll
       for (int j = 0; j < 4; ++j) raw[j] = *(const uint4_t*)(smem + L.act + addr::ring_act_lds(m * chunks + cc[it], j));
       if constexpr (F16) {
-        permute_act(act[m][it], raw);
+        permute_act<LAYOUT>(act[m][it], raw);
       } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j) actn[it][j] = raw[j];
@@ -757,10 +768,10 @@ __global__ __launch_bounds__(1024) void gemv_w4a16_ring_kernel(const T* __restri
       }
       if (__builtin_amdgcn_ballot_w64(integral) == ~0ull) {
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) acc += chunk_term_dot2<true>(w[it], actn[it], sv[it], zv[it], mg);
+        for (int it = 0; it < ITERS; ++it) acc += chunk_term_dot2<true, LAYOUT>(w[it], actn[it], sv[it], zv[it], mg);
       } else {
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) acc += chunk_term_dot2<false>(w[it], actn[it], sv[it], zv[it], mg);
+        for (int it = 0; it < ITERS; ++it) acc += chunk_term_dot2<false, LAYOUT>(w[it], actn[it], sv[it], zv[it], mg);
       }
     }
     const float v = wave_sum_to_lane63(acc);
@@ -982,10 +993,10 @@ static RingPlan plan_gemv_ring(int64_t batch, int64_t M, int64_t N, int64_t K, i
   return p;
 }
 
-template <typename T, int ITERS, int D, int MT>
+template <typename T, int ITERS, int D, int MT, int LAYOUT>
 static int launch_gemv_ring(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int N, int K,
                             int group_shift, float zero_scalar, int out_dtype, const RingPlan& p, hipStream_t st) {
-  auto kern = gemv_w4a16_ring_kernel<T, ITERS, D, MT>;
+  auto kern = gemv_w4a16_ring_kernel<T, ITERS, D, MT, LAYOUT>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -997,17 +1008,17 @@ static int launch_gemv_ring(const void* A, const void* Wp, const void* scales, c
   }
   kern<<<p.blocks, 64 * p.waves, p.lds_bytes, st>>>((const T*)A, (const uint8_t*)Wp, (const T*)scales, (const T*)zeros, C, N, K,
                                                   group_shift, zero_scalar, out_dtype, p.rows_per_block);
-  return check_launch("tlq_gemm_w4a16(gemv)", "gemv_w4a16_ring_kernel") ? 0 : 1;
+  return check_launch("tlq_gemm_w4a16(gemv)", LAYOUT == 1 ? "gemv_w4a16_ring_kernel, interleaved words" : "gemv_w4a16_ring_kernel") ? 0 : 1;
 }
 
 // 1 (default): the ring kernel where it applies; 0: never
 static thread_local int g_gemv_ring = 1;
 
-template <typename T, int MT>
+template <typename T, int MT, int LAYOUT = 0>
 static int dispatch_gemv_ring(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int N, int K,
                               int group_shift, float zero_scalar, int out_dtype, const RingPlan& p, hipStream_t st) {
 #define TLQ_RING_CASE(IT, DD) \
-  return launch_gemv_ring<T, IT, DD, MT>(A, Wp, scales, zeros, C, N, K, group_shift, zero_scalar, out_dtype, p, st)
+  return launch_gemv_ring<T, IT, DD, MT, LAYOUT>(A, Wp, scales, zeros, C, N, K, group_shift, zero_scalar, out_dtype, p, st)
   if (p.iters == 1) {
     if (p.depth == 1) TLQ_RING_CASE(1, 1);
     if (p.depth == 2 || MT > 1) TLQ_RING_CASE(1, 2);
@@ -1028,6 +1039,23 @@ bool gemv_ring_applies(int64_t M, int64_t N, int64_t K, int64_t group, int in_dt
   int shift = 0;
   while (((int64_t)1 << shift) < group) ++shift;
   return plan_gemv_ring(1, M, N, K, shift, cu_count()).ok;
+}
+
+// The ring kernel on weights whose 32-bit words went through interleave_weight (fp16 target).  -1: the kernel does not take
+// the problem (nothing launched).  The sums pair other elements than with plain words (the nibble masks pick neighbours in
+// k), so results agree with the plain layout to the last bits of the fp32 sums, not bit for bit.
+int gemv_w4a16_ring_interleaved(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
+                                int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st) {
+  if (!gemv_ring_applies(M, N, K, group, in_dtype, scales, zeros)) return -1;
+  int shift = 0;
+  while (((int64_t)1 << shift) < group) ++shift;
+  const RingPlan rp = plan_gemv_ring(1, M, N, K, shift, cu_count());
+  if (!rp.ok) return -1;
+  if (in_dtype == TLQ_F16) {
+    if (M == 1) return dispatch_gemv_ring<half_t, 1, 1>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st);
+    return dispatch_gemv_ring<half_t, 2, 1>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st);
+  }
+  return dispatch_gemv_ring<bf16_t, 1, 1>(A, Wp, scales, zeros, C, (int)N, (int)K, shift, zero_scalar, out_dtype, rp, st);
 }
 
 // wavefronts per work-group and work-groups per CU of the rows kernel for this K
