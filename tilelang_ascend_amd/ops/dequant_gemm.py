@@ -179,8 +179,9 @@ def w4a16_gemm(M: int, N: int, K: int, block_M: int = 128, block_N: int = 256, b
     call, as the reference allocates its workspace_idx buffers per call, so launches on different streams do not share one;
     when the launch stream (forward(stream=...)) is not torch's current stream the block is recorded on it (_abi.scratch).
     weight_layout: "plain" (general_compress order) or "interleaved" (B_packed went through interleave_weight for the
-    float16 target, e.g. quantize.gpu.pack_int4(..., interleave="float16")); interleaved weights are read by the "decode" and
-    "stream" kernels and the two passes, with results bit-identical to the plain layout.
+    float16 target, e.g. quantize.gpu.pack_int4(..., interleave="float16")); interleaved weights are read by the "gemv" (one row,
+    two fp16 rows), "decode", "stream" and panel kernels and the two passes, with results bit-identical to the plain layout
+    (the GEMV: to the rounding of its fp32 sums).
     tile: rows of activations per work-group of the MFMA kernel (16, 32, 64, 128, 256; 0 = chosen by the
     library); gemv_tuning = (rows_per_wave, waves, blocks_per_cu, depth) and skinny_tuning = (waves,
     row_tiles) select among the pre-built variants of those kernels.  These are the tunable parameters an
