@@ -21,8 +21,12 @@ def run_ws(A, Wp, s, z, group, algo, workspace=True):
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
     C = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
     print(f"kernel choice M={M} N={N} K={K} g={group} algo={algo} workspace={need}", flush=True)
-    _abi.check(lib.tlq_gemm_w4a16_ws(P(dA), P(dW), P(dS), P(dZ), P(C), M, N, K, group, 0.0, _abi.F16, _abi.F16, algo,
-                                     P(ws) if workspace else None, need, torch.cuda.current_stream().cuda_stream))
+    lib.tlq_debug_launch_log(1)
+    rc = lib.tlq_gemm_w4a16_ws(P(dA), P(dW), P(dS), P(dZ), P(C), M, N, K, group, 0.0, _abi.F16, _abi.F16, algo,
+                               P(ws) if workspace else None, need, torch.cuda.current_stream().cuda_stream)
+    run_ws.log = lib.tlq_debug_launch_log_text().decode()
+    lib.tlq_debug_launch_log(0)
+    _abi.check(rc)
     torch.cuda.synchronize()
     return C.cpu()
 
@@ -47,7 +51,7 @@ def cases():
         (384, 10240, 2048, 128, _abi.ALGO_STREAM),  # three blocks of 128 activation rows: streaming kernel whatever the tile kernels' fill
         (512, 8192, 1024, 128, _abi.ALGO_STREAM),   # four blocks, 32 x 4 x 1 = 128 streaming work-groups: they fit the machine at once
         (768, 8192, 4096, 128, _abi.ALGO_PANEL256),  # above 512 rows where the 256-row panel kernel's work-groups fill the machine: 3 x 32 tiles x 2 K slices on 256 CUs
-        (2048, 4096, 2048, 128, _abi.ALGO_TWO_PASS),  # 8 x 16 panel tiles and too few steps to cut: half the CUs idle, the two passes keep it
+        (2048, 4096, 2048, 128, _abi.ALGO_PANELM),  # 8 x 16 tiles of 256 rows and too few steps to cut (half the CUs idle) against 16 x 16 tiles of 128 rows: the middle-M kernel by estimate
         (224, 28672, 8192, 128, _abi.ALGO_MFMA),    # largest matrices from 192 rows on: tile kernel over two long K slices
         (256, 14336, 4096, 128, _abi.ALGO_PANELM),  # 256 .. 512 rows on 2^25 weights or more: the middle-M panel kernel
     ]
@@ -61,6 +65,9 @@ def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(cas
     A = torch.randn(M, K, generator=gen(90 + case)).to(torch.float16)
     Wp, s, z = make_w4(N, K, group, torch.float16, "int", seed=110 + case)
     auto = run_ws(A, Wp, s, z, group, _abi.ALGO_AUTO)
+    auto_log = run_ws.log
     want = run_ws(A, Wp, s, z, group, algo)
     assert_bit_equal(auto, want, f"automatic choice vs algo {algo} for M={M} N={N} K={K}")
+    # (the two four-wavefront panel kernels add up in the same order: told apart by the launch log)
+    assert auto_log == run_ws.log, (auto_log, run_ws.log)
     check_float_output(auto, w4a16_reference(A, Wp, s, z, group), "automatic choice vs oracle")

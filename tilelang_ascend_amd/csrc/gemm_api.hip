@@ -363,7 +363,7 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (b > n[0]) n[0] = b;
   }, tuned);
   if (tuned[0] > need) need = tuned[0];
-  if (panelm_preferred(M, N, K)) {
+  if (panelm_preferred(M, N, K) || M > 512) {  // (above 512 rows: where its estimate beats the 256-row kernel's)
     const int64_t pm = panelm_workspace_bytes(M, N, K);
     if (pm > need) need = pm;
   }
@@ -385,6 +385,25 @@ int64_t tlq_w4a16_workspace_bytes_min(int64_t M, int64_t N, int64_t K) {
   const int64_t partial = w4a16_partial_sum_bytes(M, N, K);
   if (partial > 0) return partial;
   return M >= kTwoPassMinM ? N * K * 2 : 0;
+}
+
+// Estimated time of a panel kernel's launch (us): rounds of work-groups x (steps per K slice x step time + fixed part), plus
+// the pass that adds the slices' partial tiles (a launch, their write and their read) where K is cut.
+static double panel_estimate_us(int tiles_m, int tiles_n, int split, int slice_steps, double step_us, double fixed_us, int64_t M,
+                                int64_t N, int64_t cus) {
+  const int64_t wgs = (int64_t)tiles_m * tiles_n * split;
+  const double rounds = (double)ceil_div(wgs, cus);
+  return rounds * ((double)slice_steps * step_us + fixed_us) + (split > 1 ? 3.0 + (double)(split + 1) * (double)M * (double)N * 4.0 / 4e6 : 0.0);
+}
+// Above 512 rows: does the middle-M kernel (128-row tiles) beat the 256-row kernel by estimate?
+static bool panelm_estimate_wins(int64_t M, int64_t N, int64_t K, int64_t group) {
+  const int64_t cus_now = cu_count_or_default();
+  const PanelMPlan pm = w4a16_panelm_plan(M, N, K, group, (int)cus_now);
+  const Panel2Plan p2 = w4a16_panel256_plan(M, N, K, group, (int)cus_now);
+  if (!pm.ok || !p2.ok || pm.tm != 8) return false;
+  const double est_m = panel_estimate_us(pm.tiles_m, pm.tiles_n, pm.split, pm.slice_steps, 2.2, 6.0, M, N, cus_now);
+  const double est_2 = panel_estimate_us(p2.tiles_m, p2.tiles_n, p2.split, p2.slice_steps, 3.3, 8.0, M, N, cus_now);
+  return est_m < 0.88 * est_2;
 }
 
 // The automatic choice takes the 256-row panel kernel where the last round of its work-groups fills 0.55 of the CUs or more.
@@ -612,6 +631,18 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
   // 1.50 - 1.56 x), 0.98 - 0.99 on a few of the largest fp16 problems -- and 2 - 21 % behind below that fill (N = K = 4096,
   // M <= 1024: 96 work-groups).  The 128-row kernel is ahead of it nowhere by more than 4 % and stays an explicit choice.
   if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && M > 512 && K > 0 && group > 0 && N >= 1 && N < kMaxDim && K < kMaxDim && M < kMaxDim) {
+    // The middle-M kernel's 128-row tiles first where an estimate of both kernels' times says so: rounds of work-groups x
+    // (steps per K slice x the time of a step + a fixed part) + the pass over the slices' partial tiles, with the step
+    // times measured at a full machine (2.2 us on 128 rows, 3.3 us on 256) and fixed parts of 6 / 8 us.  On ten (N, K)
+    // pairs x M = 576 .. 3072, fp16 with a zero-point tensor and bf16 with a scalar one (144 cases where both kernels
+    // apply), taking the 128-row kernel where its estimate is below 0.88 of the other's never lost against the choice
+    // without it and gains 4 % on average: N = 11008, K = 4096, M = 576 - 640 (5 x 43 tiles fill the machine once, 3 x 43
+    // half of it) 69 against 102 - 106 us; N = 8192, K = 2048, M <= 1024 35 - 43 against 50 - 54 us; N = K = 4096, M = 1024
+    // 50 against 62 us; N = 2048, K = 8192, M <= 1024 42 - 51 against 47 - 59 us.
+    if (panelm_estimate_wins(M, N, K, group)) {
+      const int rc = try_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, workspace, workspace_bytes, stream);
+      if (rc >= 0) return rc;
+    }
     if (panel256_fills(M, N, K, group)) {
       const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
                                   workspace_bytes, stream);
