@@ -459,8 +459,9 @@ def tune_w4a16_choice(M: int, N: int, K: int, group_size: int = 128, dtype: str 
             continue
         alive.append(n)
     times: Dict[str, List[float]] = {n: [] for n in alive}
-    for _ in range(max(1, rounds)):
-        for n in alive:
+    for r in range(max(1, rounds)):
+        # (the families take turns in a rotating order: whoever runs first after a pause is measured a little slow)
+        for n in alive[r % len(alive):] + alive[:r % len(alive)]:
             for _ in range(3):
                 call(n)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

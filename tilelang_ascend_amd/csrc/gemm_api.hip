@@ -367,7 +367,7 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int64_t pm = panelm_workspace_bytes(M, N, K);
     if (pm > need) need = pm;
   }
-  if (M > 512) {
+  if (M > 512 || panelm_preferred(M, N, K)) {  // (256 .. 512 rows: where the 256-row kernel's estimate beats the middle-M kernel's)
     const int64_t pn = panel_workspace_bytes(M, N, K);
     if (pn > need) need = pn;
   }
@@ -403,7 +403,17 @@ static bool panelm_estimate_wins(int64_t M, int64_t N, int64_t K, int64_t group)
   if (!pm.ok || !p2.ok || pm.tm != 8) return false;
   const double est_m = panel_estimate_us(pm.tiles_m, pm.tiles_n, pm.split, pm.slice_steps, 2.2, 6.0, M, N, cus_now);
   const double est_2 = panel_estimate_us(p2.tiles_m, p2.tiles_n, p2.split, p2.slice_steps, 3.3, 8.0, M, N, cus_now);
-  return est_m < 0.88 * est_2;
+  return est_m < 0.94 * est_2;
+}
+// 256 .. 512 rows: does the 256-row kernel beat the middle-M kernel by the same estimate?
+static bool panel256_estimate_wins(int64_t M, int64_t N, int64_t K, int64_t group) {
+  const int64_t cus_now = cu_count_or_default();
+  const PanelMPlan pm = w4a16_panelm_plan(M, N, K, group, (int)cus_now);
+  const Panel2Plan p2 = w4a16_panel256_plan(M, N, K, group, (int)cus_now);
+  if (!pm.ok || !p2.ok) return false;
+  const double est_m = panel_estimate_us(pm.tiles_m, pm.tiles_n, pm.split, pm.slice_steps, pm.tm == 8 ? 2.2 : 1.8, 6.0, M, N, cus_now);
+  const double est_2 = panel_estimate_us(p2.tiles_m, p2.tiles_n, p2.split, p2.slice_steps, 3.3, 8.0, M, N, cus_now);
+  return est_2 < 0.9 * est_m;
 }
 
 // The automatic choice takes the 256-row panel kernel where the last round of its work-groups fills 0.55 of the CUs or more.
@@ -561,6 +571,13 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                 (long long)need, (long long)workspace_bytes);
   // 256 .. 512 activation rows on large matrices: the middle-M panel kernel
   if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && panelm_preferred(M, N, K) && group > 0) {
+    // (very wide matrices: where the 128-row tiles need a second round of work-groups and the 256-row tiles do not, the
+    // 256-row kernel by the same estimate -- N = 28672, K = 4096, M = 512: 104 against 129 us)
+    if (panel256_estimate_wins(M, N, K, group)) {
+      const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
+                                  workspace_bytes, stream);
+      if (rc >= 0) return rc;
+    }
     const int rc = try_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, workspace, workspace_bytes, stream);
     if (rc >= 0) return rc;
   }
@@ -635,7 +652,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     // (steps per K slice x the time of a step + a fixed part) + the pass over the slices' partial tiles, with the step
     // times measured at a full machine (2.2 us on 128 rows, 3.3 us on 256) and fixed parts of 6 / 8 us.  On ten (N, K)
     // pairs x M = 576 .. 3072, fp16 with a zero-point tensor and bf16 with a scalar one (144 cases where both kernels
-    // apply), taking the 128-row kernel where its estimate is below 0.88 of the other's never lost against the choice
+    // apply), taking the 128-row kernel where its estimate is below 0.94 of the other's never lost against the choice
     // without it and gains 4 % on average: N = 11008, K = 4096, M = 576 - 640 (5 x 43 tiles fill the machine once, 3 x 43
     // half of it) 69 against 102 - 106 us; N = 8192, K = 2048, M <= 1024 35 - 43 against 50 - 54 us; N = K = 4096, M = 1024
     // 50 against 62 us; N = 2048, K = 8192, M <= 1024 42 - 51 against 47 - 59 us.
