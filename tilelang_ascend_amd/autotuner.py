@@ -404,7 +404,8 @@ def tune_w4a16_choice(M: int, N: int, K: int, group_size: int = 128, dtype: str 
     Every family in ``candidates`` (default: all) is run through ``tlq_gemm_w4a16_ws`` by name with the workspace it asks
     for (``tlq_w4a16_workspace_bytes_for``); families that refuse the shape are recorded under ``"skipped"`` with the
     library's message, a family whose output is not close to the rule-based choice's is recorded under ``"rejected"``.
-    Timings are medians over ``rounds`` rounds of ``rep`` back-to-back launches, the families taking turns inside a round.
+    Timings are medians over ``rounds`` rounds of ``rep`` back-to-back launches (more for short kernels: half a
+    millisecond per timed region at least), the families taking turns inside a round in a rotating order.
     The winner is installed (``tlq_w4a16_choice_set``) when it beats the rule-based choice by ``min_gain`` or more;
     otherwise any earlier entry for the signature is removed.  ``persist`` rewrites the device's choice file.
 
@@ -459,6 +460,16 @@ def tune_w4a16_choice(M: int, N: int, K: int, group_size: int = 128, dtype: str 
             continue
         alive.append(n)
     times: Dict[str, List[float]] = {n: [] for n in alive}
+    # short kernels: enough launches per timed region (half a millisecond or more) for the differences to be real
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    call("auto")
+    e0.record()
+    for _ in range(4):
+        call("auto")
+    e1.record()
+    torch.cuda.synchronize()
+    per_call_us = max(e0.elapsed_time(e1) * 1000.0 / 4, 1.0)
+    rep = max(rep, min(200, int(500.0 / per_call_us) + 1))
     for r in range(max(1, rounds)):
         # (the families take turns in a rotating order: whoever runs first after a pause is measured a little slow)
         for n in alive[r % len(alive):] + alive[:r % len(alive)]:
