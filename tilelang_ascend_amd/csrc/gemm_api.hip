@@ -627,7 +627,12 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const bool stream_first = ((M <= 384 && !thin_second_round) || stream_wgs <= cus_now) && !long_tile_slices && !short_windows;
     const bool slices_too_short = group < 128 && (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
                                   w4a16_mid_fill(M, N, K, group) >= 0.66;
-    if (sp.ok && args_ok && ws_ok &&
+    // One full tile height of the tile kernel (97 .. 128 rows) on up to 2^23 weights: the tile kernel over K slices is ahead of the
+    // streaming kernel (128 rows, seven (N, K) pairs, fp16 and bf16: 13.6 - 18.2 against 15.3 - 18.8 us; level at 96 rows and
+    // at 4096 x 4096, a third behind from 160 rows on).
+    const bool tile_band = algo == TLQ_ALGO_AUTO && M > 96 && M <= 128 && N * K <= ((int64_t)1 << 23) && w4a16_mid_split(M, N, K, group) > 1 &&
+                           workspace != nullptr && workspace_bytes >= w4a16_mid_split(M, N, K, group) * M * N * 4;
+    if (sp.ok && args_ok && ws_ok && !tile_band &&
         (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && !long_tile_slices && !short_windows && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
