@@ -416,13 +416,16 @@ static bool panel256_estimate_wins(int64_t M, int64_t N, int64_t K, int64_t grou
   return est_2 < 0.9 * est_m;
 }
 
-// The automatic choice takes the 256-row panel kernel where the last round of its work-groups fills 0.55 of the CUs or more.
+// The automatic choice takes the 256-row panel kernel where the last round of its work-groups fills more than half of the CUs
+// (measured: 2 - 21 % behind the two passes at 0.375 -- 96 work-groups --, 3 % behind at exactly one half, ahead from there on:
+// N = 11008, K = 4096, M = 768, 129 work-groups: 92 against 107 us).
+static const double kPanel256Fill = 0.502;
 static bool panel256_fills(int64_t M, int64_t N, int64_t K, int64_t group) {
   const int64_t cus_now = cu_count_or_default();
   const Panel2Plan pp = w4a16_panel256_plan(M, N, K, group, (int)cus_now);
   if (!pp.ok) return false;
   const int64_t wgs = (int64_t)pp.tiles_m * pp.tiles_n * pp.split;
-  return (double)wgs / (double)(ceil_div(wgs, cus_now) * cus_now) >= 0.55;
+  return (double)wgs / (double)(ceil_div(wgs, cus_now) * cus_now) >= kPanel256Fill;
 }
 
 // The panel kernel (large M, one launch, weights dequantised on the operand read).  Returns -1 when it does not take the
@@ -647,7 +650,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
   // Above 512 rows: the 256-row panel kernel (one launch, no dequantised matrix) where its work-groups fill the machine.
   // Measured against the choice without it (two passes, tile kernel over K slices) and against the 128-row panel kernel
   // on ten (N, K) pairs x eleven values of M from 576 to 8192, fp16 with a zero-point tensor and bf16 with a scalar one,
-  // groups of 128: wherever its last round of work-groups fills 0.55 of the CUs or more it is level or ahead -- by 3 - 16 %
+  // groups of 128: wherever its last round of work-groups fills more than half of the CUs it is level or ahead -- by 3 - 16 %
   // from 3072 rows on (4096 x 4096 x 4096 bf16: 104 against 113 - 119 us; 8192 x 8192 x 8192: 1.11 x), by 10 - 56 % between
   // 576 and 2048 rows on wide or long matrices (N = 28672, K = 4096, M = 768: 1.40 - 1.54 x; N = 4096, K = 14336, M = 1280:
   // 1.50 - 1.56 x), 0.98 - 0.99 on a few of the largest fp16 problems -- and 2 - 21 % behind below that fill (N = K = 4096,
