@@ -53,12 +53,14 @@ def cases():
         (768, 16384, 4096, 128, _abi.ALGO_PANEL256),  # above 512 rows where the 256-row panel kernel's work-groups fill the machine (3 x 64 tiles) and 128-row tiles would need a second round
         (768, 8192, 4096, 128, _abi.ALGO_PANELM),  # 6 x 32 tiles of 128 rows in one round against 3 x 32 x 2 K slices of 256 rows and their partial tiles: the middle-M kernel by estimate (65 against 71 us)
         (2048, 4096, 2048, 128, _abi.ALGO_PANELM),  # 8 x 16 tiles of 256 rows and too few steps to cut (half the CUs idle) against 16 x 16 tiles of 128 rows: the middle-M kernel by estimate
-        (224, 28672, 8192, 128, _abi.ALGO_MFMA),    # largest matrices from 192 rows on: tile kernel over two long K slices
-        (256, 14336, 4096, 128, _abi.ALGO_PANELM),  # 256 .. 512 rows on 2^25 weights or more: the middle-M panel kernel
+        (192, 28672, 8192, 128, _abi.ALGO_STREAM),  # largest matrices at 192 rows: the streaming kernel (122 us against 154 us for the tile kernel over two long K slices)
+        (224, 28672, 8192, 128, _abi.ALGO_PANELM),  # 196 .. 256 rows on wide or very large matrices: the middle-M panel kernel (two tiles of 128 rows)
+        (256, 6144, 6144, 128, _abi.ALGO_STREAM),   # 256 rows on fewer than 56 million weights and fewer than 10240 outputs: the streaming kernel
+        (256, 14336, 4096, 128, _abi.ALGO_PANELM),  # 257 .. 512 rows on 2^25 weights or more, 256 rows on 10240 outputs or more: the middle-M panel kernel
     ]
 
 
-@pytest.mark.parametrize("case", range(19))
+@pytest.mark.parametrize("case", range(21))
 def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
     from tilelang_ascend_amd import _abi
 

@@ -318,12 +318,20 @@ static int64_t panelm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return need;
 }
 
-// The automatic choice takes the middle-M panel kernel from 256 to 512 activation rows on matrices of 2^25 weights or more
+// The automatic choice takes the middle-M panel kernel from 257 to 512 activation rows on matrices of 2^25 weights or more
 // (measured against the streaming kernel on five (N, K) pairs, groups of 128 and 64, fp16 with a zero-point tensor:
 // 14336 x 4096 and 4096 x 14336: 43.5 - 43.9 against 45.8 - 47.0 us at 256 rows, 56 - 59 against 65 - 71 us at 384, 62 - 76 against
 // 70 - 80 us at 512; 8192 x 8192: 47 / 66 / 77 against 49 / 74 / 82 us; below 256 rows and on 4096 x 4096 or 5120 x 5120 the
-// streaming kernel is level or ahead by up to 15 %).
-static bool panelm_preferred(int64_t M, int64_t N, int64_t K) { return M >= 256 && M <= 512 && N * K >= ((int64_t)1 << 25); }
+// streaming kernel is level or ahead by up to 15 %).  From 196 to 256 rows (two tiles of 128 rows, the second more than half
+// full) the matrix has to be larger: 44 million weights with 10240 outputs or more, 56 million with fewer (10240 x 4096 at
+// 196 - 252 rows: 36 - 41 us for the streaming kernel against 40 - 43 us; at 256 rows the streaming kernel takes
+// 36 - 41 against 41 - 45 us on 6144 x 6144, 5120 x 8192 and 8192 x 5120 and 44 - 48 against 46 - 51 us on 7168 x 7168; at
+// 200 - 248 rows the middle-M kernel takes 112 - 125 against 130 - 145 us on 28672 x 8192, 59 - 67 against 67 - 79 us on
+// 28672 x 4096 and is 2 - 7 % ahead on 11008 x 4096, 12288 x 4096, 14336 x 4096, 4096 x 14336 and 8192 x 8192).
+static bool panelm_preferred(int64_t M, int64_t N, int64_t K) {
+  if (M < 196 || M > 512 || N * K < ((int64_t)1 << 25)) return false;
+  return M > 256 || N * K >= (N >= 10240 ? 44000000 : 56000000);
+}
 
 // What an explicitly named kernel family may ask of the workspace for any group size.
 int64_t tlq_w4a16_workspace_bytes_for(int64_t M, int64_t N, int64_t K, int algo) {
@@ -615,19 +623,15 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const int64_t cus_now = cu_count_or_default();
     const bool thin_second_round = M > 256 && have && N % 8 == 0 && stream_wgs > cus_now && stream_wgs * 2 <= cus_now * 3 &&
                                    w4a16_mid_split(M, N, K, group) <= 1;
-    // On the largest matrices the tile kernel finds a K cut that fills the machine with long slices (3072 values or more
-    // per work-group) and is ahead from 192 rows on: N = 28672, K = 8192, M = 256: 164 against 189 us; N = 8192,
-    // K = 28672: 168 against 185 us (at 128 rows the streaming kernel leads by 20 %, on smaller matrices at every M).
-    const int64_t tile_split = M >= 192 && M <= 256 ? w4a16_mid_split(M, N, K, group) : 1;
-    const bool long_tile_slices = tile_split > 1 && K / tile_split >= 3072 && w4a16_mid_fill(M, N, K, group) >= 0.85 &&
-                                  workspace != nullptr && workspace_bytes >= tile_split * M * N * 4;
+    // A K cut of the tile kernel into long slices -- 3072 values or more per work-group -- does not pay between 192 and 256 rows
+    // either: N = 28672, K = 8192, M = 192: 154 against 122 us for the streaming kernel; N = 8192, K = 28672: 156 against 121 us.
     // Groups of 32 values give the streaming kernel windows of four steps, each with a round trip to memory of its own:
     // from 320 rows on, the tile kernel over K slices is 2 - 11 % ahead wherever its cut fills the machine (N = 4096,
     // K = 14336, M = 384: 77 against 84 us; N = 5120, K = 13824: 89 against 97 us); where it cannot cut K (rows of 11008
     // values) the streaming kernel is far ahead (64 against 160 us) and stays.
     const bool short_windows = group < 64 && M > 256 && sp.ok && (int64_t)sp.slice_steps * 128 > 2 * 16 * group &&
                                w4a16_mid_split(M, N, K, group) > 1 && w4a16_mid_fill(M, N, K, group) >= 0.8;
-    const bool stream_first = ((M <= 384 && !thin_second_round) || stream_wgs <= cus_now) && !long_tile_slices && !short_windows;
+    const bool stream_first = ((M <= 384 && !thin_second_round) || stream_wgs <= cus_now) && !short_windows;
     const bool slices_too_short = group < 128 && (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
                                   w4a16_mid_fill(M, N, K, group) >= 0.66;
     // One full tile height of the tile kernel (97 .. 128 rows) on up to 2^23 weights: the tile kernel over K slices is ahead of the
@@ -636,7 +640,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const bool tile_band = algo == TLQ_ALGO_AUTO && M > 96 && M <= 128 && N * K <= ((int64_t)1 << 23) && w4a16_mid_split(M, N, K, group) > 1 &&
                            workspace != nullptr && workspace_bytes >= w4a16_mid_split(M, N, K, group) * M * N * 4;
     if (sp.ok && args_ok && ws_ok && !tile_band &&
-        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && !long_tile_slices && !short_windows && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
+        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && !short_windows && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
     if (algo == TLQ_ALGO_STREAM) {
