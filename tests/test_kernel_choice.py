@@ -49,7 +49,10 @@ def cases():
         (16, 5120, 5120, 128, _abi.ALGO_DECODE),   # rows of 5120 values, 320 tiles of 16 weight rows (more than CUs): decode kernel on K chunks
         (512, 4096, 2048, 128, _abi.ALGO_STREAM),  # 512 rows on 4096 weight rows: the tile kernels would fill half the machine
         (384, 10240, 2048, 128, _abi.ALGO_STREAM),  # three blocks of 128 activation rows: streaming kernel whatever the tile kernels' fill
-        (512, 8192, 1024, 128, _abi.ALGO_STREAM),   # four blocks, 32 x 4 x 1 = 128 streaming work-groups: they fit the machine at once
+        (512, 8192, 2048, 128, _abi.ALGO_STREAM),   # four blocks, 32 x 4 x 2 = 256 streaming work-groups: they fit the machine at once
+        (512, 8192, 1024, 128, _abi.ALGO_MFMA),     # short rows, one round of 128 x 128 tiles: the tile kernel in one launch (19 against 23 us)
+        (48, 8192, 1024, 128, _abi.ALGO_SKINNY),    # short rows, 33 .. 64 activation rows, up to 2^24 weights: the skinny kernel's one launch
+        (448, 5120, 13824, 128, _abi.ALGO_PANEL256),  # 108 groups per row (the middle-M kernel wants multiples of eight): two 256-row tiles against four streaming blocks by estimate
         (768, 16384, 4096, 128, _abi.ALGO_PANEL256),  # above 512 rows where the 256-row panel kernel's work-groups fill the machine (3 x 64 tiles) and 128-row tiles would need a second round
         (768, 8192, 4096, 128, _abi.ALGO_PANELM),  # 6 x 32 tiles of 128 rows in one round against 3 x 32 x 2 K slices of 256 rows and their partial tiles: the middle-M kernel by estimate (65 against 71 us)
         (2048, 4096, 2048, 128, _abi.ALGO_PANELM),  # 8 x 16 tiles of 256 rows and too few steps to cut (half the CUs idle) against 16 x 16 tiles of 128 rows: the middle-M kernel by estimate
@@ -60,7 +63,7 @@ def cases():
     ]
 
 
-@pytest.mark.parametrize("case", range(21))
+@pytest.mark.parametrize("case", range(24))
 def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
     from tilelang_ascend_amd import _abi
 

@@ -375,7 +375,7 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int64_t pm = panelm_workspace_bytes(M, N, K);
     if (pm > need) need = pm;
   }
-  if (M > 512 || panelm_preferred(M, N, K)) {  // (256 .. 512 rows: where the 256-row kernel's estimate beats the middle-M kernel's)
+  if (M > 256 || panelm_preferred(M, N, K)) {  // (257 .. 512 rows: where the 256-row kernel's estimate beats the middle-M or the streaming kernel's)
     const int64_t pn = panel_workspace_bytes(M, N, K);
     if (pn > need) need = pn;
   }
@@ -422,6 +422,22 @@ static bool panel256_estimate_wins(int64_t M, int64_t N, int64_t K, int64_t grou
   const double est_m = panel_estimate_us(pm.tiles_m, pm.tiles_n, pm.split, pm.slice_steps, pm.tm == 8 ? 2.2 : 1.8, 6.0, M, N, cus_now);
   const double est_2 = panel_estimate_us(p2.tiles_m, p2.tiles_n, p2.split, p2.slice_steps, 3.3, 8.0, M, N, cus_now);
   return est_2 < 0.9 * est_m;
+}
+
+// 257 .. 512 rows: does the 256-row kernel beat the streaming kernel's blocks of 128 rows by the same estimate (a streaming
+// step of a 128-row block: 2.2 us, fixed part 8 us)?  It matters where the middle-M kernel does not take K (group counts
+// that are no multiple of eight) and four blocks of 128 rows meet two tiles of 256: N = 5120, K = 13824, M = 448 - 512:
+// 82 - 85 against 102 us; N = 3584, K = 18944: 81 - 85 against 102 - 106 us; N = 18944, K = 3584: 82 against 118 - 128 us;
+// on 30 measured cases the estimated ratio is 4 - 25 % above the measured one, hence the bar of 0.95 (N = 8192, K = 6912,
+// where the 256-row kernel is 2 - 5 % ahead, stays with the streaming kernel; N = 4096, K = 11008, where it is 6 % behind, too).
+static bool panel256_beats_stream(int64_t M, int64_t N, int64_t K, int64_t group, const StreamPlan& sp) {
+  if (M <= 256 || !sp.ok || sp.tm != 8) return false;
+  const int64_t cus_now = cu_count_or_default();
+  const Panel2Plan p2 = w4a16_panel256_plan(M, N, K, group, (int)cus_now);
+  if (!p2.ok) return false;
+  const double est_s = panel_estimate_us(sp.m_blocks, sp.n_blocks, sp.split, sp.slice_steps, 2.2, 8.0, M, N, cus_now);
+  const double est_2 = panel_estimate_us(p2.tiles_m, p2.tiles_n, p2.split, p2.slice_steps, 3.3, 8.0, M, N, cus_now);
+  return est_2 < 0.95 * est_s;
 }
 
 // The automatic choice takes the 256-row panel kernel where the last round of its work-groups fills more than half of the CUs
@@ -564,9 +580,26 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     // pass) costs more than it saves.  Measured: 256^3 6.5 against 9.5 us, M = 128 on 1024 x 512 9.7 against 12.4 us,
     // M = 64 on 1024^2 6.7 against 11.4 us and on 2048^2 11.0 against 13.0 us; the streaming kernel with its K slices is
     // ahead from M = 256 on 1024^2 (15.5 against 20.8 us) and for M = 40 on 1024 rows of 4096 values (13.0 against 16.5 us).
+    // Short rows (K <= 2048) on up to 2^24 weights, 33 .. 64 activation rows: the skinny kernel's single launch is ahead of the
+    // streaming kernel, whose launch has 8 us that do not depend on K (N = 8192, K = 1024: 7.9 / 8.4 against 12.5 / 13.4 us at
+    // 40 / 64 rows; N = 16384, K = 1024: 10.7 / 12.4 against 13.8 / 15.6 us; N = 8192, K = 2048: 12.0 / 14.9 against 14.7 / 16.4 us;
+    // behind from 2^25 weights on and with rows of 3072 values).
     const int64_t nk = N * K;
-    if ((M <= 64 && (nk <= ((int64_t)1 << 21) || (nk <= ((int64_t)1 << 22) && K <= 2048))) || nk <= ((int64_t)1 << 19))
+    // (rows of more than 1280 values only where the skinny kernel's work-groups, one per 16 weight rows, run in one round or
+    // fill their last round: N = 6144, K = 2048, 384 work-groups: 16 - 22 against 14 - 15 us)
+    const bool skinny_fills = ceil_div(N, (int64_t)16) <= cu_count_or_default() || tile_fill(1, 16, N, 16) >= 0.8;
+    if ((M <= 64 && (nk <= ((int64_t)1 << 21) || (nk <= ((int64_t)1 << 24) && (K <= 1280 || (K <= 2048 && skinny_fills))))) || nk <= ((int64_t)1 << 19))
       return tlq_gemm_w4a16(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, stream);
+    // Short rows, 96 .. 512 activation rows, one round of 128 x 128 tiles: the tile kernel in one launch takes 4.5 us + 1.45 us
+    // per 128 values of K whatever M and N, the streaming kernel 11 - 15 us at K = 512 and 19 - 30 us at K = 1024 .. 1536.
+    // Measured on five values of N from 2048 to 32768 x six of M: ahead by 1.1 - 1.4 x on all 23 cases at K = 512, by
+    // 1.07 - 1.4 x at K = 1024 from 96 tiles on (level or behind with 64 tiles and fewer), by 1.1 - 1.27 x at K = 1536 from 128
+    // tiles and 128 rows on; behind at K = 2048.  Out of sample (eight values of K from 384 to 2560 x seven of N x seven of M, both
+    // types, against the build before): 1.1 - 1.5 x on the cases that change, none more than 3 % slower.
+    const int64_t tiles128 = ceil_div(M, (int64_t)128) * ceil_div(N, (int64_t)128);
+    if (M >= 96 && M <= 512 && N % 4 == 0 && tiles128 <= cu_count_or_default() &&
+        (K <= 512 || (K <= 1024 && tiles128 >= 96) || (K <= 1536 && tiles128 >= 128 && (M == 128 || M > 192))))  // (129 .. 192 rows: the streaming kernel's blocks of 96 rows are level there)
+      return tlq_gemm_w4a16(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_MFMA, stream);
     // 17 .. 32 activation rows whose K is one chunk of the decode kernel: that kernel, which needs no workspace
     // (M = 32, N = 14336, K = 4096: 16.8 against 20 us for the streaming kernel)
     if (M > 16 && M <= 32 && g_w4a16_decode && group > 0) {
@@ -602,6 +635,11 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                          (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) && (M * N) % 4 == 0 &&
                          ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0 && K > 0 && fits32(M, K * 2) && fits32(N, K / 2);
     const bool ws_ok = sp.ok && (sp.split == 1 || (workspace && aligned16(workspace) && workspace_bytes >= (int64_t)sp.split * M * N * 4));
+    if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && group > 0 && panel256_beats_stream(M, N, K, group, sp)) {
+      const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace,
+                                  workspace_bytes, stream);
+      if (rc >= 0) return rc;
+    }
     // measured on the MLP shapes: 20 - 35 % ahead of the tile kernel up to 256 rows, level with it at 512 -- unless the
     // tile kernels cannot fill the machine there (M = 512 on 4096 weight rows: 128 tiles of 128 x 128; K = 11008: 89
     // against 137 us for the two passes, K = 4096: 34 against 43 us)
