@@ -405,7 +405,11 @@ def tune_w4a16_choice(M: int, N: int, K: int, group_size: int = 128, dtype: str 
     for (``tlq_w4a16_workspace_bytes_for``); families that refuse the shape are recorded under ``"skipped"`` with the
     library's message, a family whose output is not close to the rule-based choice's is recorded under ``"rejected"``.
     Timings are medians over ``rounds`` rounds of ``rep`` back-to-back launches (more for short kernels: half a
-    millisecond per timed region at least), the families taking turns inside a round in a rotating order.
+    millisecond per timed region at least), the families taking turns inside a round in a rotating order.  What is
+    measured is therefore the rate of a queue of identical launches, in which the head of one launch overlaps the tail of the
+    one before; for kernels of a few microseconds that can differ from a single launch's duration by a microsecond (kernels of
+    many small work-groups overlap more than one work-group per CU does), so a gain below a microsecond on such a problem
+    says little about a program that runs other kernels in between.
     The winner is installed (``tlq_w4a16_choice_set``) when it beats the rule-based choice by ``min_gain`` or more;
     otherwise any earlier entry for the signature is removed.  ``persist`` rewrites the device's choice file.
 

@@ -594,11 +594,12 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     // per 128 values of K whatever M and N, the streaming kernel 11 - 15 us at K = 512 and 19 - 30 us at K = 1024 .. 1536.
     // Measured on five values of N from 2048 to 32768 x six of M: ahead by 1.1 - 1.4 x on all 23 cases at K = 512, by
     // 1.07 - 1.4 x at K = 1024 from 96 tiles on (level or behind with 64 tiles and fewer), by 1.1 - 1.27 x at K = 1536 from 128
-    // tiles and 128 rows on; behind at K = 2048.  Out of sample (eight values of K from 384 to 2560 x seven of N x seven of M, both
+    // tiles and 128 rows on; behind at K = 2048.  (Groups of 32 values at K = 1024: from 192 tiles on; fp16 with a zero-point
+    // tensor is 3 - 16 % behind on 96 - 128 tiles.)  Out of sample (eight values of K from 384 to 2560 x seven of N x seven of M, both
     // types, against the build before): 1.1 - 1.5 x on the cases that change, none more than 3 % slower.
     const int64_t tiles128 = ceil_div(M, (int64_t)128) * ceil_div(N, (int64_t)128);
     if (M >= 96 && M <= 512 && N % 4 == 0 && tiles128 <= cu_count_or_default() &&
-        (K <= 512 || (K <= 1024 && tiles128 >= 96) || (K <= 1536 && tiles128 >= 128 && (M == 128 || M > 192))))  // (129 .. 192 rows: the streaming kernel's blocks of 96 rows are level there)
+        (K <= 512 || (K <= 768 && tiles128 >= 96) || (K <= 1024 && tiles128 >= (group < 64 ? 192 : 96)) || (K <= 1536 && tiles128 >= 128 && (M == 128 || M > 192))))  // (129 .. 192 rows: the streaming kernel's blocks of 96 rows are level there)
       return tlq_gemm_w4a16(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_MFMA, stream);
     // 17 .. 32 activation rows whose K is one chunk of the decode kernel: that kernel, which needs no workspace
     // (M = 32, N = 14336, K = 4096: 16.8 against 20 us for the streaming kernel)
@@ -663,13 +664,18 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                                    w4a16_mid_split(M, N, K, group) <= 1;
     // A K cut of the tile kernel into long slices -- 3072 values or more per work-group -- does not pay between 192 and 256 rows
     // either: N = 28672, K = 8192, M = 192: 154 against 122 us for the streaming kernel; N = 8192, K = 28672: 156 against 121 us.
+    // With groups of 32 values, where neither the middle-M kernel nor long windows are to be had, it does (N = 8192, K = 28672,
+    // bf16, M = 196 - 252: 139 - 147 against 153 - 156 us).
+    const int64_t tile_split = group < 64 && M >= 192 && M <= 256 ? w4a16_mid_split(M, N, K, group) : 1;
+    const bool long_tile_slices = tile_split > 1 && K / tile_split >= 3072 && w4a16_mid_fill(M, N, K, group) >= 0.85 &&
+                                  workspace != nullptr && workspace_bytes >= tile_split * M * N * 4;
     // Groups of 32 values give the streaming kernel windows of four steps, each with a round trip to memory of its own:
     // from 320 rows on, the tile kernel over K slices is 2 - 11 % ahead wherever its cut fills the machine (N = 4096,
     // K = 14336, M = 384: 77 against 84 us; N = 5120, K = 13824: 89 against 97 us); where it cannot cut K (rows of 11008
     // values) the streaming kernel is far ahead (64 against 160 us) and stays.
     const bool short_windows = group < 64 && M > 256 && sp.ok && (int64_t)sp.slice_steps * 128 > 2 * 16 * group &&
                                w4a16_mid_split(M, N, K, group) > 1 && w4a16_mid_fill(M, N, K, group) >= 0.8;
-    const bool stream_first = ((M <= 384 && !thin_second_round) || stream_wgs <= cus_now) && !short_windows;
+    const bool stream_first = ((M <= 384 && !thin_second_round) || stream_wgs <= cus_now) && !long_tile_slices && !short_windows;
     const bool slices_too_short = group < 128 && (int64_t)sp.split * M * 4 >= K && (int64_t)sp.split * M * N * 4 > ((int64_t)40 << 20) &&
                                   w4a16_mid_fill(M, N, K, group) >= 0.66;
     // One full tile height of the tile kernel (97 .. 128 rows) on up to 2^23 weights: the tile kernel over K slices is ahead of the
@@ -678,7 +684,7 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     const bool tile_band = algo == TLQ_ALGO_AUTO && M > 96 && M <= 128 && N * K <= ((int64_t)1 << 23) && w4a16_mid_split(M, N, K, group) > 1 &&
                            workspace != nullptr && workspace_bytes >= w4a16_mid_split(M, N, K, group) * M * N * 4;
     if (sp.ok && args_ok && ws_ok && !tile_band &&
-        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && !short_windows && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
+        (algo == TLQ_ALGO_STREAM || (stream_first && !slices_too_short) || (!slices_too_short && !thin_second_round && !long_tile_slices && !short_windows && tile_fill(1, M, N, 128) < 0.65 && (K <= 8192 || w4a16_mid_split(M, N, K, group) <= 1))))
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, sp, (float*)workspace,
                                (hipStream_t)stream);
     if (algo == TLQ_ALGO_STREAM) {
