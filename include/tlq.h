@@ -145,6 +145,19 @@ int tlq_decode_i4_interleaved_offset(const void* words, const void* scales, cons
                                      int64_t words_per_group, int64_t n_scales, int64_t n_zeros, int offset, int zero_offset,
                                      int group_offset, int is_signed, int zeros_mode, void* stream);
 
+/* The fast decoders for interleaved 2-bit and 1-bit weights (tilelang/quantize/lop3.py:423-890 fp16 targets, :892-996 int8
+ * targets, :1048-1087 2-bit -> packed 4-bit; the device functions are in csrc/decode_lowbit.h under the reference's names).
+ * A unit is what one call of a decoder handles: out_bits 16 (fp16): 8 outputs from 16 (source_bit 2) or 8 (source_bit 1)
+ * source bits, out = f0 f4 f1 f5 f2 f6 f3 f7 of the source's fields f_j; out_bits 8 (int8): 16 outputs from 32 or 16 source
+ * bits; out_bits 4 (source_bit 2 only): 16 nibbles in two 32-bit words from 32 source bits.  src holds n_units source
+ * units back to back, out n_units x 16 bytes (8 bytes for out_bits 4).  scales / zeros (fp16 targets only): fp16, one per
+ * units_per_group consecutive units; zeros_mode 0 none | 1 original rn(rn(u - z) s) | 2 rescale (2-bit: rn(rn(u s) - z),
+ * 1-bit: fma(u, s, -|z|)) | 3 quantized (2-bit only; zeros are 16-bit integers) -- zeros with unsigned sources only.
+ * is_signed: 2-bit u - 2, 1-bit 2 u - 1 (the 2-bit -> 4-bit form ignores it, as the reference's does). */
+int tlq_decode_lowbit_interleaved(const void* src, const void* scales, const void* zeros, void* out, int64_t n_units,
+                                  int64_t units_per_group, int source_bit, int out_bits, int is_signed, int zeros_mode,
+                                  void* stream);
+
 /* Fused weight-only GEMM / GEMV, replaces dequant_gemm_fp16_wrapper + fp16_gemm
  * (example_dequant_gemm_fine_grained.py:60-115,176-223) extended with per-group scale / zero:
  *   C[M,N] = rn_out( sum_k f32(A[m,k]) * f32(W[n,k]) ),  W as in tlq_dequant_w4, fp32 accumulate.

@@ -27,6 +27,13 @@ operand fails a test):
 * rescale epilogues: pure functions of (acc, scale) -- compared with a float64
   evaluation rounded once.
 * lop3 decoders: closed forms (u-8 for signed, (u-z)*s, fma(u,s,-z), (u-qz)*s).
+* lop3 decoders for 2-bit and 1-bit sources (lop3_decode_lowbit_to_f16 / _to_i8, lop3_decode_i2_to_i4): the reference
+  holds no vectors for them and its own interleave_weight cannot produce their fp16 layouts (see above), so they are
+  pinned by what the arithmetic fixes: every one of the 2^16 / 2^8 sources against field-by-field closed forms that index
+  the fields by division instead of the decoders' shifts and masks (order f0 f4 f1 f5 f2 f6 f3 f7; u - 2 and 2u - 1 for
+  signed; two roundings against one for the 2-bit rescale form, told apart by constants chosen for that), and, for the
+  2-bit int8 target, decode(interleave_weight(q, 2, "int8")) == the plain unpack, the one low-bit layout the reference's
+  interleave_weight does produce.
 * act_quant_torch (per-token int8 quantiser): hand-built rows with known answers (ties at
   .5 fix round-half-to-even, the row maximum maps to +-127, all-zero rows give the 1e-4 / 127
   scale), invariants (odd symmetry, exact invariance under power-of-two rescaling,
@@ -379,6 +386,88 @@ def lop3_decode_i4_to_f16(words_u32, signed=False, scale=None, zeros=None, zeros
         else:
             h = (h * sc).astype(np.float16)
     return h
+
+
+# --------------------------------------------------------------------------------------
+# The 2-bit and 1-bit lop3 decoders (tilelang/quantize/lop3.py:423-996, 1048-1087), restated step by step: the spread of
+# the source bits, the shift + mask + OR of the magic number per output pair, then the packed fp16 arithmetic in the
+# reference's order (every operation rounds to fp16).  tests/test_oracle.py pins them on all 2^16 / 2^8 sources against
+# field-by-field closed forms written independently of the shifts used here.
+# --------------------------------------------------------------------------------------
+def _f16_from_bits(u16):
+    return np.asarray(u16, dtype=np.uint16).view(np.float16)
+
+
+def lop3_decode_lowbit_to_f16(src, source_bit, signed=False, scale=None, zeros=None, zeros_mode=None):
+    """src: uint16 array (2-bit: 8 fields per element) or uint8 array (1-bit: 8 bits per element) -> [n, 8] fp16.
+    2-bit (lop3.py:423-676): i2s = (w & 0xff) | ((w & 0xff00) << 8); h[i] = ((i2s >> 2i) & 0x00030003) | 0x64006400,
+    minus 0x6400 (unsigned) or 0x6402 (signed: u - 2); then scale: fma(h, s, 0); original: (h - z) then fma(., s, 0);
+    rescale: fma(h, s, 0) then - z (two roundings, :626-627); quantized: h + (0xe400 | qz) then fma(., s, 0) (:656,668-669).
+    1-bit (lop3.py:678-890): i1s = (b & 0x0f) | ((b & 0xf0) << 12); h[i] = ((i1s >> i) & 0x00010001) | 0x64006400, minus
+    0x6400; signed: h + h, then + 0xbc00 (-1) (:712-716); scale: fma(h, s, 0); original: (h - z) then fma(., s, 0);
+    rescale: fma(h, s, 0x8000 | z) -- one rounding, the addend with its sign bit forced (:870,880)."""
+    assert source_bit in (2, 1)
+    f16 = np.float16
+    if source_bit == 2:
+        w = np.asarray(src, dtype=np.uint16).reshape(-1).astype(np.uint32)
+        spread = (w & np.uint32(0x00FF)) | ((w & np.uint32(0xFF00)) << np.uint32(8))
+        mask, step = np.uint32(0x00030003), 2
+    else:
+        w = np.asarray(src, dtype=np.uint8).reshape(-1).astype(np.uint32)
+        spread = (w & np.uint32(0x0F)) | ((w & np.uint32(0xF0)) << np.uint32(12))
+        mask, step = np.uint32(0x00010001), 1
+    out = np.empty((w.size, 8), dtype=f16)
+    for i in range(4):
+        h = ((spread >> np.uint32(step * i)) & mask) | np.uint32(0x64006400)
+        for half, col in ((h & np.uint32(0xFFFF), 2 * i), (h >> np.uint32(16), 2 * i + 1)):
+            x = _f16_from_bits(half.astype(np.uint16))
+            if zeros_mode == "quantized":
+                assert source_bit == 2
+                qz = np.uint16(np.int16(zeros)) if np.ndim(zeros) == 0 else np.asarray(zeros, dtype=np.int16).view(np.uint16)
+                x = (x + _f16_from_bits(np.uint16(0xE400) | qz)).astype(f16)
+            else:
+                median = 0x6402 if (source_bit == 2 and signed) else 0x6400
+                x = (x - _f16_from_bits(np.uint16(median))).astype(f16)
+                if source_bit == 1 and signed:
+                    x = (x + x).astype(f16)
+                    x = (x + _f16_from_bits(np.uint16(0xBC00))).astype(f16)
+            if zeros_mode == "original":
+                x = (x - f16(zeros)).astype(f16)
+            if scale is not None:
+                if zeros_mode == "rescale" and source_bit == 1:
+                    nz = _f16_from_bits(np.asarray(f16(zeros)).view(np.uint16) | np.uint16(0x8000))
+                    x = (x.astype(np.float64) * np.float64(f16(scale)) + nz.astype(np.float64)).astype(f16)
+                else:
+                    x = (x.astype(np.float64) * np.float64(f16(scale))).astype(f16)  # fma with a zero addend: one rounding
+                    if zeros_mode == "rescale":
+                        x = (x - f16(zeros)).astype(f16)
+            out[:, col] = x
+    return out
+
+
+def lop3_decode_lowbit_to_i8(src, source_bit, signed=False):
+    """2-bit (lop3.py:949-996): src uint32, word i of the output = (w >> 2i) & 0x03030303, signed: minus 2 per byte.
+    1-bit (lop3.py:892-947): src uint16, i1b = (w & 0x0f0f) | ((w & 0xf0f0) << 12), word i = (i1b >> i) & 0x01010101,
+    signed: per byte x + x, then + 0xff (:916-917).  Returns [n, 16] int8 in memory order (word i, byte lane b at 4i + b)."""
+    assert source_bit in (2, 1)
+    if source_bit == 2:
+        w = np.asarray(src, dtype=np.uint32).reshape(-1)
+        words = [(w >> np.uint32(2 * i)) & np.uint32(0x03030303) for i in range(4)]
+    else:
+        w16 = np.asarray(src, dtype=np.uint16).reshape(-1).astype(np.uint32)
+        i1b = (w16 & np.uint32(0x0F0F)) | ((w16 & np.uint32(0xF0F0)) << np.uint32(12))
+        words = [(i1b >> np.uint32(i)) & np.uint32(0x01010101) for i in range(4)]
+    by = np.stack(words, axis=1).astype("<u4").view(np.uint8).reshape(-1, 16)
+    if signed:
+        by = (by - np.uint8(2)) if source_bit == 2 else ((by + by) + np.uint8(0xFF))  # uint8 arithmetic wraps per byte
+    return by.astype(np.uint8).view(np.int8)
+
+
+def lop3_decode_i2_to_i4(src):
+    """lop3.py:1048-1087 (N = 16): word i of the output = (w >> 2 (i % 2)) & 0x33333333 for i = 0, 1 (i / 2 = 0: the one
+    source word); the signed form's body is a comment, so signed and unsigned agree.  Returns [n, 2] uint32."""
+    w = np.asarray(src, dtype=np.uint32).reshape(-1)
+    return np.stack([(w >> np.uint32(2 * (i % 2))) & np.uint32(0x33333333) for i in range(2)], axis=1)
 
 
 # --------------------------------------------------------------------------------------

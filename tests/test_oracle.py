@@ -396,3 +396,74 @@ def test_golden_fixtures_still_match_the_oracle():
         assert set(f.files) == set(fresh)
         for k in f.files:
             assert np.array_equal(f[k], fresh[k]), k
+
+
+# ---- the 2-bit / 1-bit lop3 decoders: every source value against closed forms that index the fields arithmetically ----
+F16_ORDER = (0, 4, 1, 5, 2, 6, 3, 7)
+
+
+def _fields(values, bits, count):
+    """field j of every value, by division (not by the shifts the oracle uses)"""
+    v = np.asarray(values, dtype=np.int64)
+    return np.stack([(v // (2 ** (bits * j))) % (2 ** bits) for j in range(count)], axis=1)
+
+
+def _rn16(x):
+    return np.asarray(x, dtype=np.float64).astype(np.float16)
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+def test_lowbit_lop3_decoders_to_fp16_on_every_source(bits):
+    src = np.arange(2 ** (8 * bits), dtype=np.uint16 if bits == 2 else np.uint8)
+    u = _fields(src, bits, 8)[:, F16_ORDER].astype(np.float64)
+    assert np.array_equal(ref.lop3_decode_lowbit_to_f16(src, bits), _rn16(u))
+    signed = u - 2 if bits == 2 else 2 * u - 1
+    assert np.array_equal(ref.lop3_decode_lowbit_to_f16(src, bits, signed=True), _rn16(signed))
+    s, z = np.float16(0.0371), np.float16(1.3125)
+    assert np.array_equal(ref.lop3_decode_lowbit_to_f16(src, bits, scale=s), _rn16(u * float(s)))
+    assert np.array_equal(ref.lop3_decode_lowbit_to_f16(src, bits, signed=True, scale=s), _rn16(signed * float(s)))
+    orig = _rn16(_rn16(u - float(z)).astype(np.float64) * float(s))
+    assert np.array_equal(ref.lop3_decode_lowbit_to_f16(src, bits, scale=s, zeros=z, zeros_mode="original"), orig)
+    got = ref.lop3_decode_lowbit_to_f16(src, bits, scale=s, zeros=z, zeros_mode="rescale")
+    if bits == 2:  # the product is rounded, then the zero point subtracted (lop3.py:626-627)
+        assert np.array_equal(got, _rn16(_rn16(u * float(s)).astype(np.float64) - float(z)))
+        s2, z2 = np.float16(0.74658203125), np.float16(1.287109375)  # constants that tell two roundings from one (at u = 3)
+        got2 = ref.lop3_decode_lowbit_to_f16(src, bits, scale=s2, zeros=z2, zeros_mode="rescale")
+        assert np.array_equal(got2, _rn16(_rn16(u * float(s2)).astype(np.float64) - float(z2)))
+        assert not np.array_equal(got2, _rn16(u * float(s2) - float(z2)))
+        qz = 3
+        assert np.array_equal(ref.lop3_decode_lowbit_to_f16(src, bits, scale=s, zeros=qz, zeros_mode="quantized"), _rn16((u - qz) * float(s)))
+    else:          # one multiply-add whose addend has its sign bit forced (lop3.py:870,880): -|z| for either sign of z
+        assert np.array_equal(got, _rn16(u * float(s) - float(z)))
+        assert np.array_equal(ref.lop3_decode_lowbit_to_f16(src, bits, scale=s, zeros=-z, zeros_mode="rescale"), got)
+        s2, z2 = np.float16(0.74658203125), np.float16(1.287109375)
+        assert np.array_equal(ref.lop3_decode_lowbit_to_f16(src, bits, scale=s2, zeros=z2, zeros_mode="rescale"), _rn16(u * float(s2) - float(z2)))
+
+
+def test_lowbit_lop3_decoders_to_int8_and_int4():
+    rng = np.random.default_rng(5)
+    w32 = np.concatenate([rng.integers(0, 2 ** 32, 4096, dtype=np.uint64).astype(np.uint32), np.array([0, 0xFFFFFFFF, 0x1B1B1B1B], dtype=np.uint32)])
+    f = _fields(w32, 2, 16)
+    want = np.stack([f[:, 4 * b + i] for i in range(4) for b in range(4)], axis=1)  # word i, byte lane b holds field 4 b + i
+    assert np.array_equal(ref.lop3_decode_lowbit_to_i8(w32, 2), want.astype(np.int8))
+    assert np.array_equal(ref.lop3_decode_lowbit_to_i8(w32, 2, signed=True), (want - 2).astype(np.int8))
+    w16 = np.arange(65536, dtype=np.uint16)
+    b = _fields(w16, 1, 16)
+    lanes = lambda i: (i, 8 + i, 4 + i, 12 + i)  # noqa: E731
+    want1 = np.stack([b[:, j] for i in range(4) for j in lanes(i)], axis=1)
+    assert np.array_equal(ref.lop3_decode_lowbit_to_i8(w16, 1), want1.astype(np.int8))
+    assert np.array_equal(ref.lop3_decode_lowbit_to_i8(w16, 1, signed=True), (2 * want1 - 1).astype(np.int8))
+    # 2-bit -> nibbles: nibble n of output word i holds field 2 n + i
+    got = ref.lop3_decode_i2_to_i4(w32)
+    nib = np.stack([_fields(got[:, i], 4, 8) for i in range(2)], axis=1)  # [n, word, nibble]
+    assert np.array_equal(nib, np.stack([f[:, [2 * n + i for n in range(8)]] for i in range(2)], axis=1))
+
+
+def test_lowbit_int8_decoder_undoes_the_reference_interleave():
+    """interleave_weight(q, 2, "int8") (tilelang/quantize/utils.py:73-101, the one low-bit branch the reference can run) puts
+    field 4 i + b of a word at byte lane b, slot i: decode_i2u_to_i8s of the result is the plain unpack in logical order."""
+    q = torch.randint(-128, 128, (6, 16), dtype=torch.int8, generator=_rng(21))
+    inter = ref.interleave_weight(q, 2, "int8")
+    words = inter.contiguous().view(torch.int32).numpy().view(np.uint32).reshape(-1)
+    plain = _fields(q.contiguous().view(torch.int32).numpy().view(np.uint32).reshape(-1), 2, 16)
+    assert np.array_equal(ref.lop3_decode_lowbit_to_i8(words, 2), plain.astype(np.int8))

@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 import torch
 
+from helpers import assert_bit_equal
 from oracle import ref
 from tilelang_ascend_amd import quantize as Q
 
@@ -108,8 +109,22 @@ def test_lop3_group_naming_grammar():
         Q.get_lop3_intrin_group("float16", source_format="float")
     with pytest.raises(AssertionError):
         Q.get_lop3_intrin_group("float32")
-    with pytest.raises(NotImplementedError):
-        Q.get_lop3_intrin_group("float16", source_bit=2)
+    # 2-bit and 1-bit sources: the names of the reference's table (lop3.py:1147-1170), KeyError for what it does not hold
+    for kw, name in ((dict(source_bit=2), "decode_i2u_to_f16"), (dict(source_bit=2, source_format="int", with_scaling=True), "decode_i2s_to_f16_scale"),
+                     (dict(source_bit=2, with_scaling=True, with_zeros=True, zeros_mode="quantized"), "decode_i2u_to_f16_scale_zeros_quantized"),
+                     (dict(source_bit=2, with_scaling=True, with_zeros=True, zeros_mode="rescale"), "decode_i2u_to_f16_scale_zeros_rescale"),
+                     (dict(source_bit=1, source_format="int"), "decode_i1s_to_f16"), (dict(source_bit=1, with_scaling=True), "decode_i1u_to_f16_scale"),
+                     (dict(source_bit=1, with_scaling=True, with_zeros=True, zeros_mode="original"), "decode_i1u_to_f16_scale_zeros_original")):
+        g = Q.get_lop3_intrin_group("float16", **kw)
+        assert g["func_name"] == name and f" {name}(" in g["c_source"]
+    assert Q.get_lop3_intrin_group("int8", source_bit=2, source_format="int")["func_name"] == "decode_i2s_to_i8s"
+    assert Q.get_lop3_intrin_group("int8", source_bit=1)["func_name"] == "decode_i1u_to_i8s"
+    for bad in (dict(out_dtype="float16", source_bit=1, with_scaling=True, with_zeros=True, zeros_mode="quantized"),
+                dict(out_dtype="float16", source_bit=2, with_scaling=True, storage_scope="warp"),
+                dict(out_dtype="int4", source_bit=1), dict(out_dtype="int8", source_bit=2, with_scaling=True),
+                dict(out_dtype="float16", source_bit=3)):
+        with pytest.raises(KeyError):
+            Q.get_lop3_intrin_group(**bad)
     # storage_scope "warp" with scaling selects the two-group forms (lop3.py:1178-1180, 1196-1197)
     for kw, name in ((dict(), "decode_i4u_to_f16_scale_offset"),
                      (dict(source_format="int"), "decode_i4s_to_f16_scale_offset"),
@@ -119,8 +134,9 @@ def test_lop3_group_naming_grammar():
         g = Q.get_lop3_intrin_group("float16", with_scaling=True, storage_scope="warp", **kw)
         assert g["func_name"] == name and f" {name}(" in g["c_source"]
     assert Q.get_lop3_intrin_group("float16", storage_scope="warp")["func_name"] == "decode_i4u_to_f16"  # no scaling: no suffix
-    with pytest.raises(NotImplementedError):
-        Q.get_lop3_intrin_group("int4", source_bit=2)
+    assert Q.get_lop3_intrin_group("int4", source_bit=2, source_format="int")["func_name"] == "decode_i2s_to_i4s"
+    with pytest.raises(KeyError):
+        Q.get_lop3_intrin_group("int4")  # (4-bit sources have no 4-bit target)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -234,3 +250,66 @@ def test_gpu_decode_offset_rejects_short_parameter_arrays():
         lop3.decode_offset(w, torch.ones(5, dtype=torch.float16), 1, zeros=s, zeros_mode="original", group_size=32)
     with pytest.raises(RuntimeError, match="group_offset"):
         lop3.decode_offset(w, s, 0, zeros=torch.zeros(4, dtype=torch.int32), zeros_mode="quantized", group_size=32, group_offset=8)
+
+
+# ------------------------------------------------------------------------------------------------
+# 2-bit / 1-bit fast decoders on the GPU (csrc/decode_lowbit.h through tlq_decode_lowbit_interleaved) against the oracle's
+# step-by-step restatement of lop3.py:423-996, 1048-1087, on every source value
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits", [2, 1])
+def test_gpu_lowbit_decoders_to_fp16_on_every_source(bits):
+    from tilelang_ascend_amd.quantize import lop3
+
+    n = 2 ** (8 * bits)
+    src_np = np.arange(n, dtype=np.uint16 if bits == 2 else np.uint8)
+    src = torch.from_numpy(src_np.view(np.uint8).copy()).cuda()
+    s, z = 0.0371, 1.3125
+    cases = [dict(), dict(signed=True), dict(scale=s), dict(signed=True, scale=s), dict(scale=s, zeros=z, zeros_mode="original"),
+             dict(scale=s, zeros=z, zeros_mode="rescale"), dict(scale=s, zeros=-z, zeros_mode="rescale"),
+             dict(scale=0.74658203125, zeros=1.287109375, zeros_mode="rescale")]  # (the last: one rounding and two differ at u = 3)
+    if bits == 2:
+        cases.append(dict(scale=s, zeros=3, zeros_mode="quantized"))
+    for kw in cases:
+        want = ref.lop3_decode_lowbit_to_f16(src_np, bits, **kw)
+        sc = None if "scale" not in kw else torch.tensor([kw["scale"]], dtype=torch.float16)
+        zs = None if "zeros" not in kw else torch.tensor([kw["zeros"]], dtype=torch.int16 if kw["zeros_mode"] == "quantized" else torch.float16)
+        got = lop3.decode_lowbit(src, bits, "float16", "int" if kw.get("signed") else "uint", scale=sc, zeros=zs, zeros_mode=kw.get("zeros_mode"))
+        assert got.shape == (n * 8,) and got.dtype == torch.float16
+        assert_bit_equal(got.cpu().view(n, 8), torch.from_numpy(want), f"{bits}-bit {kw}")
+    # one scale / zero per group of 16 weights (two units)
+    sg = (torch.arange(n // 2, dtype=torch.float32) % 37 * 0.01 + 0.02).half()
+    zg = (torch.arange(n // 2, dtype=torch.float32) % 5 * 0.25).half()
+    got = lop3.decode_lowbit(src, bits, "float16", scale=sg, zeros=zg, zeros_mode="original", group_size=16).cpu().view(n, 8)
+    for g in (0, 1, 77, n // 2 - 1):
+        want = ref.lop3_decode_lowbit_to_f16(src_np[2 * g:2 * g + 2], bits, scale=sg[g].item(), zeros=zg[g].item(), zeros_mode="original")
+        assert_bit_equal(got[2 * g:2 * g + 2], torch.from_numpy(want), f"group {g}")
+
+
+@pytest.mark.gpu
+def test_gpu_lowbit_decoders_to_int8_and_int4():
+    from tilelang_ascend_amd import _abi
+    from tilelang_ascend_amd.quantize import lop3
+
+    rng = np.random.default_rng(9)
+    w32 = np.concatenate([rng.integers(0, 2 ** 32, 5000, dtype=np.uint64).astype(np.uint32), np.array([0, 0xFFFFFFFF, 0x1B1B1B1B], dtype=np.uint32)])
+    src32 = torch.from_numpy(w32.view(np.uint8).copy()).cuda()
+    w16 = np.arange(65536, dtype=np.uint16)
+    src16 = torch.from_numpy(w16.view(np.uint8).copy()).cuda()
+    for signed in (False, True):
+        fmt = "int" if signed else "uint"
+        got = lop3.decode_lowbit(src32, 2, "int8", fmt).cpu().view(-1, 16)
+        assert_bit_equal(got, torch.from_numpy(ref.lop3_decode_lowbit_to_i8(w32, 2, signed)), f"2-bit -> int8 {fmt}")
+        got = lop3.decode_lowbit(src16, 1, "int8", fmt).cpu().view(-1, 16)
+        assert_bit_equal(got, torch.from_numpy(ref.lop3_decode_lowbit_to_i8(w16, 1, signed)), f"1-bit -> int8 {fmt}")
+        got = lop3.decode_lowbit(src32, 2, "int4", fmt).cpu().numpy().view(np.uint32).reshape(-1, 2)
+        assert np.array_equal(got, ref.lop3_decode_i2_to_i4(w32)), f"2-bit -> int4 {fmt}"
+    # empty input, and what the entry point refuses
+    assert lop3.decode_lowbit(src32[:0], 2, "int8").numel() == 0
+    lib, P = _abi.load(), _abi.ptr
+    out = torch.empty(64, dtype=torch.uint8, device="cuda")
+    one = torch.ones(1, dtype=torch.float16, device="cuda")
+    for args, word in (((P(src32), None, None, P(out), 1, 1, 3, 16, 0, 0), "source_bit"), ((P(src32), None, None, P(out), 1, 1, 1, 4, 0, 0), "2-bit sources only"),
+                       ((P(src32), P(one), P(one), P(out), 1, 1, 1, 16, 0, 3), "quantized"), ((P(src32), P(one), P(one), P(out), 1, 1, 2, 16, 1, 1), "signed"),
+                       ((P(src32), P(one), None, P(out), 1, 1, 2, 8, 0, 0), "integer targets"), ((P(src32[1:]), None, None, P(out), 1, 1, 2, 16, 0, 0), "misaligned")):
+        assert lib.tlq_decode_lowbit_interleaved(*args, None) != 0 and word in _abi.last_error(), (word, _abi.last_error())

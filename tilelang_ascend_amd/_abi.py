@@ -33,6 +33,7 @@ SIGNATURES = {
     "tlq_dequant_w4": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _int, _vp]),
     "tlq_decode_i4_interleaved": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]),
     "tlq_decode_i4_interleaved_offset": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
+    "tlq_decode_lowbit_interleaved": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int, _int, _vp]),
     "tlq_gemm_w4a16": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _vp]),
     "tlq_gemv_w4a16_batched": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _int, _int, _vp]),
     "tlq_gemm_f16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int, _vp]),

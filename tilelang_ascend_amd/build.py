@@ -31,6 +31,7 @@ SOURCES = [
     "abi.hip",
     "unpack_dequant.hip",
     "decode_i4.hip",
+    "decode_lowbit.hip",
     "act_quant.hip",
     "repack.hip",
     "gemv_plain.hip",
