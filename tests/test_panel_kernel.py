@@ -63,10 +63,23 @@ def test_plan_and_host_walk(kernel, M, N, K, group):
     bm, bn = TILE[kernel]
     assert p["tiles_m"] == -(-M // bm) and p["tiles_n"] == -(-N // bn)
     assert p["split"] == -(-steps // p["slice_steps"])
-    assert p["split"] == 1 or p["slice_steps"] % unit == 0
+    assert p["split"] == 1 or p["slice_steps"] % unit == 0 or (kernel == "panel256" and unit % p["slice_steps"] == 0)
     walk(kernel, M, N, K, group, p["slice_steps"])
     if steps > unit:  # the shortest slices the plan may take
         walk(kernel, M, N, K, group, unit)
+
+
+def test_256_row_kernel_cuts_k_inside_a_group_that_is_longer_than_a_slice():
+    """One scale per weight row (group = K) and few tiles: the plan of the 256-row kernel cuts K into power-of-two parts of
+    the group (every step takes its group from its position in K), the host walk covers such slices, and a part that does
+    not divide the group is refused by the walk."""
+    from tilelang_ascend_amd import _abi
+
+    ok, p = plan_of(768, 4096, 8192, 8192, kernel="panel256")
+    assert ok and p["split"] > 1 and 64 % p["slice_steps"] == 0 and p["slice_steps"] >= 16, p
+    walk("panel256", 768, 4096, 8192, 8192, p["slice_steps"])
+    walk("panel256", 260, 528, 4096, 4096, 8)
+    assert _abi.load().tlq_debug_check_panel256_addressing(260, 528, 4096, 4096, 12) != 0 and "even part" in _abi.last_error()
 
 
 def test_schedule_of_the_256_row_kernel_on_the_host():
@@ -155,6 +168,19 @@ def test_panel_against_the_oracle(kernel, in_dtype, M, N, K, group, zeros_kind):
         Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=61)
     got = run_panel(A, Wp, s, z, group, kernel=kernel)
     check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"{kernel} {in_dtype} {M}x{N}x{K} g{group} {zeros_kind}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K,group,slice_steps,zeros_kind", [
+    (768, 2048, 8192, 8192, 0, "int"), (1024, 1024, 4096, 4096, 16, "frac"), (260, 528, 4096, 4096, 8, "scalar8"), (516, 1040, 8192, 2048, 4, "int"),
+])
+def test_256_row_kernel_with_slices_inside_one_group(in_dtype, M, N, K, group, slice_steps, zeros_kind):
+    dt = DT[in_dtype]
+    A = torch.randn(M, K, generator=gen(67)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=68)
+    got = run_panel(A, Wp, s, z, group, kernel="panel256", slice_steps=slice_steps)
+    check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"panel256 {in_dtype} {M}x{N}x{K} g{group} slices of {slice_steps} {zeros_kind}")
 
 
 @pytest.mark.gpu

@@ -40,6 +40,9 @@ def run_stream(A, Wp, s, z, group, out_dtype=None, algo=None):
     (17, 256, 128, 128, "int"), (32, 260, 256, 32, "frac"), (33, 1000, 512, 64, "scalar8"), (64, 2048, 4096, 128, "int"),
     (65, 520, 1152, 128, None), (100, 4096, 2048, 256, "int"), (128, 3072, 1024, 64, "frac"), (200, 516, 640, 128, "int"),
     (512, 1024, 2048, 128, "scalar8"), (48, 14336, 4096, 128, "int"), (96, 4096, 14336, 64, "int"),
+    # one scale per weight row (group = K) and other groups longer than a K slice: the slices are parts of one group
+    (64, 2048, 4096, 4096, "int"), (200, 1024, 2048, 1024, "frac"), (48, 4096, 8192, 8192, "scalar8"), (300, 512, 4096, 2048, "int"),
+    (128, 3072, 4096, 4096, None),
 ])
 def test_stream_against_the_oracle(in_dtype, M, N, K, group, zeros_kind):
     dt = DT[in_dtype]
@@ -74,6 +77,8 @@ def test_stream_one_hot_rows_return_the_dequantised_weights(in_dtype, zeros_kind
     (256, 2048, 4096, 64, 0, "int"), (256, 14336, 4096, 64, 0, "int"),
     # large groups: windows of 32 and 64 steps
     (64, 256, 128 * 80, 256, 80, "int"), (40, 260, 128 * 72, 512, 72, "frac"),
+    # slices that are a part of one group (4, 8 and 16 steps of groups of 32 steps; 2 steps of groups of 4)
+    (64, 256, 128 * 32, 4096, 8, "int"), (100, 516, 128 * 64, 4096, 4, "frac"), (200, 260, 128 * 32, 4096, 16, "mixed"), (24, 256, 128 * 8, 512, 2, "int"),
 ])
 def test_stream_windows_of_a_long_slice(in_dtype, M, N, K, group, slice_steps, zeros_kind):
     from tilelang_ascend_amd import _abi

@@ -444,7 +444,8 @@ int check_panel256(int64_t M, int64_t N, int64_t K, int64_t group, int slice_ste
   CHECK_OR_FAIL(N * (K / 2) < ((int64_t)1 << 32) && M * K * 2 < ((int64_t)1 << 32) && N * groups * 2 < ((int64_t)1 << 32),
                 "panel256: a matrix spans 4 GiB or more");
   const int steps_total = (int)(K / 128);
-  CHECK_OR_FAIL(slice_steps >= 1 && (slice_steps * 128 % group == 0 || slice_steps >= steps_total), "panel256: slices of %d steps are not whole groups", slice_steps);
+  CHECK_OR_FAIL(slice_steps >= 1 && (slice_steps * 128 % group == 0 || group % (slice_steps * 128) == 0 || slice_steps >= steps_total),
+                "panel256: slices of %d steps are neither whole groups nor an even part of one", slice_steps);
   const int TM = addr::kPanel2TM, TN = addr::kPanel2TN;
   const int64_t w_extent = N * (K / 2), a_extent = M * K * 2, s_extent = N * groups * 2;
   CHECK_OR_FAIL(2 * addr::kPanel2Slot <= 160 * 1024, "panel256: %u bytes of LDS", 2 * addr::kPanel2Slot);

@@ -413,17 +413,25 @@ Panel2Plan w4a16_panel256_plan(int64_t M, int64_t N, int64_t K, int64_t group, i
   p.tiles_m = (int)ceil_div(M, (int64_t)Panel2Cfg::BM);
   p.tiles_n = (int)ceil_div(N, (int64_t)Panel2Cfg::BN);
   const int steps_total = (int)(K / 128);
-  const int unit = group > 128 ? (int)(group / 128) : 1;  // a slice is a whole number of groups
+  // a slice is a whole number of groups or, with groups longer than a slice (one scale per weight row, say), a power-of-two
+  // part of one group: the kernel takes every step's group from the step's position in K
+  const int unit = group > 128 ? (int)(group / 128) : 1;
+  auto whole_or_part = [&](int64_t steps) {
+    if (steps >= unit) return ceil_div(steps, (int64_t)unit) * unit;
+    int64_t part = 1;
+    while (part < steps) part *= 2;
+    return part;
+  };
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (cus <= 0) cus = 256;
   int64_t ss = steps_total;
   if (g_panel2_slice_steps > 0) {
-    ss = ceil_div((int64_t)g_panel2_slice_steps, (int64_t)unit) * unit;
+    ss = whole_or_part((int64_t)g_panel2_slice_steps);
   } else if (tiles * 2 <= cus) {
     // K slices only where the tiles leave most of the machine idle: the cut that fills it best with slices of 16 steps or more
     double best = (double)ceil_div(tiles, (int64_t)cus) * (steps_total + 8);
     for (int64_t want = 2; want <= 16; ++want) {
-      int64_t cand = ceil_div(ceil_div((int64_t)steps_total, want), (int64_t)unit) * unit;
+      int64_t cand = whole_or_part(ceil_div((int64_t)steps_total, want));
       if (cand < 16 || cand >= steps_total) continue;
       const int64_t sl = ceil_div((int64_t)steps_total, cand);
       const double t = (double)ceil_div(tiles * sl, (int64_t)cus) * (double)(cand + 8) + (double)sl * (double)M * (double)N * 4.0 / 3e6 / 3.0;

@@ -186,7 +186,9 @@ __global__ __launch_bounds__(512, 2) void w4a16_stream_kernel(const T* __restric
     // of them (lane l: row l / 2, half l % 2), issued ahead of the ring so that the first step's wait covers it.
     // Otherwise 2-byte gathers, four groups per instruction (they keep the address unit busy for about a cycle per lane,
     // so they go behind the weight loads, whose trip to HBM they overlap).
-    const int G = (wsteps << 7) >> gshift;  // groups in this window (>= 1: a slice is a whole number of groups)
+    // groups in this window: a slice is a whole number of groups, or a part of ONE group (large groups, K cut below the group
+    // size: the plan takes slice lengths that divide the group, so the slice lies inside the group of its first step)
+    const int G = ((wsteps << 7) >> gshift) > 0 ? ((wsteps << 7) >> gshift) : 1;
     const int g0 = ((step0 + w0) << 7) >> gshift;
     const bool wide = (groups & 7) == 0 && (g0 & 7) == 0 && g0 + kStreamMaxGroups <= groups &&
                       (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0;  // uniform
@@ -341,7 +343,9 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   p.m_blocks = (int)ceil_div(M, (int64_t)16 * p.tm);
   p.n_blocks = (int)ceil_div(N, (int64_t)256);
   const int steps_total = (int)(K / 128);
-  const int unit = group > 128 ? (int)(group / 128) : 1;  // a slice is a whole number of groups
+  // a slice is a whole number of groups, or -- groups of more than 128 values, e.g. one scale per weight row -- a power-of-two
+  // part of one group (K % group == 0: such slices tile K, each inside one group, whose scale every step of the slice uses)
+  const int unit = group > 128 ? (int)(group / 128) : 1;
   const int window = (int)(kStreamMaxGroups * group / 128);  // steps whose groups the scale area holds; the ring restarts per window
   // K slices: the cut with the lowest estimate of rounds of work-groups (one work-group per CU) x steps per slice, plus the
   // cost of writing and adding the slices' partial tiles.  (Filling the chip once is usually that cut; but 43 x 3 blocks on
@@ -356,11 +360,18 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
   int64_t best_ss = 0;
   if (g_stream_slice_steps > 0) {
     best_ss = ceil_div((int64_t)g_stream_slice_steps, (int64_t)unit) * unit;
+    if (g_stream_slice_steps < unit && unit % g_stream_slice_steps == 0) best_ss = g_stream_slice_steps;  // a part of one group
     if (best_ss > steps_total) best_ss = steps_total;
   }
   for (int64_t want = 1; want <= 16 && g_stream_slice_steps <= 0; ++want) {
     int64_t ss = ceil_div((int64_t)steps_total, want);
-    ss = ceil_div(ss, (int64_t)unit) * unit;
+    if (ss >= unit) {
+      ss = ceil_div(ss, (int64_t)unit) * unit;
+    } else {
+      int64_t part = 1;
+      while (part < ss) part *= 2;
+      ss = part;  // (unit is a power of two: part divides it)
+    }
     if (ss < 4 && steps_total >= 4) continue;  // at least four steps per work-group
     if (ss > steps_total) ss = steps_total;
     const int64_t sl = ceil_div((int64_t)steps_total, ss);
@@ -368,7 +379,7 @@ StreamPlan w4a16_stream_plan(int64_t M, int64_t N, int64_t K, int64_t group, int
     const int64_t rounds = ceil_div(blocks * sl, (int64_t)(cus > 0 ? cus : 256));
     const int64_t windows = ceil_div(ss, (int64_t)window);
     // slices that do not start at a multiple of eight groups gather their scales two bytes at a time
-    const bool gathers = sl > 1 && (ss * 128 / group) % 8 != 0;
+    const bool gathers = sl > 1 && (ss * 128 < group || (ss * 128 / group) % 8 != 0);
     const double t = (double)rounds * ((double)(ss + 2) * t_step + (double)(windows - 1) * t_window + (gathers ? t_gather : 0.0)) +
                      (sl > 1 ? (double)sl * t_slice : 0.0);
     if (best_ss == 0 || t < best * 0.97) best = t, best_ss = ss;
