@@ -52,6 +52,8 @@ def cases():
         (512, 8192, 2048, 128, _abi.ALGO_STREAM),   # four blocks, 32 x 4 x 2 = 256 streaming work-groups: they fit the machine at once
         (512, 8192, 1024, 128, _abi.ALGO_MFMA),     # short rows, one round of 128 x 128 tiles: the tile kernel in one launch (19 against 23 us)
         (48, 8192, 1024, 128, _abi.ALGO_SKINNY),    # short rows, 33 .. 64 activation rows, up to 2^24 weights: the skinny kernel's one launch
+        (112, 32768, 4096, 128, _abi.ALGO_PANELM),    # one tile of 128 rows on 2^27 weights or more: the middle-M kernel
+        (144, 50304, 4096, 128, _abi.ALGO_PANEL256),  # two streaming blocks of 96 rows in two rounds against one round of 256-row tiles, by estimate
         (448, 5120, 13824, 128, _abi.ALGO_PANEL256),  # 108 groups per row (the middle-M kernel wants multiples of eight): two 256-row tiles against four streaming blocks by estimate
         (768, 16384, 4096, 128, _abi.ALGO_PANEL256),  # above 512 rows where the 256-row panel kernel's work-groups fill the machine (3 x 64 tiles) and 128-row tiles would need a second round
         (768, 8192, 4096, 128, _abi.ALGO_PANELM),  # 6 x 32 tiles of 128 rows in one round against 3 x 32 x 2 K slices of 256 rows and their partial tiles: the middle-M kernel by estimate (65 against 71 us)
@@ -63,7 +65,7 @@ def cases():
     ]
 
 
-@pytest.mark.parametrize("case", range(24))
+@pytest.mark.parametrize("case", range(26))
 def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
     from tilelang_ascend_amd import _abi
 

@@ -333,6 +333,11 @@ static bool panelm_preferred(int64_t M, int64_t N, int64_t K) {
   return M > 256 || N * K >= (N >= 10240 ? 44000000 : 56000000);
 }
 
+// One tile of 128 rows (97 .. 128 activation rows) on matrices of 2^27 weights or more: the middle-M kernel is 9 - 18 % ahead of
+// the streaming kernel (N = 50304, K = 4096, M = 128: 64.5 against 76.1 us; N = 65536, K = 8192: 144 against 154 us;
+// N = 28672, K = 8192, M = 112: 74 against 82 us; N = 8192, K = 28672: 76 against 81 us; level at 64 and 96 rows).
+static bool panelm_one_tile(int64_t M, int64_t N, int64_t K) { return M > 96 && M <= 128 && N * K >= ((int64_t)1 << 27); }
+
 // What an explicitly named kernel family may ask of the workspace for any group size.
 int64_t tlq_w4a16_workspace_bytes_for(int64_t M, int64_t N, int64_t K, int algo) {
   if (M <= 0 || N <= 0 || K <= 0 || M >= kMaxDim || N >= kMaxDim || K >= kMaxDim) return 0;
@@ -371,11 +376,11 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (b > n[0]) n[0] = b;
   }, tuned);
   if (tuned[0] > need) need = tuned[0];
-  if (panelm_preferred(M, N, K) || M > 512) {  // (above 512 rows: where its estimate beats the 256-row kernel's)
+  if (panelm_preferred(M, N, K) || panelm_one_tile(M, N, K) || M > 512) {  // (above 512 rows: where its estimate beats the 256-row kernel's)
     const int64_t pm = panelm_workspace_bytes(M, N, K);
     if (pm > need) need = pm;
   }
-  if (M > 256 || panelm_preferred(M, N, K)) {  // (257 .. 512 rows: where the 256-row kernel's estimate beats the middle-M or the streaming kernel's)
+  if (M > 128 || panelm_preferred(M, N, K)) {  // (129 .. 512 rows: where the 256-row kernel's estimate beats the middle-M or the streaming kernel's)
     const int64_t pn = panel_workspace_bytes(M, N, K);
     if (pn > need) need = pn;
   }
@@ -431,11 +436,13 @@ static bool panel256_estimate_wins(int64_t M, int64_t N, int64_t K, int64_t grou
 // on 30 measured cases the estimated ratio is 4 - 25 % above the measured one, hence the bar of 0.95 (N = 8192, K = 6912,
 // where the 256-row kernel is 2 - 5 % ahead, stays with the streaming kernel; N = 4096, K = 11008, where it is 6 % behind, too).
 static bool panel256_beats_stream(int64_t M, int64_t N, int64_t K, int64_t group, const StreamPlan& sp) {
-  if (M <= 256 || !sp.ok || sp.tm != 8) return false;
+  // (256 rows: one tile against two blocks -- N = 151936, K = 3584: 278 against 333 us; 129 .. 192 rows in two blocks of 96
+  // rows, 1.75 us a step, on very wide matrices: N = 50304 .. 128256, K = 4096 .. 8192, M = 160: 100 - 238 against 128 - 277 us)
+  if (M <= 128 || !sp.ok || (sp.tm != 8 && sp.tm != 6)) return false;
   const int64_t cus_now = cu_count_or_default();
   const Panel2Plan p2 = w4a16_panel256_plan(M, N, K, group, (int)cus_now);
   if (!p2.ok) return false;
-  const double est_s = panel_estimate_us(sp.m_blocks, sp.n_blocks, sp.split, sp.slice_steps, 2.2, 8.0, M, N, cus_now);
+  const double est_s = panel_estimate_us(sp.m_blocks, sp.n_blocks, sp.split, sp.slice_steps, sp.tm == 8 ? 2.2 : 1.75, 8.0, M, N, cus_now);
   const double est_2 = panel_estimate_us(p2.tiles_m, p2.tiles_n, p2.split, p2.slice_steps, 3.3, 8.0, M, N, cus_now);
   return est_2 < 0.95 * est_s;
 }
@@ -623,6 +630,10 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                                   workspace_bytes, stream);
       if (rc >= 0) return rc;
     }
+    const int rc = try_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, workspace, workspace_bytes, stream);
+    if (rc >= 0) return rc;
+  }
+  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && panelm_one_tile(M, N, K) && group > 0) {
     const int rc = try_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, workspace, workspace_bytes, stream);
     if (rc >= 0) return rc;
   }
