@@ -833,6 +833,12 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
   if (algo != TLQ_ALGO_TWO_PASS) {
     const StreamPlan sp = w4a16_stream_plan(M, N, K, group, cu_count_or_default());
     const bool ws_ok = sp.ok && (M * N) % 4 == 0 && (sp.split == 1 || (ws_aligned && workspace_bytes >= (int64_t)sp.split * M * N * 4));
+    // (129 .. 512 rows: the 256-row kernel where its estimate beats the streaming kernel's, as for the plain layout)
+    if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && group > 0 && panel256_beats_stream(M, N, K, group, sp)) {
+      const int rc = try_panel256(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, workspace,
+                                  workspace_bytes, stream);
+      if (rc >= 0) return rc;
+    }
     if (ws_ok && (algo == TLQ_ALGO_STREAM || M <= 384 || (int64_t)sp.m_blocks * sp.n_blocks * sp.split <= cu_count_or_default() || tile_fill(1, M, N, 128) < 0.65 || !(ws_aligned && workspace_bytes >= N * K * 2)))  // (no tile kernel reads this layout: the alternative is the two passes)
       return gemm_w4a16_stream(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, sp,
                                (float*)workspace, (hipStream_t)stream);
