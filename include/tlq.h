@@ -180,7 +180,9 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
  * tiles) -- which is the structure of the reference's own wrapper (example_dequant_gemm_fine_grained.py:176-223 unpacks,
  * then calls fp16_gemm) and is faster than converting the weights again in every row block of the fused kernel.  The
  * workspace holds nothing between calls.
- * algo: as tlq_gemm_w4a16, or TLQ_ALGO_TWO_PASS to force the two passes (workspace required). */
+ * algo: as tlq_gemm_w4a16, or TLQ_ALGO_TWO_PASS to force the two passes (workspace required).
+ * With TLQ_ALGO_AUTO and more than 512 rows, a row count that is no multiple of four runs as two calls on the stream: the
+ * multiple of four below (the large-M kernels take such counts only), then the last one to three rows. */
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 /* The least workspace with which tlq_gemm_w4a16_ws still takes a workspace-based kernel for this shape (the partial sums
  * of the K-slice kernels where they apply, else the dequantised matrix of the two passes); for callers short of memory. */

@@ -79,3 +79,29 @@ def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(cas
     # (the two four-wavefront panel kernels add up in the same order: told apart by the launch log)
     assert auto_log == run_ws.log, (auto_log, run_ws.log)
     check_float_output(auto, w4a16_reference(A, Wp, s, z, group), "automatic choice vs oracle")
+
+
+@pytest.mark.parametrize("M,N,K,group", [(601, 4096, 2048, 128), (1003, 2048, 4096, 64), (2049, 1024, 1024, 128), (513, 11008, 4096, 128)])
+def test_row_counts_that_are_no_multiple_of_four_run_as_head_and_tail(M, N, K, group):
+    """Above 512 rows the automatic choice runs M - M % 4 rows through the choice for that count (the panel kernels take
+    multiples of four) and the last rows through the small-M kernels: the result's rows are bit for bit those of the two
+    calls made separately, and the whole agrees with the oracle."""
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    A = torch.randn(M, K, generator=gen(700 + M)).to(torch.float16)
+    Wp, s, z = make_w4(N, K, group, torch.float16, "int", seed=800 + M)
+    whole = run_ws(A, Wp, s, z, group, _abi.ALGO_AUTO)
+    log = run_ws.log
+    head = M - M % 4
+    first = run_ws(A[:head].contiguous(), Wp, s, z, group, _abi.ALGO_AUTO)
+    assert log.startswith(run_ws.log.strip()), (log, run_ws.log)  # the head's launches come first, then the tail's
+    assert len(log.strip().split(" + ")) > len(run_ws.log.strip().split(" + "))
+    assert_bit_equal(whole[:head], first, f"rows 0 .. {head - 1}")
+    dA, dW, dS, dZ = A[head:].contiguous().cuda(), Wp.cuda(), s.cuda(), z.cuda()
+    C = torch.empty(M - head, N, dtype=torch.float16, device="cuda")
+    _abi.check(lib.tlq_gemm_w4a16(P(dA), P(dW), P(dS), P(dZ), P(C), M - head, N, K, group, 0.0, _abi.F16, _abi.F16, _abi.ALGO_AUTO,
+                                  torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert_bit_equal(whole[head:], C.cpu(), f"rows {head} .. {M - 1}")
+    check_float_output(whole, w4a16_reference(A, Wp, s, z, group), "head and tail vs oracle")

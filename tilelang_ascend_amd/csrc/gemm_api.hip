@@ -367,6 +367,11 @@ int64_t tlq_w4a16_workspace_bytes_for(int64_t M, int64_t N, int64_t K, int algo)
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
   int64_t need = w4a16_partial_sum_bytes(M, N, K);
+  // (above 512 rows a row count that is no multiple of four runs as the multiple below plus a tail: room for that call)
+  if (M > 512 && (M & 3) != 0) {
+    const int64_t head = tlq_w4a16_workspace_bytes(M & ~(int64_t)3, N, K);
+    if (head > need) need = head;
+  }
   // tuned choices for this shape (any group, any type): room for the chosen family as well
   int64_t tuned[4] = {0, M, N, K};
   w4a16_choice_for_shape(M, N, K, [](int algo, void* ctx) {
@@ -530,6 +535,24 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                                        workspace_bytes, stream);
       if (rc == 0 || launch_count() != before) return rc;
       set_error("%s", "");
+    }
+  }
+  // Above 512 rows the panel kernels are the fast path, and they take row counts that are multiples of four (their direct
+  // loads move four activation rows).  Any other count -- prompt lengths are what they are -- runs as its multiple of four
+  // below through the same choice plus the last one to three rows through the small-M kernels, which is one short launch
+  // more instead of the two passes for everything (measured: M = 1001, N = 14336, K = 4096: 147 us in one piece, 128 us for
+  // 1000 rows; M = 2049, N = K = 8192: 392 against 249 us; M = 601, N = K = 8192: 164 against 120 us; the tail takes 6 - 15 us).
+  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && M > 512 && (M & 3) != 0 && M < kMaxDim && N >= 16 && N % 16 == 0 && N < kMaxDim && K > 0 &&
+      K < kMaxDim && group > 0 && A && C && (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) &&
+      (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32)) {
+    const int64_t head = M & ~(int64_t)3;
+    if (w4a16_panel256_plan(head, N, K, group, cu_count_or_default()).ok) {
+      const int rc = tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, head, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, workspace,
+                                       workspace_bytes, stream);
+      if (rc != 0) return rc;
+      const int64_t out_bytes = out_dtype == TLQ_F32 ? 4 : 2;
+      return tlq_gemm_w4a16((const uint8_t*)A + head * K * 2, w_packed, scales, zeros, (uint8_t*)C + head * N * out_bytes, M - head, N, K, group,
+                            zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, stream);
     }
   }
   if (algo == TLQ_ALGO_PANELM) {
