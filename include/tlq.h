@@ -166,7 +166,8 @@ int tlq_decode_lowbit_interleaved(const void* src, const void* scales, const voi
  * N % 4 == 0 and a power-of-two group (32, 64, 128, ...); the GEMV kernel (M <= 16) takes any such group;
  * the skinny kernel (M <= 64) needs K % 128 == 0.  TLQ_ALGO_AUTO: M = 1 GEMV (fp16; bf16 up to K = 8192; fp16 also M = 2 with
  * K <= 4096), otherwise the decode kernel (TLQ_ALGO_DECODE) where M <= 32, K % 256 == 0, K <= 4096, the group is a power of two and the
- * scale / zero tensors are dword aligned, else M <= 64 skinny where its conditions hold (else GEMV up to M = 4), else MFMA. */
+ * scale / zero tensors are dword aligned, else M <= 64 skinny where its conditions hold (else GEMV up to M = 4), else -- more than
+ * 64 rows -- what tlq_gemm_w4a16_ws takes when it is given no workspace: the streaming and panel kernels where they do not cut K, else MFMA. */
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                    int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                    void* stream);
