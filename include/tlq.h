@@ -183,7 +183,11 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
  * workspace holds nothing between calls.
  * algo: as tlq_gemm_w4a16, or TLQ_ALGO_TWO_PASS to force the two passes (workspace required).
  * With TLQ_ALGO_AUTO and more than 512 rows, a row count that is no multiple of four runs as two calls on the stream: the
- * multiple of four below (the large-M kernels take such counts only), then the last one to three rows. */
+ * multiple of four below (the large-M kernels take such counts only), then the last one to three rows.
+ * One scale / zero point per weight row (group == K) on rows whose length is no power of two: the kernels over K slices take
+ * power-of-two groups, so the per-row values are first written out per group of min(K & -K, 1024) values into the last
+ * 2 * align16(N * K / group * 2) + 16 bytes of the workspace (tlq_w4a16_workspace_bytes counts them) and the call runs with
+ * that group: bit for bit what a caller gets who replicates the values.  A smaller workspace: the call runs with group == K. */
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 /* The least workspace with which tlq_gemm_w4a16_ws still takes a workspace-based kernel for this shape (the partial sums
  * of the K-slice kernels where they apply, else the dequantised matrix of the two passes); for callers short of memory. */

@@ -240,7 +240,10 @@ def test_w4a16_workspace_entry_point_rules():
     assert lib.tlq_w4a16_workspace_bytes(2048, 256, 512) == 256 * 512 * 2       # two passes: the dequantised matrix
     assert lib.tlq_w4a16_workspace_bytes(255, 256, 512) == 0                     # K too short to cut, M below the two passes
     assert lib.tlq_w4a16_workspace_bytes(16, 4096, 4096) == 0                    # decode sizes use no workspace
-    assert lib.tlq_w4a16_workspace_bytes(64, 4096, 14336) == 16 * 64 * 4096 * 4  # 16 K slices of fp32 partial sums
+    # 16 K slices of fp32 partial sums, and (rows of 14336 = 7 x 2048 values are no power of two) room for one scale and
+    # one zero point per weight row written out per group of 1024: two tensors of 4096 x 14 16-bit values, plus 16 bytes
+    assert lib.tlq_w4a16_workspace_bytes(64, 4096, 14336) == 16 * 64 * 4096 * 4 + 2 * 4096 * 14 * 2 + 16
+    assert lib.tlq_w4a16_workspace_bytes(64, 4096, 16384) == 16 * 64 * 4096 * 4
     M, N, K, g = 64, 128, 256, 128
     A = torch.randn(M, K, generator=gen(62)).half()
     Wp, s, z = make_w4(N, K, g, torch.float16, "int", seed=63)

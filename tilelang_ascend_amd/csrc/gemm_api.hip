@@ -109,6 +109,19 @@ void w4a16_choice_for_shape(int64_t M, int64_t N, int64_t K, void (*fn)(int algo
 
 }  // namespace tlq
 
+// One scale / zero point per weight row (group = K) where K is no power of two: the fast kernels index groups by shifts, so
+// the row's value is written out once per power-of-two group (the largest power of two that divides K, 1024 at most) into
+// the tail of the workspace and the call runs with that group size -- the same arithmetic per weight, hence the same bits.
+__global__ __launch_bounds__(256) void expand_row_values_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, int64_t n_out,
+                                                                int groups) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_out; i += (int64_t)gridDim.x * blockDim.x) out[i] = in[i / groups];
+}
+static int64_t row_group_for(int64_t K) {  // largest power of two dividing K, 1024 at most
+  int64_t g = K & -K;
+  return g > 1024 ? 1024 : g;
+}
+static int64_t row_group_tensor_bytes(int64_t N, int64_t K) { return (N * (K / row_group_for(K)) * 2 + 15) / 16 * 16; }
+
 using namespace tlq;
 
 #define TLQ_CHECK_DIMS(name)                                                                                      \
@@ -374,12 +387,21 @@ int64_t tlq_w4a16_workspace_bytes_for(int64_t M, int64_t N, int64_t K, int algo)
   }
 }
 
+static int64_t w4a16_kernel_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
+  const int64_t need = w4a16_kernel_workspace_bytes(M, N, K);
+  // (rows whose length is no power of two with one group per row: room behind everything else for the scales and zero points
+  // written out per power-of-two group)
+  if ((K & (K - 1)) != 0 && K % 64 == 0) return (need + 15) / 16 * 16 + 2 * row_group_tensor_bytes(N, K) + 16;
+  return need;
+}
+// what the kernels themselves may ask for
+static int64_t w4a16_kernel_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   int64_t need = w4a16_partial_sum_bytes(M, N, K);
   // (above 512 rows a row count that is no multiple of four runs as the multiple below plus a tail: room for that call)
   if (M > 512 && (M & 3) != 0) {
-    const int64_t head = tlq_w4a16_workspace_bytes(M & ~(int64_t)3, N, K);
+    const int64_t head = w4a16_kernel_workspace_bytes(M & ~(int64_t)3, N, K);
     if (head > need) need = head;
   }
   // tuned choices for this shape (any group, any type): room for the chosen family as well
@@ -535,6 +557,37 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
   TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_PANELM, "tlq_gemm_w4a16_ws: bad algo %d", algo);
+  // One group per weight row on rows whose length is no power of two (K = 11008, 5120, 3584 ...): only the oldest kernels take
+  // such a group (M = 64, N = 4096, K = 11008: 59 us against 23 us with groups of 128).  The row's scale / zero point is
+  // written out per power-of-two group into the tail of the workspace (one small launch) and the call goes on with that group.
+  // (not for the two passes by name: their dequantisation pass takes any group as it is)
+  if (M >= 1 && N >= 1 && N < kMaxDim && K >= 64 && K < kMaxDim && group == K && (K & (K - 1)) != 0 && K % 64 == 0 &&
+      algo != TLQ_ALGO_TWO_PASS && (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16)) {
+    const int64_t g_eff = row_group_for(K), groups = K / g_eff, tensor_bytes = row_group_tensor_bytes(N, K);
+    if (!scales && !zeros)  // no tensors: any group size says the same
+      return tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, g_eff, zero_scalar, in_dtype, out_dtype, algo, workspace, workspace_bytes, stream);
+    const int64_t tail = ((scales ? 1 : 0) + (zeros ? 1 : 0)) * tensor_bytes;
+    const int64_t head_bytes = (workspace_bytes - tail) & ~(int64_t)15;
+    if (workspace && aligned16(workspace) && workspace_bytes >= tail + 16 && ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0) {
+      uint8_t* const base = (uint8_t*)workspace + head_bytes;
+      const int64_t n_out = N * groups;
+      const int grid = (int)((n_out + 255) / 256 > 4096 ? 4096 : (n_out + 255) / 256);
+      const void* s_eff = scales;
+      const void* z_eff = zeros;
+      if (scales) {
+        expand_row_values_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)scales, (uint16_t*)base, n_out, (int)groups);
+        if (!check_launch("tlq_gemm_w4a16 (one scale per row, written out per group)", "expand_row_values_kernel")) return 1;
+        s_eff = base;
+      }
+      if (zeros) {
+        uint8_t* const zb = base + (scales ? tensor_bytes : 0);
+        expand_row_values_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)zeros, (uint16_t*)zb, n_out, (int)groups);
+        if (!check_launch("tlq_gemm_w4a16 (one zero point per row, written out per group)", "expand_row_values_kernel")) return 1;
+        z_eff = zb;
+      }
+      return tlq_gemm_w4a16_ws(A, w_packed, s_eff, z_eff, C, M, N, K, g_eff, zero_scalar, in_dtype, out_dtype, algo, workspace, head_bytes, stream);
+    }
+  }
   if (algo == TLQ_ALGO_AUTO && M >= 1 && N >= 1) {
     // a tuned choice for this call signature goes first (as in tlq_gemm_w4a16); a kernel that refuses the call -- its shape
     // rules, the alignment of an operand, a workspace smaller than it needs -- has launched nothing, and the rules decide
