@@ -112,7 +112,12 @@ def test_gemv_headline(ops, rows, waves):
 
 
 @pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
-@pytest.mark.parametrize("N,K,group", [(49152, 8192, 128), (8192, 16384, 64), (1031, 16384, 32)])
+@pytest.mark.parametrize("N,K,group", [
+    (49152, 8192, 128), (8192, 16384, 64), (1031, 16384, 32),
+    # 28 and 86 groups per row (no multiples of eight: the scales of a work-group's rows are still whole 16-byte pieces), more
+    # rows per CU than LDS holds scales for (several equal work-groups per CU), and a row count with which they are no whole pieces
+    (152064, 3584, 128), (16384, 11008, 128), (12000, 8192, 32), (10001, 3584, 128),
+])
 def test_gemv_long_rows_and_many_rows(ops, in_dtype, N, K, group):
     """Output-projection-sized decode shapes: rows of 8192 and 16384 values, whose activations alone take 18 - 36 KB of
     the GEMV's LDS, so that the rows a work-group may own are limited by what is left of 64 KB (or the streaming kernel

@@ -463,7 +463,9 @@ __device__ __forceinline__ void gemv_rows_body(const T* __restrict__ A, const ui
   for (int j = 0; j < 4; ++j) araw[j] = ((const uint4_t*)(A + ((int64_t)tchunk << 5)))[j];
   const int n_sz = (r1 - r0) * groups;  // values per tensor
   const int64_t sz0 = (int64_t)r0 * groups;
-  const bool wide = (groups & 7) == 0 && (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0;  // r0 * groups is a multiple of 8 too
+  // 16-byte pieces: every work-group's values (rows_per_block * groups of them from r0 * groups on, fewer in the last one)
+  // and every problem's (N * groups) must be whole pieces -- 28 or 86 groups per row with rows in fours qualify
+  const bool wide = ((rows_per_block * groups) & 7) == 0 && (((int64_t)N * groups) & 7) == 0 && (((uintptr_t)scales | (uintptr_t)zeros) & 15) == 0;
   uint4_t s_raw = {0, 0, 0, 0}, z_raw = {0, 0, 0, 0};
   const int t8 = threadIdx.x << 3;
   if (wide && t8 < n_sz) {  // a work-group of 1024 threads covers 8192 values per tensor in one go
@@ -926,7 +928,11 @@ static RowsPlan plan_gemv_rows(int batch, int N, int K, int group_shift, int wav
   if (rpb_max > (48 * 1024) / (4 * groups)) rpb_max = (48 * 1024) / (4 * groups);  // at most 48 KB of scales and zero points
   rpb_max &= ~3;
   if (rpb_max < waves_per_block) return p;
-  if (rpb > rpb_max) rpb = rpb_max;
+  // more rows per work-group than LDS holds: an equal number of smaller work-groups for every CU instead of full ones and a
+  // short last round (N = 28672, K = 8192, groups of 64: 312 work-groups of 92 rows on 256 CUs took 31.7 us, the same
+  // matrix with groups of 128 -- 256 work-groups of 112 rows -- 23.3 us)
+  if (rpb > rpb_max) rpb = (int)ceil_div(N, (int64_t)blocks * ceil_div(rpb, rpb_max));
+  if (rpb < waves_per_block) rpb = waves_per_block;
   rpb = (rpb + 3) & ~3;  // keeps the zero-point block of LDS 16-byte aligned for any group count
   if (rpb > rpb_max) rpb = rpb_max;
   p.rows_per_block = rpb;
