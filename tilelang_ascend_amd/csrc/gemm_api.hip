@@ -361,6 +361,16 @@ static bool panelm_preferred(int64_t M, int64_t N, int64_t K) {
 // N = 28672, K = 8192, M = 112: 74 against 82 us; N = 8192, K = 28672: 76 against 81 us; level at 64 and 96 rows).
 static bool panelm_one_tile(int64_t M, int64_t N, int64_t K) { return M > 96 && M <= 128 && N * K >= ((int64_t)1 << 27); }
 
+// 65 .. 128 rows on output-layer widths: the 128-row panel kernel, whose work-groups own 512 weight rows, where they fill more
+// than five eighths of the machine in ONE round -- the streaming kernel's work-groups (256 weight rows) then need two, the second
+// one partly empty (N = 102400, K = 4096, M = 96: 106 against 124 us; K = 5120: 133 against 159 us; N = 128256, K = 4096: 123
+// against 136 us; N = 81920: 100 against 111 us).  Not with longer rows (N = 81920, K = 8192: 208 against 204 us).
+static bool panel_one_round(int64_t M, int64_t N, int64_t K) {
+  const int64_t cus_now = cu_count_or_default();
+  const int64_t tiles = ceil_div(N, (int64_t)512);
+  return M > 64 && M <= 128 && K <= 5120 && tiles <= cus_now && tiles * 8 >= cus_now * 5;
+}
+
 // What an explicitly named kernel family may ask of the workspace for any group size.
 int64_t tlq_w4a16_workspace_bytes_for(int64_t M, int64_t N, int64_t K, int algo) {
   if (M <= 0 || N <= 0 || K <= 0 || M >= kMaxDim || N >= kMaxDim || K >= kMaxDim) return 0;
@@ -417,7 +427,7 @@ static int64_t w4a16_kernel_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int64_t pm = panelm_workspace_bytes(M, N, K);
     if (pm > need) need = pm;
   }
-  if (M > 128 || panelm_preferred(M, N, K)) {  // (129 .. 512 rows: where the 256-row kernel's estimate beats the middle-M or the streaming kernel's)
+  if (M > 128 || panelm_preferred(M, N, K) || panel_one_round(M, N, K)) {  // (129 .. 512 rows: where the 256-row kernel's estimate beats the middle-M or the streaming kernel's)
     const int64_t pn = panel_workspace_bytes(M, N, K);
     if (pn > need) need = pn;
   }
@@ -717,6 +727,10 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
       if (rc >= 0) return rc;
     }
     const int rc = try_panelm(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, workspace, workspace_bytes, stream);
+    if (rc >= 0) return rc;
+  }
+  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && panel_one_round(M, N, K) && group > 0) {
+    const int rc = try_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace, workspace_bytes, stream);
     if (rc >= 0) return rc;
   }
   if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && panelm_one_tile(M, N, K) && group > 0) {
