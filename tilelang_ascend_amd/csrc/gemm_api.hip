@@ -185,6 +185,13 @@ int tlq_debug_decode_plan(int64_t M, int64_t N, int64_t K, int64_t group, int cu
 // Activation rows from which the decode kernel is ahead of the GEMV kernels, whose time grows with every row: from three
 // rows on, and with two rows once the weights are large enough for the second pass over them to show (measured: level at
 // 4096 x 4096, 10.4 against 12.8 us (fp16) and 11.1 against 15.3 us (bf16, skinny kernel) at 11008 x 4096).
+// Whether the skinny kernel's work-groups (one per 16 weight rows; one round of one per CU, or rounds of two per CU) leave a
+// fifth or more of their last round's places empty.
+static bool skinny_leaves_cus_idle(int64_t N) {
+  if (tile_fill(1, 16, N, 16) < 0.8) return true;
+  const int64_t wgs = ceil_div(N, (int64_t)16), places = 2 * cu_count_or_default();
+  return wgs > places / 2 && (double)wgs / (double)(ceil_div(wgs, places) * places) < 0.8;
+}
 static bool decode_preferred(int64_t M, int64_t N, int64_t K) { return M > 2 || (M == 2 && N * K >= ((int64_t)1 << 24)); }
 
 int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
@@ -665,8 +672,11 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     // K = 28672: 32 against 49 us for the generic GEMV;
     // from 64 MB of weights on -- N = 28672, K = 8192, M = 16: 31.6 against 45.6 us -- and where the skinny kernel's
     // work-groups, one per 16 weight rows, would leave a fifth of the machine or more idle in their last round:
-    // N = 5120, K = 13824: 15.8 against 23.6 us; with 8192 or 13824 weight rows the skinny kernel is level or ahead)
-    if (dp.ok && dp.chunks > 1 && (algo == TLQ_ALGO_DECODE || M > 16 || K > 16384 || N * (K / 2) >= ((int64_t)64 << 20) || tile_fill(1, 16, N, 16) < 0.8) && args_ok && (M * N) % 4 == 0 && workspace && aligned16(workspace) &&
+    // N = 5120, K = 13824: 15.8 against 23.6 us; with 8192 or 13824 weight rows the skinny kernel is level or ahead.
+    // Two of its work-groups share a CU, so that holds for rounds of twice the CU count as well: N = 10240, K = 8192
+    // (640 work-groups on 512 places): 15 against 20 - 26 us; N = 12288, K = 6144 (768): 14 - 15 against 17 - 21 us;
+    // N = 17408, K = 5120 (1088): 17 - 19 against 20 - 24 us; with 512 or 960 work-groups the skinny kernel is ahead)
+    if (dp.ok && dp.chunks > 1 && (algo == TLQ_ALGO_DECODE || M > 16 || K > 16384 || N * (K / 2) >= ((int64_t)64 << 20) || skinny_leaves_cus_idle(N)) && args_ok && (M * N) % 4 == 0 && workspace && aligned16(workspace) &&
         workspace_bytes >= (int64_t)dp.chunks * M * N * 4)
       return gemm_w4a16_decode(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, dp,
                                (float*)workspace, (hipStream_t)stream);
