@@ -86,7 +86,7 @@ def test_streaming_kernel_on_interleaved_words(in_dtype, M, N, K, group, zeros_k
 
 
 @pytest.mark.parametrize("in_dtype,out_dtype", [("float16", "float16"), ("bfloat16", "float32")])
-@pytest.mark.parametrize("M,N,K,group", [(300, 1024, 512, 128), (1024, 2048, 1024, 64), (448, 5120, 13824, 128)])
+@pytest.mark.parametrize("M,N,K,group", [(300, 1024, 512, 128), (1024, 2048, 1024, 64), (448, 5120, 13824, 128), (80, 81920, 1024, 128)])
 def test_two_passes_and_automatic_choice_on_interleaved_words(in_dtype, out_dtype, M, N, K, group):
     from tilelang_ascend_amd import _abi
 
@@ -96,7 +96,8 @@ def test_two_passes_and_automatic_choice_on_interleaved_words(in_dtype, out_dtyp
     # what the automatic choice takes for interleaved words: the streaming kernel for 300 rows on 1024 weight rows (the
     # tile kernels of the two passes would leave most of the machine idle), the two passes for 1024 rows
     # (448 rows on 5120 x 13824: two tiles of the 256-row kernel against four streaming blocks, by estimate)
-    taken = {300: _abi.ALGO_STREAM, 1024: _abi.ALGO_TWO_PASS, 448: _abi.ALGO_PANEL256}[M]
+    # (80 rows on 81920 weight rows: 160 work-groups of the 128-row panel kernel in one round)
+    taken = {300: _abi.ALGO_STREAM, 1024: _abi.ALGO_TWO_PASS, 448: _abi.ALGO_PANEL256, 80: _abi.ALGO_PANEL}[M]
     for algo, plain_algo in ((_abi.ALGO_TWO_PASS, _abi.ALGO_TWO_PASS), (_abi.ALGO_AUTO, taken)):
         rc, plain = run_layout(A, Wp, s, z, group, _abi.W_PLAIN, plain_algo, DT[out_dtype])
         assert rc == 0, _abi.last_error()

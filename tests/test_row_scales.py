@@ -63,3 +63,31 @@ def test_without_room_for_the_values_the_call_still_answers():
     got = run(A, Wp, s, z, 1408, workspace_bytes=0)
     assert "written out per group" not in run.log
     check_float_output(got, w4a16_reference(A, Wp, s, z, 1408), "no workspace")
+
+
+@pytest.mark.parametrize("M,N,K,zeros_kind", [(16, 512, 2816, "int"), (64, 1024, 1408, "frac"), (300, 1024, 2816, "int")])
+def test_interleaved_words_with_one_group_per_row(M, N, K, zeros_kind):
+    """tlq_gemm_w4a16_layout_ws writes the values out the same way: the bits of the plain layout on the same logical weights."""
+    from oracle import ref
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    A = torch.randn(M, K, generator=gen(960 + M)).half()
+    Wp, s, z = make_w4(N, K, K, torch.float16, zeros_kind, seed=961 + M)
+    # (the kernel that reads interleaved words at this size, by name on the plain ones: the sums must be added in the same order)
+    plain = run(A, Wp, s, z, K, algo=_abi.ALGO_DECODE if M <= 32 else _abi.ALGO_STREAM)
+    Wi = ref.interleave_weight(Wp.view(torch.int8), 4, "float16").view(torch.uint8).contiguous()
+    dA, dW, dS, dZ = A.cuda(), Wi.cuda(), s.cuda(), z.cuda()
+    need = max(lib.tlq_w4a16_workspace_bytes(M, N, K), 16)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    print(f"row scales, interleaved words M={M} N={N} K={K} workspace={need}", flush=True)
+    lib.tlq_debug_launch_log(1)
+    rc = lib.tlq_gemm_w4a16_layout_ws(P(dA), P(dW), P(dS), P(dZ), P(C), M, N, K, K, 0.0, _abi.F16, _abi.F16, _abi.ALGO_AUTO,
+                                      _abi.W_INTERLEAVED_F16, P(ws), need, torch.cuda.current_stream().cuda_stream)
+    log = lib.tlq_debug_launch_log_text().decode()
+    lib.tlq_debug_launch_log(0)
+    _abi.check(rc)
+    torch.cuda.synchronize()
+    assert "written out per group" in log and "dequant" not in log, log
+    assert_bit_equal(C.cpu(), plain, "interleaved vs plain words, one group per row")

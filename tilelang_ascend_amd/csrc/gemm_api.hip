@@ -570,40 +570,55 @@ static int try_panelm(const void* A, const void* w_packed, const void* scales, c
                            (hipStream_t)stream);
 }
 
+// One group per weight row on rows whose length is no power of two (K = 11008, 5120, 3584 ...): only the oldest kernels take
+// such a group (M = 64, N = 4096, K = 11008: 59 us against 23 us with groups of 128).  The row's scale / zero point is
+// written out per power-of-two group into the tail of the workspace (one small launch per tensor) and the call goes on with
+// that group and the workspace in front of the tail.  Returns 0 where that does not apply (no such group, no room: the call
+// goes on as it is), 1 with `out` filled in, -1 after a failed launch.
+struct RowValues {
+  const void* scales;
+  const void* zeros;
+  int64_t group, workspace_bytes;
+};
+static int write_out_row_values(const void* scales, const void* zeros, int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype,
+                                void* workspace, int64_t workspace_bytes, void* stream, RowValues& out) {
+  if (!(M >= 1 && N >= 1 && N < kMaxDim && K >= 64 && K < kMaxDim && group == K && (K & (K - 1)) != 0 && K % 64 == 0 &&
+        (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16)))
+    return 0;
+  const int64_t g_eff = row_group_for(K), groups = K / g_eff, tensor_bytes = row_group_tensor_bytes(N, K);
+  out = RowValues{scales, zeros, g_eff, workspace_bytes};
+  if (!scales && !zeros) return 1;  // no tensors: any group size says the same
+  const int64_t tail = ((scales ? 1 : 0) + (zeros ? 1 : 0)) * tensor_bytes;
+  const int64_t head_bytes = (workspace_bytes - tail) & ~(int64_t)15;
+  if (!(workspace && aligned16(workspace) && workspace_bytes >= tail + 16 && ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0)) return 0;
+  uint8_t* const base = (uint8_t*)workspace + head_bytes;
+  const int64_t n_out = N * groups;
+  const int grid = (int)((n_out + 255) / 256 > 4096 ? 4096 : (n_out + 255) / 256);
+  if (scales) {
+    expand_row_values_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)scales, (uint16_t*)base, n_out, (int)groups);
+    if (!check_launch("tlq_gemm_w4a16 (one scale per row, written out per group)", "expand_row_values_kernel")) return -1;
+    out.scales = base;
+  }
+  if (zeros) {
+    uint8_t* const zb = base + (scales ? tensor_bytes : 0);
+    expand_row_values_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)zeros, (uint16_t*)zb, n_out, (int)groups);
+    if (!check_launch("tlq_gemm_w4a16 (one zero point per row, written out per group)", "expand_row_values_kernel")) return -1;
+    out.zeros = zb;
+  }
+  out.workspace_bytes = head_bytes;
+  return 1;
+}
+
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
   TLQ_REQUIRE(algo >= TLQ_ALGO_AUTO && algo <= TLQ_ALGO_PANELM, "tlq_gemm_w4a16_ws: bad algo %d", algo);
-  // One group per weight row on rows whose length is no power of two (K = 11008, 5120, 3584 ...): only the oldest kernels take
-  // such a group (M = 64, N = 4096, K = 11008: 59 us against 23 us with groups of 128).  The row's scale / zero point is
-  // written out per power-of-two group into the tail of the workspace (one small launch) and the call goes on with that group.
-  // (not for the two passes by name: their dequantisation pass takes any group as it is)
-  if (M >= 1 && N >= 1 && N < kMaxDim && K >= 64 && K < kMaxDim && group == K && (K & (K - 1)) != 0 && K % 64 == 0 &&
-      algo != TLQ_ALGO_TWO_PASS && (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16)) {
-    const int64_t g_eff = row_group_for(K), groups = K / g_eff, tensor_bytes = row_group_tensor_bytes(N, K);
-    if (!scales && !zeros)  // no tensors: any group size says the same
-      return tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, C, M, N, K, g_eff, zero_scalar, in_dtype, out_dtype, algo, workspace, workspace_bytes, stream);
-    const int64_t tail = ((scales ? 1 : 0) + (zeros ? 1 : 0)) * tensor_bytes;
-    const int64_t head_bytes = (workspace_bytes - tail) & ~(int64_t)15;
-    if (workspace && aligned16(workspace) && workspace_bytes >= tail + 16 && ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0) {
-      uint8_t* const base = (uint8_t*)workspace + head_bytes;
-      const int64_t n_out = N * groups;
-      const int grid = (int)((n_out + 255) / 256 > 4096 ? 4096 : (n_out + 255) / 256);
-      const void* s_eff = scales;
-      const void* z_eff = zeros;
-      if (scales) {
-        expand_row_values_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)scales, (uint16_t*)base, n_out, (int)groups);
-        if (!check_launch("tlq_gemm_w4a16 (one scale per row, written out per group)", "expand_row_values_kernel")) return 1;
-        s_eff = base;
-      }
-      if (zeros) {
-        uint8_t* const zb = base + (scales ? tensor_bytes : 0);
-        expand_row_values_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)zeros, (uint16_t*)zb, n_out, (int)groups);
-        if (!check_launch("tlq_gemm_w4a16 (one zero point per row, written out per group)", "expand_row_values_kernel")) return 1;
-        z_eff = zb;
-      }
-      return tlq_gemm_w4a16_ws(A, w_packed, s_eff, z_eff, C, M, N, K, g_eff, zero_scalar, in_dtype, out_dtype, algo, workspace, head_bytes, stream);
-    }
+  if (algo != TLQ_ALGO_TWO_PASS) {  // (not for the two passes by name: their dequantisation pass takes any group as it is)
+    RowValues rv;
+    const int wrote = write_out_row_values(scales, zeros, M, N, K, group, in_dtype, workspace, workspace_bytes, stream, rv);
+    if (wrote < 0) return 1;
+    if (wrote > 0)
+      return tlq_gemm_w4a16_ws(A, w_packed, rv.scales, rv.zeros, C, M, N, K, rv.group, zero_scalar, in_dtype, out_dtype, algo, workspace, rv.workspace_bytes, stream);
   }
   if (algo == TLQ_ALGO_AUTO && M >= 1 && N >= 1) {
     // a tuned choice for this call signature goes first (as in tlq_gemm_w4a16); a kernel that refuses the call -- its shape
@@ -894,6 +909,14 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
   TLQ_REQUIRE(aligned16(A) && aligned16(w_packed) && aligned16(C), "tlq_gemm_w4a16_layout_ws: A, w_packed and C must be 16-byte aligned");
   TLQ_REQUIRE(((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0, "tlq_gemm_w4a16_layout_ws: scales / zeros misaligned");
   TLQ_REQUIRE(fits32(M, K * 2) && fits32(N, K / 2), "tlq_gemm_w4a16_layout_ws: a matrix spans 4 GiB or more");
+  if (algo != TLQ_ALGO_TWO_PASS) {  // one scale / zero point per row on rows that are no power of two: as for plain words
+    RowValues rv;
+    const int wrote = write_out_row_values(scales, zeros, M, N, K, group, in_dtype, workspace, workspace_bytes, stream, rv);
+    if (wrote < 0) return 1;
+    if (wrote > 0)
+      return tlq_gemm_w4a16_layout_ws(A, w_packed, rv.scales, rv.zeros, C, M, N, K, rv.group, zero_scalar, in_dtype, out_dtype, algo, w_layout, workspace,
+                                      rv.workspace_bytes, stream);
+  }
   const bool ws_aligned = workspace && aligned16(workspace);
   // one or two activation rows: the ring GEMV where the plain layout takes it too (one row; two fp16 rows on 8192 weight
   // rows or more), or when asked for by name
@@ -939,6 +962,10 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
     TLQ_REQUIRE(false, "tlq_gemm_w4a16_layout_ws: the panel kernel does not take M=%lld N=%lld K=%lld group=%lld with a "
                 "workspace of %lld bytes (K %% 128 == 0, M %% 4 == 0, N %% 16 == 0, a power-of-two group with (K / group) %% 8 == 0, 16-byte "
                 "aligned scale / zero tensors)", (long long)M, (long long)N, (long long)K, (long long)group, (long long)workspace_bytes);
+  }
+  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && panel_one_round(M, N, K)) {  // (65 .. 128 rows on output-layer widths, as for plain words)
+    const int rc = try_panel(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, workspace, workspace_bytes, stream);
+    if (rc >= 0) return rc;
   }
   if (algo != TLQ_ALGO_TWO_PASS) {
     const StreamPlan sp = w4a16_stream_plan(M, N, K, group, cu_count_or_default());
