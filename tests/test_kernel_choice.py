@@ -61,12 +61,13 @@ def cases():
         (192, 28672, 8192, 128, _abi.ALGO_STREAM),  # largest matrices at 192 rows: the streaming kernel (122 us against 154 us for the tile kernel over two long K slices)
         (224, 28672, 8192, 128, _abi.ALGO_PANELM),  # 196 .. 256 rows on wide or very large matrices: the middle-M panel kernel (two tiles of 128 rows)
         (256, 6144, 6144, 128, _abi.ALGO_STREAM),   # 256 rows on fewer than 56 million weights and fewer than 10240 outputs: the streaming kernel
+        (256, 14336, 4096, 512, _abi.ALGO_STREAM),  # groups of 512 values up to 256 rows: the panel kernels' windows of eight groups leave K uncut, the streaming kernel cuts inside a group
         (80, 81920, 1024, 128, _abi.ALGO_PANEL),    # 65 .. 128 rows on output-layer widths: 160 .. 256 work-groups of the 128-row panel kernel (512 weight rows each) in one round
         (256, 14336, 4096, 128, _abi.ALGO_PANELM),  # 257 .. 512 rows on 2^25 weights or more, 256 rows on 10240 outputs or more: the middle-M panel kernel
     ]
 
 
-@pytest.mark.parametrize("case", range(27))
+@pytest.mark.parametrize("case", range(28))
 def test_automatic_choice_returns_the_bits_of_the_kernel_it_is_meant_to_take(case):
     from tilelang_ascend_amd import _abi
 

@@ -743,7 +743,10 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     TLQ_REQUIRE(have, "tlq_gemm_w4a16_ws: the two-pass path needs a 16-byte aligned workspace of %lld bytes (got %lld)",
                 (long long)need, (long long)workspace_bytes);
   // 256 .. 512 activation rows on large matrices: the middle-M panel kernel
-  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && panelm_preferred(M, N, K) && group > 0) {
+  // (not up to 256 rows with groups of 512 values or more: the panel kernels cut K into windows of eight groups -- 32 steps and
+  // more -- and run uncut or nearly so, the streaming kernel cuts inside a group: N = 14336, K = 4096, M = 256: 50 against 59 us;
+  // N = 11008: 47 against 58 us; N = K = 8192: 52 against 61 us; from 384 rows on the panel kernels are ahead again)
+  if (algo == TLQ_ALGO_AUTO && !g_w4a16_panel && panelm_preferred(M, N, K) && group > 0 && !(M <= 256 && group >= 512)) {
     // (very wide matrices: where the 128-row tiles need a second round of work-groups and the 256-row tiles do not, the
     // 256-row kernel by the same estimate -- N = 28672, K = 4096, M = 512: 104 against 129 us)
     if (panel256_estimate_wins(M, N, K, group)) {
