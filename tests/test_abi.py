@@ -212,6 +212,12 @@ def test_workspace_size_rules():
         assert lib.tlq_f16_workspace_bytes(1, M, N, K) > 0
     assert ws(1024, 14336, 4096) == 14336 * 4096 * 2  # many output tiles already: no K slices, two passes
     assert ws(64, 0, 4096) == 0 and ws(64, 128, 0) == 0
+    # a weight-row count that is no multiple of four, more than 32 activation rows: what the multiple of 16 below asks for, then
+    # its packed result (sized for fp32 outputs)
+    a16 = lambda b: (b + 15) // 16 * 16  # noqa: E731
+    assert ws(100, 1001, 512) == a16(ws(100, 992, 512)) + a16(100 * 992 * 4)
+    assert ws(300, 50257, 4096) == a16(ws(300, 50256, 4096)) + a16(300 * 50256 * 4)
+    assert ws(32, 1001, 512) == ws(32, 1000, 512) and ws(100, 1004, 512) == 0
 
 
 def test_tuning_hooks_are_per_thread():

@@ -7,6 +7,8 @@ namespace tlq {
 int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t batch, int64_t M,
                int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 bool gemv_ring_applies(int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype, const void* scales, const void* zeros);
+int w4a16_tail_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t rows, int64_t K,
+                    int64_t group, float zero_scalar, int in_dtype, int out_dtype, int64_t ldc, int64_t col0, hipStream_t st);
 int gemv_w4a16_ring_interleaved(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                                 int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
@@ -116,6 +118,36 @@ __global__ __launch_bounds__(256) void expand_row_values_kernel(const uint16_t* 
                                                                 int groups) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_out; i += (int64_t)gridDim.x * blockDim.x) out[i] = in[i / groups];
 }
+// A matrix of `cols` columns (rows packed) into the first `cols` columns of a matrix whose rows lie `ldc` elements apart.
+template <typename E>
+__global__ __launch_bounds__(256) void copy_into_wider_rows_kernel(const E* __restrict__ in, E* __restrict__ out, int64_t M, int64_t cols, int64_t ldc) {
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  for (int64_t m = blockIdx.y; m < M; m += gridDim.y) out[m * ldc + c] = in[m * cols + c];
+}
+// The same for 16-bit elements, two at a time: pairs that are aligned in the OUTPUT (a row starts at element m * ldc, whose
+// parity moves the pairs by one column), one 4-byte store each; the first or last column of a row alone where a pair straddles it.
+__global__ __launch_bounds__(256) void copy_pairs_into_wider_rows_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, int64_t M,
+                                                                        int64_t cols, int64_t ldc) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (int64_t m = blockIdx.y; m < M; m += gridDim.y) {
+    const int64_t o = m * ldc;
+    const int64_t c0 = 2 * t - (o & 1);
+    if (c0 >= cols) continue;
+    const uint16_t* const src = in + m * cols;
+    if (c0 >= 0 && c0 + 1 < cols)
+      *(uint32_t*)(out + o + c0) = (uint32_t)src[c0] | ((uint32_t)src[c0 + 1] << 16);
+    else if (c0 >= 0)
+      out[o + c0] = src[c0];
+    else
+      out[o] = src[0];
+  }
+}
+// A weight-row count that is no multiple of four (vocabularies of 50257 or 32001 rows): the multiple of 16 below runs through the
+// usual choice into a packed result behind the workspace, which is then copied into C; the last rows go straight into C.
+static int64_t ragged_head(int64_t N) { return N & ~(int64_t)15; }
+static bool ragged_rows_apply(int64_t M, int64_t N) { return M > 32 && (N & 3) != 0 && N > 16 && M < tlq::kMaxDim && N < tlq::kMaxDim; }
+static int64_t ragged_result_bytes(int64_t M, int64_t N, int out_bytes) { return (M * ragged_head(N) * out_bytes + 15) / 16 * 16; }
 static int64_t row_group_for(int64_t K) {  // largest power of two dividing K, 1024 at most
   int64_t g = K & -K;
   return g > 1024 ? 1024 : g;
@@ -407,7 +439,9 @@ int64_t tlq_w4a16_workspace_bytes_for(int64_t M, int64_t N, int64_t K, int algo)
 static int64_t w4a16_kernel_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
-  const int64_t need = w4a16_kernel_workspace_bytes(M, N, K);
+  int64_t need = w4a16_kernel_workspace_bytes(M, N, K);
+  // (a weight-row count that is no multiple of four: what the multiple of 16 below asks for, then its packed result, sized for fp32)
+  if (ragged_rows_apply(M, N)) need = (w4a16_kernel_workspace_bytes(M, ragged_head(N), K) + 15) / 16 * 16 + ragged_result_bytes(M, N, 4);
   // (rows whose length is no power of two with one group per row: room behind everything else for the scales and zero points
   // written out per power-of-two group)
   if ((K & (K - 1)) != 0 && K % 64 == 0) return (need + 15) / 16 * 16 + 2 * row_group_tensor_bytes(N, K) + 16;
@@ -619,6 +653,32 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     if (wrote < 0) return 1;
     if (wrote > 0)
       return tlq_gemm_w4a16_ws(A, w_packed, rv.scales, rv.zeros, C, M, N, K, rv.group, zero_scalar, in_dtype, out_dtype, algo, workspace, rv.workspace_bytes, stream);
+  }
+  // A weight-row count that is no multiple of four, more than 32 activation rows: only the skinny kernel (up to 64 rows) takes it as
+  // it is (N = 32001, K = 4096, M = 64: 88 us against 42 us for N = 32000; more rows were refused).  With room behind the workspace
+  // for the packed result of the first N - N % 16 rows: those through the usual choice, a copy into C, the last rows straight into C.
+  if (algo == TLQ_ALGO_AUTO && ragged_rows_apply(M, N) && K > 0 && K % 64 == 0 && group > 0 && K % group == 0 && group % 32 == 0 && A && w_packed && C &&
+      (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) && (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) &&
+      ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0 && workspace && aligned16(workspace)) {
+    const int out_bytes = out_dtype == TLQ_F32 ? 4 : 2;
+    const int64_t head = ragged_head(N), result_bytes = ragged_result_bytes(M, N, out_bytes);
+    if (workspace_bytes >= result_bytes) {
+      const int64_t front = (workspace_bytes - result_bytes) & ~(int64_t)15;
+      uint8_t* const packed = (uint8_t*)workspace + front;
+      const int64_t groups = K / group;
+      if (int rc = tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, packed, M, head, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, workspace, front, stream)) return rc;
+      const dim3 grid((unsigned)ceil_div(head, (int64_t)256), (unsigned)(M > 4096 ? 4096 : M));
+      if (out_bytes == 4)
+        copy_into_wider_rows_kernel<uint32_t><<<grid, 256, 0, (hipStream_t)stream>>>((const uint32_t*)packed, (uint32_t*)C, M, head, N);
+      else
+        copy_pairs_into_wider_rows_kernel<<<dim3((unsigned)ceil_div(head / 2 + 1, (int64_t)256), grid.y), 256, 0, (hipStream_t)stream>>>(
+            (const uint16_t*)packed, (uint16_t*)C, M, head, N);
+      if (!check_launch("tlq_gemm_w4a16 (packed result into C)", out_bytes == 4 ? "copy_into_wider_rows_kernel" : "copy_pairs_into_wider_rows_kernel")) return 1;
+      const int eb = 2;  // scales and zero points: 16-bit values
+      return w4a16_tail_rows(A, (const uint8_t*)w_packed + head * (K / 2), scales ? (const uint8_t*)scales + head * groups * eb : nullptr,
+                             zeros ? (const uint8_t*)zeros + head * groups * eb : nullptr, C, M, N - head, K, group, zero_scalar, in_dtype, out_dtype, N, head,
+                             (hipStream_t)stream);
+    }
   }
   if (algo == TLQ_ALGO_AUTO && M >= 1 && N >= 1) {
     // a tuned choice for this call signature goes first (as in tlq_gemm_w4a16); a kernel that refuses the call -- its shape

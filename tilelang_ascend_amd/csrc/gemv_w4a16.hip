@@ -864,6 +864,56 @@ __global__ __launch_bounds__(256) void gemv_w4a16_kernel(const T* __restrict__ A
   }
 }
 
+// A few weight rows (the last N % 16 of a matrix whose row count is no multiple of 16) against ALL activation rows, written
+// into an output whose rows lie `ldc` elements apart, from column `col0` on: one wavefront per activation row, the generic
+// kernel's arithmetic (every weight dequantised as the reference rounds it, fp32 sums).
+template <typename T>
+__global__ __launch_bounds__(256) void w4a16_tail_rows_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
+                                                              const T* __restrict__ scales, const T* __restrict__ zeros,
+                                                              void* __restrict__ C, int M, int rows, int K, int group,
+                                                              float zero_scalar, int out_dtype, int64_t ldc, int64_t col0) {
+  typedef typename ActOf<T>::type Act;
+  const int lane = threadIdx.x & 63;
+  const int64_t m = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (m >= M) return;  // whole wavefront leaves together
+  const int chunks = K >> 5;
+  const int groups = K / group;
+  const int64_t row_bytes = K >> 1;
+  const T one = from_float<T>(1.0f);
+  const T zs = from_float<T>(zero_scalar);
+  for (int r = 0; r < rows; ++r) {
+    float acc = 0.f;
+    for (int c = lane; c < chunks; c += 64) {
+      const uint4_t w = *(const uint4_t*)(Wp + r * row_bytes + ((int64_t)c << 4));
+      const int g = (c << 5) / group;
+      const T s = scales ? scales[(int64_t)r * groups + g] : one;
+      const T z = zeros ? zeros[(int64_t)r * groups + g] : zs;
+      Act act;
+      load_act(act, A, m * K + ((int64_t)c << 5));
+      acc += chunk_term(w, act, s, z);
+    }
+    const float v = wave_sum(acc);
+    if (lane == 0) store_out(C, m * ldc + col0 + r, v, out_dtype);
+  }
+}
+
+// Wp, scales and zeros point at the first of the `rows` weight rows.
+int w4a16_tail_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t rows, int64_t K,
+                    int64_t group, float zero_scalar, int in_dtype, int out_dtype, int64_t ldc, int64_t col0, hipStream_t st) {
+  if (M < 1 || rows < 1 || rows > 64 || K < 32 || K % 32 != 0 || group < 1 || K % group != 0 || group % 32 != 0 || M > 0x7fffffff || K > 0x7fffffff) {
+    set_error("tlq_gemm_w4a16 (last weight rows): bad shape M=%lld rows=%lld K=%lld group=%lld", (long long)M, (long long)rows, (long long)K, (long long)group);
+    return 1;
+  }
+  const unsigned blocks = (unsigned)ceil_div(M, (int64_t)4);
+  if (in_dtype == TLQ_F16)
+    w4a16_tail_rows_kernel<half_t><<<blocks, 256, 0, st>>>((const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C,
+                                                           (int)M, (int)rows, (int)K, (int)group, zero_scalar, out_dtype, ldc, col0);
+  else
+    w4a16_tail_rows_kernel<bf16_t><<<blocks, 256, 0, st>>>((const bf16_t*)A, (const uint8_t*)Wp, (const bf16_t*)scales, (const bf16_t*)zeros, C,
+                                                           (int)M, (int)rows, (int)K, (int)group, zero_scalar, out_dtype, ldc, col0);
+  return check_launch("tlq_gemm_w4a16 (last weight rows)", "w4a16_tail_rows_kernel") ? 0 : 1;
+}
+
 template <typename T, int R, int MT>
 static void launch_gemv(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int batch, int M,
                         int N, int K, int group, float zero_scalar, int out_dtype, int waves_per_block, hipStream_t st) {
