@@ -188,7 +188,8 @@ int tlq_gemm_w4a16(const void* A, const void* w_packed, const void* scales, cons
  * power-of-two groups, so the per-row values are first written out per group of min(K & -K, 1024) values into the last
  * 2 * align16(N * K / group * 2) + 16 bytes of the workspace (tlq_w4a16_workspace_bytes counts them) and the call runs with
  * that group: bit for bit what a caller gets who replicates the values.  A smaller workspace: the call runs with group == K.
- * A weight-row count N that is no multiple of four (vocabularies of 50257 or 32001 rows) with more than 32 activation rows: the
+ * A weight-row count N that is no multiple of four (vocabularies of 50257 or 32001 rows) with more than 32 activation rows, or a
+ * multiple of four that is no multiple of eight with more than 512 (while the packed result stays below 1 GiB): the
  * first N - N % 16 weight rows run through the usual choice into a packed [M, N - N % 16] result kept in the last
  * align16(M * (N - N % 16) * sizeof(out)) bytes of the workspace, one launch copies it into C and one more computes the last
  * weight rows straight into C (tlq_w4a16_workspace_bytes counts that room, sized for fp32 outputs).  Without it such a count

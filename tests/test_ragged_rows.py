@@ -1,4 +1,5 @@
-"""Weight-row counts that are no multiple of four (vocabularies of 50257 or 32001 rows) with more than 32 activation rows:
+"""Weight-row counts that are no multiple of four (vocabularies of 50257 or 32001 rows) with more than 32 activation rows, and
+multiples of four that are no multiples of eight above 512 rows:
 tlq_gemm_w4a16_ws runs the first N - N % 16 rows through its usual choice into a packed result behind the workspace, copies
 that into C and computes the last rows straight into C.  The first columns must be, bit for bit, what the same call returns
 for those weight rows alone, and the whole must agree with the oracle (ref_program_fp16 extended by scales / zero points,
@@ -42,6 +43,7 @@ def run(A, Wp, s, z, group, out_dtype=None, workspace_bytes=None):
     (40, 1001, 512, 128, "int"), (64, 5001, 1024, 64, "frac"), (100, 1003, 512, 128, "scalar8"), (300, 2050, 1024, 128, "int"),
     (700, 1037, 2048, 128, None), (601, 1029, 1024, 32, "int"), (129, 8207, 256, 256, "frac"), (33, 31, 512, 128, "int"),
     (256, 4099, 1408, 1408, "int"),  # with one scale per row on rows that are no power of two as well
+    (600, 1036, 1024, 128, "int"), (1024, 4100, 512, 64, "scalar8"),  # a multiple of four that is no multiple of eight, above 512 rows
 ])
 def test_row_counts_that_are_no_multiple_of_four(in_dtype, out_dtype, M, N, K, group, zeros_kind):
     from tilelang_ascend_amd import _abi

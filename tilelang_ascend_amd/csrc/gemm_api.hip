@@ -146,8 +146,16 @@ __global__ __launch_bounds__(256) void copy_pairs_into_wider_rows_kernel(const u
 // A weight-row count that is no multiple of four (vocabularies of 50257 or 32001 rows): the multiple of 16 below runs through the
 // usual choice into a packed result behind the workspace, which is then copied into C; the last rows go straight into C.
 static int64_t ragged_head(int64_t N) { return N & ~(int64_t)15; }
-static bool ragged_rows_apply(int64_t M, int64_t N) { return M > 32 && (N & 3) != 0 && N > 16 && M < tlq::kMaxDim && N < tlq::kMaxDim; }
 static int64_t ragged_result_bytes(int64_t M, int64_t N, int out_bytes) { return (M * ragged_head(N) * out_bytes + 15) / 16 * 16; }
+// (Also a multiple of four that is no multiple of eight above 512 rows, where the panel kernels are the choice and want multiples
+// of 16 and the two passes multiples of eight, which leaves the tile kernel through registers: N = 4100, K = 4096, M = 1024 .. 4096:
+// 63 - 150 against 92 - 239 us; N = 32004: 228 - 1082 against 275 - 1135 us -- while the packed result stays below 1 GiB.  With
+// multiples of eight the two passes are level or ahead from 2048 rows on: N = 14344, M = 4096: 430 against 512 us.)
+static bool ragged_rows_apply(int64_t M, int64_t N) {
+  if (!(N > 16 && M < tlq::kMaxDim && N < tlq::kMaxDim)) return false;
+  if ((N & 3) != 0) return M > 32;
+  return (N & 7) != 0 && M > 512 && ragged_result_bytes(M, N, 4) <= ((int64_t)1 << 30);
+}
 static int64_t row_group_for(int64_t K) {  // largest power of two dividing K, 1024 at most
   int64_t g = K & -K;
   return g > 1024 ? 1024 : g;
