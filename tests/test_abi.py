@@ -218,6 +218,7 @@ def test_workspace_size_rules():
     assert ws(100, 1001, 512) == a16(ws(100, 992, 512)) + a16(100 * 992 * 4)
     assert ws(300, 50257, 4096) == a16(ws(300, 50256, 4096)) + a16(300 * 50256 * 4)
     assert ws(32, 1001, 512) == ws(32, 1000, 512) and ws(100, 1004, 512) == 0
+    assert ws(100, 7, 512) == 0 and ws(1000, 15, 4096) == 0  # fewer than 16 weight rows: the last-rows kernel alone, no packed result
     assert ws(600, 1036, 1024) == a16(ws(600, 1024, 1024)) + a16(600 * 1024 * 4)  # (above 512 rows: multiples of four that are no multiples of eight, too)
 
 

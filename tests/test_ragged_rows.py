@@ -43,7 +43,7 @@ def run(A, Wp, s, z, group, out_dtype=None, workspace_bytes=None):
     (40, 1001, 512, 128, "int"), (64, 5001, 1024, 64, "frac"), (100, 1003, 512, 128, "scalar8"), (300, 2050, 1024, 128, "int"),
     (700, 1037, 2048, 128, None), (601, 1029, 1024, 32, "int"), (129, 8207, 256, 256, "frac"), (33, 31, 512, 128, "int"),
     (256, 4099, 1408, 1408, "int"),  # with one scale per row on rows that are no power of two as well
-    (600, 1036, 1024, 128, "int"), (1024, 4100, 512, 64, "scalar8"),  # a multiple of four that is no multiple of eight, above 512 rows
+    (100, 7, 512, 128, "int"), (600, 1036, 1024, 128, "int"), (1024, 4100, 512, 64, "scalar8"),  # a multiple of four that is no multiple of eight, above 512 rows
 ])
 def test_row_counts_that_are_no_multiple_of_four(in_dtype, out_dtype, M, N, K, group, zeros_kind):
     from tilelang_ascend_amd import _abi
@@ -54,8 +54,11 @@ def test_row_counts_that_are_no_multiple_of_four(in_dtype, out_dtype, M, N, K, g
     rc, got = run(A, Wp, s, z, group, DT[out_dtype])
     assert rc == 0, _abi.last_error()
     log = run.log
-    assert "packed result into C" in log and "last weight rows" in log, log
     head = N - N % 16
+    assert ("packed result into C" in log or head == 0) and "last weight rows" in log, log
+    if head == 0:  # fewer than 16 weight rows: the last-rows kernel alone
+        check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"{N} weight rows")
+        return
     cut = lambda t: t[:head].contiguous() if torch.is_tensor(t) else t  # noqa: E731
     rc, first = run(A, Wp[:head].contiguous(), cut(s), cut(z), group, DT[out_dtype])
     assert rc == 0, _abi.last_error()

@@ -152,8 +152,9 @@ static int64_t ragged_result_bytes(int64_t M, int64_t N, int out_bytes) { return
 // 63 - 150 against 92 - 239 us; N = 32004: 228 - 1082 against 275 - 1135 us -- while the packed result stays below 1 GiB.  With
 // multiples of eight the two passes are level or ahead from 2048 rows on: N = 14344, M = 4096: 430 against 512 us.)
 static bool ragged_rows_apply(int64_t M, int64_t N) {
-  if (!(N > 16 && M < tlq::kMaxDim && N < tlq::kMaxDim)) return false;
-  if ((N & 3) != 0) return M > 32;
+  if (!(N >= 1 && M < tlq::kMaxDim && N < tlq::kMaxDim)) return false;
+  if ((N & 3) != 0) return M > 32;  // (fewer than 16 weight rows: the last-rows kernel alone)
+  if (N <= 16) return false;
   return (N & 7) != 0 && M > 512 && ragged_result_bytes(M, N, 4) <= ((int64_t)1 << 30);
 }
 static int64_t row_group_for(int64_t K) {  // largest power of two dividing K, 1024 at most
@@ -449,7 +450,7 @@ int64_t tlq_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (N <= 0 || K <= 0) return 0;
   int64_t need = w4a16_kernel_workspace_bytes(M, N, K);
   // (a weight-row count that is no multiple of four: what the multiple of 16 below asks for, then its packed result, sized for fp32)
-  if (ragged_rows_apply(M, N)) need = (w4a16_kernel_workspace_bytes(M, ragged_head(N), K) + 15) / 16 * 16 + ragged_result_bytes(M, N, 4);
+  if (ragged_rows_apply(M, N)) need = ragged_head(N) == 0 ? 0 : (w4a16_kernel_workspace_bytes(M, ragged_head(N), K) + 15) / 16 * 16 + ragged_result_bytes(M, N, 4);
   // (rows whose length is no power of two with one group per row: room behind everything else for the scales and zero points
   // written out per power-of-two group)
   if ((K & (K - 1)) != 0 && K % 64 == 0) return (need + 15) / 16 * 16 + 2 * row_group_tensor_bytes(N, K) + 16;
@@ -667,21 +668,23 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
   // for the packed result of the first N - N % 16 rows: those through the usual choice, a copy into C, the last rows straight into C.
   if (algo == TLQ_ALGO_AUTO && ragged_rows_apply(M, N) && K > 0 && K % 64 == 0 && group > 0 && K % group == 0 && group % 32 == 0 && A && w_packed && C &&
       (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) && (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) &&
-      ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0 && workspace && aligned16(workspace)) {
+      ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0 && aligned16(A) && aligned16(w_packed) && aligned16(C)) {
     const int out_bytes = out_dtype == TLQ_F32 ? 4 : 2;
     const int64_t head = ragged_head(N), result_bytes = ragged_result_bytes(M, N, out_bytes);
-    if (workspace_bytes >= result_bytes) {
-      const int64_t front = (workspace_bytes - result_bytes) & ~(int64_t)15;
+    if (head == 0 || (workspace && aligned16(workspace) && workspace_bytes >= result_bytes)) {
+      const int64_t front = head == 0 ? 0 : (workspace_bytes - result_bytes) & ~(int64_t)15;
       uint8_t* const packed = (uint8_t*)workspace + front;
       const int64_t groups = K / group;
-      if (int rc = tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, packed, M, head, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, workspace, front, stream)) return rc;
-      const dim3 grid((unsigned)ceil_div(head, (int64_t)256), (unsigned)(M > 4096 ? 4096 : M));
-      if (out_bytes == 4)
-        copy_into_wider_rows_kernel<uint32_t><<<grid, 256, 0, (hipStream_t)stream>>>((const uint32_t*)packed, (uint32_t*)C, M, head, N);
-      else
-        copy_pairs_into_wider_rows_kernel<<<dim3((unsigned)ceil_div(head / 2 + 1, (int64_t)256), grid.y), 256, 0, (hipStream_t)stream>>>(
-            (const uint16_t*)packed, (uint16_t*)C, M, head, N);
-      if (!check_launch("tlq_gemm_w4a16 (packed result into C)", out_bytes == 4 ? "copy_into_wider_rows_kernel" : "copy_pairs_into_wider_rows_kernel")) return 1;
+      if (head > 0) {
+        if (int rc = tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, packed, M, head, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, workspace, front, stream)) return rc;
+        const dim3 grid((unsigned)ceil_div(head, (int64_t)256), (unsigned)(M > 4096 ? 4096 : M));
+        if (out_bytes == 4)
+          copy_into_wider_rows_kernel<uint32_t><<<grid, 256, 0, (hipStream_t)stream>>>((const uint32_t*)packed, (uint32_t*)C, M, head, N);
+        else
+          copy_pairs_into_wider_rows_kernel<<<dim3((unsigned)ceil_div(head / 2 + 1, (int64_t)256), grid.y), 256, 0, (hipStream_t)stream>>>(
+              (const uint16_t*)packed, (uint16_t*)C, M, head, N);
+        if (!check_launch("tlq_gemm_w4a16 (packed result into C)", out_bytes == 4 ? "copy_into_wider_rows_kernel" : "copy_pairs_into_wider_rows_kernel")) return 1;
+      }
       const int eb = 2;  // scales and zero points: 16-bit values
       return w4a16_tail_rows(A, (const uint8_t*)w_packed + head * (K / 2), scales ? (const uint8_t*)scales + head * groups * eb : nullptr,
                              zeros ? (const uint8_t*)zeros + head * groups * eb : nullptr, C, M, N - head, K, group, zero_scalar, in_dtype, out_dtype, N, head,
