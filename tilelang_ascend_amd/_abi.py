@@ -110,6 +110,7 @@ SIGNATURES = {
 
 _lock = threading.Lock()
 _lib = None
+_build_failure = None
 
 
 def library_path() -> str:
@@ -132,9 +133,13 @@ def load():
         # lock, so concurrent processes compile once), or say so when that is impossible
         if path == _build.LIB_PATH and _build.is_stale():
             state = "not found" if not os.path.exists(path) else "older than the kernel sources"
+            global _build_failure
+            if _build_failure is not None:  # one attempt per process: sources that do not compile fail every caller at once
+                raise RuntimeError(f"libtlq.so at {path} is {state} and could not be built ({_build_failure})")
             try:
                 path = _build.build_library(force=False)
             except Exception as e:  # noqa: BLE001
+                _build_failure = e
                 raise RuntimeError(
                     f"libtlq.so at {path} is {state} and could not be built ({e}); "
                     "run `python -m tilelang_ascend_amd.build`"
