@@ -981,7 +981,9 @@ static RowsPlan plan_gemv_rows(int batch, int N, int K, int group_shift, int wav
   // more rows per work-group than LDS holds: an equal number of smaller work-groups for every CU instead of full ones and a
   // short last round (N = 28672, K = 8192, groups of 64: 312 work-groups of 92 rows on 256 CUs took 31.7 us, the same
   // matrix with groups of 128 -- 256 work-groups of 112 rows -- 23.3 us)
-  if (rpb > rpb_max) rpb = (int)ceil_div(N, (int64_t)blocks * ceil_div(rpb, rpb_max));
+  // (one problem per launch only: with many, the work-groups of all problems share the rounds, and full ones were faster --
+  // 24 problems of N = 11008, K = 4096: 94 us with 29 work-groups of 384 rows each, 104 us with 33 of 336)
+  if (rpb > rpb_max && batch == 1) rpb = (int)ceil_div(N, (int64_t)blocks * ceil_div(rpb, rpb_max));
   if (rpb < waves_per_block) rpb = waves_per_block;
   rpb = (rpb + 3) & ~3;  // keeps the zero-point block of LDS 16-byte aligned for any group count
   if (rpb > rpb_max) rpb = rpb_max;
