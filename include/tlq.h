@@ -213,7 +213,8 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
  * 16-bit values).  Other shapes are rejected.  Results are bit-identical to the plain layout on the same logical weights,
  * except for the GEMV, whose dot products pair neighbouring elements instead of elements four apart: there the two
  * layouts agree to the rounding of the fp32 sums (and bit for bit on one-hot activations).  One scale / zero point per row on
- * rows whose length is no power of two is written out per group into the workspace's tail as in tlq_gemm_w4a16_ws. */
+ * rows whose length is no power of two is written out per group into the workspace's tail as in tlq_gemm_w4a16_ws, and ragged
+ * weight-row counts run as the multiple of 16 below plus the last rows in the same way. */
 int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                              int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                              int w_layout, void* workspace, int64_t workspace_bytes, void* stream);

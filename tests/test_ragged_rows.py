@@ -81,3 +81,40 @@ def test_without_room_for_the_packed_result_the_call_answers_as_before():
     A = torch.randn(200, 512, generator=gen(1102)).half()
     rc, _ = run(A, Wp, s, z, 128, workspace_bytes=0)
     assert rc != 0 and "N" in _abi.last_error()
+
+
+@pytest.mark.parametrize("in_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K,group,zeros_kind", [(40, 1001, 512, 128, "int"), (300, 2050, 1024, 64, "frac"), (700, 1037, 2048, 128, "scalar8"), (100, 7, 512, 128, "int")])
+def test_interleaved_words_with_ragged_row_counts(in_dtype, M, N, K, group, zeros_kind):
+    """tlq_gemm_w4a16_layout_ws takes the same route for words repacked by interleave_weight: against the oracle, and the last
+    columns (the last-rows kernel puts each word back in plain order) bit for bit those of the plain layout."""
+    from oracle import ref
+    from tilelang_ascend_amd import _abi
+
+    lib, P = _abi.load(), _abi.ptr
+    dt = DT[in_dtype]
+    A = torch.randn(M, K, generator=gen(1200 + M)).to(dt)
+    Wp, s, z = make_w4(N, K, group, dt, zeros_kind, seed=1201 + M)
+    rc, plain = run(A, Wp, s, z, group)
+    assert rc == 0, _abi.last_error()
+    Wi = ref.interleave_weight(Wp.view(torch.int8), 4, "float16").view(torch.uint8).contiguous()
+    zt = z if torch.is_tensor(z) else None
+    zs = 0.0 if (torch.is_tensor(z) or z is None) else float(z)
+    dA, dW, dS = A.cuda(), Wi.cuda(), s.cuda()
+    dZ = zt.cuda() if zt is not None else None
+    need = max(lib.tlq_w4a16_workspace_bytes(M, N, K), 16)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    C = torch.full((M, N), float("nan"), dtype=dt, device="cuda")
+    print(f"ragged rows, interleaved words M={M} N={N} K={K} g={group} {in_dtype} workspace={need}", flush=True)
+    lib.tlq_debug_launch_log(1)
+    rc = lib.tlq_gemm_w4a16_layout_ws(P(dA), P(dW), P(dS), P(dZ), P(C), M, N, K, group, zs, CODE[dt], CODE[dt], _abi.ALGO_AUTO,
+                                      _abi.W_INTERLEAVED_F16, P(ws), need, torch.cuda.current_stream().cuda_stream)
+    log = lib.tlq_debug_launch_log_text().decode()
+    lib.tlq_debug_launch_log(0)
+    torch.cuda.synchronize()
+    assert rc == 0, _abi.last_error()
+    assert "last weight rows" in log, log
+    got = C.cpu()
+    head = N - N % 16
+    assert_bit_equal(got[:, head:].contiguous(), plain[:, head:].contiguous(), f"columns {head} .. {N - 1}")
+    check_float_output(got, w4a16_reference(A, Wp, s, z, group), f"interleaved, ragged {M}x{N}x{K} {in_dtype}")

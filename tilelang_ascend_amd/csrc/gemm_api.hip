@@ -8,7 +8,7 @@ int gemv_w4a16(const void* A, const void* Wp, const void* scales, const void* ze
                int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 bool gemv_ring_applies(int64_t M, int64_t N, int64_t K, int64_t group, int in_dtype, const void* scales, const void* zeros);
 int w4a16_tail_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t rows, int64_t K,
-                    int64_t group, float zero_scalar, int in_dtype, int out_dtype, int64_t ldc, int64_t col0, hipStream_t st);
+                    int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, int64_t ldc, int64_t col0, hipStream_t st);
 int gemv_w4a16_ring_interleaved(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
                                 int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, hipStream_t st);
 int gemm_w4a16_mfma(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t N,
@@ -652,6 +652,43 @@ static int write_out_row_values(const void* scales, const void* zeros, int64_t M
   return 1;
 }
 
+// A weight-row count that is no multiple of four, more than 32 activation rows: only the skinny kernel (up to 64 rows) takes it as
+// it is (N = 32001, K = 4096, M = 64: 88 us against 42 us for N = 32000; more rows were refused).  With room behind the workspace
+// for the packed result of the first N - N % 16 rows: those through the usual choice, a copy into C, the last rows straight into C.
+// `taken` says whether the call was answered here (the return value is then its result).
+static int run_ragged_rows(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M, int64_t N, int64_t K,
+                           int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, void* workspace, int64_t workspace_bytes,
+                           void* stream, bool& taken) {
+  taken = false;
+  if (!(ragged_rows_apply(M, N) && K > 0 && K % 64 == 0 && group > 0 && K % group == 0 && group % 32 == 0 && A && w_packed && C &&
+        (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) && (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) &&
+        ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0 && aligned16(A) && aligned16(w_packed) && aligned16(C)))
+    return 0;
+  const int out_bytes = out_dtype == TLQ_F32 ? 4 : 2;
+  const int64_t head = ragged_head(N), result_bytes = ragged_result_bytes(M, N, out_bytes);
+  if (!(head == 0 || (workspace && aligned16(workspace) && workspace_bytes >= result_bytes))) return 0;
+  taken = true;
+  const int64_t front = head == 0 ? 0 : (workspace_bytes - result_bytes) & ~(int64_t)15;
+  uint8_t* const packed = (uint8_t*)workspace + front;
+  const int64_t groups = K / group;
+  if (head > 0) {
+    if (int rc = tlq_gemm_w4a16_layout_ws(A, w_packed, scales, zeros, packed, M, head, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, w_layout,
+                                          workspace, front, stream))
+      return rc;
+    const dim3 grid((unsigned)ceil_div(head, (int64_t)256), (unsigned)(M > 4096 ? 4096 : M));
+    if (out_bytes == 4)
+      copy_into_wider_rows_kernel<uint32_t><<<grid, 256, 0, (hipStream_t)stream>>>((const uint32_t*)packed, (uint32_t*)C, M, head, N);
+    else
+      copy_pairs_into_wider_rows_kernel<<<dim3((unsigned)ceil_div(head / 2 + 1, (int64_t)256), grid.y), 256, 0, (hipStream_t)stream>>>(
+          (const uint16_t*)packed, (uint16_t*)C, M, head, N);
+    if (!check_launch("tlq_gemm_w4a16 (packed result into C)", out_bytes == 4 ? "copy_into_wider_rows_kernel" : "copy_pairs_into_wider_rows_kernel")) return 1;
+  }
+  const int eb = 2;  // scales and zero points: 16-bit values
+  return w4a16_tail_rows(A, (const uint8_t*)w_packed + head * (K / 2), scales ? (const uint8_t*)scales + head * groups * eb : nullptr,
+                         zeros ? (const uint8_t*)zeros + head * groups * eb : nullptr, C, M, N - head, K, group, zero_scalar, in_dtype, out_dtype, w_layout, N,
+                         head, (hipStream_t)stream);
+}
+
 int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, const void* zeros, void* C, int64_t M,
                       int64_t N, int64_t K, int64_t group, float zero_scalar, int in_dtype, int out_dtype, int algo,
                       void* workspace, int64_t workspace_bytes, void* stream) {
@@ -663,33 +700,10 @@ int tlq_gemm_w4a16_ws(const void* A, const void* w_packed, const void* scales, c
     if (wrote > 0)
       return tlq_gemm_w4a16_ws(A, w_packed, rv.scales, rv.zeros, C, M, N, K, rv.group, zero_scalar, in_dtype, out_dtype, algo, workspace, rv.workspace_bytes, stream);
   }
-  // A weight-row count that is no multiple of four, more than 32 activation rows: only the skinny kernel (up to 64 rows) takes it as
-  // it is (N = 32001, K = 4096, M = 64: 88 us against 42 us for N = 32000; more rows were refused).  With room behind the workspace
-  // for the packed result of the first N - N % 16 rows: those through the usual choice, a copy into C, the last rows straight into C.
-  if (algo == TLQ_ALGO_AUTO && ragged_rows_apply(M, N) && K > 0 && K % 64 == 0 && group > 0 && K % group == 0 && group % 32 == 0 && A && w_packed && C &&
-      (in_dtype == TLQ_F16 || in_dtype == TLQ_BF16) && (out_dtype == TLQ_F16 || out_dtype == TLQ_BF16 || out_dtype == TLQ_F32) &&
-      ((uintptr_t)scales & 1) == 0 && ((uintptr_t)zeros & 1) == 0 && aligned16(A) && aligned16(w_packed) && aligned16(C)) {
-    const int out_bytes = out_dtype == TLQ_F32 ? 4 : 2;
-    const int64_t head = ragged_head(N), result_bytes = ragged_result_bytes(M, N, out_bytes);
-    if (head == 0 || (workspace && aligned16(workspace) && workspace_bytes >= result_bytes)) {
-      const int64_t front = head == 0 ? 0 : (workspace_bytes - result_bytes) & ~(int64_t)15;
-      uint8_t* const packed = (uint8_t*)workspace + front;
-      const int64_t groups = K / group;
-      if (head > 0) {
-        if (int rc = tlq_gemm_w4a16_ws(A, w_packed, scales, zeros, packed, M, head, K, group, zero_scalar, in_dtype, out_dtype, TLQ_ALGO_AUTO, workspace, front, stream)) return rc;
-        const dim3 grid((unsigned)ceil_div(head, (int64_t)256), (unsigned)(M > 4096 ? 4096 : M));
-        if (out_bytes == 4)
-          copy_into_wider_rows_kernel<uint32_t><<<grid, 256, 0, (hipStream_t)stream>>>((const uint32_t*)packed, (uint32_t*)C, M, head, N);
-        else
-          copy_pairs_into_wider_rows_kernel<<<dim3((unsigned)ceil_div(head / 2 + 1, (int64_t)256), grid.y), 256, 0, (hipStream_t)stream>>>(
-              (const uint16_t*)packed, (uint16_t*)C, M, head, N);
-        if (!check_launch("tlq_gemm_w4a16 (packed result into C)", out_bytes == 4 ? "copy_into_wider_rows_kernel" : "copy_pairs_into_wider_rows_kernel")) return 1;
-      }
-      const int eb = 2;  // scales and zero points: 16-bit values
-      return w4a16_tail_rows(A, (const uint8_t*)w_packed + head * (K / 2), scales ? (const uint8_t*)scales + head * groups * eb : nullptr,
-                             zeros ? (const uint8_t*)zeros + head * groups * eb : nullptr, C, M, N - head, K, group, zero_scalar, in_dtype, out_dtype, N, head,
-                             (hipStream_t)stream);
-    }
+  if (algo == TLQ_ALGO_AUTO) {
+    bool taken = false;
+    const int rc = run_ragged_rows(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, TLQ_W_PLAIN, workspace, workspace_bytes, stream, taken);
+    if (taken) return rc;
   }
   if (algo == TLQ_ALGO_AUTO && M >= 1 && N >= 1) {
     // a tuned choice for this call signature goes first (as in tlq_gemm_w4a16); a kernel that refuses the call -- its shape
@@ -990,6 +1004,11 @@ int tlq_gemm_w4a16_layout_ws(const void* A, const void* w_packed, const void* sc
     if (wrote > 0)
       return tlq_gemm_w4a16_layout_ws(A, w_packed, rv.scales, rv.zeros, C, M, N, K, rv.group, zero_scalar, in_dtype, out_dtype, algo, w_layout, workspace,
                                       rv.workspace_bytes, stream);
+  }
+  if (algo == TLQ_ALGO_AUTO) {  // ragged weight-row counts: as for plain words
+    bool taken = false;
+    const int rc = run_ragged_rows(A, w_packed, scales, zeros, C, M, N, K, group, zero_scalar, in_dtype, out_dtype, w_layout, workspace, workspace_bytes, stream, taken);
+    if (taken) return rc;
   }
   const bool ws_aligned = workspace && aligned16(workspace);
   // one or two activation rows: the ring GEMV where the plain layout takes it too (one row; two fp16 rows on 8192 weight

@@ -867,7 +867,14 @@ __global__ __launch_bounds__(256) void gemv_w4a16_kernel(const T* __restrict__ A
 // A few weight rows (the last N % 16 of a matrix whose row count is no multiple of 16) against ALL activation rows, written
 // into an output whose rows lie `ldc` elements apart, from column `col0` on: one wavefront per activation row, the generic
 // kernel's arithmetic (every weight dequantised as the reference rounds it, fp32 sums).
-template <typename T>
+// A 32-bit word of interleave_weight's float16 layout (field j holds element (0, 2, 4, 6, 1, 3, 5, 7)[j]) back in plain order.
+__device__ __forceinline__ uint32_t plain_word_of_interleaved(uint32_t v) {
+  const uint32_t lo = v & 0xffffu, hi = v >> 16;  // even elements | odd elements
+  const uint32_t even = ((lo & 0xf000u) << 12) | ((lo & 0x0f00u) << 8) | ((lo & 0x00f0u) << 4) | (lo & 0x000fu);
+  const uint32_t odd = ((hi & 0xf000u) << 12) | ((hi & 0x0f00u) << 8) | ((hi & 0x00f0u) << 4) | (hi & 0x000fu);
+  return even | (odd << 4);
+}
+template <typename T, int LAYOUT>
 __global__ __launch_bounds__(256) void w4a16_tail_rows_kernel(const T* __restrict__ A, const uint8_t* __restrict__ Wp,
                                                               const T* __restrict__ scales, const T* __restrict__ zeros,
                                                               void* __restrict__ C, int M, int rows, int K, int group,
@@ -884,7 +891,8 @@ __global__ __launch_bounds__(256) void w4a16_tail_rows_kernel(const T* __restric
   for (int r = 0; r < rows; ++r) {
     float acc = 0.f;
     for (int c = lane; c < chunks; c += 64) {
-      const uint4_t w = *(const uint4_t*)(Wp + r * row_bytes + ((int64_t)c << 4));
+      uint4_t w = *(const uint4_t*)(Wp + r * row_bytes + ((int64_t)c << 4));
+      if constexpr (LAYOUT == 1) w = uint4_t{plain_word_of_interleaved(w.x), plain_word_of_interleaved(w.y), plain_word_of_interleaved(w.z), plain_word_of_interleaved(w.w)};
       const int g = (c << 5) / group;
       const T s = scales ? scales[(int64_t)r * groups + g] : one;
       const T z = zeros ? zeros[(int64_t)r * groups + g] : zs;
@@ -899,18 +907,23 @@ __global__ __launch_bounds__(256) void w4a16_tail_rows_kernel(const T* __restric
 
 // Wp, scales and zeros point at the first of the `rows` weight rows.
 int w4a16_tail_rows(const void* A, const void* Wp, const void* scales, const void* zeros, void* C, int64_t M, int64_t rows, int64_t K,
-                    int64_t group, float zero_scalar, int in_dtype, int out_dtype, int64_t ldc, int64_t col0, hipStream_t st) {
+                    int64_t group, float zero_scalar, int in_dtype, int out_dtype, int w_layout, int64_t ldc, int64_t col0, hipStream_t st) {
   if (M < 1 || rows < 1 || rows > 64 || K < 32 || K % 32 != 0 || group < 1 || K % group != 0 || group % 32 != 0 || M > 0x7fffffff || K > 0x7fffffff) {
     set_error("tlq_gemm_w4a16 (last weight rows): bad shape M=%lld rows=%lld K=%lld group=%lld", (long long)M, (long long)rows, (long long)K, (long long)group);
     return 1;
   }
   const unsigned blocks = (unsigned)ceil_div(M, (int64_t)4);
-  if (in_dtype == TLQ_F16)
-    w4a16_tail_rows_kernel<half_t><<<blocks, 256, 0, st>>>((const half_t*)A, (const uint8_t*)Wp, (const half_t*)scales, (const half_t*)zeros, C,
-                                                           (int)M, (int)rows, (int)K, (int)group, zero_scalar, out_dtype, ldc, col0);
-  else
-    w4a16_tail_rows_kernel<bf16_t><<<blocks, 256, 0, st>>>((const bf16_t*)A, (const uint8_t*)Wp, (const bf16_t*)scales, (const bf16_t*)zeros, C,
-                                                           (int)M, (int)rows, (int)K, (int)group, zero_scalar, out_dtype, ldc, col0);
+#define TLQ_TAIL_CASE(TT, LL)                                                                                                        \
+  w4a16_tail_rows_kernel<TT, LL><<<blocks, 256, 0, st>>>((const TT*)A, (const uint8_t*)Wp, (const TT*)scales, (const TT*)zeros, C, (int)M, \
+                                                         (int)rows, (int)K, (int)group, zero_scalar, out_dtype, ldc, col0)
+  if (in_dtype == TLQ_F16) {
+    if (w_layout == TLQ_W_PLAIN) TLQ_TAIL_CASE(half_t, 0);
+    else TLQ_TAIL_CASE(half_t, 1);
+  } else {
+    if (w_layout == TLQ_W_PLAIN) TLQ_TAIL_CASE(bf16_t, 0);
+    else TLQ_TAIL_CASE(bf16_t, 1);
+  }
+#undef TLQ_TAIL_CASE
   return check_launch("tlq_gemm_w4a16 (last weight rows)", "w4a16_tail_rows_kernel") ? 0 : 1;
 }
 
